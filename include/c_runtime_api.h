@@ -1,0 +1,258 @@
+/*
+ * C ABI of libc_runtime_api.so for MI355X (gfx950).
+ *
+ * Drop-in for the GPU operator layer of Athena/TSplit: every entry point below
+ * has the name, argument order and argument meaning of the symbol the
+ * reference's ctypes layer binds (python/athena/gpu_links/<Op>Link.py ->
+ * _LIB.<symbol>), as declared in the reference's src/common/c_runtime_api.h
+ * (cited per declaration as "ref:").  Where the reference's header and its
+ * implementation disagree, the implementation -- i.e. what its Python call
+ * sites really pass -- wins, and the comment says so.
+ *
+ * Conventions (ref: src/common/dlarray.h:22-63, src/common/runtime_base.h:13-47):
+ *  - every tensor is dense, C-contiguous float32; 4-D tensors are NCHW, filters OIHW;
+ *  - a DLStreamHandle of NULL means the default stream; all operator calls are
+ *    asynchronous on their stream unless a non-NULL ProfilerHandle is given, in
+ *    which case the call blocks and fills the Profiler (time in ms, sizes in MiB);
+ *  - return 0 on success, -1 on failure (a message goes to stderr).
+ */
+#ifndef TSPLIT_AMD_C_RUNTIME_API_H_
+#define TSPLIT_AMD_C_RUNTIME_API_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#else
+#include <stdbool.h>
+#endif
+
+/* ---- types (ref: src/common/dlarray.h:22-63, src/common/profiler.h:13-22) ---- */
+typedef enum { kCPU = 1, kGPU = 2 } DLDeviceType;
+
+typedef struct {
+  int device_id;
+  DLDeviceType device_type;
+} DLContext;
+
+typedef struct {
+  void *data;       /* device (kGPU) or host (kCPU) pointer; never owned by a micro-tensor view */
+  DLContext ctx;
+  int ndim;
+  int64_t *shape;
+} DLArray;          /* 32 bytes */
+
+typedef struct {
+  int device_id;
+  void *handle;     /* points to a heap hipStream_t */
+} DLStream;
+
+typedef struct {
+  int device_id;
+  void *handle;     /* points to a heap hipEvent_t */
+} DLEvent;
+
+typedef struct Profiler {
+  float time;              /* ms */
+  float input_memory;      /* MiB */
+  float output_memory;     /* MiB */
+  float workspace_memory;  /* MiB */
+} Profiler;
+
+typedef int64_t index_t;
+typedef DLArray *DLArrayHandle;
+typedef DLStream *DLStreamHandle;
+typedef DLEvent *DLEventHandle;
+typedef Profiler *ProfilerHandle;
+
+/* ---- runtime: profiler, streams, events (ref: c_runtime_api.h:33-52; impl
+ *      src/common/c_runtime_api.cc:110-115, src/cuda_common/gpu_runtime.cc:64-126) ---- */
+int ProfilerAlloc(ProfilerHandle *handle);            /* fields start at -1 */
+int DLStreamCreate(size_t dev_id, DLStreamHandle *handle);
+int DLStreamDestroy(DLStreamHandle handle);
+int DLStreamSync(DLStreamHandle handle);
+int DLEventCreate(size_t dev_id, DLEventHandle *handle);
+int DLEventDestroy(DLEventHandle handle);
+int DLEventRecord(DLStreamHandle stream_handle, DLEventHandle event_handle);
+int DLEventSync(DLEventHandle handle);
+/* ref declares `bool`; the ctypes caller reads an int, so a clean 0/1 int is exported. */
+int DLEventQuery(DLEventHandle handle);
+
+/* ---- runtime: library-handle hooks.  The reference creates cuDNN/cuBLAS/cuSPARSE
+ *      handles here (gpu_runtime.h:100-105, gpu_runtime.cc:13-62); this library has
+ *      no such handles, the calls only select the device. ---- */
+void cudnn_init(size_t dev_id, DLStreamHandle stream);
+void cublas_init(size_t dev_id, DLStreamHandle stream);
+void cusp_init(size_t dev_id, DLStreamHandle stream);
+void cuda_init(void);
+
+/* ---- runtime: pooled allocator introspection (ref: c_runtime_api.h:49-51; impl
+ *      c_runtime_api.cc:308-347 over src/cuda_common/gpu_memory_manager.cc:201-318) ---- */
+void DLMemoryManager_PrintState(void *t, int type);   /* *(int*)t = number of free chunks; type!=0 prints */
+void DLMemoryManager_Try_to_Malloc(size_t memory_size, void *p);  /* *(int*)p = 1 if it would succeed */
+void DLMemoryManager_GPU_Usage(size_t *used_size, size_t *unused_unavailable_size,
+                               size_t *unused_available_size);
+
+/* ---- runtime: arrays (ref: c_runtime_api.h:64-106; impl c_runtime_api.cc:137-306).
+ *      MEMORY_MANAGE_RULE 0 = raw device malloc/free per tensor, != 0 = pool. ---- */
+int DLArrayAlloc(const index_t *shape, index_t ndim, DLContext ctx, DLArrayHandle *out,
+                 int MEMORY_MANAGE_RULE);
+int DLArrayAllocSelf(DLArrayHandle handle, int MEMORY_MANAGE_RULE);
+int DLArrayFree(DLArrayHandle handle, int MEMORY_MANAGE_RULE);
+int DLArrayFreeSelf(DLArrayHandle handle, int MEMORY_MANAGE_RULE);
+int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream);
+/* One allocation holding an output (at the base) and an input (flush with the end) that
+ * overlap by `overlap_pieces` of the input's `pieces` micro-tensors (impl c_runtime_api.cc:164-210). */
+int DLArrayReuseAlloc(DLContext ctx, int MEMORY_MANAGE_RULE, const index_t *input_shape,
+                      index_t input_ndim, DLArrayHandle *input, const index_t *output_shape,
+                      index_t output_ndim, DLArrayHandle *output, int pieces, int overlap_pieces);
+/* Zero-copy view of micro-tensor `index` of `total_number` along dimension 0 (batch) or 1
+ * (impl c_runtime_api.cc:212-271).  The view owns its DLArray and shape, not the data. */
+int DLArraySliceForMicroTensor(DLArrayHandle input, DLArrayHandle *output, int total_number,
+                               int index, int dimension);
+
+/* ---- graph-closure elementwise ops (ref: c_runtime_api.h:115,140-141,151-152,162-163,
+ *      173-174,342; impl src/ops/ArraySet.cu:9, AddElewise.cu:9, AddConst.cu:9,
+ *      MultiplyElewise.cu:9, MultiplyConst.cu:9, Reshape.cu:5) ---- */
+int DLGpuArraySet(DLArrayHandle arr, float value, DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuMatrixElementwiseAdd(const DLArrayHandle matA, const DLArrayHandle matB,
+                              DLArrayHandle output, DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuMatrixElementwiseAddByConst(const DLArrayHandle input, float val, DLArrayHandle output,
+                                     DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuMatrixElementwiseMultiply(const DLArrayHandle matA, const DLArrayHandle matB,
+                                   DLArrayHandle output, DLStreamHandle stream_handle,
+                                   ProfilerHandle p);
+int DLGpuMatrixMultiplyByConst(const DLArrayHandle input, float val, DLArrayHandle output,
+                               DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuReshape(const DLArrayHandle in_arr, DLArrayHandle out_arr, DLStreamHandle stream_handle,
+                 ProfilerHandle p);
+
+/* ---- Relu (ref: c_runtime_api.h:234,243-244; impl src/ops/Relu.cu:9,82).
+ *      Gradient is (sign(x)+1)*0.5*dy, i.e. 0.5*dy at x == 0. ---- */
+int DLGpuRelu(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle,
+              ProfilerHandle p);
+int DLGpuReluGradient(const DLArrayHandle input, const DLArrayHandle in_grad, DLArrayHandle output,
+                      DLStreamHandle stream_handle, ProfilerHandle p);
+
+/* ---- MatMul (ref: c_runtime_api.h:207-209; impl src/ops/MatrixMult.cu:4-72).
+ *      Row-major 2-D C = op(A) op(B). ---- */
+int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, const DLArrayHandle matB,
+                        bool transposeB, DLArrayHandle matC, DLStreamHandle stream_handle,
+                        ProfilerHandle p);
+
+/* ---- Softmax / SoftmaxCrossEntropy (ref: c_runtime_api.h:272,288-294; impl
+ *      src/ops/Softmax.cu:24, src/ops/SoftmaxCrossEntropy.cu:44,106).  Rows = product of
+ *      all but the last dimension; loss has one element = mean over rows; the gradient
+ *      is (softmax(a) - b) * c[0] / a.shape[0]. ---- */
+int DLGpuSoftmax(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle,
+                 ProfilerHandle p);
+int DLGpuSoftmaxCrossEntropy(const DLArrayHandle input_a, const DLArrayHandle input_b,
+                             DLArrayHandle output, DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuSoftmaxCrossEntropy_Gradient(const DLArrayHandle input_a, const DLArrayHandle input_b,
+                                      const DLArrayHandle input_c, DLArrayHandle output,
+                                      DLStreamHandle stream_handle, ProfilerHandle p);
+
+/* ---- Conv2d, cross-correlation, no bias, square stride, dilation 1.
+ *      `CuDNN_` symbols (ref: c_runtime_api.h:348-352; impl src/ops/CudnnConv2d.cu:6,207,410)
+ *      take (pad_h, pad_w, stride); they are the ones the graph ops call
+ *      (python/athena/gpu_ops/Conv2d.py:116-118).  Output/gradient shapes are taken from
+ *      the pre-allocated output array. ---- */
+int CuDNN_DLGpuConv2d(const DLArrayHandle input_x, const DLArrayHandle input_f,
+                      DLArrayHandle output, const int padding, const int padding2,
+                      const int stride, DLStreamHandle stream_handle, ProfilerHandle p);
+int CuDNN_DLGpuConv2d_Gradient_of_Filter(const DLArrayHandle input_x,
+                                         const DLArrayHandle gradient_y, DLArrayHandle gradient_f,
+                                         const int padding, const int padding2, const int stride,
+                                         DLStreamHandle stream_handle, ProfilerHandle p);
+int CuDNN_DLGpuConv2d_Gradient_of_Data(const DLArrayHandle input_f, const DLArrayHandle gradient_y,
+                                       DLArrayHandle gradient_x, const int padding,
+                                       const int padding2, const int stride,
+                                       DLStreamHandle stream_handle, ProfilerHandle p);
+/*      Plain symbols: the reference header lists (padding1, padding2)
+ *      (c_runtime_api.h:296-304) but its implementation and Python call sites pass ONE
+ *      padding int (src/ops/Conv2d.cu:52,172,241; gpu_links/Conv2dLink.py:13-14,31-32,40-41):
+ *      the implementation's signature is exported.  The caller-provided im2col workspaces
+ *      are accepted and left untouched (the implicit-GEMM kernels need none). */
+int DLGpuConv2d(const DLArrayHandle input_x, const DLArrayHandle input_f, DLArrayHandle output,
+                DLArrayHandle workspace_arr, const int padding, const int stride,
+                DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuConv2d_Gradient_of_Data(const DLArrayHandle input_f, const DLArrayHandle gradient_y,
+                                 DLArrayHandle gradient_x, DLArrayHandle workspace_im2col,
+                                 const int padding, const int stride,
+                                 DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuConv2d_Gradient_of_Filter(const DLArrayHandle input_x, const DLArrayHandle gradient_y,
+                                   DLArrayHandle gradient_f, DLArrayHandle workspace_im2col,
+                                   DLArrayHandle workspace_batch_filter, const int padding,
+                                   const int stride, DLStreamHandle stream_handle,
+                                   ProfilerHandle p);
+
+/* ---- BatchNorm, training mode, spatial, biased batch variance (ref: c_runtime_api.h:371-376;
+ *      impl src/ops/CudnnBn.cu:12,212).  scale/bias/dscale/dbias/save_* hold C elements.
+ *      save_mean_arr / save_var_arr may be NULL; when given, forward writes (batch mean,
+ *      1/sqrt(var+eps)) and the gradient reads them instead of recomputing (the cuDNN
+ *      convention the reference relies on).  `momentum` is accepted and unused: the
+ *      reference computes running statistics into throw-away scratch (CudnnBn.cu:164-176). ---- */
+int CuDNN_DLGpuBatch_Normalization(const DLArrayHandle input_X, const DLArrayHandle bn_scale,
+                                   const DLArrayHandle bn_bias, DLArrayHandle output_Y,
+                                   float momentum, float eps, DLArrayHandle save_mean_arr,
+                                   DLArrayHandle save_var_arr, DLStreamHandle stream_handle,
+                                   ProfilerHandle p);
+int CuDNN_DLGpuBatch_Normalization_gradient(const DLArrayHandle gradient_Y,
+                                            const DLArrayHandle input_X,
+                                            const DLArrayHandle bn_scale, DLArrayHandle gradient_X,
+                                            DLArrayHandle gradient_bn_scale,
+                                            DLArrayHandle gradient_bn_bias, float eps,
+                                            DLArrayHandle save_mean_arr,
+                                            DLArrayHandle save_var_arr,
+                                            DLStreamHandle stream_handle, ProfilerHandle p);
+
+/* ---- MaxPool (ref: c_runtime_api.h:334-338,366-368; impl src/ops/MaxPool.cu:45,138,
+ *      src/ops/CudnnMaxPool.cu:3,103).  Windows are clipped to the image; the maximum is the
+ *      first strict maximum in row-major scan; the gradient accumulates in window order and
+ *      zero-fills the rest of gradient_X itself.  Note the differing argument orders and
+ *      integer types of the two families. ---- */
+int DLGpuMax_Pooling2d(const DLArrayHandle input, const int kernel_H, const int kernel_W,
+                       DLArrayHandle output, const int padding, const int stride,
+                       DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuMax_Pooling2d_gradient(const DLArrayHandle input, const DLArrayHandle output_grad,
+                                const int kernel_H, const int kernel_W, DLArrayHandle input_grad,
+                                const int padding, const int stride, DLStreamHandle stream_handle,
+                                ProfilerHandle p);
+int CuDNN_DLGpuMax_Pooling2d(const DLArrayHandle input, const size_t kernel_H,
+                             const size_t kernel_W, DLArrayHandle output, const size_t padding,
+                             const size_t stride, DLStreamHandle stream_handle, ProfilerHandle p);
+int CuDNN_DLGpuMax_Pooling2d_gradient(const DLArrayHandle output_Y, const DLArrayHandle gradient_Y,
+                                      const DLArrayHandle input_X, const size_t kernel_H,
+                                      const size_t kernel_W, DLArrayHandle gradient_X,
+                                      const size_t padding, const size_t stride,
+                                      DLStreamHandle stream_handle, ProfilerHandle p);
+
+/* ---- Concat / Slice copies (ref: c_runtime_api.h:382-384,394-396; impl
+ *      src/ops/Concat.cu:22,127, src/ops/Slice.cu:30,118).  begin_pos is a host array of
+ *      ndim int64. ---- */
+int DLGpuConcat(const DLArrayHandle input_x, const DLArrayHandle input_y, DLArrayHandle output,
+                int axis, DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuConcat_gradient(const DLArrayHandle output_gradient, DLArrayHandle input_gradient,
+                         int axis, int id, DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuSlice(const DLArrayHandle in_arr, DLArrayHandle out_arr, int64_t *begin_pos,
+               DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuSliceGradient(const DLArrayHandle in_arr, DLArrayHandle out_arr, int64_t *begin_pos,
+                       DLStreamHandle stream_handle, ProfilerHandle p);
+
+/* ---- Optimizer updates, in place, no ProfilerHandle (ref: c_runtime_api.h:399-410; impl
+ *      src/ops/Optimizers.cu:9,48,87,122).  beta1t/beta2t are the host-accumulated powers. ---- */
+int SGDOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, float lr,
+                       DLStreamHandle stream_handle);
+int MomentumOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, DLArrayHandle velocity,
+                            float lr, float momentum, bool nesterov, DLStreamHandle stream_handle);
+int AdaGradOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, DLArrayHandle acc,
+                           float lr, float eps, DLStreamHandle stream_handle);
+int AdamOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, DLArrayHandle expavg,
+                        DLArrayHandle expavgsq, float lr, float beta1, float beta2, float beta1t,
+                        float beta2t, float eps, DLStreamHandle stream_handle);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+#endif /* TSPLIT_AMD_C_RUNTIME_API_H_ */

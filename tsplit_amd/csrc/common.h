@@ -1,0 +1,90 @@
+// Shared host-side helpers of the operator library: argument checks, stream lookup,
+// the ProfilerHandle contract, and per-stream scratch memory for kernels that need it.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/c_runtime_api.h"
+
+namespace tsplit {
+
+inline int64_t numel(const DLArray *a) {
+  int64_t n = 1;
+  for (int i = 0; i < a->ndim; ++i) n *= a->shape[i];
+  return n;
+}
+
+inline hipStream_t stream_of(DLStreamHandle h) {
+  return h ? *static_cast<hipStream_t *>(h->handle) : static_cast<hipStream_t>(nullptr);
+}
+
+inline float mib(int64_t elems) { return static_cast<float>(elems) * 4.0f / (1024.0f * 1024.0f); }
+
+// Grow-only device scratch, one buffer per (stream, slot), kept until the process ends.
+// Kernels launched on one stream are ordered, so a buffer may be reused by the next op on
+// that stream without waiting; ops on different streams never share one.
+void *scratch_get(hipStream_t stream, int slot, size_t bytes);
+
+#define TS_FAIL(...)                                  \
+  do {                                                \
+    std::fprintf(stderr, "[libc_runtime_api] ");      \
+    std::fprintf(stderr, __VA_ARGS__);                \
+    std::fprintf(stderr, "\n");                       \
+    return -1;                                        \
+  } while (0)
+
+#define TS_REQUIRE(cond, ...) \
+  do {                        \
+    if (!(cond)) TS_FAIL(__VA_ARGS__); \
+  } while (0)
+
+#define TS_HIP(call)                                                                        \
+  do {                                                                                      \
+    hipError_t e_ = (call);                                                                 \
+    if (e_ != hipSuccess) TS_FAIL("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
+  } while (0)
+
+// ProfilerHandle contract of the reference (e.g. src/ops/Relu.cu:15-51): with a non-NULL
+// profiler the call records operand sizes in MiB, times the launch with events and blocks
+// until it has finished.  Usage:
+//   ProfileScope ps(p, stream, in_elems, out_elems, ws_elems);  ... launches ...  return ps.finish();
+class ProfileScope {
+ public:
+  ProfileScope(ProfilerHandle p, hipStream_t s, int64_t in_elems, int64_t out_elems, int64_t ws_elems)
+      : p_(p), s_(s) {
+    if (!p_) return;
+    p_->input_memory = mib(in_elems);
+    p_->output_memory = mib(out_elems);
+    p_->workspace_memory = mib(ws_elems);
+    ok_ = hipEventCreate(&a_) == hipSuccess && hipEventCreate(&b_) == hipSuccess &&
+          hipEventRecord(a_, s_) == hipSuccess;
+  }
+  int finish() {
+    hipError_t le = hipGetLastError();
+    if (le != hipSuccess) {
+      std::fprintf(stderr, "[libc_runtime_api] kernel launch failed: %s\n", hipGetErrorString(le));
+      return -1;
+    }
+    if (!p_) return 0;
+    if (!ok_) return -1;
+    float ms = -1.f;
+    bool good = hipEventRecord(b_, s_) == hipSuccess && hipEventSynchronize(b_) == hipSuccess &&
+                hipEventElapsedTime(&ms, a_, b_) == hipSuccess;
+    (void)hipEventDestroy(a_);
+    (void)hipEventDestroy(b_);
+    p_->time = ms;
+    return good ? 0 : -1;
+  }
+
+ private:
+  ProfilerHandle p_;
+  hipStream_t s_;
+  hipEvent_t a_{}, b_{};
+  bool ok_ = false;
+};
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace tsplit

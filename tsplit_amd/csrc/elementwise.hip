@@ -1,0 +1,341 @@
+// HBM-streaming elementwise kernels: graph-closure ops, Relu and the optimizer updates.
+//
+// One template serves all of them.  Every thread moves UNROLL x 16 bytes per array with
+// all loads issued before any arithmetic (so a wave keeps UNROLL dwordx4 loads per array
+// in flight), consecutive lanes touch consecutive 16-byte words, and a block covers one
+// contiguous 16 KiB span per array.  Arrays that are not 16-byte aligned (micro-tensor
+// views can start anywhere on a 4-byte boundary) take the scalar variant.
+#include "common.h"
+
+namespace tsplit {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;
+
+template <int N>
+struct Ptrs {
+  float *p[N];
+};
+
+// Op contract: static constexpr int N (arrays), LOAD / STORE bit masks over the arrays,
+// and  __device__ void apply(float (&v)[N]) const  transforming one element of each.
+template <class Op>
+__global__ __launch_bounds__(kThreads) void ew_vec_kernel(Op op, Ptrs<Op::N> a, int64_t n) {
+  constexpr int N = Op::N;
+  const int64_t n4 = n >> 2;
+  const int64_t first = (static_cast<int64_t>(blockIdx.x) * kUnroll) * kThreads + threadIdx.x;
+  float4 v[kUnroll][N];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const int64_t i = first + static_cast<int64_t>(u) * kThreads;
+    if (i < n4) {
+#pragma unroll
+      for (int k = 0; k < N; ++k)
+        if (Op::LOAD & (1 << k)) v[u][k] = reinterpret_cast<const float4 *>(a.p[k])[i];
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const int64_t i = first + static_cast<int64_t>(u) * kThreads;
+    if (i < n4) {
+      float e[4][N];
+#pragma unroll
+      for (int k = 0; k < N; ++k) {
+        e[0][k] = v[u][k].x;
+        e[1][k] = v[u][k].y;
+        e[2][k] = v[u][k].z;
+        e[3][k] = v[u][k].w;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) op.apply(e[j]);
+#pragma unroll
+      for (int k = 0; k < N; ++k)
+        if (Op::STORE & (1 << k))
+          reinterpret_cast<float4 *>(a.p[k])[i] = make_float4(e[0][k], e[1][k], e[2][k], e[3][k]);
+    }
+  }
+  // the last (n % 4) elements
+  if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    const int64_t i = (n4 << 2) + threadIdx.x;
+    float e[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k)
+      if (Op::LOAD & (1 << k)) e[k] = a.p[k][i];
+    op.apply(e);
+#pragma unroll
+    for (int k = 0; k < N; ++k)
+      if (Op::STORE & (1 << k)) a.p[k][i] = e[k];
+  }
+}
+
+template <class Op>
+__global__ __launch_bounds__(kThreads) void ew_scalar_kernel(Op op, Ptrs<Op::N> a, int64_t n) {
+  constexpr int N = Op::N;
+  const int64_t first = (static_cast<int64_t>(blockIdx.x) * kUnroll) * kThreads + threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const int64_t i = first + static_cast<int64_t>(u) * kThreads;
+    if (i < n) {
+      float e[N];
+#pragma unroll
+      for (int k = 0; k < N; ++k)
+        if (Op::LOAD & (1 << k)) e[k] = a.p[k][i];
+      op.apply(e);
+#pragma unroll
+      for (int k = 0; k < N; ++k)
+        if (Op::STORE & (1 << k)) a.p[k][i] = e[k];
+    }
+  }
+}
+
+template <class Op>
+void launch(Op op, Ptrs<Op::N> a, int64_t n, hipStream_t s) {
+  if (n <= 0) return;
+  bool vec = true;
+  for (int k = 0; k < Op::N; ++k) vec = vec && aligned16(a.p[k]);
+  const int64_t per_block = static_cast<int64_t>(kThreads) * kUnroll;
+  if (vec) {
+    const int64_t n4 = n >> 2;
+    int64_t blocks = (n4 + per_block - 1) / per_block;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(ew_vec_kernel<Op>, dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s, op, a, n);
+  } else {
+    const int64_t blocks = (n + per_block - 1) / per_block;
+    hipLaunchKernelGGL(ew_scalar_kernel<Op>, dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s, op, a, n);
+  }
+}
+
+// ---- ops.  Array 0 is the output unless noted. ----
+struct SetOp {   // out = c
+  static constexpr int N = 1, LOAD = 0, STORE = 1;
+  float c;
+  __device__ void apply(float (&v)[1]) const { v[0] = c; }
+};
+struct CopyOp {  // out = a
+  static constexpr int N = 2, LOAD = 2, STORE = 1;
+  __device__ void apply(float (&v)[2]) const { v[0] = v[1]; }
+};
+struct AddOp {   // out = a + b
+  static constexpr int N = 3, LOAD = 6, STORE = 1;
+  __device__ void apply(float (&v)[3]) const { v[0] = v[1] + v[2]; }
+};
+struct MulOp {
+  static constexpr int N = 3, LOAD = 6, STORE = 1;
+  __device__ void apply(float (&v)[3]) const { v[0] = v[1] * v[2]; }
+};
+struct AddConstOp {
+  static constexpr int N = 2, LOAD = 2, STORE = 1;
+  float c;
+  __device__ void apply(float (&v)[2]) const { v[0] = v[1] + c; }
+};
+struct MulConstOp {
+  static constexpr int N = 2, LOAD = 2, STORE = 1;
+  float c;
+  __device__ void apply(float (&v)[2]) const { v[0] = v[1] * c; }
+};
+struct ReluOp {
+  static constexpr int N = 2, LOAD = 2, STORE = 1;
+  __device__ void apply(float (&v)[2]) const { v[0] = fmaxf(v[1], 0.f); }
+};
+struct ReluGradOp {   // out = (sign(x)+1)*0.5*dy ; arrays: out, x, dy
+  static constexpr int N = 3, LOAD = 6, STORE = 1;
+  __device__ void apply(float (&v)[3]) const {
+    const float x = v[1];
+    const float sgn = x > 0.f ? 1.f : (x < 0.f ? -1.f : x);   // keeps +-0 and NaN like np.sign
+    v[0] = (sgn + 1.f) * 0.5f * v[2];
+  }
+};
+// optimizers: arrays param, grad, state...; evaluation order of src/ops/Optimizers.cu
+struct SgdOp {
+  static constexpr int N = 2, LOAD = 3, STORE = 1;
+  float lr;
+  __device__ void apply(float (&v)[2]) const { v[0] = v[0] - lr * v[1]; }
+};
+struct MomentumOp {   // param, grad, velocity
+  static constexpr int N = 3, LOAD = 7, STORE = 5;
+  float lr, mom;
+  __device__ void apply(float (&v)[3]) const {
+    v[2] = mom * v[2] - lr * v[1];
+    v[0] = v[0] + v[2];
+  }
+};
+struct NesterovOp {
+  static constexpr int N = 3, LOAD = 7, STORE = 5;
+  float lr, mom;
+  __device__ void apply(float (&v)[3]) const {
+    const float t = lr * v[1];
+    v[2] = mom * (v[2] - t);
+    v[0] = v[0] + v[2] - t;
+  }
+};
+struct AdaGradOp {    // param, grad, acc
+  static constexpr int N = 3, LOAD = 7, STORE = 5;
+  float lr, eps;
+  __device__ void apply(float (&v)[3]) const {
+    v[2] = v[2] + v[1] * v[1];
+    v[0] = v[0] - lr * v[1] / (sqrtf(v[2]) + eps);
+  }
+};
+struct AdamOp {       // param, grad, m, v
+  static constexpr int N = 4, LOAD = 15, STORE = 13;
+  float lr, b1, b2, b1t, b2t, eps;
+  __device__ void apply(float (&v)[4]) const {
+    v[2] = b1 * v[2] + (1.f - b1) * v[1];
+    v[3] = b2 * v[3] + (1.f - b2) * v[1] * v[1];
+    const float mc = v[2] / (1.f - b1t);
+    const float vc = v[3] / (1.f - b2t);
+    v[0] = v[0] - lr * mc / (sqrtf(vc) + eps);
+  }
+};
+
+inline float *fp(const DLArray *a) { return static_cast<float *>(a->data); }
+
+}  // namespace
+}  // namespace tsplit
+
+using namespace tsplit;
+
+#define SAME_SIZE(a, b, name) \
+  TS_REQUIRE(numel(a) == numel(b), name ": operand sizes differ (%lld vs %lld)", (long long)numel(a), (long long)numel(b))
+
+extern "C" {
+
+int DLGpuArraySet(DLArrayHandle arr, float value, DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(arr && arr->data, "DLGpuArraySet: NULL array");
+  hipStream_t s = stream_of(stream_handle);
+  const int64_t n = numel(arr);
+  ProfileScope ps(p, s, 0, n, 0);
+  launch(SetOp{value}, Ptrs<1>{{fp(arr)}}, n, s);
+  return ps.finish();
+}
+
+int DLGpuMatrixElementwiseAdd(const DLArrayHandle matA, const DLArrayHandle matB, DLArrayHandle output,
+                              DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(matA && matB && output, "DLGpuMatrixElementwiseAdd: NULL array");
+  SAME_SIZE(matA, output, "DLGpuMatrixElementwiseAdd");
+  SAME_SIZE(matB, output, "DLGpuMatrixElementwiseAdd");
+  hipStream_t s = stream_of(stream_handle);
+  const int64_t n = numel(output);
+  ProfileScope ps(p, s, 2 * n, n, 0);
+  launch(AddOp{}, Ptrs<3>{{fp(output), fp(matA), fp(matB)}}, n, s);
+  return ps.finish();
+}
+
+int DLGpuMatrixElementwiseMultiply(const DLArrayHandle matA, const DLArrayHandle matB, DLArrayHandle output,
+                                   DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(matA && matB && output, "DLGpuMatrixElementwiseMultiply: NULL array");
+  SAME_SIZE(matA, output, "DLGpuMatrixElementwiseMultiply");
+  SAME_SIZE(matB, output, "DLGpuMatrixElementwiseMultiply");
+  hipStream_t s = stream_of(stream_handle);
+  const int64_t n = numel(output);
+  ProfileScope ps(p, s, 2 * n, n, 0);
+  launch(MulOp{}, Ptrs<3>{{fp(output), fp(matA), fp(matB)}}, n, s);
+  return ps.finish();
+}
+
+int DLGpuMatrixElementwiseAddByConst(const DLArrayHandle input, float val, DLArrayHandle output,
+                                     DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(input && output, "DLGpuMatrixElementwiseAddByConst: NULL array");
+  SAME_SIZE(input, output, "DLGpuMatrixElementwiseAddByConst");
+  hipStream_t s = stream_of(stream_handle);
+  const int64_t n = numel(output);
+  ProfileScope ps(p, s, n, n, 0);
+  launch(AddConstOp{val}, Ptrs<2>{{fp(output), fp(input)}}, n, s);
+  return ps.finish();
+}
+
+int DLGpuMatrixMultiplyByConst(const DLArrayHandle input, float val, DLArrayHandle output,
+                               DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(input && output, "DLGpuMatrixMultiplyByConst: NULL array");
+  SAME_SIZE(input, output, "DLGpuMatrixMultiplyByConst");
+  hipStream_t s = stream_of(stream_handle);
+  const int64_t n = numel(output);
+  ProfileScope ps(p, s, n, n, 0);
+  launch(MulConstOp{val}, Ptrs<2>{{fp(output), fp(input)}}, n, s);
+  return ps.finish();
+}
+
+int DLGpuReshape(const DLArrayHandle in_arr, DLArrayHandle out_arr, DLStreamHandle stream_handle,
+                 ProfilerHandle p) {
+  TS_REQUIRE(in_arr && out_arr, "DLGpuReshape: NULL array");
+  SAME_SIZE(in_arr, out_arr, "DLGpuReshape");
+  hipStream_t s = stream_of(stream_handle);
+  const int64_t n = numel(out_arr);
+  ProfileScope ps(p, s, n, n, 0);
+  if (in_arr->data != out_arr->data) launch(CopyOp{}, Ptrs<2>{{fp(out_arr), fp(in_arr)}}, n, s);
+  return ps.finish();
+}
+
+int DLGpuRelu(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(input && output, "DLGpuRelu: NULL array");
+  SAME_SIZE(input, output, "DLGpuRelu");
+  hipStream_t s = stream_of(stream_handle);
+  const int64_t n = numel(output);
+  ProfileScope ps(p, s, n, n, 0);
+  launch(ReluOp{}, Ptrs<2>{{fp(output), fp(input)}}, n, s);
+  return ps.finish();
+}
+
+int DLGpuReluGradient(const DLArrayHandle input, const DLArrayHandle in_grad, DLArrayHandle output,
+                      DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(input && in_grad && output, "DLGpuReluGradient: NULL array");
+  SAME_SIZE(input, output, "DLGpuReluGradient");
+  SAME_SIZE(in_grad, output, "DLGpuReluGradient");
+  hipStream_t s = stream_of(stream_handle);
+  const int64_t n = numel(output);
+  ProfileScope ps(p, s, 2 * n, n, 0);
+  launch(ReluGradOp{}, Ptrs<3>{{fp(output), fp(input), fp(in_grad)}}, n, s);
+  return ps.finish();
+}
+
+int SGDOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, float lr, DLStreamHandle stream_handle) {
+  TS_REQUIRE(param && grad, "SGDOptimizerUpdate: NULL array");
+  SAME_SIZE(param, grad, "SGDOptimizerUpdate");
+  hipStream_t s = stream_of(stream_handle);
+  ProfileScope ps(nullptr, s, 0, 0, 0);
+  launch(SgdOp{lr}, Ptrs<2>{{fp(param), fp(grad)}}, numel(param), s);
+  return ps.finish();
+}
+
+int MomentumOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, DLArrayHandle velocity, float lr,
+                            float momentum, bool nesterov, DLStreamHandle stream_handle) {
+  TS_REQUIRE(param && grad && velocity, "MomentumOptimizerUpdate: NULL array");
+  SAME_SIZE(param, grad, "MomentumOptimizerUpdate");
+  SAME_SIZE(param, velocity, "MomentumOptimizerUpdate");
+  hipStream_t s = stream_of(stream_handle);
+  ProfileScope ps(nullptr, s, 0, 0, 0);
+  Ptrs<3> a{{fp(param), fp(grad), fp(velocity)}};
+  if (nesterov)
+    launch(NesterovOp{lr, momentum}, a, numel(param), s);
+  else
+    launch(MomentumOp{lr, momentum}, a, numel(param), s);
+  return ps.finish();
+}
+
+int AdaGradOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, DLArrayHandle acc, float lr, float eps,
+                           DLStreamHandle stream_handle) {
+  TS_REQUIRE(param && grad && acc, "AdaGradOptimizerUpdate: NULL array");
+  SAME_SIZE(param, grad, "AdaGradOptimizerUpdate");
+  SAME_SIZE(param, acc, "AdaGradOptimizerUpdate");
+  hipStream_t s = stream_of(stream_handle);
+  ProfileScope ps(nullptr, s, 0, 0, 0);
+  launch(AdaGradOp{lr, eps}, Ptrs<3>{{fp(param), fp(grad), fp(acc)}}, numel(param), s);
+  return ps.finish();
+}
+
+int AdamOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, DLArrayHandle expavg, DLArrayHandle expavgsq,
+                        float lr, float beta1, float beta2, float beta1t, float beta2t, float eps,
+                        DLStreamHandle stream_handle) {
+  TS_REQUIRE(param && grad && expavg && expavgsq, "AdamOptimizerUpdate: NULL array");
+  SAME_SIZE(param, grad, "AdamOptimizerUpdate");
+  SAME_SIZE(param, expavg, "AdamOptimizerUpdate");
+  SAME_SIZE(param, expavgsq, "AdamOptimizerUpdate");
+  hipStream_t s = stream_of(stream_handle);
+  ProfileScope ps(nullptr, s, 0, 0, 0);
+  launch(AdamOp{lr, beta1, beta2, beta1t, beta2t, eps}, Ptrs<4>{{fp(param), fp(grad), fp(expavg), fp(expavgsq)}},
+         numel(param), s);
+  return ps.finish();
+}
+
+}  // extern "C"

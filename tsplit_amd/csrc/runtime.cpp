@@ -1,0 +1,426 @@
+// Runtime half of the C ABI: array lifecycle, copies, streams, events, the pooled
+// allocator's public face, micro-tensor views.  No kernels here.
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <new>
+#include <set>
+#include <stdexcept>
+
+#include "common.h"
+#include "pool.h"
+
+namespace tsplit {
+namespace {
+
+std::mutex g_mu;
+
+// ---------------------------------------------------------------- device pool
+size_t env_bytes(const char *name, size_t dflt) {
+  const char *v = std::getenv(name);
+  if (!v || !*v) return dflt;
+  return static_cast<size_t>(std::strtoull(v, nullptr, 10));
+}
+
+void *dev_alloc(size_t bytes, void *) {
+  void *p = nullptr;
+  if (hipMalloc(&p, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  return p;
+}
+void dev_release(void *p, void *) { (void)hipFree(p); }
+size_t dev_available(void *) {
+  size_t free_b = 0, total_b = 0;
+  if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) return 0;
+  // head-room for kernels' code objects, scratch and the runtime itself
+  // (the reference keeps 500 MB back: gpu_memory_manager.cc:246)
+  const size_t keep = 512ull << 20;
+  return free_b > keep ? free_b - keep : 0;
+}
+
+std::map<int, BinnedPool *> g_pools;
+
+BinnedPool *pool_for(int dev) {
+  auto it = g_pools.find(dev);
+  if (it != g_pools.end()) return it->second;
+  PoolBacking b{dev_alloc, dev_release, dev_available, nullptr};
+  size_t slab = env_bytes("TSPLIT_POOL_SLAB_BYTES", 1ull << 30);
+  size_t limit = env_bytes("TSPLIT_POOL_LIMIT_BYTES", ~size_t(0));
+  BinnedPool *p = new BinnedPool(b, slab, limit);
+  g_pools[dev] = p;
+  return p;
+}
+
+int current_or(int dev) {
+  (void)hipSetDevice(dev);
+  return dev;
+}
+
+// ---------------------------------------------------------------- host memory
+// Host tensors are pinned when a device is present (the reference's GPU build does the
+// same: src/common/cpu_device_api.cc:30-36) so that stream copies really are asynchronous;
+// on a machine without a device they are plain aligned memory.
+std::set<void *> g_pinned;
+
+void *host_alloc(size_t bytes) {
+  if (bytes == 0) bytes = 4;
+  void *p = nullptr;
+  int n = 0;
+  if (hipGetDeviceCount(&n) == hipSuccess && n > 0) {
+    if (hipHostMalloc(&p, bytes, hipHostMallocDefault) == hipSuccess) {
+      g_pinned.insert(p);
+      return p;
+    }
+    (void)hipGetLastError();
+  } else {
+    (void)hipGetLastError();
+  }
+  if (posix_memalign(&p, 256, bytes) != 0) return nullptr;
+  return p;
+}
+
+void host_free(void *p) {
+  auto it = g_pinned.find(p);
+  if (it != g_pinned.end()) {
+    g_pinned.erase(it);
+    (void)hipHostFree(p);
+  } else {
+    std::free(p);
+  }
+}
+
+size_t byte_size(const DLArray *a) { return static_cast<size_t>(numel(a)) * 4; }
+
+void *data_alloc(DLContext ctx, size_t bytes, int rule) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (ctx.device_type == kCPU) return host_alloc(bytes);
+  if (ctx.device_type != kGPU) throw std::runtime_error("unknown device type");
+  current_or(ctx.device_id);
+  void *p = nullptr;
+  if (rule == 0) {
+    if (hipMalloc(&p, bytes ? bytes : 4) != hipSuccess) {
+      (void)hipGetLastError();
+      p = nullptr;
+    }
+  } else {
+    p = pool_for(ctx.device_id)->Malloc(bytes);
+  }
+  if (!p) throw std::runtime_error("out of device memory");
+  return p;
+}
+
+void data_free(DLContext ctx, void *p, int rule) {
+  if (!p) return;
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (ctx.device_type == kCPU) {
+    host_free(p);
+    return;
+  }
+  current_or(ctx.device_id);
+  if (rule != 0) {
+    if (pool_for(ctx.device_id)->Free(p)) return;
+    throw std::runtime_error("pointer was not allocated from the pool");
+  }
+  (void)hipFree(p);
+}
+
+DLArray *new_array(const index_t *shape, index_t ndim, DLContext ctx) {
+  DLArray *a = new DLArray();
+  a->data = nullptr;
+  a->ctx = ctx;
+  a->ndim = static_cast<int>(ndim);
+  a->shape = new int64_t[ndim > 0 ? ndim : 1];
+  for (index_t i = 0; i < ndim; ++i) a->shape[i] = shape[i];
+  return a;
+}
+
+// ---------------------------------------------------------------- scratch
+struct ScratchKey {
+  hipStream_t s;
+  int slot;
+  bool operator<(const ScratchKey &o) const { return s != o.s ? s < o.s : slot < o.slot; }
+};
+struct ScratchBuf {
+  void *p;
+  size_t bytes;
+};
+std::map<ScratchKey, ScratchBuf> g_scratch;
+
+}  // namespace
+
+void *scratch_get(hipStream_t stream, int slot, size_t bytes) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  ScratchBuf &b = g_scratch[ScratchKey{stream, slot}];
+  if (b.bytes >= bytes && b.p) return b.p;
+  if (b.p) {
+    // the old buffer may still be read by a kernel in flight on this stream
+    (void)hipStreamSynchronize(stream);
+    (void)hipFree(b.p);
+    b.p = nullptr;
+    b.bytes = 0;
+  }
+  size_t want = (bytes + (1 << 20) - 1) >> 20 << 20;
+  if (hipMalloc(&b.p, want) != hipSuccess) {
+    (void)hipGetLastError();
+    b.p = nullptr;
+    return nullptr;
+  }
+  b.bytes = want;
+  return b.p;
+}
+
+}  // namespace tsplit
+
+using namespace tsplit;
+
+#define API_BEGIN() try {
+#define API_END()                                                        \
+  }                                                                      \
+  catch (const std::exception &e) {                                      \
+    std::fprintf(stderr, "[libc_runtime_api] %s\n", e.what());           \
+    return -1;                                                           \
+  }                                                                      \
+  return 0;
+
+extern "C" {
+
+int ProfilerAlloc(ProfilerHandle *handle) {
+  Profiler *p = new Profiler();
+  p->time = p->input_memory = p->output_memory = p->workspace_memory = -1.f;
+  *handle = p;
+  return 0;
+}
+
+// ------------------------------------------------------------ streams / events
+int DLStreamCreate(size_t dev_id, DLStreamHandle *handle) {
+  TS_HIP(hipSetDevice(static_cast<int>(dev_id)));
+  hipStream_t *s = new hipStream_t();
+  hipError_t e = hipStreamCreate(s);   // default priority, blocking w.r.t. the NULL stream
+  if (e != hipSuccess) {
+    delete s;
+    TS_FAIL("hipStreamCreate failed: %s", hipGetErrorString(e));
+  }
+  DLStream *h = new DLStream();
+  h->device_id = static_cast<int>(dev_id);
+  h->handle = s;
+  *handle = h;
+  return 0;
+}
+
+int DLStreamDestroy(DLStreamHandle handle) {
+  if (!handle) return 0;
+  hipStream_t *s = static_cast<hipStream_t *>(handle->handle);
+  if (s) {
+    (void)hipStreamSynchronize(*s);
+    TS_HIP(hipStreamDestroy(*s));
+    delete s;
+  }
+  delete handle;
+  return 0;
+}
+
+int DLStreamSync(DLStreamHandle handle) {
+  TS_HIP(hipStreamSynchronize(stream_of(handle)));
+  return 0;
+}
+
+int DLEventCreate(size_t dev_id, DLEventHandle *handle) {
+  TS_HIP(hipSetDevice(static_cast<int>(dev_id)));
+  hipEvent_t *ev = new hipEvent_t();
+  hipError_t e = hipEventCreate(ev);
+  if (e != hipSuccess) {
+    delete ev;
+    TS_FAIL("hipEventCreate failed: %s", hipGetErrorString(e));
+  }
+  DLEvent *h = new DLEvent();
+  h->device_id = static_cast<int>(dev_id);
+  h->handle = ev;
+  *handle = h;
+  return 0;
+}
+
+int DLEventDestroy(DLEventHandle handle) {
+  if (!handle) return 0;
+  hipEvent_t *ev = static_cast<hipEvent_t *>(handle->handle);
+  if (ev) {
+    TS_HIP(hipEventDestroy(*ev));
+    delete ev;
+  }
+  delete handle;
+  return 0;
+}
+
+int DLEventRecord(DLStreamHandle stream_handle, DLEventHandle event_handle) {
+  TS_REQUIRE(event_handle != nullptr, "DLEventRecord: NULL event");
+  TS_HIP(hipEventRecord(*static_cast<hipEvent_t *>(event_handle->handle), stream_of(stream_handle)));
+  return 0;
+}
+
+int DLEventSync(DLEventHandle handle) {
+  TS_REQUIRE(handle != nullptr, "DLEventSync: NULL event");
+  TS_HIP(hipEventSynchronize(*static_cast<hipEvent_t *>(handle->handle)));
+  return 0;
+}
+
+int DLEventQuery(DLEventHandle handle) {
+  if (!handle) return 0;
+  hipError_t e = hipEventQuery(*static_cast<hipEvent_t *>(handle->handle));
+  if (e == hipSuccess) return 1;
+  (void)hipGetLastError();   // hipErrorNotReady is sticky in the last-error slot otherwise
+  return 0;
+}
+
+void cuda_init(void) {
+  int d = 0;
+  if (hipGetDevice(&d) == hipSuccess) (void)hipSetDevice(d);
+}
+void cudnn_init(size_t dev_id, DLStreamHandle) { (void)hipSetDevice(static_cast<int>(dev_id)); }
+void cublas_init(size_t dev_id, DLStreamHandle) { (void)hipSetDevice(static_cast<int>(dev_id)); }
+void cusp_init(size_t dev_id, DLStreamHandle) { (void)hipSetDevice(static_cast<int>(dev_id)); }
+
+// ------------------------------------------------------------ pool introspection
+static int current_device() {
+  int d = 0;
+  if (hipGetDevice(&d) != hipSuccess) {
+    (void)hipGetLastError();
+    d = 0;
+  }
+  return d;
+}
+
+void DLMemoryManager_PrintState(void *t, int type) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  *static_cast<int *>(t) = pool_for(current_device())->FreeChunkCount(type != 0);
+}
+
+void DLMemoryManager_Try_to_Malloc(size_t memory_size, void *p) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  *static_cast<int *>(p) = pool_for(current_device())->Try(memory_size) ? 1 : 0;
+}
+
+void DLMemoryManager_GPU_Usage(size_t *used_size, size_t *unused_unavailable_size,
+                               size_t *unused_available_size) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  pool_for(current_device())->Usage(used_size, unused_unavailable_size, unused_available_size);
+}
+
+// ------------------------------------------------------------ arrays
+int DLArrayAlloc(const index_t *shape, index_t ndim, DLContext ctx, DLArrayHandle *out,
+                 int MEMORY_MANAGE_RULE) {
+  DLArray *a = nullptr;
+  try {
+    a = new_array(shape, ndim, ctx);
+    a->data = data_alloc(ctx, byte_size(a), MEMORY_MANAGE_RULE);
+    *out = a;
+  } catch (const std::exception &e) {
+    std::fprintf(stderr, "[libc_runtime_api] DLArrayAlloc: %s\n", e.what());
+    if (a) {
+      delete[] a->shape;
+      delete a;
+    }
+    return -1;
+  }
+  return 0;
+}
+
+int DLArrayAllocSelf(DLArrayHandle handle, int MEMORY_MANAGE_RULE) {
+  API_BEGIN();
+  handle->data = data_alloc(handle->ctx, byte_size(handle), MEMORY_MANAGE_RULE);
+  API_END();
+}
+
+int DLArrayFree(DLArrayHandle handle, int MEMORY_MANAGE_RULE) {
+  API_BEGIN();
+  if (handle) {
+    void *d = handle->data;
+    DLContext ctx = handle->ctx;
+    delete[] handle->shape;
+    delete handle;
+    data_free(ctx, d, MEMORY_MANAGE_RULE);
+  }
+  API_END();
+}
+
+int DLArrayFreeSelf(DLArrayHandle handle, int MEMORY_MANAGE_RULE) {
+  API_BEGIN();
+  void *d = handle->data;
+  handle->data = nullptr;
+  data_free(handle->ctx, d, MEMORY_MANAGE_RULE);
+  API_END();
+}
+
+int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle stream) {
+  TS_REQUIRE(from && to, "DLArrayCopyFromTo: NULL array");
+  size_t bytes = byte_size(from);
+  TS_REQUIRE(bytes == byte_size(to), "DLArrayCopyFromTo: sizes differ (%zu vs %zu bytes)", bytes,
+             byte_size(to));
+  if (bytes == 0) return 0;
+  const bool fg = from->ctx.device_type == kGPU, tg = to->ctx.device_type == kGPU;
+  if (!fg && !tg) {
+    std::memcpy(to->data, from->data, bytes);
+    return 0;
+  }
+  hipMemcpyKind kind = fg && tg ? hipMemcpyDeviceToDevice : (fg ? hipMemcpyDeviceToHost : hipMemcpyHostToDevice);
+  TS_HIP(hipSetDevice(fg ? from->ctx.device_id : to->ctx.device_id));
+  if (stream) {
+    TS_HIP(hipMemcpyAsync(to->data, from->data, bytes, kind, stream_of(stream)));
+  } else {
+    TS_HIP(hipMemcpy(to->data, from->data, bytes, kind));
+  }
+  return 0;
+}
+
+int DLArrayReuseAlloc(DLContext ctx, int MEMORY_MANAGE_RULE, const index_t *input_shape,
+                      index_t input_ndim, DLArrayHandle *input, const index_t *output_shape,
+                      index_t output_ndim, DLArrayHandle *output, int pieces, int overlap_pieces) {
+  TS_REQUIRE(pieces > 0 && overlap_pieces >= 0 && overlap_pieces <= pieces,
+             "DLArrayReuseAlloc: bad pieces/overlap (%d/%d)", pieces, overlap_pieces);
+  DLArray *in = nullptr, *out = nullptr;
+  try {
+    in = new_array(input_shape, input_ndim, ctx);
+    out = new_array(output_shape, output_ndim, ctx);
+    const size_t in_b = byte_size(in), out_b = byte_size(out);
+    const size_t total = out_b + in_b / pieces * (pieces - overlap_pieces);
+    if (total < in_b) throw std::runtime_error("DLArrayReuseAlloc: output smaller than the overlapped part of the input");
+    char *base = static_cast<char *>(data_alloc(ctx, total, MEMORY_MANAGE_RULE));
+    out->data = base;                      // output at the base
+    in->data = base + (total - in_b);      // input flush with the end
+    *input = in;
+    *output = out;
+  } catch (const std::exception &e) {
+    std::fprintf(stderr, "[libc_runtime_api] %s\n", e.what());
+    for (DLArray *a : {in, out})
+      if (a) {
+        delete[] a->shape;
+        delete a;
+      }
+    return -1;
+  }
+  return 0;
+}
+
+int DLArraySliceForMicroTensor(DLArrayHandle input, DLArrayHandle *output, int total_number,
+                               int index, int dimension) {
+  TS_REQUIRE(input && input->ndim >= 1, "DLArraySliceForMicroTensor: bad input");
+  TS_REQUIRE(total_number > 0 && index >= 0 && index < total_number,
+             "DLArraySliceForMicroTensor: index %d of %d", index, total_number);
+  const int d = dimension == 0 ? 0 : 1;
+  TS_REQUIRE(d < input->ndim, "DLArraySliceForMicroTensor: dimension %d of a %d-d array", d, input->ndim);
+  DLArray *v = new_array(input->shape, input->ndim, input->ctx);
+  const int64_t D = input->shape[d];
+  const int64_t len = D ? numel(input) / D : 0;   // elements per index of the split dimension
+  const int64_t base = D / total_number, extra = D % total_number;
+  // pieces [0, extra) hold base+1 indices, the rest hold base
+  const int64_t before = static_cast<int64_t>(index) * base + (index < extra ? index : extra);
+  v->shape[d] = base + (index < extra ? 1 : 0);
+  // For d == 1 this is, like the reference, a contiguous chunk re-labelled [N, C/k, ...]:
+  // a true channel slice only when N == 1.
+  v->data = static_cast<float *>(input->data) + before * len;
+  *output = v;
+  return 0;
+}
+
+}  // extern "C"

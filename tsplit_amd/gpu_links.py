@@ -1,0 +1,221 @@
+"""One thin Python function per operator symbol of the C ABI.
+
+Mirror of the reference's python/athena/gpu_links/*.py: same function names, argument
+order and defaults (cited per function), so a graph op written against the reference's
+`gpu_links` runs unchanged on this library.  Return values of the C calls are checked
+here (the reference's wrappers ignore them).
+"""
+import ctypes
+
+from . import ndarray as _nd
+from ._base import _LIB, check_call
+
+__all__ = [
+    "array_set", "matrix_elementwise_add", "matrix_elementwise_add_by_const",
+    "matrix_elementwise_multiply", "matrix_elementwise_multiply_by_const", "array_reshape",
+    "relu", "relu_gradient", "matrix_multiply", "softmax", "softmax_cross_entropy",
+    "softmax_cross_entropy_gradient", "CuDNN_conv2d", "CuDNN_conv2d_gradient_of_data",
+    "CuDNN_conv2d_gradient_of_filter", "conv2d", "conv2d_gradient_of_data",
+    "conv2d_gradient_of_filter", "CuDNN_Batch_Normalization", "CuDNN_Batch_Normalization_gradient",
+    "max_pooling2d", "max_pooling2d_gradient", "CuDNN_max_pooling2d", "CuDNN_max_pooling2d_gradient",
+    "concat", "concat_gradient", "matrix_slice", "matrix_slice_gradient",
+    "sgd_update", "momentum_update", "adagrad_update", "adam_update",
+]
+
+
+def _h(arr):
+    assert isinstance(arr, _nd.NDArray)
+    return arr.handle
+
+
+def _s(stream):
+    return stream.handle if stream else None
+
+
+def _p(profiler):
+    return ctypes.byref(profiler) if profiler else None
+
+
+# ---- graph-closure ops (gpu_links/ArraySetLink.py:8, AddElewiseLink.py, AddConstLink.py,
+#      MultiplyElewiseLink.py, MultiplyConstLink.py, ReshapeLink.py:8) ----
+def array_set(arr, value, stream=None, profiler=None):
+    check_call(_LIB.DLGpuArraySet(_h(arr), ctypes.c_float(value), _s(stream), _p(profiler)))
+
+
+def matrix_elementwise_add(matA, matB, matC, stream=None, profiler=None):
+    check_call(_LIB.DLGpuMatrixElementwiseAdd(_h(matA), _h(matB), _h(matC), _s(stream), _p(profiler)))
+
+
+def matrix_elementwise_add_by_const(in_mat, val, out_mat, stream=None, profiler=None):
+    check_call(_LIB.DLGpuMatrixElementwiseAddByConst(_h(in_mat), ctypes.c_float(val), _h(out_mat),
+                                                     _s(stream), _p(profiler)))
+
+
+def matrix_elementwise_multiply(matA, matB, matC, stream=None, profiler=None):
+    check_call(_LIB.DLGpuMatrixElementwiseMultiply(_h(matA), _h(matB), _h(matC), _s(stream), _p(profiler)))
+
+
+def matrix_elementwise_multiply_by_const(in_mat, val, out_mat, stream=None, profiler=None):
+    check_call(_LIB.DLGpuMatrixMultiplyByConst(_h(in_mat), ctypes.c_float(val), _h(out_mat),
+                                               _s(stream), _p(profiler)))
+
+
+def array_reshape(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuReshape(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+# ---- Relu (gpu_links/ReluLink.py:8,14) ----
+def relu(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuRelu(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def relu_gradient(in_arr, in_grad_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuReluGradient(_h(in_arr), _h(in_grad_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+# ---- MatMul (gpu_links/MatrixMultLink.py:8) ----
+def matrix_multiply(matA, transA, matB, transB, matC, stream=None, profiler=None):
+    check_call(_LIB.DLGpuMatrixMultiply(_h(matA), ctypes.c_bool(bool(transA)), _h(matB),
+                                        ctypes.c_bool(bool(transB)), _h(matC), _s(stream), _p(profiler)))
+
+
+# ---- Softmax / CE (gpu_links/SoftmaxLink.py, SoftmaxCrossEntropyLink.py:8,17) ----
+def softmax(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuSoftmax(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def softmax_cross_entropy(in_arr_a, in_arr_b, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuSoftmaxCrossEntropy(_h(in_arr_a), _h(in_arr_b), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def softmax_cross_entropy_gradient(in_arr_a, in_arr_b, in_arr_c, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuSoftmaxCrossEntropy_Gradient(_h(in_arr_a), _h(in_arr_b), _h(in_arr_c), _h(out_arr),
+                                                      _s(stream), _p(profiler)))
+
+
+# ---- Conv2d (gpu_links/CudnnConv2d.py:8,21,33; gpu_links/Conv2dLink.py:8,24,35) ----
+def CuDNN_conv2d(in_arr_x, in_arr_f, out_arr, padding=0, padding2=None, stride=1, stream=None, profiler=None):
+    pad2 = padding if padding2 is None else padding2
+    check_call(_LIB.CuDNN_DLGpuConv2d(_h(in_arr_x), _h(in_arr_f), _h(out_arr), int(padding), int(pad2),
+                                      int(stride), _s(stream), _p(profiler)))
+
+
+def CuDNN_conv2d_gradient_of_filter(in_arr_x, in_gradient_y, out_gradient_f, padding=0, padding2=None,
+                                    stride=1, stream=None, profiler=None):
+    pad2 = padding if padding2 is None else padding2
+    check_call(_LIB.CuDNN_DLGpuConv2d_Gradient_of_Filter(_h(in_arr_x), _h(in_gradient_y), _h(out_gradient_f),
+                                                         int(padding), int(pad2), int(stride),
+                                                         _s(stream), _p(profiler)))
+
+
+def CuDNN_conv2d_gradient_of_data(in_arr_f, in_gradient_y, out_gradient_x, padding=0, padding2=None,
+                                  stride=1, stream=None, profiler=None):
+    pad2 = padding if padding2 is None else padding2
+    check_call(_LIB.CuDNN_DLGpuConv2d_Gradient_of_Data(_h(in_arr_f), _h(in_gradient_y), _h(out_gradient_x),
+                                                       int(padding), int(pad2), int(stride),
+                                                       _s(stream), _p(profiler)))
+
+
+def conv2d(in_arr_x, in_arr_f, out_arr, workspace_arr, padding=0, stride=1, stream=None, profiler=None):
+    check_call(_LIB.DLGpuConv2d(_h(in_arr_x), _h(in_arr_f), _h(out_arr), _h(workspace_arr),
+                                int(padding), int(stride), _s(stream), _p(profiler)))
+
+
+def conv2d_gradient_of_filter(in_arr_x, in_gradient_y, out_gradient_f, workspace_im2col,
+                              workspace_batch_filter, padding=0, stride=1, stream=None, profiler=None):
+    check_call(_LIB.DLGpuConv2d_Gradient_of_Filter(_h(in_arr_x), _h(in_gradient_y), _h(out_gradient_f),
+                                                   _h(workspace_im2col), _h(workspace_batch_filter),
+                                                   int(padding), int(stride), _s(stream), _p(profiler)))
+
+
+def conv2d_gradient_of_data(in_arr_f, in_gradient_y, out_gradient_x, workspace_im2col, padding=0,
+                            stride=1, stream=None, profiler=None):
+    check_call(_LIB.DLGpuConv2d_Gradient_of_Data(_h(in_arr_f), _h(in_gradient_y), _h(out_gradient_x),
+                                                 _h(workspace_im2col), int(padding), int(stride),
+                                                 _s(stream), _p(profiler)))
+
+
+# ---- BatchNorm (gpu_links/CudnnBnLink.py:8,17) ----
+def CuDNN_Batch_Normalization(in_arr, bn_scale_arr, bn_bias_arr, out_arr, save_mean, save_var,
+                              momentum=0.99, eps=0.001, stream=None, profiler=None):
+    check_call(_LIB.CuDNN_DLGpuBatch_Normalization(
+        _h(in_arr), _h(bn_scale_arr), _h(bn_bias_arr), _h(out_arr), ctypes.c_float(momentum),
+        ctypes.c_float(eps), save_mean.handle if save_mean else None,
+        save_var.handle if save_var else None, _s(stream), _p(profiler)))
+
+
+def CuDNN_Batch_Normalization_gradient(in_gradient_y, in_arr_x, in_bn_scale, out_gradient_x,
+                                       out_gradient_bn_scale, out_gradient_bn_bias, saved_mean, saved_var,
+                                       eps=0.001, stream=None, profiler=None):
+    check_call(_LIB.CuDNN_DLGpuBatch_Normalization_gradient(
+        _h(in_gradient_y), _h(in_arr_x), _h(in_bn_scale), _h(out_gradient_x), _h(out_gradient_bn_scale),
+        _h(out_gradient_bn_bias), ctypes.c_float(eps), saved_mean.handle if saved_mean else None,
+        saved_var.handle if saved_var else None, _s(stream), _p(profiler)))
+
+
+# ---- MaxPool (gpu_links/MaxPoolLink.py:8,15; gpu_links/CudnnMaxPoolLink.py:8,15) ----
+def max_pooling2d(in_arr, kernel_H, kernel_W, pooled_layer, padding=0, stride=1, stream=None, profiler=None):
+    check_call(_LIB.DLGpuMax_Pooling2d(_h(in_arr), int(kernel_H), int(kernel_W), _h(pooled_layer),
+                                       int(padding), int(stride), _s(stream), _p(profiler)))
+
+
+def max_pooling2d_gradient(in_arr, in_grad_arr, kernel_H, kernel_W, out_grad_arr, padding=0, stride=1,
+                           stream=None, profiler=None):
+    check_call(_LIB.DLGpuMax_Pooling2d_gradient(_h(in_arr), _h(in_grad_arr), int(kernel_H), int(kernel_W),
+                                                _h(out_grad_arr), int(padding), int(stride),
+                                                _s(stream), _p(profiler)))
+
+
+def CuDNN_max_pooling2d(in_arr, kernel_H, kernel_W, pooled_layer, padding=0, stride=1, stream=None,
+                        profiler=None):
+    check_call(_LIB.CuDNN_DLGpuMax_Pooling2d(_h(in_arr), ctypes.c_size_t(kernel_H), ctypes.c_size_t(kernel_W),
+                                             _h(pooled_layer), ctypes.c_size_t(padding),
+                                             ctypes.c_size_t(stride), _s(stream), _p(profiler)))
+
+
+def CuDNN_max_pooling2d_gradient(in_arr_y, in_gradient_y, in_arr_x, kernel_H, kernel_W, out_gradient_x,
+                                 padding=0, stride=1, stream=None, profiler=None):
+    check_call(_LIB.CuDNN_DLGpuMax_Pooling2d_gradient(
+        _h(in_arr_y), _h(in_gradient_y), _h(in_arr_x), ctypes.c_size_t(kernel_H), ctypes.c_size_t(kernel_W),
+        _h(out_gradient_x), ctypes.c_size_t(padding), ctypes.c_size_t(stride), _s(stream), _p(profiler)))
+
+
+# ---- Concat / Slice (gpu_links/ConcatLink.py:8,14; gpu_links/SliceLink.py:8,16) ----
+def concat(in_arr1, in_arr2, out_arr, axis=0, stream=None, profiler=None):
+    check_call(_LIB.DLGpuConcat(_h(in_arr1), _h(in_arr2), _h(out_arr), int(axis), _s(stream), _p(profiler)))
+
+
+def concat_gradient(out_grad_arr, in_arr, axis=0, idx=0, stream=None, profiler=None):
+    check_call(_LIB.DLGpuConcat_gradient(_h(out_grad_arr), _h(in_arr), int(axis), int(idx),
+                                         _s(stream), _p(profiler)))
+
+
+def matrix_slice(in_arr, out_arr, begin_pos, stream=None, profiler=None):
+    pos = (ctypes.c_int64 * len(begin_pos))(*list(begin_pos))
+    check_call(_LIB.DLGpuSlice(_h(in_arr), _h(out_arr), pos, _s(stream), _p(profiler)))
+
+
+def matrix_slice_gradient(in_arr, out_arr, begin_pos, stream=None, profiler=None):
+    pos = (ctypes.c_int64 * len(begin_pos))(*list(begin_pos))
+    check_call(_LIB.DLGpuSliceGradient(_h(in_arr), _h(out_arr), pos, _s(stream), _p(profiler)))
+
+
+# ---- Optimizers (gpu_links/OptimizerLink.py:7-30) ----
+def sgd_update(param, grad, lr, stream=None):
+    check_call(_LIB.SGDOptimizerUpdate(_h(param), _h(grad), ctypes.c_float(lr), _s(stream)))
+
+
+def momentum_update(param, grad, velocity, lr, momentum, nesterov, stream=None):
+    check_call(_LIB.MomentumOptimizerUpdate(_h(param), _h(grad), _h(velocity), ctypes.c_float(lr),
+                                            ctypes.c_float(momentum), ctypes.c_bool(bool(nesterov)), _s(stream)))
+
+
+def adagrad_update(param, grad, accumulation, lr, eps, stream=None):
+    check_call(_LIB.AdaGradOptimizerUpdate(_h(param), _h(grad), _h(accumulation), ctypes.c_float(lr),
+                                           ctypes.c_float(eps), _s(stream)))
+
+
+def adam_update(param, grad, expavg, expavgsq, lr, beta1, beta2, beta1t, beta2t, eps, stream=None):
+    check_call(_LIB.AdamOptimizerUpdate(_h(param), _h(grad), _h(expavg), _h(expavgsq), ctypes.c_float(lr),
+                                        ctypes.c_float(beta1), ctypes.c_float(beta2), ctypes.c_float(beta1t),
+                                        ctypes.c_float(beta2t), ctypes.c_float(eps), _s(stream)))
