@@ -1,0 +1,397 @@
+// Training-mode spatial BatchNorm, forward and backward, NCHW float32.
+//
+// Per channel the N*H*W elements sit in N contiguous planes of H*W.  Both directions are
+// two streaming passes over a (split, channel) grid:
+//   forward : [stats]  partial (sum x, sum x^2) per block          -> scratch (double)
+//             [apply]  every block folds the partials of its channel, then y = a*x + b
+//   backward: [reduce] partial (sum dy, sum dy*x, sum x, sum x^2)   -> scratch (double)
+//             [dx]     folds them, then dx = k1*dy + k2*x + k3; split 0 writes dgamma/dbeta
+// Threads walk a per-channel virtual index (in 16-byte words when H*W % 4 == 0) that is
+// mapped to (plane, offset) with a multiply-shift division, so consecutive lanes read
+// consecutive words of one plane.  Per-thread accumulation is float32 over a few hundred
+// values; everything across threads and blocks is folded in double, which keeps
+// E[x^2]-E[x]^2 and sum(dy*x)-mean*sum(dy) accurate.
+// Algorithmic traffic is 8 B/elem forward and 12 B/elem backward; these kernels move
+// 12 and 20 B/elem (x, and dy, are read by both passes).
+#include "common.h"
+#include "fastdiv.h"
+#include "reduce.h"
+
+namespace tsplit {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / kWave;
+
+struct Geo {
+  FastDiv plane;      // divides by words per plane
+  uint32_t wpp;       // words per plane (H*W / VEC)
+  uint32_t words;     // words per channel (N * wpp)
+  uint32_t chunk;     // words per block
+  int C;
+};
+
+template <int VEC>
+struct Word;
+template <>
+struct Word<4> {
+  using T = float4;
+};
+template <>
+struct Word<1> {
+  using T = float;
+};
+
+template <int VEC>
+__device__ __forceinline__ int64_t word_addr(const Geo &g, uint32_t i, int c) {
+  const uint32_t n = g.plane.div(i);
+  const uint32_t j = i - n * g.wpp;
+  return (static_cast<int64_t>(n) * g.C + c) * g.wpp + j;
+}
+
+__device__ __forceinline__ void acc2(const float4 &v, float &s, float &q) {
+  s += (v.x + v.y) + (v.z + v.w);
+  q += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+}
+__device__ __forceinline__ void acc2(const float &v, float &s, float &q) {
+  s += v;
+  q += v * v;
+}
+__device__ __forceinline__ void acc_dot(const float4 &a, const float4 &b, float &s, float &d) {
+  s += (a.x + a.y) + (a.z + a.w);
+  d += (a.x * b.x + a.y * b.y) + (a.z * b.z + a.w * b.w);
+}
+__device__ __forceinline__ void acc_dot(const float &a, const float &b, float &s, float &d) {
+  s += a;
+  d += a * b;
+}
+__device__ __forceinline__ float4 axpb(const float4 &x, float a, float b) {
+  return make_float4(a * x.x + b, a * x.y + b, a * x.z + b, a * x.w + b);
+}
+__device__ __forceinline__ float axpb(const float &x, float a, float b) { return a * x + b; }
+__device__ __forceinline__ float4 lin2(const float4 &dy, const float4 &x, float k1, float k2, float k3) {
+  return make_float4(k1 * dy.x + k2 * x.x + k3, k1 * dy.y + k2 * x.y + k3, k1 * dy.z + k2 * x.z + k3,
+                     k1 * dy.w + k2 * x.w + k3);
+}
+__device__ __forceinline__ float lin2(const float &dy, const float &x, float k1, float k2, float k3) {
+  return k1 * dy + k2 * x + k3;
+}
+
+// partial layout: [C][S][NQ] doubles
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void bn_stats_kernel(const float *__restrict__ x, double *__restrict__ part,
+                                                            Geo g, int S) {
+  using W = typename Word<VEC>::T;
+  __shared__ double sm[kWaves];
+  const int c = blockIdx.y, s = blockIdx.x;
+  const uint32_t begin = s * g.chunk;
+  const uint32_t end = min(begin + g.chunk, g.words);
+  const W *xw = reinterpret_cast<const W *>(x);
+  float sum = 0.f, sq = 0.f;
+  uint32_t i = begin + threadIdx.x;
+  for (; i + 3 * kThreads < end; i += 4 * kThreads) {
+    W v0 = xw[word_addr<VEC>(g, i, c)];
+    W v1 = xw[word_addr<VEC>(g, i + kThreads, c)];
+    W v2 = xw[word_addr<VEC>(g, i + 2 * kThreads, c)];
+    W v3 = xw[word_addr<VEC>(g, i + 3 * kThreads, c)];
+    acc2(v0, sum, sq);
+    acc2(v1, sum, sq);
+    acc2(v2, sum, sq);
+    acc2(v3, sum, sq);
+  }
+  for (; i < end; i += kThreads) acc2(xw[word_addr<VEC>(g, i, c)], sum, sq);
+  const double ds = block_sum<double, kWaves>(static_cast<double>(sum), sm);
+  const double dq = block_sum<double, kWaves>(static_cast<double>(sq), sm);
+  if (threadIdx.x == 0) {
+    double *o = part + (static_cast<int64_t>(c) * S + s) * 2;
+    o[0] = ds;
+    o[1] = dq;
+  }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void bn_apply_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                            const float *__restrict__ gamma,
+                                                            const float *__restrict__ beta,
+                                                            const double *__restrict__ part, int S, Geo g, float eps,
+                                                            double inv_m, float *__restrict__ save_mean,
+                                                            float *__restrict__ save_istd) {
+  using W = typename Word<VEC>::T;
+  __shared__ float coef[2];
+  const int c = blockIdx.y;
+  if (threadIdx.x == 0) {
+    double s = 0.0, q = 0.0;
+    for (int k = 0; k < S; ++k) {
+      s += part[(static_cast<int64_t>(c) * S + k) * 2];
+      q += part[(static_cast<int64_t>(c) * S + k) * 2 + 1];
+    }
+    const double mean = s * inv_m;
+    double var = q * inv_m - mean * mean;
+    if (var < 0.0) var = 0.0;
+    const double istd = 1.0 / sqrt(var + static_cast<double>(eps));
+    const double a = static_cast<double>(gamma[c]) * istd;
+    coef[0] = static_cast<float>(a);
+    coef[1] = static_cast<float>(static_cast<double>(beta[c]) - mean * a);
+    if (blockIdx.x == 0) {
+      if (save_mean) save_mean[c] = static_cast<float>(mean);
+      if (save_istd) save_istd[c] = static_cast<float>(istd);
+    }
+  }
+  __syncthreads();
+  const float a = coef[0], b = coef[1];
+  const uint32_t begin = blockIdx.x * g.chunk;
+  const uint32_t end = min(begin + g.chunk, g.words);
+  const W *xw = reinterpret_cast<const W *>(x);
+  W *yw = reinterpret_cast<W *>(y);
+  uint32_t i = begin + threadIdx.x;
+  for (; i + 3 * kThreads < end; i += 4 * kThreads) {
+    const int64_t a0 = word_addr<VEC>(g, i, c), a1 = word_addr<VEC>(g, i + kThreads, c),
+                  a2 = word_addr<VEC>(g, i + 2 * kThreads, c), a3 = word_addr<VEC>(g, i + 3 * kThreads, c);
+    W v0 = xw[a0], v1 = xw[a1], v2 = xw[a2], v3 = xw[a3];
+    yw[a0] = axpb(v0, a, b);
+    yw[a1] = axpb(v1, a, b);
+    yw[a2] = axpb(v2, a, b);
+    yw[a3] = axpb(v3, a, b);
+  }
+  for (; i < end; i += kThreads) {
+    const int64_t a0 = word_addr<VEC>(g, i, c);
+    yw[a0] = axpb(xw[a0], a, b);
+  }
+}
+
+// partials per block: sum dy, sum dy*x, sum x, sum x^2
+template <int VEC, bool STATS>
+__global__ __launch_bounds__(kThreads) void bn_bwd_reduce_kernel(const float *__restrict__ dy,
+                                                                 const float *__restrict__ x,
+                                                                 double *__restrict__ part, Geo g, int S) {
+  using W = typename Word<VEC>::T;
+  __shared__ double sm[kWaves];
+  const int c = blockIdx.y, s = blockIdx.x;
+  const uint32_t begin = s * g.chunk;
+  const uint32_t end = min(begin + g.chunk, g.words);
+  const W *xw = reinterpret_cast<const W *>(x);
+  const W *dw = reinterpret_cast<const W *>(dy);
+  float sdy = 0.f, sdx = 0.f, sx = 0.f, sq = 0.f;
+  uint32_t i = begin + threadIdx.x;
+  for (; i + kThreads < end; i += 2 * kThreads) {
+    const int64_t a0 = word_addr<VEC>(g, i, c), a1 = word_addr<VEC>(g, i + kThreads, c);
+    W x0 = xw[a0], d0 = dw[a0], x1 = xw[a1], d1 = dw[a1];
+    acc_dot(d0, x0, sdy, sdx);
+    acc_dot(d1, x1, sdy, sdx);
+    if (STATS) {
+      acc2(x0, sx, sq);
+      acc2(x1, sx, sq);
+    }
+  }
+  for (; i < end; i += kThreads) {
+    const int64_t a0 = word_addr<VEC>(g, i, c);
+    W x0 = xw[a0], d0 = dw[a0];
+    acc_dot(d0, x0, sdy, sdx);
+    if (STATS) acc2(x0, sx, sq);
+  }
+  const double r0 = block_sum<double, kWaves>(static_cast<double>(sdy), sm);
+  const double r1 = block_sum<double, kWaves>(static_cast<double>(sdx), sm);
+  double r2 = 0.0, r3 = 0.0;
+  if (STATS) {
+    r2 = block_sum<double, kWaves>(static_cast<double>(sx), sm);
+    r3 = block_sum<double, kWaves>(static_cast<double>(sq), sm);
+  }
+  if (threadIdx.x == 0) {
+    double *o = part + (static_cast<int64_t>(c) * S + s) * 4;
+    o[0] = r0;
+    o[1] = r1;
+    o[2] = r2;
+    o[3] = r3;
+  }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void bn_bwd_dx_kernel(const float *__restrict__ dy, const float *__restrict__ x,
+                                                             float *__restrict__ dx, const float *__restrict__ gamma,
+                                                             const double *__restrict__ part, int S, Geo g, float eps,
+                                                             double inv_m, const float *__restrict__ save_mean,
+                                                             const float *__restrict__ save_istd,
+                                                             float *__restrict__ dgamma, float *__restrict__ dbeta) {
+  using W = typename Word<VEC>::T;
+  __shared__ float coef[3];
+  const int c = blockIdx.y;
+  if (threadIdx.x == 0) {
+    double sdy = 0.0, sdx = 0.0, sx = 0.0, sq = 0.0;
+    for (int k = 0; k < S; ++k) {
+      const double *o = part + (static_cast<int64_t>(c) * S + k) * 4;
+      sdy += o[0];
+      sdx += o[1];
+      sx += o[2];
+      sq += o[3];
+    }
+    double mean, istd;
+    if (save_mean && save_istd) {
+      mean = static_cast<double>(save_mean[c]);
+      istd = static_cast<double>(save_istd[c]);
+    } else {
+      mean = sx * inv_m;
+      double var = sq * inv_m - mean * mean;
+      if (var < 0.0) var = 0.0;
+      istd = 1.0 / sqrt(var + static_cast<double>(eps));
+    }
+    const double dbias = sdy;
+    const double dscale = (sdx - mean * sdy) * istd;
+    const double k1 = static_cast<double>(gamma[c]) * istd;
+    const double k2 = -k1 * istd * dscale * inv_m;
+    const double k3 = -k1 * dbias * inv_m - k2 * mean;
+    coef[0] = static_cast<float>(k1);
+    coef[1] = static_cast<float>(k2);
+    coef[2] = static_cast<float>(k3);
+    if (blockIdx.x == 0) {
+      if (dgamma) dgamma[c] = static_cast<float>(dscale);
+      if (dbeta) dbeta[c] = static_cast<float>(dbias);
+    }
+  }
+  __syncthreads();
+  const float k1 = coef[0], k2 = coef[1], k3 = coef[2];
+  const uint32_t begin = blockIdx.x * g.chunk;
+  const uint32_t end = min(begin + g.chunk, g.words);
+  const W *xw = reinterpret_cast<const W *>(x);
+  const W *dw = reinterpret_cast<const W *>(dy);
+  W *ow = reinterpret_cast<W *>(dx);
+  uint32_t i = begin + threadIdx.x;
+  for (; i + kThreads < end; i += 2 * kThreads) {
+    const int64_t a0 = word_addr<VEC>(g, i, c), a1 = word_addr<VEC>(g, i + kThreads, c);
+    W x0 = xw[a0], d0 = dw[a0], x1 = xw[a1], d1 = dw[a1];
+    ow[a0] = lin2(d0, x0, k1, k2, k3);
+    ow[a1] = lin2(d1, x1, k1, k2, k3);
+  }
+  for (; i < end; i += kThreads) {
+    const int64_t a0 = word_addr<VEC>(g, i, c);
+    ow[a0] = lin2(dw[a0], xw[a0], k1, k2, k3);
+  }
+}
+
+struct Plan {
+  Geo g;
+  int S;
+  int vec;
+  int64_t m;
+};
+
+// words_per_block: how much of a channel one block streams
+bool make_plan(const DLArray *x, bool all_aligned, uint32_t words_per_block, int max_blocks, Plan &pl) {
+  if (x->ndim != 4) return false;
+  const int64_t N = x->shape[0], C = x->shape[1], HW = x->shape[2] * x->shape[3];
+  if (N <= 0 || C <= 0 || HW <= 0) return false;
+  pl.m = N * HW;
+  pl.vec = (HW % 4 == 0 && all_aligned) ? 4 : 1;
+  const int64_t words = pl.m / pl.vec;
+  if (words >= (1ll << 31) || C > 65535) return false;
+  int64_t S = (words + words_per_block - 1) / words_per_block;
+  const int64_t cap = max_blocks / C > 0 ? max_blocks / C : 1;
+  if (S > cap) S = cap;
+  if (S < 1) S = 1;
+  int64_t chunk = (words + S - 1) / S;
+  chunk = (chunk + kThreads - 1) / kThreads * kThreads;
+  S = (words + chunk - 1) / chunk;
+  pl.S = static_cast<int>(S);
+  pl.g.wpp = static_cast<uint32_t>(HW / pl.vec);
+  pl.g.plane = FastDiv(pl.g.wpp);
+  pl.g.words = static_cast<uint32_t>(words);
+  pl.g.chunk = static_cast<uint32_t>(chunk);
+  pl.g.C = static_cast<int>(C);
+  return true;
+}
+
+inline const float *cf(const DLArray *a) { return static_cast<const float *>(a->data); }
+inline float *mf(DLArray *a) { return static_cast<float *>(a->data); }
+
+}  // namespace
+}  // namespace tsplit
+
+using namespace tsplit;
+
+extern "C" {
+
+int CuDNN_DLGpuBatch_Normalization(const DLArrayHandle input_X, const DLArrayHandle bn_scale,
+                                   const DLArrayHandle bn_bias, DLArrayHandle output_Y, float momentum, float eps,
+                                   DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                                   DLStreamHandle stream_handle, ProfilerHandle p) {
+  (void)momentum;
+  TS_REQUIRE(input_X && bn_scale && bn_bias && output_Y, "BatchNorm: NULL array");
+  TS_REQUIRE(input_X->ndim == 4 && output_Y->ndim == 4, "BatchNorm: input and output must be 4-D NCHW");
+  TS_REQUIRE(numel(input_X) == numel(output_Y), "BatchNorm: input/output sizes differ");
+  const int64_t C = input_X->shape[1];
+  TS_REQUIRE(numel(bn_scale) == C && numel(bn_bias) == C, "BatchNorm: scale/bias must hold C=%lld elements", (long long)C);
+  TS_REQUIRE(!save_mean_arr || numel(save_mean_arr) == C, "BatchNorm: save_mean must hold C elements");
+  TS_REQUIRE(!save_var_arr || numel(save_var_arr) == C, "BatchNorm: save_var must hold C elements");
+  hipStream_t s = stream_of(stream_handle);
+  const bool al = aligned16(input_X->data) && aligned16(output_Y->data);
+  Plan st, ap;
+  TS_REQUIRE(make_plan(input_X, al, 64 * kThreads, 4096, st), "BatchNorm: unsupported shape");
+  TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 1 << 20, ap), "BatchNorm: unsupported shape");
+  double *part = static_cast<double *>(scratch_get(s, 1, static_cast<size_t>(C) * st.S * 2 * sizeof(double)));
+  TS_REQUIRE(part, "BatchNorm: no scratch memory");
+  ProfileScope ps(p, s, numel(input_X) + 2 * C, numel(output_Y), C * st.S * 4);
+  const double inv_m = 1.0 / static_cast<double>(st.m);
+  float *sm = save_mean_arr ? mf(save_mean_arr) : nullptr;
+  float *sv = save_var_arr ? mf(save_var_arr) : nullptr;
+  dim3 gs(st.S, static_cast<unsigned>(C)), ga(ap.S, static_cast<unsigned>(C));
+  if (st.vec == 4) {
+    hipLaunchKernelGGL(bn_stats_kernel<4>, gs, dim3(kThreads), 0, s, cf(input_X), part, st.g, st.S);
+    hipLaunchKernelGGL(bn_apply_kernel<4>, ga, dim3(kThreads), 0, s, cf(input_X), mf(output_Y), cf(bn_scale),
+                       cf(bn_bias), part, st.S, ap.g, eps, inv_m, sm, sv);
+  } else {
+    hipLaunchKernelGGL(bn_stats_kernel<1>, gs, dim3(kThreads), 0, s, cf(input_X), part, st.g, st.S);
+    hipLaunchKernelGGL(bn_apply_kernel<1>, ga, dim3(kThreads), 0, s, cf(input_X), mf(output_Y), cf(bn_scale),
+                       cf(bn_bias), part, st.S, ap.g, eps, inv_m, sm, sv);
+  }
+  return ps.finish();
+}
+
+int CuDNN_DLGpuBatch_Normalization_gradient(const DLArrayHandle gradient_Y, const DLArrayHandle input_X,
+                                            const DLArrayHandle bn_scale, DLArrayHandle gradient_X,
+                                            DLArrayHandle gradient_bn_scale, DLArrayHandle gradient_bn_bias,
+                                            float eps, DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                                            DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(gradient_Y && input_X && bn_scale && gradient_X, "BatchNorm gradient: NULL array");
+  TS_REQUIRE(input_X->ndim == 4, "BatchNorm gradient: input must be 4-D NCHW");
+  TS_REQUIRE(numel(input_X) == numel(gradient_Y) && numel(input_X) == numel(gradient_X),
+             "BatchNorm gradient: x, dy, dx sizes differ");
+  const int64_t C = input_X->shape[1];
+  TS_REQUIRE(numel(bn_scale) == C, "BatchNorm gradient: scale must hold C elements");
+  TS_REQUIRE(!gradient_bn_scale || numel(gradient_bn_scale) == C, "BatchNorm gradient: dscale must hold C elements");
+  TS_REQUIRE(!gradient_bn_bias || numel(gradient_bn_bias) == C, "BatchNorm gradient: dbias must hold C elements");
+  const bool saved = save_mean_arr && save_var_arr;
+  TS_REQUIRE(!saved || (numel(save_mean_arr) == C && numel(save_var_arr) == C),
+             "BatchNorm gradient: saved statistics must hold C elements");
+  hipStream_t s = stream_of(stream_handle);
+  const bool al = aligned16(input_X->data) && aligned16(gradient_Y->data) && aligned16(gradient_X->data);
+  Plan rd, dxp;
+  TS_REQUIRE(make_plan(input_X, al, 32 * kThreads, 4096, rd), "BatchNorm gradient: unsupported shape");
+  TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 1 << 20, dxp), "BatchNorm gradient: unsupported shape");
+  double *part = static_cast<double *>(scratch_get(s, 1, static_cast<size_t>(C) * rd.S * 4 * sizeof(double)));
+  TS_REQUIRE(part, "BatchNorm gradient: no scratch memory");
+  ProfileScope ps(p, s, 2 * numel(input_X) + C, numel(gradient_X) + 2 * C, C * rd.S * 8);
+  const double inv_m = 1.0 / static_cast<double>(rd.m);
+  const float *sm = saved ? cf(save_mean_arr) : nullptr;
+  const float *sv = saved ? cf(save_var_arr) : nullptr;
+  float *dg = gradient_bn_scale ? mf(gradient_bn_scale) : nullptr;
+  float *db = gradient_bn_bias ? mf(gradient_bn_bias) : nullptr;
+  dim3 gr(rd.S, static_cast<unsigned>(C)), gd(dxp.S, static_cast<unsigned>(C));
+#define BN_BWD(V)                                                                                                   \
+  do {                                                                                                              \
+    if (saved)                                                                                                      \
+      hipLaunchKernelGGL((bn_bwd_reduce_kernel<V, false>), gr, dim3(kThreads), 0, s, cf(gradient_Y), cf(input_X),   \
+                         part, rd.g, rd.S);                                                                         \
+    else                                                                                                            \
+      hipLaunchKernelGGL((bn_bwd_reduce_kernel<V, true>), gr, dim3(kThreads), 0, s, cf(gradient_Y), cf(input_X),    \
+                         part, rd.g, rd.S);                                                                         \
+    hipLaunchKernelGGL(bn_bwd_dx_kernel<V>, gd, dim3(kThreads), 0, s, cf(gradient_Y), cf(input_X), mf(gradient_X),  \
+                       cf(bn_scale), part, rd.S, dxp.g, eps, inv_m, sm, sv, dg, db);                                \
+  } while (0)
+  if (rd.vec == 4)
+    BN_BWD(4);
+  else
+    BN_BWD(1);
+#undef BN_BWD
+  return ps.finish();
+}
+
+}  // extern "C"

@@ -1,0 +1,246 @@
+// MaxPool 2-D forward and backward, NCHW float32.
+//
+// Semantics (src/ops/MaxPool.cu:3-43, python/athena/gpu_ops/MaxPool.py:8-68): the window is
+// clipped to the image, the maximum is the first strict maximum in row-major scan order.
+// The backward pass is a gather: one thread per input element looks at the (at most
+// ceil(k/s)^2) windows that contain it, recomputes each window's argmax and adds that
+// window's dy when the argmax is this element -- in ascending window order, which is the
+// accumulation order of the reference's scatter loop, without atomics and without a
+// separate zero-fill pass (every dx element is written exactly once).
+// The 2x2 / stride 2 / no padding case (every VGG pool) has a vectorised path: a thread
+// owns two adjacent windows, i.e. one 16-byte word from each of two input rows.
+#include "common.h"
+
+namespace tsplit {
+namespace {
+
+constexpr int kThreads = 256;
+
+struct PoolGeo {
+  int H, W, pH, pW, kH, kW, pad, stride;
+};
+
+__device__ __forceinline__ int window_argmax(const float *__restrict__ plane, const PoolGeo &g, int oh, int ow) {
+  int hs = oh * g.stride - g.pad, ws = ow * g.stride - g.pad;
+  const int he = min(hs + g.kH, g.H), we = min(ws + g.kW, g.W);
+  hs = max(hs, 0);
+  ws = max(ws, 0);
+  int best = hs * g.W + ws;
+  float bv = plane[best];
+  for (int i = hs; i < he; ++i)
+    for (int j = ws; j < we; ++j) {
+      const float v = plane[i * g.W + j];
+      if (v > bv) {
+        bv = v;
+        best = i * g.W + j;
+      }
+    }
+  return best;
+}
+
+__global__ __launch_bounds__(kThreads) void pool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                            PoolGeo g, int64_t total) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx >= total) return;
+  const int ow = static_cast<int>(idx % g.pW);
+  const int64_t t = idx / g.pW;
+  const int oh = static_cast<int>(t % g.pH);
+  const int64_t nc = t / g.pH;
+  const float *plane = x + nc * g.H * g.W;
+  y[idx] = plane[window_argmax(plane, g, oh, ow)];
+}
+
+__global__ __launch_bounds__(kThreads) void pool_bwd_kernel(const float *__restrict__ x, const float *__restrict__ dy,
+                                                            float *__restrict__ dx, PoolGeo g, int64_t total) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx >= total) return;
+  const int w = static_cast<int>(idx % g.W);
+  const int64_t t = idx / g.W;
+  const int h = static_cast<int>(t % g.H);
+  const int64_t nc = t / g.H;
+  const float *plane = x + nc * g.H * g.W;
+  const float *dplane = dy + nc * g.pH * g.pW;
+  // windows oh with oh*s - pad <= h < oh*s - pad + kH
+  const int oh_lo = max(0, (h + g.pad - g.kH + g.stride) / g.stride);   // ceil((h+pad-kH+1)/s) for the non-negative case
+  const int oh_hi = min(g.pH - 1, (h + g.pad) / g.stride);
+  const int ow_lo = max(0, (w + g.pad - g.kW + g.stride) / g.stride);
+  const int ow_hi = min(g.pW - 1, (w + g.pad) / g.stride);
+  const int me = h * g.W + w;
+  float acc = 0.f;
+  for (int oh = oh_lo; oh <= oh_hi; ++oh)
+    for (int ow = ow_lo; ow <= ow_hi; ++ow)
+      if (window_argmax(plane, g, oh, ow) == me) acc += dplane[oh * g.pW + ow];
+  dx[idx] = acc;
+}
+
+// ---- 2x2 stride 2 pad 0, W % 4 == 0, H % 2 == 0, 16-byte aligned x/dx and 8-byte aligned y/dy ----
+// thread -> (plane, oh, q): input words (2oh, q) and (2oh+1, q), outputs (oh, 2q) and (oh, 2q+1)
+__global__ __launch_bounds__(kThreads) void pool2x2_fwd_kernel(const float4 *__restrict__ x, float2 *__restrict__ y,
+                                                               int W4, int pH, int64_t total) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx >= total) return;
+  const int q = static_cast<int>(idx % W4);
+  const int64_t row = idx / W4;                 // plane * pH + oh
+  const int64_t in = (row * 2) * W4 + q;        // (plane*H + 2*oh) * W4 + q, H = 2*pH
+  const float4 a = x[in], b = x[in + W4];
+  float2 o;
+  // scan order: (0,0) (0,1) (1,0) (1,1); strict > keeps the first maximum
+  float m = a.x;
+  m = a.y > m ? a.y : m;
+  m = b.x > m ? b.x : m;
+  m = b.y > m ? b.y : m;
+  o.x = m;
+  m = a.z;
+  m = a.w > m ? a.w : m;
+  m = b.z > m ? b.z : m;
+  m = b.w > m ? b.w : m;
+  o.y = m;
+  y[idx] = o;
+}
+
+__device__ __forceinline__ void route2x2(float v00, float v01, float v10, float v11, float g, float &o00, float &o01,
+                                         float &o10, float &o11) {
+  int k = 0;
+  float m = v00;
+  if (v01 > m) { m = v01; k = 1; }
+  if (v10 > m) { m = v10; k = 2; }
+  if (v11 > m) { m = v11; k = 3; }
+  o00 = k == 0 ? g : 0.f;
+  o01 = k == 1 ? g : 0.f;
+  o10 = k == 2 ? g : 0.f;
+  o11 = k == 3 ? g : 0.f;
+}
+
+__global__ __launch_bounds__(kThreads) void pool2x2_bwd_kernel(const float4 *__restrict__ x,
+                                                               const float2 *__restrict__ dy, float4 *__restrict__ dx,
+                                                               int W4, int64_t total) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx >= total) return;
+  const int q = static_cast<int>(idx % W4);
+  const int64_t row = idx / W4;
+  const int64_t in = (row * 2) * W4 + q;
+  const float4 a = x[in], b = x[in + W4];
+  const float2 g = dy[idx];
+  float4 oa, ob;
+  route2x2(a.x, a.y, b.x, b.y, g.x, oa.x, oa.y, ob.x, ob.y);
+  route2x2(a.z, a.w, b.z, b.w, g.y, oa.z, oa.w, ob.z, ob.w);
+  dx[in] = oa;
+  dx[in + W4] = ob;
+}
+
+inline bool aligned8(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 7) == 0; }
+
+int check_geo(const char *who, const DLArray *x, const DLArray *y, int64_t kH, int64_t kW, int64_t pad, int64_t stride,
+              PoolGeo &g) {
+  TS_REQUIRE(x && y, "%s: NULL array", who);
+  TS_REQUIRE(x->ndim == 4 && y->ndim == 4, "%s: arrays must be 4-D NCHW", who);
+  TS_REQUIRE(kH > 0 && kW > 0 && stride > 0 && pad >= 0, "%s: bad kernel/stride/padding", who);
+  TS_REQUIRE(pad < kH && pad < kW, "%s: padding must be smaller than the kernel", who);
+  TS_REQUIRE(x->shape[0] == y->shape[0] && x->shape[1] == y->shape[1], "%s: N,C of input and output differ", who);
+  g.H = static_cast<int>(x->shape[2]);
+  g.W = static_cast<int>(x->shape[3]);
+  g.pH = static_cast<int>(y->shape[2]);
+  g.pW = static_cast<int>(y->shape[3]);
+  g.kH = static_cast<int>(kH);
+  g.kW = static_cast<int>(kW);
+  g.pad = static_cast<int>(pad);
+  g.stride = static_cast<int>(stride);
+  TS_REQUIRE(g.H + 2 * g.pad >= g.kH && g.W + 2 * g.pad >= g.kW, "%s: kernel larger than the padded image", who);
+  const int eh = (g.H + 2 * g.pad - g.kH) / g.stride + 1, ew = (g.W + 2 * g.pad - g.kW) / g.stride + 1;
+  TS_REQUIRE(g.pH == eh && g.pW == ew, "%s: output is %dx%d, expected %dx%d", who, g.pH, g.pW, eh, ew);
+  return 0;
+}
+
+bool fast2x2(const PoolGeo &g, const void *x, const void *y, const void *dx) {
+  return g.kH == 2 && g.kW == 2 && g.stride == 2 && g.pad == 0 && g.W % 4 == 0 && g.H % 2 == 0 && aligned16(x) &&
+         aligned8(y) && (dx == nullptr || aligned16(dx));
+}
+
+int pool_forward(const char *who, const DLArray *x, DLArray *y, int64_t kH, int64_t kW, int64_t pad, int64_t stride,
+                 DLStreamHandle sh, ProfilerHandle p) {
+  PoolGeo g;
+  if (check_geo(who, x, y, kH, kW, pad, stride, g)) return -1;
+  hipStream_t s = stream_of(sh);
+  ProfileScope ps(p, s, numel(x), numel(y), 0);
+  const int64_t planes = x->shape[0] * x->shape[1];
+  if (numel(y) > 0) {
+    if (fast2x2(g, x->data, y->data, nullptr)) {
+      const int64_t total = planes * g.pH * (g.W / 4);
+      hipLaunchKernelGGL(pool2x2_fwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
+                         dim3(kThreads), 0, s, static_cast<const float4 *>(x->data), static_cast<float2 *>(y->data),
+                         g.W / 4, g.pH, total);
+    } else {
+      const int64_t total = numel(y);
+      hipLaunchKernelGGL(pool_fwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
+                         dim3(kThreads), 0, s, static_cast<const float *>(x->data), static_cast<float *>(y->data), g,
+                         total);
+    }
+  }
+  return ps.finish();
+}
+
+int pool_backward(const char *who, const DLArray *x, const DLArray *dy, DLArray *dx, int64_t kH, int64_t kW,
+                  int64_t pad, int64_t stride, DLStreamHandle sh, ProfilerHandle p) {
+  PoolGeo g;
+  TS_REQUIRE(dx, "%s: NULL array", who);
+  if (check_geo(who, x, dy, kH, kW, pad, stride, g)) return -1;
+  TS_REQUIRE(dx->ndim == 4 && numel(dx) == numel(x), "%s: input gradient must have the input's shape", who);
+  hipStream_t s = stream_of(sh);
+  ProfileScope ps(p, s, numel(x) + numel(dy), numel(dx), 0);
+  const int64_t planes = x->shape[0] * x->shape[1];
+  if (numel(dx) > 0) {
+    if (fast2x2(g, x->data, dy->data, dx->data)) {
+      const int64_t total = planes * g.pH * (g.W / 4);
+      hipLaunchKernelGGL(pool2x2_bwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
+                         dim3(kThreads), 0, s, static_cast<const float4 *>(x->data),
+                         static_cast<const float2 *>(dy->data), static_cast<float4 *>(dx->data), g.W / 4, total);
+    } else {
+      const int64_t total = numel(dx);
+      hipLaunchKernelGGL(pool_bwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
+                         dim3(kThreads), 0, s, static_cast<const float *>(x->data),
+                         static_cast<const float *>(dy->data), static_cast<float *>(dx->data), g, total);
+    }
+  }
+  return ps.finish();
+}
+
+}  // namespace
+}  // namespace tsplit
+
+using namespace tsplit;
+
+extern "C" {
+
+int DLGpuMax_Pooling2d(const DLArrayHandle input, const int kernel_H, const int kernel_W, DLArrayHandle output,
+                       const int padding, const int stride, DLStreamHandle stream_handle, ProfilerHandle p) {
+  return pool_forward("DLGpuMax_Pooling2d", input, output, kernel_H, kernel_W, padding, stride, stream_handle, p);
+}
+
+int DLGpuMax_Pooling2d_gradient(const DLArrayHandle input, const DLArrayHandle output_grad, const int kernel_H,
+                                const int kernel_W, DLArrayHandle input_grad, const int padding, const int stride,
+                                DLStreamHandle stream_handle, ProfilerHandle p) {
+  return pool_backward("DLGpuMax_Pooling2d_gradient", input, output_grad, input_grad, kernel_H, kernel_W, padding,
+                       stride, stream_handle, p);
+}
+
+int CuDNN_DLGpuMax_Pooling2d(const DLArrayHandle input, const size_t kernel_H, const size_t kernel_W,
+                             DLArrayHandle output, const size_t padding, const size_t stride,
+                             DLStreamHandle stream_handle, ProfilerHandle p) {
+  return pool_forward("CuDNN_DLGpuMax_Pooling2d", input, output, static_cast<int64_t>(kernel_H),
+                      static_cast<int64_t>(kernel_W), static_cast<int64_t>(padding), static_cast<int64_t>(stride),
+                      stream_handle, p);
+}
+
+int CuDNN_DLGpuMax_Pooling2d_gradient(const DLArrayHandle output_Y, const DLArrayHandle gradient_Y,
+                                      const DLArrayHandle input_X, const size_t kernel_H, const size_t kernel_W,
+                                      DLArrayHandle gradient_X, const size_t padding, const size_t stride,
+                                      DLStreamHandle stream_handle, ProfilerHandle p) {
+  // output_Y is not needed: the argmax is recomputed from input_X (first strict maximum), which
+  // is what the plain symbol does and what the numpy reference defines.
+  (void)output_Y;
+  return pool_backward("CuDNN_DLGpuMax_Pooling2d_gradient", input_X, gradient_Y, gradient_X,
+                       static_cast<int64_t>(kernel_H), static_cast<int64_t>(kernel_W), static_cast<int64_t>(padding),
+                       static_cast<int64_t>(stride), stream_handle, p);
+}
+
+}  // extern "C"
