@@ -1,0 +1,84 @@
+// DLGpuMatrixMultiply: row-major 2-D C = op(A) op(B) on the fp32 MFMA tile engine.
+//
+// The four transpose combinations only change which loader stages each operand (a
+// transposed operand is simply one whose other index is contiguous); nothing is ever
+// transposed in memory.  Skinny problems (M <= 64, the fully-connected layers at batch 64)
+// use 64x256 tiles; when the tile count cannot fill 256 CUs the K range is split across
+// blocks and folded by a second deterministic kernel (the 64x25088x4096 layer streams a
+// 392 MiB weight matrix and needs every CU pulling on HBM).
+#include "common.h"
+#include "mfma_gemm.h"
+
+namespace tsplit {
+namespace {
+
+using namespace mg;
+
+template <int BM, int BN, int WM, int WN, bool TA, bool TB>
+int launch_gemm(const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int M, int N, int K,
+                hipStream_t s, int64_t *ws_elems) {
+  using AL = typename std::conditional<TA, MnContigLoader<BM>, KContigLoader<BM>>::type;
+  using BL = typename std::conditional<TB, KContigLoader<BN>, MnContigLoader<BN>>::type;
+  typename AL::Params ap{A, lda, M, lda % 4 == 0 && aligned16(A)};
+  typename BL::Params bp{B, ldb, N, ldb % 4 == 0 && aligned16(B)};
+  const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+  int S, kchunk;
+  plan_splitk(tm * tn, K, 64, S, kchunk);
+  float *out = C;
+  const int64_t mn = static_cast<int64_t>(M) * N;
+  if (S > 1) {
+    out = static_cast<float *>(scratch_get(s, 2, static_cast<size_t>(S) * mn * 4));
+    TS_REQUIRE(out, "DLGpuMatrixMultiply: no scratch memory for split-K");
+    *ws_elems = S * mn;
+  }
+  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>), dim3(tn, tm, S), dim3(kThreads), 0, s,
+                     ap, bp, out, mn, static_cast<int64_t>(N), RowMajorCols{}, M, N, K, kchunk);
+  if (S > 1)
+    hipLaunchKernelGGL(splitk_fold_kernel, dim3(static_cast<unsigned>((mn + 255) / 256)), dim3(256), 0, s, out, C, mn,
+                       mn, S);
+  return 0;
+}
+
+template <bool TA, bool TB>
+int dispatch_tile(const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int M, int N, int K,
+                  hipStream_t s, int64_t *ws) {
+  if (M <= 64) return launch_gemm<64, 256, 1, 4, TA, TB>(A, lda, B, ldb, C, M, N, K, s, ws);
+  return launch_gemm<128, 128, 2, 2, TA, TB>(A, lda, B, ldb, C, M, N, K, s, ws);
+}
+
+}  // namespace
+}  // namespace tsplit
+
+using namespace tsplit;
+
+extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, const DLArrayHandle matB,
+                                   bool transposeB, DLArrayHandle matC, DLStreamHandle stream_handle,
+                                   ProfilerHandle p) {
+  TS_REQUIRE(matA && matB && matC, "DLGpuMatrixMultiply: NULL array");
+  TS_REQUIRE(matA->ndim == 2 && matB->ndim == 2 && matC->ndim == 2, "DLGpuMatrixMultiply: 2-D arrays only");
+  const int64_t M = matC->shape[0], N = matC->shape[1];
+  const int64_t K = transposeA ? matA->shape[0] : matA->shape[1];
+  const int64_t Am = transposeA ? matA->shape[1] : matA->shape[0];
+  const int64_t Bk = transposeB ? matB->shape[1] : matB->shape[0];
+  const int64_t Bn = transposeB ? matB->shape[0] : matB->shape[1];
+  TS_REQUIRE(Am == M && Bn == N && Bk == K, "DLGpuMatrixMultiply: shapes do not conform: op(A) %lldx%lld, op(B) %lldx%lld, C %lldx%lld",
+             (long long)Am, (long long)K, (long long)Bk, (long long)Bn, (long long)M, (long long)N);
+  TS_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) - 64, "DLGpuMatrixMultiply: dimension too large");
+  hipStream_t s = stream_of(stream_handle);
+  int64_t ws = 0;
+  ProfileScope ps(p, s, numel(matA) + numel(matB), M * N, 0);
+  int rc = 0;
+  if (M > 0 && N > 0) {
+    const float *A = static_cast<const float *>(matA->data), *B = static_cast<const float *>(matB->data);
+    float *C = static_cast<float *>(matC->data);
+    const int64_t lda = matA->shape[1], ldb = matB->shape[1];
+    const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
+    if (!transposeA && !transposeB) rc = dispatch_tile<false, false>(A, lda, B, ldb, C, m, n, k, s, &ws);
+    if (!transposeA && transposeB) rc = dispatch_tile<false, true>(A, lda, B, ldb, C, m, n, k, s, &ws);
+    if (transposeA && !transposeB) rc = dispatch_tile<true, false>(A, lda, B, ldb, C, m, n, k, s, &ws);
+    if (transposeA && transposeB) rc = dispatch_tile<true, true>(A, lda, B, ldb, C, m, n, k, s, &ws);
+  }
+  if (p) p->workspace_memory = mib(ws);
+  if (rc) return rc;
+  return ps.finish();
+}

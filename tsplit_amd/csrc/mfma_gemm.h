@@ -1,0 +1,291 @@
+// fp32 MFMA tile engine shared by MatMul and the three convolutions.
+//
+// D[M,N] = A[M,K] * B[K,N] with v_mfma_f32_32x32x2_f32.  A block of 256 threads (4 waves)
+// owns a BM x BN tile; each wave owns a 64x64 sub-tile = 2x2 MFMA blocks (64 accumulator
+// VGPRs), so one k-pair costs 2+2 operand registers for 4 MFMAs.  K advances in steps of
+// BK = 16 through double-buffered LDS: the loads of step t+1 are issued before the MFMAs of
+// step t and parked in registers, then written to the other LDS stage; one barrier per step.
+//
+// Each operand is staged in LDS in the orientation it has in memory, never transposed:
+//   * "k-major"  [BK][MN+8]  for operands whose M/N index is contiguous in memory
+//   * "mn-major" [MN][BK+4]  for operands whose K index is contiguous in memory
+// This works because an MFMA only needs both operands to agree on WHICH k each lane
+// supplies, not on the order: within a 16-wide step, lanes 0-31 supply k = 8j+i and lanes
+// 32-63 supply k = 8j+4+i (j = 0,1; i = 0..3).  An mn-major operand then reads its four
+// values with one 16-byte LDS read per lane; a k-major one with four 4-byte reads that are
+// conflict-free because consecutive lanes touch consecutive addresses.
+//
+// Operand loaders (global -> registers -> LDS) are policy classes; the convolutions plug in
+// gather loaders that compute im2col addresses on the fly.  The epilogue writes
+// out[row_stride * m + colmap(n)], which covers row-major matrices, NCHW activations and the
+// split-K partial buffers alike.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace tsplit {
+namespace mg {
+
+constexpr int BK = 16;
+constexpr int kThreads = 256;
+constexpr int kMnPad = 8;   // k-major rows: MN + 8 floats
+constexpr int kKPad = 4;    // mn-major rows: BK + 4 floats
+
+typedef float acc16 __attribute__((ext_vector_type(16)));
+
+template <int MN>
+struct KMajorLds {   // [BK][MN + 8]
+  static constexpr int kStride = MN + kMnPad;
+  static constexpr int kFloats = BK * kStride;
+  // the 4 k-values (group j) this lane supplies for the 32-wide block starting at mn0
+  static __device__ __forceinline__ void frag(const float *lds, int mn0, int j, int lane, float (&v)[4]) {
+    const float *p = lds + (8 * j + 4 * (lane >> 5)) * kStride + mn0 + (lane & 31);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = p[i * kStride];
+  }
+};
+
+template <int MN>
+struct MnMajorLds {  // [MN][BK + 4]
+  static constexpr int kStride = BK + kKPad;
+  static constexpr int kFloats = MN * kStride;
+  static __device__ __forceinline__ void frag(const float *lds, int mn0, int j, int lane, float (&v)[4]) {
+    const float4 q = *reinterpret_cast<const float4 *>(lds + (mn0 + (lane & 31)) * kStride + 8 * j + 4 * (lane >> 5));
+    v[0] = q.x;
+    v[1] = q.y;
+    v[2] = q.z;
+    v[3] = q.w;
+  }
+};
+
+// ------------------------------------------------------------------ dense-matrix loaders
+// Operand whose K index is contiguous: element (mn, k) at p[mn * ld + k].
+template <int MN>
+struct KContigLoader {
+  using Lds = MnMajorLds<MN>;
+  struct Params {
+    const float *p;
+    int64_t ld;
+    int mn_total;
+    bool vec;   // ld % 4 == 0 and p 16-byte aligned
+  };
+  static constexpr int kPasses = MN / 64;   // 64 rows x 4 quads per pass
+  float4 r[kPasses];
+  const float *base[kPasses];
+  bool row_ok[kPasses];
+  int kq;
+  bool vec;
+
+  __device__ __forceinline__ void init(const Params &P, int mn0, int tid) {
+    kq = tid & 3;
+    vec = P.vec;
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s) {
+      const int row = mn0 + (tid >> 2) + 64 * s;
+      row_ok[s] = row < P.mn_total;
+      base[s] = P.p + static_cast<int64_t>(row_ok[s] ? row : 0) * P.ld;
+    }
+  }
+  __device__ __forceinline__ void load(int k0, int kend) {
+    const int k = k0 + 4 * kq;
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (row_ok[s]) {
+        if (vec && k + 3 < kend) {
+          v = *reinterpret_cast<const float4 *>(base[s] + k);
+        } else {
+          if (k < kend) v.x = base[s][k];
+          if (k + 1 < kend) v.y = base[s][k + 1];
+          if (k + 2 < kend) v.z = base[s][k + 2];
+          if (k + 3 < kend) v.w = base[s][k + 3];
+        }
+      }
+      r[s] = v;
+    }
+  }
+  __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s)
+      *reinterpret_cast<float4 *>(lds + ((tid >> 2) + 64 * s) * Lds::kStride + 4 * kq) = r[s];
+  }
+};
+
+// Operand whose M/N index is contiguous: element (k, mn) at p[k * ld + mn].
+template <int MN>
+struct MnContigLoader {
+  using Lds = KMajorLds<MN>;
+  struct Params {
+    const float *p;
+    int64_t ld;
+    int mn_total;
+    bool vec;
+  };
+  static constexpr int kQuads = MN / 4;                 // 16-byte words per row
+  static constexpr int kRowsPerPass = kThreads / kQuads;
+  static constexpr int kPasses = BK / kRowsPerPass;
+  float4 r[kPasses];
+  const float *p;
+  int64_t ld;
+  int col, krow, ncols;   // first column of this thread's word, row within a pass, valid columns
+  bool vec;
+
+  __device__ __forceinline__ void init(const Params &P, int mn0, int tid) {
+    p = P.p;
+    ld = P.ld;
+    vec = P.vec;
+    col = mn0 + 4 * (tid % kQuads);
+    krow = tid / kQuads;
+    ncols = P.mn_total - col;   // <= 0: nothing valid
+  }
+  __device__ __forceinline__ void load(int k0, int kend) {
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s) {
+      const int k = k0 + krow + s * kRowsPerPass;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (k < kend && ncols > 0) {
+        const float *q = p + static_cast<int64_t>(k) * ld + col;
+        if (vec && ncols >= 4) {
+          v = *reinterpret_cast<const float4 *>(q);
+        } else {
+          v.x = q[0];
+          if (ncols > 1) v.y = q[1];
+          if (ncols > 2) v.z = q[2];
+          if (ncols > 3) v.w = q[3];
+        }
+      }
+      r[s] = v;
+    }
+  }
+  __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s)
+      *reinterpret_cast<float4 *>(lds + (krow + s * kRowsPerPass) * Lds::kStride + 4 * (tid % kQuads)) = r[s];
+  }
+};
+
+// ------------------------------------------------------------------ column maps
+struct RowMajorCols {   // out[m * row_stride + n]
+  __device__ __forceinline__ int64_t operator()(int n) const { return n; }
+};
+
+// ------------------------------------------------------------------ the kernel
+// grid: x = N tiles, y = M tiles, z = K splits.  Split z writes to out + z * z_stride.
+template <int BM, int BN, int WM, int WN, class ALoader, class BLoader, class ColMap>
+__global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::Params ap, typename BLoader::Params bp,
+                                                             float *__restrict__ out, int64_t z_stride,
+                                                             int64_t row_stride, ColMap colmap, int M, int N, int K,
+                                                             int kchunk) {
+  static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
+  using ALds = typename ALoader::Lds;
+  using BLds = typename BLoader::Lds;
+  __shared__ __attribute__((aligned(16))) float lds_a[2][ALds::kFloats];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][BLds::kFloats];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
+  const int kbegin = blockIdx.z * kchunk;
+  const int kend = min(K, kbegin + kchunk);
+
+  ALoader la;
+  BLoader lb;
+  la.init(ap, m0, tid);
+  lb.init(bp, n0, tid);
+
+  acc16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  if (kbegin < kend) {
+    la.load(kbegin, kend);
+    lb.load(kbegin, kend);
+    la.store(lds_a[0], tid);
+    lb.store(lds_b[0], tid);
+  }
+  __syncthreads();
+
+  int stage = 0;
+  for (int k0 = kbegin; k0 < kend; k0 += BK) {
+    const bool more = k0 + BK < kend;
+    if (more) {
+      la.load(k0 + BK, kend);
+      lb.load(k0 + BK, kend);
+    }
+    const float *sa = lds_a[stage], *sb = lds_b[stage];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      float fa[2][4], fb[2][4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        ALds::frag(sa, wm0 + 32 * i, j, lane, fa[i]);
+        BLds::frag(sb, wn0 + 32 * i, j, lane, fb[i]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < 2; ++ni)
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
+    }
+    if (more) {
+      la.store(lds_a[stage ^ 1], tid);
+      lb.store(lds_b[stage ^ 1], tid);
+    }
+    __syncthreads();
+    stage ^= 1;
+  }
+
+  // epilogue: accumulator register e of a 32x32 block holds row 8*(e/4) + 4*(lane/32) + e%4,
+  // column lane%32
+  float *o = out + static_cast<int64_t>(blockIdx.z) * z_stride;
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const int n = n0 + wn0 + 32 * ni + (lane & 31);
+    if (n >= N) continue;
+    const int64_t coff = colmap(n);
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+      const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = mb + 8 * (e >> 2) + (e & 3);
+        if (m < M) o[static_cast<int64_t>(m) * row_stride + coff] = acc[mi][ni][e];
+      }
+    }
+  }
+}
+
+// out[i] = sum_z part[z * stride + i], z ascending (deterministic split-K fold)
+__global__ __launch_bounds__(256) void splitk_fold_kernel(const float *__restrict__ part, float *__restrict__ out,
+                                                          int64_t n, int64_t stride, int S) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n) return;
+  float s = part[i];
+  for (int z = 1; z < S; ++z) s += part[z * stride + i];
+  out[i] = s;
+}
+
+// How many K splits to use so that the launch fills the chip; kchunk is a multiple of BK.
+inline void plan_splitk(int tiles, int K, int max_split, int &S, int &kchunk) {
+  const int target = 2 * 256;   // about two blocks per CU
+  int s = tiles >= target ? 1 : (target + tiles - 1) / tiles;
+  const int ksteps = (K + BK - 1) / BK;
+  if (s > ksteps / 4) s = ksteps / 4;   // at least 4 k-steps per split
+  if (s > max_split) s = max_split;
+  if (s < 1) s = 1;
+  int per = (ksteps + s - 1) / s;
+  if (per < 1) per = 1;
+  kchunk = per * BK;
+  S = (K + kchunk - 1) / kchunk;
+  if (S < 1) S = 1;
+}
+
+}  // namespace mg
+}  // namespace tsplit
