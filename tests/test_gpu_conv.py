@@ -1,0 +1,124 @@
+"""GPU parity of the three convolutions (implicit GEMM on fp32 MFMA) against the CPU oracle,
+through both symbol families.  Tolerance 2e-3 max relative error; measured errors are ~1e-6."""
+import numpy as np
+import pytest
+
+from oracle import ops as O
+from util import assert_close
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+CASES = [
+    # N, C, H, W, O, kH, kW, ph, pw, stride
+    (2, 3, 6, 6, 4, 3, 3, 1, 1, 1),
+    (1, 2, 7, 7, 3, 3, 3, 1, 1, 2),
+    (2, 2, 8, 8, 3, 3, 3, 1, 1, 2),        # stride 2 with flooring
+    (1, 3, 9, 9, 2, 7, 7, 3, 3, 2),        # ResNet stem class
+    (1, 2, 5, 8, 3, 1, 7, 0, 3, 1),        # 1x7, asymmetric padding
+    (1, 2, 8, 5, 3, 7, 1, 3, 0, 1),        # 7x1
+    (2, 4, 5, 5, 3, 1, 1, 0, 0, 1),        # 1x1
+    (1, 2, 6, 6, 2, 3, 3, 0, 0, 1),        # valid
+    (2, 3, 32, 32, 64, 3, 3, 1, 1, 1),     # VGG conv1_1 class: K = 27, 64x256 tiles
+    (2, 64, 28, 28, 64, 3, 3, 1, 1, 1),    # 64 -> 64
+    (4, 64, 56, 56, 128, 3, 3, 1, 1, 1),   # 128x128 tiles
+    (2, 128, 14, 14, 256, 3, 3, 1, 1, 1),  # two M tiles, N = 392 (ragged)
+    (3, 20, 17, 13, 70, 3, 3, 1, 1, 1),    # everything ragged
+    (2, 16, 15, 15, 24, 3, 3, 1, 1, 2),    # stride 2, odd output 8x8
+    (2, 8, 7, 7, 40, 1, 1, 0, 0, 1),       # oH*oW = 49: not a multiple of 4
+    (2, 6, 12, 12, 130, 5, 5, 2, 2, 1),
+]
+
+
+def _run(case, family, rng):
+    from tsplit_amd import gpu_links as L, ndarray
+    ctx = ndarray.gpu(0)
+    N, C, H, W, Oc, kH, kW, ph, pw, s = case
+    x = rng.normal(size=(N, C, H, W)).astype(np.float32)
+    w = (rng.normal(size=(Oc, C, kH, kW)) / np.sqrt(C * kH * kW)).astype(np.float32)
+    ref_y = O.conv2d(x, w, ph, pw, s)
+    dy = rng.normal(size=ref_y.shape).astype(np.float32)
+    gx, gw, gdy = ndarray.array(x, ctx), ndarray.array(w, ctx), ndarray.array(dy, ctx)
+    y, dx, dw = ndarray.empty(ref_y.shape, ctx), ndarray.empty(x.shape, ctx), ndarray.empty(w.shape, ctx)
+    if family == "cudnn":
+        L.CuDNN_conv2d(gx, gw, y, ph, pw, s)
+        L.CuDNN_conv2d_gradient_of_data(gw, gdy, dx, ph, pw, s)
+        L.CuDNN_conv2d_gradient_of_filter(gx, gdy, dw, ph, pw, s)
+    else:
+        ws = ndarray.empty((1,), ctx)          # the im2col workspaces are accepted and unused
+        L.conv2d(gx, gw, y, ws, ph, s)
+        L.conv2d_gradient_of_data(gw, gdy, dx, ws, ph, s)
+        L.conv2d_gradient_of_filter(gx, gdy, dw, ws, ws, ph, s)
+    e1 = assert_close(y.asnumpy(), ref_y, TOL, f"conv fwd {case}")
+    e2 = assert_close(dx.asnumpy(), O.conv2d_grad_data(w, dy, x.shape, ph, pw, s), TOL, f"conv bwd-data {case}")
+    e3 = assert_close(dw.asnumpy(), O.conv2d_grad_filter(x, dy, w.shape, ph, pw, s), TOL, f"conv bwd-filter {case}")
+    assert max(e1, e2, e3) < 1e-4
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_conv_cudnn_family(case, rng):
+    _run(case, "cudnn", rng)
+
+
+@pytest.mark.parametrize("case", [c for c in CASES if c[7] == c[8]][:8])
+def test_conv_plain_family(case, rng):
+    _run(case, "plain", rng)
+
+
+def test_conv_micro_tensor_split_is_bit_identical(rng):
+    """Conv is per-sample: running it on 4 batch views gives exactly the unsplit result."""
+    from tsplit_amd import gpu_links as L, ndarray
+    ctx = ndarray.gpu(0)
+    x = rng.normal(size=(8, 16, 20, 20)).astype(np.float32)
+    w = rng.normal(size=(32, 16, 3, 3)).astype(np.float32)
+    gx, gw = ndarray.array(x, ctx), ndarray.array(w, ctx)
+    whole, parts = ndarray.empty((8, 32, 20, 20), ctx), ndarray.empty((8, 32, 20, 20), ctx)
+    L.CuDNN_conv2d(gx, gw, whole, 1, 1, 1)
+    gx.split_tensor(4); parts.split_tensor(4)
+    for i in range(4):
+        L.CuDNN_conv2d(gx.sTensor[i], gw, parts.sTensor[i], 1, 1, 1)
+    np.testing.assert_array_equal(whole.asnumpy(), parts.asnumpy())
+
+
+def test_conv_full_size_properties(rng):
+    """Size-independent checks at a full VGG layer shape (64 x 64 x 224 x 224 -> 64, 236.8 GFLOP):
+    a delta filter copies one input channel (exact), and the adjoint identity
+    <conv(x,w),dy> = <x,bwd_data(w,dy)> = <w,bwd_filter(x,dy)> holds."""
+    from tsplit_amd import gpu_links as L, ndarray
+    ctx = ndarray.gpu(0)
+    shape = (64, 64, 224, 224)
+    # build inputs on the host in float32 without large temporaries
+    x = rng.standard_normal(size=shape).astype(np.float32)
+    gx = ndarray.array(x, ctx)
+    w = np.zeros((64, 64, 3, 3), np.float32)
+    perm = rng.permutation(64)
+    w[np.arange(64), perm, 1, 1] = 1.0            # output channel o = input channel perm[o]
+    y = ndarray.empty(shape, ctx)
+    L.CuDNN_conv2d(gx, ndarray.array(w, ctx), y, 1, 1, 1)
+    got = y.asnumpy()
+    assert np.array_equal(got, x[:, perm])
+    del got
+    w2 = (rng.standard_normal(size=(64, 64, 3, 3)) / 24.0).astype(np.float32)
+    gw2 = ndarray.array(w2, ctx)
+    L.CuDNN_conv2d(gx, gw2, y, 1, 1, 1)
+    yv = y.asnumpy()
+    dy = rng.standard_normal(size=shape).astype(np.float32)
+    gdy = ndarray.array(dy, ctx)
+    lhs = float(np.vdot(yv.astype(np.float64, copy=False).ravel(), dy.ravel())) if False else float(
+        np.sum(yv.reshape(64, -1).astype(np.float64) * dy.reshape(64, -1)))
+    dx, dw = ndarray.empty(shape, ctx), ndarray.empty(w2.shape, ctx)
+    L.CuDNN_conv2d_gradient_of_data(gw2, gdy, dx, 1, 1, 1)
+    L.CuDNN_conv2d_gradient_of_filter(gx, gdy, dw, 1, 1, 1)
+    r1 = float(np.sum(dx.asnumpy().reshape(64, -1).astype(np.float64) * x.reshape(64, -1)))
+    r2 = float(np.sum(dw.asnumpy().astype(np.float64) * w2))
+    assert abs(r1 - lhs) <= 1e-4 * abs(lhs) and abs(r2 - lhs) <= 1e-4 * abs(lhs), (lhs, r1, r2)
+
+
+def test_conv_shape_errors():
+    from tsplit_amd import gpu_links as L, ndarray
+    ctx = ndarray.gpu(0)
+    x, w = ndarray.empty((1, 3, 8, 8), ctx), ndarray.empty((4, 3, 3, 3), ctx)
+    with pytest.raises(RuntimeError):
+        L.CuDNN_conv2d(x, w, ndarray.empty((1, 4, 7, 8), ctx), 1, 1, 1)      # wrong output size
+    with pytest.raises(RuntimeError):
+        L.CuDNN_conv2d(x, ndarray.empty((4, 2, 3, 3), ctx), ndarray.empty((1, 4, 8, 8), ctx), 1, 1, 1)

@@ -1,0 +1,518 @@
+// Conv2d forward, backward-data and backward-filter as implicit GEMMs on the fp32 MFMA tile
+// engine.  NCHW activations, OIHW filters, cross-correlation, no bias, square stride,
+// dilation 1, separate (pad_h, pad_w).  No im2col buffer is ever materialised: the gather
+// loaders below compute im2col addresses on the fly while staging tiles into LDS.
+//
+//   forward     y[img,o,p]  : M = O,  N = imgs*oH*oW, K = C*kH*kW
+//                 A = filter [O][K] as it lies in memory (K contiguous)
+//                 B = gather of x: (k=(c,kh,kw), n=(img,oh,ow)) -> x[img,c,oh*s-ph+kh,ow*s-pw+kw]
+//   bwd-data    dx[img,c,q] : M = C,  N = imgs*H*W,   K = O*kH*kW
+//                 A = filter re-laid as [C][O*kH*kW] by a small kernel (<= 9.4 MB per VGG layer)
+//                 B = gather of dy: (k=(o,kh,kw), n=(img,h,w)) -> dy[img,o,(h+ph-kh)/s,(w+pw-kw)/s]
+//   bwd-filter  dw[o,j]     : M = O,  N = C*kH*kW,    K = imgs*oH*oW   (split-K, folded in order)
+//                 A = dy: (m=o, k=(img,p)) -> dy[img,o,p]       (K contiguous inside an image)
+//                 B = gather of x: (k=(img,oh,ow), j=(c,kh,kw)) -> x[img,c,oh*s-ph+kh,ow*s-pw+kw]
+//
+// The (c,kh,kw) -> offset decomposition is a per-geometry table built once on the host and
+// cached on the device; the (img,oh,ow) decomposition uses multiply-shift division and is
+// done once per thread (forward, bwd-data: a thread's columns never change) or once per
+// k-step (bwd-filter).
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <vector>
+
+#include "common.h"
+#include "fastdiv.h"
+#include "mfma_gemm.h"
+
+namespace tsplit {
+namespace {
+
+using namespace mg;
+
+struct ConvGeo {
+  int imgs, C, H, W, O, kH, kW, ph, pw, s, oH, oW;
+};
+
+// one entry per reduction index (c|o, kh, kw)
+struct Tap {
+  int off;      // offset of the tap inside one image of the gathered tensor
+  short kh, kw;
+};
+
+// ------------------------------------------------------------------ tap tables (host cache)
+struct TapKey {
+  int chans, kH, kW, plane_w, plane_hw, sign;
+  bool operator<(const TapKey &o) const {
+    return std::tie(chans, kH, kW, plane_w, plane_hw, sign) <
+           std::tie(o.chans, o.kH, o.kW, o.plane_w, o.plane_hw, o.sign);
+  }
+};
+std::map<TapKey, Tap *> g_taps;
+std::mutex g_taps_mu;
+
+// off = ch*plane_hw + sign*(kh*plane_w + kw)
+const Tap *tap_table(int chans, int kH, int kW, int plane_w, int plane_hw, int sign) {
+  std::lock_guard<std::mutex> lk(g_taps_mu);
+  TapKey key{chans, kH, kW, plane_w, plane_hw, sign};
+  auto it = g_taps.find(key);
+  if (it != g_taps.end()) return it->second;
+  std::vector<Tap> h(static_cast<size_t>(chans) * kH * kW);
+  size_t i = 0;
+  for (int c = 0; c < chans; ++c)
+    for (int a = 0; a < kH; ++a)
+      for (int b = 0; b < kW; ++b, ++i) {
+        h[i].off = c * plane_hw + sign * (a * plane_w + b);
+        h[i].kh = static_cast<short>(a);
+        h[i].kw = static_cast<short>(b);
+      }
+  Tap *d = nullptr;
+  if (hipMalloc(&d, h.size() * sizeof(Tap)) != hipSuccess) return nullptr;
+  if (hipMemcpy(d, h.data(), h.size() * sizeof(Tap), hipMemcpyHostToDevice) != hipSuccess) return nullptr;
+  g_taps[key] = d;
+  return d;
+}
+
+// ------------------------------------------------------------------ gather loader, k-major
+// Serves forward (gathers x) and bwd-data (gathers dy).  Column n = (img, r, c) of the GEMM
+// output; reduction index k = (ch, kh, kw).
+//   forward : src row = r*s - ph + kh           (always "divisible")
+//   bwd-data: src row = (r + ph - kh) / s       valid only when divisible and inside
+template <int BN, bool BWD_DATA>
+struct GatherColsLoader {
+  using Lds = KMajorLds<BN>;
+  struct Params {
+    const float *src;     // x (forward) or dy (bwd-data)
+    const Tap *taps;
+    FastDiv plane;        // columns per image: oH*oW (forward) or H*W (bwd-data)
+    FastDiv width;        // oW (forward) or W (bwd-data)
+    int64_t img_stride;   // elements per image of src
+    int src_h, src_w;     // extent of one plane of src
+    int ph, pw, s;
+    int n_total;
+  };
+  static constexpr int kPerThread = BN / 16;          // 16 * BN / 256
+  static constexpr int kKStep = kThreads / BN;        // 2 (BN=128) or 1 (BN=256)
+  float r[kPerThread];
+  const float *base;
+  const Tap *taps;
+  int r0, c0;            // forward: oh*s-ph, ow*s-pw ; bwd-data: h+ph, w+pw
+  int src_h, src_w, s, kfirst;
+  bool col_ok;
+
+  __device__ __forceinline__ void init(const Params &P, int n0, int tid) {
+    const int n = n0 + tid % BN;
+    kfirst = tid / BN;
+    col_ok = n < P.n_total;
+    const uint32_t nn = col_ok ? n : 0;
+    const uint32_t img = P.plane.div(nn);
+    const uint32_t p = nn - img * P.plane.d;
+    const uint32_t row = P.width.div(p);
+    const uint32_t col = p - row * P.width.d;
+    taps = P.taps;
+    src_h = P.src_h;
+    src_w = P.src_w;
+    s = P.s;
+    if (BWD_DATA) {
+      r0 = static_cast<int>(row) + P.ph;
+      c0 = static_cast<int>(col) + P.pw;
+      base = P.src + static_cast<int64_t>(img) * P.img_stride;
+    } else {
+      r0 = static_cast<int>(row) * P.s - P.ph;
+      c0 = static_cast<int>(col) * P.s - P.pw;
+      base = P.src + static_cast<int64_t>(img) * P.img_stride + static_cast<int64_t>(r0) * P.src_w + c0;
+    }
+  }
+  __device__ __forceinline__ void load(int k0, int kend) {
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) {
+      const int k = k0 + kfirst + kKStep * i;
+      float v = 0.f;
+      if (col_ok && k < kend) {
+        const Tap t = taps[k];
+        if (BWD_DATA) {
+          int rr = r0 - t.kh, cc = c0 - t.kw;
+          bool ok = rr >= 0 && cc >= 0;
+          if (s != 1) {
+            ok = ok && (rr % s == 0) && (cc % s == 0);
+            rr /= s;
+            cc /= s;
+          }
+          // tap offset already holds the channel part; the spatial part is recomputed here
+          if (ok && rr < src_h && cc < src_w)
+            v = base[static_cast<int64_t>(t.off) + static_cast<int64_t>(rr) * src_w + cc];
+        } else {
+          const int rr = r0 + t.kh, cc = c0 + t.kw;
+          if (static_cast<unsigned>(rr) < static_cast<unsigned>(src_h) &&
+              static_cast<unsigned>(cc) < static_cast<unsigned>(src_w))
+            v = base[t.off];
+        }
+      }
+      r[i] = v;
+    }
+  }
+  __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) lds[(kfirst + kKStep * i) * Lds::kStride + tid % BN] = r[i];
+  }
+};
+
+// ------------------------------------------------------------------ bwd-filter loaders, mn-major
+// A = dy: row m = output channel, k = (img, p); K contiguous inside an image.
+template <int BM>
+struct DyRowsLoader {
+  using Lds = MnMajorLds<BM>;
+  struct Params {
+    const float *dy;
+    FastDiv plane;     // oH*oW
+    int O;
+    bool vec;          // oH*oW % 4 == 0 and dy 16-byte aligned
+  };
+  static constexpr int kPasses = BM / 64;
+  float4 r[kPasses];
+  const float *dy;
+  FastDiv plane;
+  int O, row0, kq;
+  bool vec;
+
+  __device__ __forceinline__ void init(const Params &P, int m0, int tid) {
+    dy = P.dy;
+    plane = P.plane;
+    O = P.O;
+    vec = P.vec;
+    row0 = m0 + (tid >> 2);
+    kq = tid & 3;
+  }
+  __device__ __forceinline__ float one(int k, int row, int kend) const {
+    if (k >= kend) return 0.f;
+    const uint32_t img = plane.div(k);
+    const uint32_t p = k - img * plane.d;
+    return dy[(static_cast<int64_t>(img) * O + row) * plane.d + p];
+  }
+  __device__ __forceinline__ void load(int k0, int kend) {
+    const int k = k0 + 4 * kq;
+    const uint32_t img = plane.div(k);
+    const uint32_t p = k - img * plane.d;
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s) {
+      const int row = row0 + 64 * s;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (row < O) {
+        if (vec && k + 3 < kend) {
+          v = *reinterpret_cast<const float4 *>(dy + (static_cast<int64_t>(img) * O + row) * plane.d + p);
+        } else {
+          v.x = one(k, row, kend);
+          v.y = one(k + 1, row, kend);
+          v.z = one(k + 2, row, kend);
+          v.w = one(k + 3, row, kend);
+        }
+      }
+      r[s] = v;
+    }
+  }
+  __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s)
+      *reinterpret_cast<float4 *>(lds + ((tid >> 2) + 64 * s) * Lds::kStride + 4 * kq) = r[s];
+  }
+};
+
+// B = gather of x: column j = (c, kh, kw) (fixed per thread), k = (img, oh, ow).
+template <int BN>
+struct GatherRowsLoader {
+  using Lds = MnMajorLds<BN>;
+  struct Params {
+    const float *x;
+    const Tap *taps;
+    FastDiv plane;        // oH*oW
+    FastDiv width;        // oW
+    int64_t img_stride;   // C*H*W
+    int H, W, ph, pw, s;
+    int j_total;
+  };
+  static constexpr int kCols = BN / 16;   // columns per thread
+  float r[kCols];
+  int off[kCols];
+  short kh[kCols], kw[kCols];
+  const float *x;
+  FastDiv plane, width;
+  int64_t img_stride;
+  int H, W, ph, pw, s, klocal;
+
+  __device__ __forceinline__ void init(const Params &P, int j0, int tid) {
+    x = P.x;
+    plane = P.plane;
+    width = P.width;
+    img_stride = P.img_stride;
+    H = P.H;
+    W = P.W;
+    ph = P.ph;
+    pw = P.pw;
+    s = P.s;
+    klocal = tid & 15;
+#pragma unroll
+    for (int i = 0; i < kCols; ++i) {
+      const int j = j0 + (tid >> 4) + 16 * i;
+      if (j < P.j_total) {
+        const Tap t = P.taps[j];
+        off[i] = t.off;
+        kh[i] = t.kh;
+        kw[i] = t.kw;
+      } else {
+        off[i] = 0;
+        kh[i] = -20000;   // fails the range test below for any row
+        kw[i] = 0;
+      }
+    }
+  }
+  __device__ __forceinline__ void load(int k0, int kend) {
+    const int k = k0 + klocal;
+    const bool k_ok = k < kend;
+    const uint32_t kk = k_ok ? k : 0;
+    const uint32_t img = plane.div(kk);
+    const uint32_t p = kk - img * plane.d;
+    const uint32_t oh = width.div(p);
+    const uint32_t ow = p - oh * width.d;
+    const int r0 = static_cast<int>(oh) * s - ph, c0 = static_cast<int>(ow) * s - pw;
+    const float *base = x + static_cast<int64_t>(img) * img_stride + static_cast<int64_t>(r0) * W + c0;
+#pragma unroll
+    for (int i = 0; i < kCols; ++i) {
+      const int rr = r0 + kh[i], cc = c0 + kw[i];
+      float v = 0.f;
+      if (k_ok && static_cast<unsigned>(rr) < static_cast<unsigned>(H) &&
+          static_cast<unsigned>(cc) < static_cast<unsigned>(W))
+        v = base[off[i]];
+      r[i] = v;
+    }
+  }
+  __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+    for (int i = 0; i < kCols; ++i) lds[((tid >> 4) + 16 * i) * Lds::kStride + klocal] = r[i];
+  }
+};
+
+// ------------------------------------------------------------------ NCHW output columns
+struct NchwCols {   // out[img][m][p]: column n = img*plane + p -> img*img_stride + p ; row stride = plane
+  FastDiv plane;
+  int64_t img_stride;
+  __device__ __forceinline__ int64_t operator()(int n) const {
+    const uint32_t img = plane.div(n);
+    return static_cast<int64_t>(img) * img_stride + (n - img * plane.d);
+  }
+};
+
+// filter [O][C][kHW] -> [C][O][kHW]
+__global__ __launch_bounds__(256) void filter_oc_swap_kernel(const float *__restrict__ w, float *__restrict__ wt,
+                                                             int O, int C, int kHW) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= O * C * kHW) return;
+  const int r = idx % kHW;
+  const int t = idx / kHW;
+  const int o = t % O, c = t / O;
+  wt[idx] = w[(o * C + c) * kHW + r];
+}
+
+// ------------------------------------------------------------------ host side
+int geo_from(const char *who, const DLArray *x, const DLArray *w, const DLArray *y, int ph, int pw, int s,
+             ConvGeo &g) {
+  TS_REQUIRE(x && w && y, "%s: NULL array", who);
+  TS_REQUIRE(x->ndim == 4 && w->ndim == 4 && y->ndim == 4, "%s: arrays must be 4-D", who);
+  TS_REQUIRE(s >= 1 && ph >= 0 && pw >= 0, "%s: bad stride/padding", who);
+  g.imgs = static_cast<int>(x->shape[0]);
+  g.C = static_cast<int>(x->shape[1]);
+  g.H = static_cast<int>(x->shape[2]);
+  g.W = static_cast<int>(x->shape[3]);
+  g.O = static_cast<int>(w->shape[0]);
+  g.kH = static_cast<int>(w->shape[2]);
+  g.kW = static_cast<int>(w->shape[3]);
+  g.ph = ph;
+  g.pw = pw;
+  g.s = s;
+  g.oH = static_cast<int>(y->shape[2]);
+  g.oW = static_cast<int>(y->shape[3]);
+  TS_REQUIRE(w->shape[1] == g.C, "%s: filter has %lld input channels, input has %d", who, (long long)w->shape[1], g.C);
+  TS_REQUIRE(y->shape[0] == g.imgs && y->shape[1] == g.O, "%s: output N,C must be %d,%d", who, g.imgs, g.O);
+  TS_REQUIRE(g.H + 2 * ph >= g.kH && g.W + 2 * pw >= g.kW, "%s: filter larger than the padded image", who);
+  const int eh = (g.H + 2 * ph - g.kH) / s + 1, ew = (g.W + 2 * pw - g.kW) / s + 1;
+  TS_REQUIRE(g.oH == eh && g.oW == ew, "%s: output is %dx%d, expected %dx%d", who, g.oH, g.oW, eh, ew);
+  TS_REQUIRE(numel(x) < (1ll << 31) && numel(y) < (1ll << 31) && numel(w) < (1ll << 31), "%s: tensor too large", who);
+  TS_REQUIRE(g.kH < 20000 && g.kW < 20000, "%s: filter too large", who);
+  return 0;
+}
+
+inline const float *cf(const DLArray *a) { return static_cast<const float *>(a->data); }
+inline float *mf(DLArray *a) { return static_cast<float *>(a->data); }
+
+template <int BM, int BN, int WM, int WN>
+void launch_fwd(const ConvGeo &g, const float *x, const float *w, float *y, const Tap *taps, hipStream_t st) {
+  using AL = KContigLoader<BM>;
+  using BL = GatherColsLoader<BN, false>;
+  const int K = g.C * g.kH * g.kW, N = g.imgs * g.oH * g.oW, M = g.O;
+  typename AL::Params ap{w, K, M, K % 4 == 0 && aligned16(w)};
+  typename BL::Params bp{x, taps, FastDiv(g.oH * g.oW), FastDiv(g.oW), static_cast<int64_t>(g.C) * g.H * g.W,
+                         g.H, g.W, g.ph, g.pw, g.s, N};
+  NchwCols cm{FastDiv(g.oH * g.oW), static_cast<int64_t>(g.O) * g.oH * g.oW};
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, 1);
+  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, NchwCols>), grid, dim3(kThreads), 0, st, ap, bp, y,
+                     int64_t(0), static_cast<int64_t>(g.oH) * g.oW, cm, M, N, K, (K + BK - 1) / BK * BK);
+}
+
+template <int BM, int BN, int WM, int WN>
+void launch_bwd_data(const ConvGeo &g, const float *wt, const float *dy, float *dx, const Tap *taps,
+                     hipStream_t st) {
+  using AL = KContigLoader<BM>;
+  using BL = GatherColsLoader<BN, true>;
+  const int K = g.O * g.kH * g.kW, N = g.imgs * g.H * g.W, M = g.C;
+  typename AL::Params ap{wt, K, M, K % 4 == 0 && aligned16(wt)};
+  typename BL::Params bp{dy, taps, FastDiv(g.H * g.W), FastDiv(g.W), static_cast<int64_t>(g.O) * g.oH * g.oW,
+                         g.oH, g.oW, g.ph, g.pw, g.s, N};
+  NchwCols cm{FastDiv(g.H * g.W), static_cast<int64_t>(g.C) * g.H * g.W};
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, 1);
+  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, NchwCols>), grid, dim3(kThreads), 0, st, ap, bp, dx,
+                     int64_t(0), static_cast<int64_t>(g.H) * g.W, cm, M, N, K, (K + BK - 1) / BK * BK);
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_bwd_filter(const ConvGeo &g, const float *x, const float *dy, float *dw, const Tap *taps, hipStream_t st,
+                      int64_t *ws_elems) {
+  using AL = DyRowsLoader<BM>;
+  using BL = GatherRowsLoader<BN>;
+  const int K = g.imgs * g.oH * g.oW, N = g.C * g.kH * g.kW, M = g.O;
+  typename AL::Params ap{dy, FastDiv(g.oH * g.oW), g.O, (g.oH * g.oW) % 4 == 0 && aligned16(dy)};
+  typename BL::Params bp{x, taps, FastDiv(g.oH * g.oW), FastDiv(g.oW), static_cast<int64_t>(g.C) * g.H * g.W,
+                         g.H, g.W, g.ph, g.pw, g.s, N};
+  const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+  int S, kchunk;
+  plan_splitk(tm * tn, K, 1024, S, kchunk);
+  const int64_t mn = static_cast<int64_t>(M) * N;
+  float *out = dw;
+  if (S > 1) {
+    out = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(S) * mn * 4));
+    TS_REQUIRE(out, "conv bwd-filter: no scratch memory for split-K");
+    *ws_elems = S * mn;
+  }
+  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>), dim3(tn, tm, S), dim3(kThreads), 0, st,
+                     ap, bp, out, mn, static_cast<int64_t>(N), RowMajorCols{}, M, N, K, kchunk);
+  if (S > 1)
+    hipLaunchKernelGGL(splitk_fold_kernel, dim3(static_cast<unsigned>((mn + 255) / 256)), dim3(256), 0, st, out, dw,
+                       mn, mn, S);
+  return 0;
+}
+
+int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y, int ph, int pw, int s,
+                 DLStreamHandle sh, ProfilerHandle p) {
+  ConvGeo g;
+  if (geo_from(who, x, w, y, ph, pw, s, g)) return -1;
+  hipStream_t st = stream_of(sh);
+  ProfileScope ps(p, st, numel(x) + numel(w), numel(y), 0);
+  if (numel(y) > 0) {
+    const Tap *taps = tap_table(g.C, g.kH, g.kW, g.W, g.H * g.W, +1);
+    TS_REQUIRE(taps, "%s: could not build the tap table", who);
+    if (g.O <= 64)
+      launch_fwd<64, 256, 1, 4>(g, cf(x), cf(w), mf(y), taps, st);
+    else
+      launch_fwd<128, 128, 2, 2>(g, cf(x), cf(w), mf(y), taps, st);
+  }
+  return ps.finish();
+}
+
+int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray *dx, int ph, int pw, int s,
+                  DLStreamHandle sh, ProfilerHandle p) {
+  ConvGeo g;
+  if (geo_from(who, dx, w, dy, ph, pw, s, g)) return -1;
+  hipStream_t st = stream_of(sh);
+  ProfileScope ps(p, st, numel(dy) + numel(w), numel(dx), numel(w));
+  if (numel(dx) > 0) {
+    // taps index dy: off = o*oH*oW (spatial part is recomputed because of the stride test)
+    const Tap *taps = tap_table(g.O, g.kH, g.kW, 0, g.oH * g.oW, 0);
+    TS_REQUIRE(taps, "%s: could not build the tap table", who);
+    float *wt = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(numel(w)) * 4));
+    TS_REQUIRE(wt, "%s: no scratch memory", who);
+    const int total = static_cast<int>(numel(w));
+    hipLaunchKernelGGL(filter_oc_swap_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
+                       g.kH * g.kW);
+    if (g.C <= 64)
+      launch_bwd_data<64, 256, 1, 4>(g, wt, cf(dy), mf(dx), taps, st);
+    else
+      launch_bwd_data<128, 128, 2, 2>(g, wt, cf(dy), mf(dx), taps, st);
+  }
+  return ps.finish();
+}
+
+int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArray *dw, int ph, int pw, int s,
+                    DLStreamHandle sh, ProfilerHandle p) {
+  ConvGeo g;
+  if (geo_from(who, x, dw, dy, ph, pw, s, g)) return -1;
+  hipStream_t st = stream_of(sh);
+  int64_t ws = 0;
+  ProfileScope ps(p, st, numel(x) + numel(dy), numel(dw), 0);
+  int rc = 0;
+  if (numel(dw) > 0) {
+    const Tap *taps = tap_table(g.C, g.kH, g.kW, g.W, g.H * g.W, +1);
+    TS_REQUIRE(taps, "%s: could not build the tap table", who);
+    if (g.O <= 64)
+      rc = launch_bwd_filter<64, 256, 1, 4>(g, cf(x), cf(dy), mf(dw), taps, st, &ws);
+    else
+      rc = launch_bwd_filter<128, 128, 2, 2>(g, cf(x), cf(dy), mf(dw), taps, st, &ws);
+  }
+  if (p) p->workspace_memory = mib(ws);
+  if (rc) return rc;
+  return ps.finish();
+}
+
+}  // namespace
+}  // namespace tsplit
+
+using namespace tsplit;
+
+extern "C" {
+
+int CuDNN_DLGpuConv2d(const DLArrayHandle input_x, const DLArrayHandle input_f, DLArrayHandle output,
+                      const int padding, const int padding2, const int stride, DLStreamHandle stream_handle,
+                      ProfilerHandle p) {
+  return conv_forward("CuDNN_DLGpuConv2d", input_x, input_f, output, padding, padding2, stride, stream_handle, p);
+}
+
+int CuDNN_DLGpuConv2d_Gradient_of_Filter(const DLArrayHandle input_x, const DLArrayHandle gradient_y,
+                                         DLArrayHandle gradient_f, const int padding, const int padding2,
+                                         const int stride, DLStreamHandle stream_handle, ProfilerHandle p) {
+  return conv_bwd_filter("CuDNN_DLGpuConv2d_Gradient_of_Filter", input_x, gradient_y, gradient_f, padding, padding2,
+                         stride, stream_handle, p);
+}
+
+int CuDNN_DLGpuConv2d_Gradient_of_Data(const DLArrayHandle input_f, const DLArrayHandle gradient_y,
+                                       DLArrayHandle gradient_x, const int padding, const int padding2,
+                                       const int stride, DLStreamHandle stream_handle, ProfilerHandle p) {
+  return conv_bwd_data("CuDNN_DLGpuConv2d_Gradient_of_Data", input_f, gradient_y, gradient_x, padding, padding2,
+                       stride, stream_handle, p);
+}
+
+// The plain symbols take one padding int and caller-provided im2col workspaces
+// (src/ops/Conv2d.cu:52,172,241).  The workspaces are not needed and are left untouched.
+int DLGpuConv2d(const DLArrayHandle input_x, const DLArrayHandle input_f, DLArrayHandle output,
+                DLArrayHandle workspace_arr, const int padding, const int stride, DLStreamHandle stream_handle,
+                ProfilerHandle p) {
+  (void)workspace_arr;
+  return conv_forward("DLGpuConv2d", input_x, input_f, output, padding, padding, stride, stream_handle, p);
+}
+
+int DLGpuConv2d_Gradient_of_Data(const DLArrayHandle input_f, const DLArrayHandle gradient_y,
+                                 DLArrayHandle gradient_x, DLArrayHandle workspace_im2col, const int padding,
+                                 const int stride, DLStreamHandle stream_handle, ProfilerHandle p) {
+  (void)workspace_im2col;
+  return conv_bwd_data("DLGpuConv2d_Gradient_of_Data", input_f, gradient_y, gradient_x, padding, padding, stride,
+                       stream_handle, p);
+}
+
+int DLGpuConv2d_Gradient_of_Filter(const DLArrayHandle input_x, const DLArrayHandle gradient_y,
+                                   DLArrayHandle gradient_f, DLArrayHandle workspace_im2col,
+                                   DLArrayHandle workspace_batch_filter, const int padding, const int stride,
+                                   DLStreamHandle stream_handle, ProfilerHandle p) {
+  (void)workspace_im2col;
+  (void)workspace_batch_filter;
+  return conv_bwd_filter("DLGpuConv2d_Gradient_of_Filter", input_x, gradient_y, gradient_f, padding, padding, stride,
+                         stream_handle, p);
+}
+
+}  // extern "C"

@@ -263,7 +263,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::P
 }
 
 // out[i] = sum_z part[z * stride + i], z ascending (deterministic split-K fold)
-__global__ __launch_bounds__(256) void splitk_fold_kernel(const float *__restrict__ part, float *__restrict__ out,
+static __global__ __launch_bounds__(256) void splitk_fold_kernel(const float *__restrict__ part, float *__restrict__ out,
                                                           int64_t n, int64_t stride, int S) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (i >= n) return;
