@@ -1,0 +1,89 @@
+"""End-to-end parity: whole training runs through the C ABI track the CPU oracle.
+Tolerance from the task statement: loss within 1e-3 relative over 20 steps."""
+import numpy as np
+import pytest
+
+from oracle import nets
+from util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _onehot(idx, n):
+    return np.eye(n, dtype=np.float32)[idx]
+
+
+def test_mlp_20_steps_tracks_oracle():
+    """BASELINE config 1: 784-256-256-10 without bias, batch 128, 20 SGD steps, lr 0.1,
+    X ~ U[0,1), labels uniform, weights ~ N(0, 0.1)."""
+    from tsplit_amd import ndarray, trainer
+    rng = np.random.RandomState(123)
+    X = rng.uniform(0, 1, (128, 784)).astype(np.float32)
+    Y = _onehot(rng.randint(0, 10, 128), 10)
+    spec = trainer.mlp_spec()
+    params = {k: rng.normal(0, 0.1, s).astype(np.float32) for k, s in trainer.param_shapes(spec).items()}
+    ref_losses, ref_params = nets.train(spec, params, X, Y, steps=20, lr=0.1)
+    ctx = ndarray.gpu(0)
+    t = trainer.Trainer(spec, params, X.shape, 10, ctx, optimizer=("sgd", 0.1))
+    gx, gy = ndarray.array(X, ctx), ndarray.array(Y, ctx)
+    losses = []
+    for _ in range(20):
+        t.step(gx, gy)
+        losses.append(t.loss_value())
+    rel = np.max(np.abs(np.array(losses) - np.array(ref_losses)) / np.abs(ref_losses))
+    assert rel <= 1e-3, (rel, losses, ref_losses)
+    assert ref_losses[-1] < ref_losses[0]            # it does train
+    for k in params:
+        assert_close(t.params[k].asnumpy(), ref_params[k], 1e-3, k)
+
+
+def _small_convnet():
+    return [("conv", "c1", 3, 8, 3, 1, 1), ("bn", "c1_bn", 8), ("relu",),
+            ("conv", "c2", 8, 16, 3, 1, 1), ("bn", "c2_bn", 16), ("relu",), ("maxpool", 2, 0, 2),
+            ("conv", "c3", 16, 16, 3, 1, 1), ("bn", "c3_bn", 16), ("relu",), ("maxpool", 2, 0, 2),
+            ("flatten",), ("fc", "f1", 16 * 4 * 4, 32), ("fc", "f2", 32, 10)]
+
+
+@pytest.mark.parametrize("split", [None, {0: 4, 3: 4}, {3: 3}])
+def test_convnet_momentum_tracks_oracle_with_and_without_split(split):
+    from tsplit_amd import ndarray, trainer
+    rng = np.random.RandomState(7)
+    spec = _small_convnet()
+    X = rng.normal(size=(8, 3, 16, 16)).astype(np.float32)
+    Y = _onehot(rng.randint(0, 10, 8), 10)
+    params = trainer.init_params(spec, seed=5)
+    ref_losses, ref_params = nets.train(spec, params, X, Y, steps=6, lr=0.05, momentum=0.9)
+    ctx = ndarray.gpu(0)
+    t = trainer.Trainer(spec, params, X.shape, 10, ctx, optimizer=("momentum", 0.05, 0.9), split=split)
+    gx, gy = ndarray.array(X, ctx), ndarray.array(Y, ctx)
+    losses = []
+    for _ in range(6):
+        t.step(gx, gy)
+        losses.append(t.loss_value())
+    rel = np.max(np.abs(np.array(losses) - np.array(ref_losses)) / np.abs(ref_losses))
+    assert rel <= 1e-3, (rel, losses, ref_losses)
+    for k in params:
+        assert_close(t.params[k].asnumpy(), ref_params[k], 2e-3, k)
+
+
+def test_vgg16_topology_small_resolution_tracks_oracle():
+    """The full VGG-16 layer list (13 conv+BN+Relu, 5 pools, 3 FC) at 32x32, batch 4, with the
+    two largest-resolution blocks run as 2 micro-tensors: 3 momentum steps against the oracle."""
+    from tsplit_amd import ndarray, trainer
+    rng = np.random.RandomState(11)
+    spec = trainer.vgg16_spec(num_classes=10, in_hw=32)
+    X = rng.normal(size=(4, 3, 32, 32)).astype(np.float32)
+    Y = _onehot(rng.randint(0, 10, 4), 10)
+    params = trainer.init_params(spec, seed=3)
+    ref_losses, _ = nets.train(spec, params, X, Y, steps=3, lr=0.01, momentum=0.9)
+    ctx = ndarray.gpu(0)
+    conv_idx = [i for i, l in enumerate(spec) if l[0] == "conv"]
+    t = trainer.Trainer(spec, params, X.shape, 10, ctx, optimizer=("momentum", 0.01, 0.9),
+                        split={i: 2 for i in conv_idx[:4]})
+    gx, gy = ndarray.array(X, ctx), ndarray.array(Y, ctx)
+    losses = []
+    for _ in range(3):
+        t.step(gx, gy)
+        losses.append(t.loss_value())
+    rel = np.max(np.abs(np.array(losses) - np.array(ref_losses)) / np.abs(ref_losses))
+    assert rel <= 1e-3, (rel, losses, ref_losses)

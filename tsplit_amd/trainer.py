@@ -1,0 +1,285 @@
+"""Minimal executor for sequential conv nets, driving the operator library through
+`gpu_links` exactly as the reference's executor loop drives it.
+
+Reproduces, for a layer list, what the reference does for a graph: one NDArray per node
+output (python/athena/gpu_ops/executor.py:71-92), a forward sweep that calls each op's GPU
+symbol on one compute stream (executor.py:140-152), the backward nodes its autodiff creates
+(conv -> gradient_of_filter + gradient_of_data, matmul -> two transposed matmuls, relu ->
+relu_gradient, maxpool -> max_pooling2d_gradient, softmaxCE -> its gradient seeded with ones:
+executor.py:160-196), filter gradients issued before data gradients (executor.py:327-332),
+the data gradient of the first layer never evaluated, then one optimizer call per parameter
+(python/athena/optimizer.py:95-176).
+
+The TSplit part: `split={layer_index: pieces}` runs that conv layer (forward, both
+backward passes) on `pieces` zero-copy batch micro-tensors (DLArraySliceForMicroTensor);
+per-piece filter gradients are summed with DLGpuMatrixElementwiseAdd.  BatchNorm always
+sees the whole batch: its statistics are batch statistics, so a BN over a micro-batch is
+a different function.
+
+Layer spec entries:
+    ("conv", name, Cin, Cout, k, pad, stride) | ("bn", name, C) | ("relu",) |
+    ("maxpool", k, pad, stride) | ("flatten",) | ("fc", name, n_in, n_out)
+"""
+import numpy as np
+
+from . import gpu_links as L
+from . import ndarray
+from .stream import create_stream_handle
+
+
+def mlp_spec(sizes=(784, 256, 256, 10)):
+    """784 -> 256 -> 256 -> 10 without biases, Relu between layers."""
+    spec = []
+    for i in range(len(sizes) - 1):
+        spec.append(("fc", "mlp_fc%d" % (i + 1), sizes[i], sizes[i + 1]))
+        if i < len(sizes) - 2:
+            spec.append(("relu",))
+    return spec
+
+
+def vgg16_spec(num_classes=1000, in_hw=224):
+    """VGG-16 as examples/imagenet_vgg.py:24-98 builds it: 13 x (conv3x3 pad 1, BN, Relu),
+    5 max-pools 2x2/2, flatten, three bias-free fully connected layers with no activation
+    in between."""
+    spec = []
+    cin = 3
+    for bi, (n, cout) in enumerate([(2, 64), (2, 128), (3, 256), (3, 512), (3, 512)], 1):
+        for li in range(1, n + 1):
+            name = "vgg_block%d_layer%d" % (bi, li)
+            spec += [("conv", name, cin, cout, 3, 1, 1), ("bn", name + "_bn", cout), ("relu",)]
+            cin = cout
+        spec.append(("maxpool", 2, 0, 2))
+    spec.append(("flatten",))
+    feat = 512 * (in_hw // 32) ** 2
+    spec += [("fc", "vgg_fc1", feat, 4096), ("fc", "vgg_fc2", 4096, 4096), ("fc", "vgg_fc3", 4096, num_classes)]
+    return spec
+
+
+def param_shapes(spec):
+    shapes = {}
+    for layer in spec:
+        if layer[0] == "conv":
+            _, name, cin, cout, k, _, _ = layer
+            shapes[name + "_weight"] = (cout, cin, k, k)
+        elif layer[0] == "bn":
+            _, name, c = layer
+            shapes[name + "_scale"] = (1, c, 1, 1)
+            shapes[name + "_bias"] = (1, c, 1, 1)
+        elif layer[0] == "fc":
+            _, name, n_in, n_out = layer
+            shapes[name + "_weight"] = (n_in, n_out)
+    return shapes
+
+
+def init_params(spec, seed=123, scheme="he"):
+    """Seeded host-side initialisation.  "he": N(0, sqrt(2/fan_in)) weights, BN scale 1, bias 0.
+    "normal0.1": N(0, 0.1) everywhere (what examples/imagenet_vgg.py:14-21 draws)."""
+    rng = np.random.RandomState(seed)
+    params = {}
+    for name, shape in param_shapes(spec).items():
+        if scheme == "normal0.1":
+            params[name] = rng.normal(scale=0.1, size=shape).astype(np.float32)
+        elif name.endswith("_scale"):
+            params[name] = np.ones(shape, np.float32)
+        elif name.endswith("_bias"):
+            params[name] = np.zeros(shape, np.float32)
+        else:
+            fan_in = int(np.prod(shape[1:])) if len(shape) == 4 else shape[0]
+            params[name] = rng.normal(scale=np.sqrt(2.0 / fan_in), size=shape).astype(np.float32)
+    return params
+
+
+def _out_shape(layer, s):
+    kind = layer[0]
+    if kind == "conv":
+        _, _, _, cout, k, pad, stride = layer
+        return (s[0], cout, (s[2] + 2 * pad - k) // stride + 1, (s[3] + 2 * pad - k) // stride + 1)
+    if kind in ("bn", "relu"):
+        return s
+    if kind == "maxpool":
+        _, k, pad, stride = layer
+        return (s[0], s[1], (s[2] + 2 * pad - k) // stride + 1, (s[3] + 2 * pad - k) // stride + 1)
+    if kind == "flatten":
+        return (s[0], int(np.prod(s[1:])))
+    if kind == "fc":
+        return (s[0], layer[3])
+    raise ValueError(kind)
+
+
+class Trainer(object):
+    def __init__(self, spec, params, input_shape, num_classes, ctx=None, optimizer=("sgd", 0.1),
+                 split=None, bn_eps=0.01, timer=None):
+        self.spec = list(spec)
+        # optional per-call timing hook: timer.begin(stream) / timer.end(stream, tag, work, unit)
+        self.timer = timer
+        self.ctx = ctx if ctx is not None else ndarray.gpu(0)
+        self.stream = create_stream_handle(self.ctx)
+        self.optimizer = optimizer
+        self.split = dict(split or {})
+        self.eps = bn_eps
+        self.params = {k: ndarray.array(v, self.ctx) for k, v in params.items()}
+        self.grads = {k: ndarray.empty(v.shape, self.ctx) for k, v in params.items()}
+        self.state = {}
+        if optimizer[0] == "momentum":
+            self.state = {k: ndarray.array(np.zeros(v.shape, np.float32), self.ctx) for k, v in params.items()}
+        # one array per node output, one per node gradient
+        self.acts = [None]          # acts[0] is the input, bound per step
+        self.dacts = [None]
+        self.saved = {}
+        self.dw_piece = {}
+        s = tuple(input_shape)
+        self.shapes = [s]
+        for li, layer in enumerate(self.spec):
+            s = _out_shape(layer, s)
+            self.shapes.append(s)
+            self.acts.append(ndarray.empty(s, self.ctx))
+            self.dacts.append(ndarray.empty(s, self.ctx))
+            if layer[0] == "bn":
+                c = layer[2]
+                self.saved[li] = (ndarray.empty((1, c, 1, 1), self.ctx), ndarray.empty((1, c, 1, 1), self.ctx))
+            if layer[0] == "conv" and li in self.split:
+                self.acts[-1].split_tensor(self.split[li])
+                self.dacts[-1].split_tensor(self.split[li])
+                # per-piece filter gradient, summed into the layer's gradient
+                self.dw_piece[li] = ndarray.empty(param_shapes([layer])[layer[1] + "_weight"], self.ctx)
+        assert self.shapes[-1] == (input_shape[0], num_classes), (self.shapes[-1], num_classes)
+        self.loss = ndarray.empty((1,), self.ctx)
+        self.ones = ndarray.empty((1,), self.ctx)
+        L.array_set(self.ones, 1.0, self.stream)          # adjoint seed (executor.py:175)
+        for li in self.split:
+            if li > 0:
+                self.acts[li].split_tensor(self.split[li])
+                self.dacts[li].split_tensor(self.split[li])
+
+    def _run(self, tag, work, unit, fn, *args):
+        """Issue one operator call on the compute stream; `work` is its algorithmic FLOP or
+        byte count (each distinct input read once, each output written once)."""
+        if self.timer is None:
+            fn(*args, self.stream)
+        else:
+            self.timer.begin(self.stream)
+            fn(*args, self.stream)
+            self.timer.end(self.stream, tag, work, unit)
+
+    @staticmethod
+    def _n(shape):
+        return int(np.prod(shape))
+
+    @staticmethod
+    def _tile(rows):
+        return "64x256" if rows <= 64 else "128x128"
+
+    # ---------------------------------------------------------------- forward
+    def forward(self, x, labels):
+        n = self._n
+        self.acts[0] = x
+        if 0 in self.split:
+            x.split_tensor(self.split[0])
+        for li, layer in enumerate(self.spec):
+            a, out = self.acts[li], self.acts[li + 1]
+            kind = layer[0]
+            if kind == "conv":
+                _, name, cin, cout, k, pad, stride = layer
+                w = self.params[name + "_weight"]
+                tag = "conv_fwd_" + self._tile(cout)
+                pairs = list(zip(a.sTensor, out.sTensor)) if li in self.split else [(a, out)]
+                for xa, ya in pairs:
+                    self._run(tag, 2.0 * n(ya.shape) * cin * k * k, "flop", L.CuDNN_conv2d, xa, w, ya, pad, pad, stride)
+            elif kind == "bn":
+                name = layer[1]
+                sm, sv = self.saved[li]
+                self._run("bn_fwd", 8.0 * n(a.shape), "byte", L.CuDNN_Batch_Normalization, a,
+                          self.params[name + "_scale"], self.params[name + "_bias"], out, sm, sv, 0.99, self.eps)
+            elif kind == "relu":
+                self._run("relu_fwd", 8.0 * n(a.shape), "byte", L.relu, a, out)
+            elif kind == "maxpool":
+                _, k, pad, stride = layer
+                self._run("maxpool_fwd", 4.0 * (n(a.shape) + n(out.shape)), "byte", L.CuDNN_max_pooling2d, a, k, k, out,
+                          pad, stride)
+            elif kind == "flatten":
+                self._run("reshape", 8.0 * n(a.shape), "byte", L.array_reshape, a, out)
+            elif kind == "fc":
+                _, name, n_in, n_out = layer
+                self._run("matmul_" + self._tile(a.shape[0]), 2.0 * a.shape[0] * n_in * n_out, "flop",
+                          L.matrix_multiply, a, False, self.params[name + "_weight"], False, out)
+        self._run("softmax_ce_fwd", 8.0 * n(self.acts[-1].shape), "byte", L.softmax_cross_entropy, self.acts[-1],
+                  labels, self.loss)
+        return self.loss
+
+    # ---------------------------------------------------------------- backward
+    def backward(self, labels):
+        n = self._n
+        self._run("softmax_ce_bwd", 12.0 * n(self.acts[-1].shape), "byte", L.softmax_cross_entropy_gradient,
+                  self.acts[-1], labels, self.ones, self.dacts[-1])
+        for li in range(len(self.spec) - 1, -1, -1):
+            layer = self.spec[li]
+            a, g_out, g_in = self.acts[li], self.dacts[li + 1], self.dacts[li]
+            kind = layer[0]
+            first = li == 0
+            if kind == "conv":
+                _, name, cin, cout, k, pad, stride = layer
+                w, dw = self.params[name + "_weight"], self.grads[name + "_weight"]
+                split = li in self.split
+                xs = a.sTensor if split else [a]
+                gs = g_out.sTensor if split else [g_out]
+                for i, (xa, ga) in enumerate(zip(xs, gs)):
+                    # filter gradient first, as the reference reorders it (executor.py:327-332)
+                    self._run("conv_bwd_filter_" + self._tile(cout), 2.0 * n(ga.shape) * cin * k * k, "flop",
+                              L.CuDNN_conv2d_gradient_of_filter, xa, ga, dw if i == 0 else self.dw_piece[li],
+                              pad, pad, stride)
+                    if i > 0:
+                        self._run("add", 12.0 * n(dw.shape), "byte", L.matrix_elementwise_add, dw, self.dw_piece[li], dw)
+                if not first:
+                    gis = g_in.sTensor if split else [g_in]
+                    for ga, gi in zip(gs, gis):
+                        self._run("conv_bwd_data_" + self._tile(cin), 2.0 * n(ga.shape) * cin * k * k, "flop",
+                                  L.CuDNN_conv2d_gradient_of_data, w, ga, gi, pad, pad, stride)
+            elif kind == "bn":
+                name = layer[1]
+                sm, sv = self.saved[li]
+                self._run("bn_bwd", 12.0 * n(a.shape), "byte", L.CuDNN_Batch_Normalization_gradient, g_out, a,
+                          self.params[name + "_scale"], g_in, self.grads[name + "_scale"],
+                          self.grads[name + "_bias"], sm, sv, self.eps)
+            elif kind == "relu":
+                self._run("relu_bwd", 12.0 * n(a.shape), "byte", L.relu_gradient, a, g_out, g_in)
+            elif kind == "maxpool":
+                _, k, pad, stride = layer
+                self._run("maxpool_bwd", 4.0 * (2 * n(a.shape) + n(g_out.shape)), "byte",
+                          L.CuDNN_max_pooling2d_gradient, self.acts[li + 1], g_out, a, k, k, g_in, pad, stride)
+            elif kind == "flatten":
+                self._run("reshape", 8.0 * n(a.shape), "byte", L.array_reshape, g_out, g_in)
+            elif kind == "fc":
+                _, name, n_in, n_out = layer
+                w = self.params[name + "_weight"]
+                m = a.shape[0]
+                self._run("matmul_" + self._tile(n_in), 2.0 * m * n_in * n_out, "flop", L.matrix_multiply, a, True,
+                          g_out, False, self.grads[name + "_weight"])
+                if not first:
+                    self._run("matmul_" + self._tile(m), 2.0 * m * n_in * n_out, "flop", L.matrix_multiply, g_out,
+                              False, w, True, g_in)
+
+    # ---------------------------------------------------------------- update
+    def update(self):
+        for name, p in self.params.items():
+            g = self.grads[name]
+            if self.optimizer[0] == "sgd":
+                self._run("sgd", 12.0 * self._n(p.shape), "byte", L.sgd_update, p, g, self.optimizer[1])
+            elif self.optimizer[0] == "momentum":
+                self._run("momentum", 20.0 * self._n(p.shape), "byte", L.momentum_update, p, g, self.state[name],
+                          self.optimizer[1], self.optimizer[2], False)
+            else:
+                raise ValueError(self.optimizer[0])
+
+    def step(self, x, labels):
+        """One training step, asynchronous on self.stream; returns the (device) loss array."""
+        self.forward(x, labels)
+        self.backward(labels)
+        self.update()
+        return self.loss
+
+    def sync(self):
+        self.stream.sync()
+
+    def loss_value(self):
+        self.sync()
+        return float(self.loss.asnumpy()[0])
