@@ -1,0 +1,188 @@
+#!/usr/bin/env python3
+"""Benchmark of the operator hot path: VGG-16 fp32 training steps on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+A step = forward + backward + momentum-SGD update of VGG-16 (13 conv3x3+BN+Relu, 5 max-pools,
+3 bias-free FC; batch 64, 3x224x224, 1000 classes) issued through the C ABI on one stream,
+with the four largest-resolution conv layers run as 4 batch micro-tensors.  Inputs,
+labels and parameters are resident in HBM before the timed region starts.
+
+Prints ONE JSON line.  Besides the contract fields it carries
+  roofline      the kernel with the largest share of the step (a conv implicit-GEMM kernel):
+                algorithmic FLOP per launch / mean launch time, measured with HIP events
+                recorded on the compute stream around every launch inside the timed region
+  kernels       the same figures for every operator class (TFLOP/s or GB/s)
+  cpu_baseline  the numpy CPU oracle timed on this host on a bounded sample of the workload
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS_FP32_MFMA = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+class EventTimer(object):
+    """Brackets every operator call with a pair of HIP events on the compute stream; elapsed
+    times are read after the final synchronisation, so nothing blocks inside the step."""
+
+    def __init__(self, ctx):
+        from tsplit_amd.stream import create_event_handle
+        self._mk = lambda: create_event_handle(ctx)
+        self._hip = ctypes.CDLL("libamdhip64.so")
+        self._pool, self._used, self.spans = [], 0, []
+        self.enabled = False
+
+    def _ev(self):
+        if self._used == len(self._pool):
+            self._pool.append(self._mk())
+        self._used += 1
+        return self._pool[self._used - 1]
+
+    def begin(self, stream):
+        if self.enabled:
+            self._a = self._ev()
+            self._a.record(stream)
+
+    def end(self, stream, tag, work, unit):
+        if self.enabled:
+            b = self._ev()
+            b.record(stream)
+            self.spans.append((tag, work, unit, self._a, b))
+
+    def collect(self):
+        """-> {tag: dict(calls, ms_total, ms_avg, work_per_call, unit, rate)} ; rate in TFLOP/s or GB/s"""
+        out = {}
+        ms = ctypes.c_float(0)
+        for tag, work, unit, a, b in self.spans:
+            ea = ctypes.cast(a.handle.contents.handle, ctypes.POINTER(ctypes.c_void_p))[0]
+            eb = ctypes.cast(b.handle.contents.handle, ctypes.POINTER(ctypes.c_void_p))[0]
+            rc = self._hip.hipEventElapsedTime(ctypes.byref(ms), ctypes.c_void_p(ea), ctypes.c_void_p(eb))
+            if rc != 0:
+                raise RuntimeError("hipEventElapsedTime failed: %d" % rc)
+            d = out.setdefault(tag, {"calls": 0, "ms_total": 0.0, "work": 0.0, "unit": unit})
+            d["calls"] += 1
+            d["ms_total"] += ms.value
+            d["work"] += work
+        for d in out.values():
+            d["ms_avg"] = d["ms_total"] / d["calls"]
+            d["work_per_call"] = d["work"] / d["calls"]
+            sec = d["ms_total"] * 1e-3
+            d["rate"] = d["work"] / sec / (1e12 if d["unit"] == "flop" else 1e9) if sec > 0 else 0.0
+        return out
+
+
+def vgg_workload(batch, seed=123):
+    from tsplit_amd import trainer
+    rng = np.random.RandomState(seed)
+    spec = trainer.vgg16_spec(1000, 224)
+    params = trainer.init_params(spec, seed=seed, scheme="he")
+    x = rng.standard_normal(size=(batch, 3, 224, 224)).astype(np.float32)
+    labels = np.zeros((batch, 1000), np.float32)
+    labels[np.arange(batch), rng.randint(0, 1000, batch)] = 1.0
+    conv_idx = [i for i, l in enumerate(spec) if l[0] == "conv"]
+    split = {i: 4 for i in conv_idx[:4]}          # the two 224x224 and the two 112x112 layers
+    return spec, params, x, labels, split
+
+
+def cpu_baseline(sample_batch=1, seed=123):
+    """The numpy oracle (float64, as the reference's numpy path computes) on `sample_batch`
+    images of the same seeded workload: one forward+backward+momentum step."""
+    from oracle import nets, ops
+    spec, params, x, labels, _ = vgg_workload(sample_batch, seed)
+    vel = {k: np.zeros_like(v) for k, v in params.items()}
+    t0 = time.perf_counter()
+    loss, _, grads = nets.forward_backward(spec, params, x, labels, eps=0.01)
+    for k in params:
+        ops.momentum_update(params[k], grads[k], vel[k], 0.01, 0.9)
+    dt = time.perf_counter() - t0
+    try:
+        import threadpoolctl
+        cores = max([p.get("num_threads", 1) for p in threadpoolctl.threadpool_info()] or [1])
+    except Exception:
+        cores = os.cpu_count() or 1
+    return {"value": sample_batch / dt, "unit": "samples/s", "cores": int(cores), "kind": "port",
+            "sample": "one VGG-16 fwd+bwd+momentum step on %d of the 64 seeded images, numpy oracle in float64 "
+                      "(%.1f s, loss %.4f)" % (sample_batch, dt, loss)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-split", action="store_true")
+    ap.add_argument("--no-events", action="store_true", help="time the steps without per-launch events")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build is single-GPU by design (no collectives, no sharding); run with --gpus 1. "
+                 "The one-GPU figure is the whole-job throughput.")
+
+    from tsplit_amd import ndarray, trainer
+    ctx = ndarray.gpu(0)
+    spec, params, x, labels, split = vgg_workload(a.batch)
+    if a.no_split:
+        split = {}
+    timer = None if a.no_events else EventTimer(ctx)
+    t = trainer.Trainer(spec, params, x.shape, 1000, ctx, optimizer=("momentum", 1e-4, 0.9), split=split, timer=timer)
+    gx, gy = ndarray.array(x, ctx), ndarray.array(labels, ctx)      # resident before timing
+    for _ in range(a.warmup):
+        t.step(gx, gy)
+    t.sync()
+    if timer:
+        timer.enabled = True
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        t.step(gx, gy)
+    t.sync()
+    dt = time.perf_counter() - t0
+    loss = float(t.loss.asnumpy()[0])
+    ms_per_step = dt / a.steps * 1e3
+
+    out = {
+        "metric": "train samples/s, fp32, 1 MI355X; conv MFMA util %; BN/relu HBM GB/s",
+        "value": a.batch * a.steps / dt, "unit": "samples/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "VGG-16 training step (fwd+bwd+momentum SGD), fp32 NCHW, batch %d, 3x224x224, "
+                               "1000 classes, He init, %s" % (a.batch, "4 batch micro-tensors on the 4 largest conv layers"
+                                                              if split else "no micro-tensor split"),
+                   "global_batch": a.batch, "final_loss": loss},
+    }
+    if timer:
+        k = timer.collect()
+        kernels = {}
+        for tag, d in sorted(k.items(), key=lambda kv: -kv[1]["ms_total"]):
+            peak = PEAK_TFLOPS_FP32_MFMA if d["unit"] == "flop" else PEAK_HBM_GBS
+            kernels[tag] = {"calls_per_step": d["calls"] / a.steps, "ms_per_step": d["ms_total"] / a.steps,
+                            "ms_avg": d["ms_avg"], "achieved": d["rate"],
+                            "unit": "TFLOP/s" if d["unit"] == "flop" else "GB/s", "frac": d["rate"] / peak}
+        dom = next(iter(kernels))
+        dd = k[dom]
+        out["roofline"] = {"kernel": dom, "bound": "mfma" if dd["unit"] == "flop" else "hbm",
+                           "achieved": dd["rate"], "peak": PEAK_TFLOPS_FP32_MFMA if dd["unit"] == "flop" else PEAK_HBM_GBS,
+                           "unit": "TFLOP/s" if dd["unit"] == "flop" else "GB/s",
+                           "frac": dd["rate"] / (PEAK_TFLOPS_FP32_MFMA if dd["unit"] == "flop" else PEAK_HBM_GBS),
+                           "traffic": None, "per_launch": dd["work_per_call"], "ms_avg": dd["ms_avg"]}
+        conv = [d for tag, d in k.items() if tag.startswith("conv_")]
+        conv_flop, conv_ms = sum(d["work"] for d in conv), sum(d["ms_total"] for d in conv)
+        out["conv_mfma_util_pct"] = 100.0 * conv_flop / (conv_ms * 1e-3) / 1e12 / PEAK_TFLOPS_FP32_MFMA
+        out["kernels"] = kernels
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libc_runtime_api.so")
+# TSPLIT_LIB_PATH overrides the in-tree location (e.g. to try another build of the library)
+LIB_PATH = os.environ.get("TSPLIT_LIB_PATH") or os.path.join(_HERE, "lib", "libc_runtime_api.so")
 
 
 def _load_lib():

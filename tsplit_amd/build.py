@@ -24,6 +24,7 @@ ARCH = "gfx950"
 # packed-fp32 code generation is switched off for every device object of this library
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unknown-warning-option"]
+FLAGS += os.environ.get("TSPLIT_EXTRA_HIPCC_FLAGS", "").split()
 
 
 def _sources():

@@ -158,6 +158,99 @@ struct GatherColsLoader {
   }
 };
 
+
+// ------------------------------------------------------------------ tap-major gather loader
+// Fast path of forward and (stride 1) bwd-data when the channel count is a multiple of 16.
+// The reduction index is re-ordered k' = ((ch/16)*kH*kW + tap)*16 + ch%16, so one 16-wide
+// k-step covers 16 consecutive channels of ONE filter tap, and the kH*kW steps that follow
+// each other gather from the same 16 channel planes (L1 hits): the padding test is done once per
+// step and thread instead of once per element, there is no tap table, and a thread's 8 (or
+// 16) values are consecutive in k', so they go to an mn-major LDS tile with 16-byte writes
+// and are read back with 16-byte reads.  The filter is re-laid to match by a small kernel.
+template <int BN, bool BWD_DATA>
+struct TapMajorColsLoader {
+  using Lds = MnMajorLds<BN>;
+  struct Params {
+    const float *src;     // x (forward) or dy (bwd-data)
+    FastDiv plane;        // columns per image
+    FastDiv width;
+    int64_t img_stride;   // elements per image of src
+    int chan_stride;      // elements per channel plane of src
+    int src_h, src_w;
+    int ph, pw, s;
+    int chans, kW, taps_total;
+    int n_total;
+  };
+  static constexpr int kPerThread = BN / 16;      // 8 or 16 consecutive k'
+  static constexpr int kQuads = kPerThread / 4;
+  float4 r[kQuads];
+  const float *base;      // image base
+  int r0, c0;             // forward: oh*s-ph, ow*s-pw ; bwd-data: h+ph, w+pw
+  int src_h, src_w, chan_stride, kW, taps_total;
+  int klocal0;            // first k' (within a step) of this thread
+  int tap, ch0;           // running position of the current step: tap index and first channel
+  bool col_ok, started;
+
+  __device__ __forceinline__ void init(const Params &P, int n0, int tid) {
+    const int n = n0 + tid % BN;
+    klocal0 = (tid / BN) * kPerThread;
+    col_ok = n < P.n_total;
+    const uint32_t nn = col_ok ? n : 0;
+    const uint32_t img = P.plane.div(nn);
+    const uint32_t p = nn - img * P.plane.d;
+    const uint32_t row = P.width.div(p);
+    const uint32_t col = p - row * P.width.d;
+    src_h = P.src_h;
+    src_w = P.src_w;
+    chan_stride = P.chan_stride;
+    kW = P.kW;
+    taps_total = P.taps_total;
+    base = P.src + static_cast<int64_t>(img) * P.img_stride;
+    if (BWD_DATA) {
+      r0 = static_cast<int>(row) + P.ph;
+      c0 = static_cast<int>(col) + P.pw;
+    } else {
+      r0 = static_cast<int>(row) * P.s - P.ph;
+      c0 = static_cast<int>(col) * P.s - P.pw;
+    }
+    started = false;
+  }
+  __device__ __forceinline__ void load(int k0, int /*kend*/) {
+    if (!started) {            // steps arrive in order; only the first needs a division
+      const int step = k0 / BK;
+      ch0 = (step / taps_total) * BK;
+      tap = step % taps_total;
+      started = true;
+    }
+    const int kh = tap / kW, kw = tap - kh * kW;
+    const int rr = BWD_DATA ? r0 - kh : r0 + kh;
+    const int cc = BWD_DATA ? c0 - kw : c0 + kw;
+    const bool ok = col_ok && static_cast<unsigned>(rr) < static_cast<unsigned>(src_h) &&
+                    static_cast<unsigned>(cc) < static_cast<unsigned>(src_w);
+    const float *p = base + static_cast<int64_t>(ch0 + klocal0) * chan_stride + rr * src_w + cc;
+#pragma unroll
+    for (int q = 0; q < kQuads; ++q) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (ok) {
+        v.x = p[(4 * q + 0) * chan_stride];
+        v.y = p[(4 * q + 1) * chan_stride];
+        v.z = p[(4 * q + 2) * chan_stride];
+        v.w = p[(4 * q + 3) * chan_stride];
+      }
+      r[q] = v;
+    }
+    if (++tap == taps_total) {   // all taps of these 16 channels first: the gathers of
+      tap = 0;                   // consecutive steps then hit the same cache lines
+      ch0 += BK;
+    }
+  }
+  __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+    for (int q = 0; q < kQuads; ++q)
+      *reinterpret_cast<float4 *>(lds + (tid % BN) * Lds::kStride + klocal0 + 4 * q) = r[q];
+  }
+};
+
 // ------------------------------------------------------------------ bwd-filter loaders, mn-major
 // A = dy: row m = output channel, k = (img, p); K contiguous inside an image.
 template <int BM>
@@ -292,6 +385,73 @@ struct GatherRowsLoader {
   }
 };
 
+
+// Tap-major variant of the bwd-filter gather: columns are ordered j' = (kh*kW + kw)*C + c and
+// a thread owns BN/16 CONSECUTIVE columns, i.e. consecutive channels of one filter tap, so
+// the padding test is done once per step and the loads differ only by a channel stride.
+// The result comes out as dw'[o][tap][c]; the split-K fold writes it back as [o][c][tap].
+template <int BN>
+struct TapMajorRowsLoader {
+  using Lds = MnMajorLds<BN>;
+  struct Params {
+    const float *x;
+    FastDiv plane;        // oH*oW
+    FastDiv width;        // oW
+    int64_t img_stride;   // C*H*W
+    int chan_stride;      // H*W
+    int H, W, ph, pw, s;
+    int C, kW;
+    int j_total;
+  };
+  static constexpr int kCols = BN / 16;
+  float r[kCols];
+  const float *x;
+  FastDiv plane, width;
+  int64_t img_stride, col_off;
+  int chan_stride, H, W, s, klocal, jlocal0, dr, dc;   // dr = kh - ph, dc = kw - pw
+  bool cols_ok;
+
+  __device__ __forceinline__ void init(const Params &P, int j0, int tid) {
+    x = P.x;
+    plane = P.plane;
+    width = P.width;
+    img_stride = P.img_stride;
+    chan_stride = P.chan_stride;
+    H = P.H;
+    W = P.W;
+    s = P.s;
+    klocal = tid & 15;
+    jlocal0 = kCols * (tid >> 4);
+    const int j = j0 + jlocal0;
+    cols_ok = j < P.j_total;           // C % kCols == 0: a thread's columns are all valid or none
+    const int jj = cols_ok ? j : 0;
+    const int tap = jj / P.C, c = jj - tap * P.C;
+    const int kh = tap / P.kW, kw = tap - kh * P.kW;
+    dr = kh - P.ph;
+    dc = kw - P.pw;
+    col_off = static_cast<int64_t>(c) * P.chan_stride;
+  }
+  __device__ __forceinline__ void load(int k0, int kend) {
+    const int k = k0 + klocal;
+    const bool k_ok = cols_ok && k < kend;
+    const uint32_t kk = k_ok ? k : 0;
+    const uint32_t img = plane.div(kk);
+    const uint32_t p = kk - img * plane.d;
+    const uint32_t oh = width.div(p);
+    const uint32_t ow = p - oh * width.d;
+    const int rr = static_cast<int>(oh) * s + dr, cc = static_cast<int>(ow) * s + dc;
+    const bool ok = k_ok && static_cast<unsigned>(rr) < static_cast<unsigned>(H) &&
+                    static_cast<unsigned>(cc) < static_cast<unsigned>(W);
+    const float *q = x + static_cast<int64_t>(img) * img_stride + col_off + rr * W + cc;
+#pragma unroll
+    for (int i = 0; i < kCols; ++i) r[i] = ok ? q[i * chan_stride] : 0.f;
+  }
+  __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+    for (int i = 0; i < kCols; ++i) lds[(jlocal0 + i) * Lds::kStride + klocal] = r[i];
+  }
+};
+
 // ------------------------------------------------------------------ NCHW output columns
 struct NchwCols {   // out[img][m][p]: column n = img*plane + p -> img*img_stride + p ; row stride = plane
   FastDiv plane;
@@ -311,6 +471,37 @@ __global__ __launch_bounds__(256) void filter_oc_swap_kernel(const float *__rest
   const int t = idx / kHW;
   const int o = t % O, c = t / O;
   wt[idx] = w[(o * C + c) * kHW + r];
+}
+
+// re-lays of the filter [O][C][kHW] for the tap-major loaders, reduction index
+// k' = ((ch/16)*kHW + tap)*16 + ch%16:
+//   forward : out[o][k'] with ch = c     bwd-data: out[c][k'] with ch = o
+__global__ __launch_bounds__(256) void filter_tap_major_kernel(const float *__restrict__ w, float *__restrict__ out,
+                                                               int O, int C, int kHW, bool for_bwd_data) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= O * C * kHW) return;
+  const int K = (for_bwd_data ? O : C) * kHW;
+  const int row = idx / K, kp = idx - row * K;
+  const int lo = kp & 15;
+  const int t = kp >> 4;
+  const int tap = t % kHW, blk = t / kHW;
+  const int ch = blk * 16 + lo;
+  const int o = for_bwd_data ? ch : row, c = for_bwd_data ? row : ch;
+  out[idx] = w[(o * C + c) * kHW + tap];
+}
+
+// split-K fold for the tap-major bwd-filter: part[z][o][tap][c] summed over z (ascending, so the
+// result does not depend on scheduling) and written as dw[o][c][tap]
+__global__ __launch_bounds__(256) void fold_tap_major_kernel(const float *__restrict__ part, float *__restrict__ dw,
+                                                             int O, int C, int kHW, int64_t stride, int S) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;     // index into one partial: (o*kHW + tap)*C + c
+  if (idx >= O * C * kHW) return;
+  float acc = part[idx];
+  for (int z = 1; z < S; ++z) acc += part[z * stride + idx];
+  const int c = idx % C;
+  const int t = idx / C;
+  const int tap = t % kHW, o = t / kHW;
+  dw[(o * C + c) * kHW + tap] = acc;
 }
 
 // ------------------------------------------------------------------ host side
@@ -358,6 +549,21 @@ void launch_fwd(const ConvGeo &g, const float *x, const float *w, float *y, cons
                      int64_t(0), static_cast<int64_t>(g.oH) * g.oW, cm, M, N, K, (K + BK - 1) / BK * BK);
 }
 
+// forward with the tap-major reduction order; wf is the filter re-laid as [O][kHW][C]
+template <int BM, int BN, int WM, int WN>
+void launch_fwd_tap_major(const ConvGeo &g, const float *x, const float *wf, float *y, hipStream_t st) {
+  using AL = KContigLoader<BM>;
+  using BL = TapMajorColsLoader<BN, false>;
+  const int K = g.C * g.kH * g.kW, N = g.imgs * g.oH * g.oW, M = g.O;
+  typename AL::Params ap{wf, K, M, true};
+  typename BL::Params bp{x, FastDiv(g.oH * g.oW), FastDiv(g.oW), static_cast<int64_t>(g.C) * g.H * g.W, g.H * g.W,
+                         g.H, g.W, g.ph, g.pw, g.s, g.C, g.kW, g.kH * g.kW, N};
+  NchwCols cm{FastDiv(g.oH * g.oW), static_cast<int64_t>(g.O) * g.oH * g.oW};
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, 1);
+  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, NchwCols>), grid, dim3(kThreads), 0, st, ap, bp, y,
+                     int64_t(0), static_cast<int64_t>(g.oH) * g.oW, cm, M, N, K, K);
+}
+
 template <int BM, int BN, int WM, int WN>
 void launch_bwd_data(const ConvGeo &g, const float *wt, const float *dy, float *dx, const Tap *taps,
                      hipStream_t st) {
@@ -373,6 +579,21 @@ void launch_bwd_data(const ConvGeo &g, const float *wt, const float *dy, float *
                      int64_t(0), static_cast<int64_t>(g.H) * g.W, cm, M, N, K, (K + BK - 1) / BK * BK);
 }
 
+// stride-1 bwd-data with the tap-major reduction order; wt is the filter re-laid as [C][kHW][O]
+template <int BM, int BN, int WM, int WN>
+void launch_bwd_data_tap_major(const ConvGeo &g, const float *wt, const float *dy, float *dx, hipStream_t st) {
+  using AL = KContigLoader<BM>;
+  using BL = TapMajorColsLoader<BN, true>;
+  const int K = g.O * g.kH * g.kW, N = g.imgs * g.H * g.W, M = g.C;
+  typename AL::Params ap{wt, K, M, true};
+  typename BL::Params bp{dy, FastDiv(g.H * g.W), FastDiv(g.W), static_cast<int64_t>(g.O) * g.oH * g.oW, g.oH * g.oW,
+                         g.oH, g.oW, g.ph, g.pw, 1, g.O, g.kW, g.kH * g.kW, N};
+  NchwCols cm{FastDiv(g.H * g.W), static_cast<int64_t>(g.C) * g.H * g.W};
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, 1);
+  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, NchwCols>), grid, dim3(kThreads), 0, st, ap, bp, dx,
+                     int64_t(0), static_cast<int64_t>(g.H) * g.W, cm, M, N, K, K);
+}
+
 template <int BM, int BN, int WM, int WN>
 int launch_bwd_filter(const ConvGeo &g, const float *x, const float *dy, float *dw, const Tap *taps, hipStream_t st,
                       int64_t *ws_elems) {
@@ -384,7 +605,8 @@ int launch_bwd_filter(const ConvGeo &g, const float *x, const float *dy, float *
                          g.H, g.W, g.ph, g.pw, g.s, N};
   const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
   int S, kchunk;
-  plan_splitk(tm * tn, K, 1024, S, kchunk);
+  static const int occ = blocks_per_cu(mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>);
+  plan_splitk(tm * tn, K, 1024, occ, S, kchunk);
   const int64_t mn = static_cast<int64_t>(M) * N;
   float *out = dw;
   if (S > 1) {
@@ -400,6 +622,32 @@ int launch_bwd_filter(const ConvGeo &g, const float *x, const float *dy, float *
   return 0;
 }
 
+// bwd-filter with tap-major columns; always goes through the fold kernel, which also restores
+// the OIHW layout
+template <int BM, int BN, int WM, int WN>
+int launch_bwd_filter_tap_major(const ConvGeo &g, const float *x, const float *dy, float *dw, hipStream_t st,
+                                int64_t *ws_elems) {
+  using AL = DyRowsLoader<BM>;
+  using BL = TapMajorRowsLoader<BN>;
+  const int K = g.imgs * g.oH * g.oW, N = g.C * g.kH * g.kW, M = g.O;
+  typename AL::Params ap{dy, FastDiv(g.oH * g.oW), g.O, (g.oH * g.oW) % 4 == 0 && aligned16(dy)};
+  typename BL::Params bp{x, FastDiv(g.oH * g.oW), FastDiv(g.oW), static_cast<int64_t>(g.C) * g.H * g.W, g.H * g.W,
+                         g.H, g.W, g.ph, g.pw, g.s, g.C, g.kW, N};
+  const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+  int S, kchunk;
+  static const int occ = blocks_per_cu(mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>);
+  plan_splitk(tm * tn, K, 1024, occ, S, kchunk);
+  const int64_t mn = static_cast<int64_t>(M) * N;
+  float *part = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(S) * mn * 4));
+  TS_REQUIRE(part, "conv bwd-filter: no scratch memory for split-K");
+  *ws_elems = S * mn;
+  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>), dim3(tn, tm, S), dim3(kThreads), 0, st,
+                     ap, bp, part, mn, static_cast<int64_t>(N), RowMajorCols{}, M, N, K, kchunk);
+  hipLaunchKernelGGL(fold_tap_major_kernel, dim3(static_cast<unsigned>((mn + 255) / 256)), dim3(256), 0, st, part, dw,
+                     g.O, g.C, g.kH * g.kW, mn, S);
+  return 0;
+}
+
 int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y, int ph, int pw, int s,
                  DLStreamHandle sh, ProfilerHandle p) {
   ConvGeo g;
@@ -407,12 +655,24 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
   hipStream_t st = stream_of(sh);
   ProfileScope ps(p, st, numel(x) + numel(w), numel(y), 0);
   if (numel(y) > 0) {
-    const Tap *taps = tap_table(g.C, g.kH, g.kW, g.W, g.H * g.W, +1);
-    TS_REQUIRE(taps, "%s: could not build the tap table", who);
-    if (g.O <= 64)
-      launch_fwd<64, 256, 1, 4>(g, cf(x), cf(w), mf(y), taps, st);
-    else
-      launch_fwd<128, 128, 2, 2>(g, cf(x), cf(w), mf(y), taps, st);
+    if (g.C % BK == 0) {
+      float *wf = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(numel(w)) * 4));
+      TS_REQUIRE(wf, "%s: no scratch memory", who);
+      const int total = static_cast<int>(numel(w));
+      hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wf, g.O, g.C,
+                         g.kH * g.kW, false);
+      if (g.O <= 64)
+        launch_fwd_tap_major<64, 256, 1, 4>(g, cf(x), wf, mf(y), st);
+      else
+        launch_fwd_tap_major<128, 128, 2, 2>(g, cf(x), wf, mf(y), st);
+    } else {
+      const Tap *taps = tap_table(g.C, g.kH, g.kW, g.W, g.H * g.W, +1);
+      TS_REQUIRE(taps, "%s: could not build the tap table", who);
+      if (g.O <= 64)
+        launch_fwd<64, 256, 1, 4>(g, cf(x), cf(w), mf(y), taps, st);
+      else
+        launch_fwd<128, 128, 2, 2>(g, cf(x), cf(w), mf(y), taps, st);
+    }
   }
   return ps.finish();
 }
@@ -424,18 +684,27 @@ int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray 
   hipStream_t st = stream_of(sh);
   ProfileScope ps(p, st, numel(dy) + numel(w), numel(dx), numel(w));
   if (numel(dx) > 0) {
-    // taps index dy: off = o*oH*oW (spatial part is recomputed because of the stride test)
-    const Tap *taps = tap_table(g.O, g.kH, g.kW, 0, g.oH * g.oW, 0);
-    TS_REQUIRE(taps, "%s: could not build the tap table", who);
     float *wt = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(numel(w)) * 4));
     TS_REQUIRE(wt, "%s: no scratch memory", who);
     const int total = static_cast<int>(numel(w));
-    hipLaunchKernelGGL(filter_oc_swap_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
-                       g.kH * g.kW);
-    if (g.C <= 64)
-      launch_bwd_data<64, 256, 1, 4>(g, wt, cf(dy), mf(dx), taps, st);
-    else
-      launch_bwd_data<128, 128, 2, 2>(g, wt, cf(dy), mf(dx), taps, st);
+    if (g.s == 1 && g.O % BK == 0) {
+      hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
+                         g.kH * g.kW, true);
+      if (g.C <= 64)
+        launch_bwd_data_tap_major<64, 256, 1, 4>(g, wt, cf(dy), mf(dx), st);
+      else
+        launch_bwd_data_tap_major<128, 128, 2, 2>(g, wt, cf(dy), mf(dx), st);
+    } else {
+      // taps index dy: off = o*oH*oW (the spatial part is recomputed because of the stride test)
+      const Tap *taps = tap_table(g.O, g.kH, g.kW, 0, g.oH * g.oW, 0);
+      TS_REQUIRE(taps, "%s: could not build the tap table", who);
+      hipLaunchKernelGGL(filter_oc_swap_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
+                         g.kH * g.kW);
+      if (g.C <= 64)
+        launch_bwd_data<64, 256, 1, 4>(g, wt, cf(dy), mf(dx), taps, st);
+      else
+        launch_bwd_data<128, 128, 2, 2>(g, wt, cf(dy), mf(dx), taps, st);
+    }
   }
   return ps.finish();
 }
@@ -449,12 +718,19 @@ int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArra
   ProfileScope ps(p, st, numel(x) + numel(dy), numel(dw), 0);
   int rc = 0;
   if (numel(dw) > 0) {
-    const Tap *taps = tap_table(g.C, g.kH, g.kW, g.W, g.H * g.W, +1);
-    TS_REQUIRE(taps, "%s: could not build the tap table", who);
-    if (g.O <= 64)
-      rc = launch_bwd_filter<64, 256, 1, 4>(g, cf(x), cf(dy), mf(dw), taps, st, &ws);
-    else
-      rc = launch_bwd_filter<128, 128, 2, 2>(g, cf(x), cf(dy), mf(dw), taps, st, &ws);
+    if (g.C % BK == 0) {
+      if (g.O <= 64)
+        rc = launch_bwd_filter_tap_major<64, 256, 1, 4>(g, cf(x), cf(dy), mf(dw), st, &ws);
+      else
+        rc = launch_bwd_filter_tap_major<128, 128, 2, 2>(g, cf(x), cf(dy), mf(dw), st, &ws);
+    } else {
+      const Tap *taps = tap_table(g.C, g.kH, g.kW, g.W, g.H * g.W, +1);
+      TS_REQUIRE(taps, "%s: could not build the tap table", who);
+      if (g.O <= 64)
+        rc = launch_bwd_filter<64, 256, 1, 4>(g, cf(x), cf(dy), mf(dw), taps, st, &ws);
+      else
+        rc = launch_bwd_filter<128, 128, 2, 2>(g, cf(x), cf(dy), mf(dw), taps, st, &ws);
+    }
   }
   if (p) p->workspace_memory = mib(ws);
   if (rc) return rc;

@@ -23,7 +23,8 @@ int launch_gemm(const float *A, int64_t lda, const float *B, int64_t ldb, float 
   typename BL::Params bp{B, ldb, N, ldb % 4 == 0 && aligned16(B)};
   const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
   int S, kchunk;
-  plan_splitk(tm * tn, K, 64, S, kchunk);
+  static const int occ = blocks_per_cu(mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>);
+  plan_splitk(tm * tn, K, 64, occ, S, kchunk);
   float *out = C;
   const int64_t mn = static_cast<int64_t>(M) * N;
   if (S > 1) {

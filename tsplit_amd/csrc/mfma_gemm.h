@@ -213,10 +213,12 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::P
   int stage = 0;
   for (int k0 = kbegin; k0 < kend; k0 += BK) {
     const bool more = k0 + BK < kend;
+#ifndef EXP_NOLOAD
     if (more) {
       la.load(k0 + BK, kend);
       lb.load(k0 + BK, kend);
     }
+#endif
     const float *sa = lds_a[stage], *sb = lds_b[stage];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -234,11 +236,15 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::P
           for (int ni = 0; ni < 2; ++ni)
             acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
     }
+#ifndef EXP_NOSTORE
     if (more) {
       la.store(lds_a[stage ^ 1], tid);
       lb.store(lds_b[stage ^ 1], tid);
     }
+#endif
+#ifndef EXP_NOBARRIER
     __syncthreads();
+#endif
     stage ^= 1;
   }
 
@@ -272,10 +278,13 @@ static __global__ __launch_bounds__(256) void splitk_fold_kernel(const float *__
   out[i] = s;
 }
 
-// How many K splits to use so that the launch fills the chip; kchunk is a multiple of BK.
-inline void plan_splitk(int tiles, int K, int max_split, int &S, int &kchunk) {
-  const int target = 2 * 256;   // about two blocks per CU
-  int s = tiles >= target ? 1 : (target + tiles - 1) / tiles;
+// How many K splits to use so that the launch fills the chip.  The aim is ONE full wave of
+// resident blocks (blocks_per_cu on each of the 256 CUs): fewer leaves CUs idle, and a count
+// such as 2.1 blocks per CU makes some CUs do 3 units of work while others do 2.
+// kchunk is a multiple of BK.
+inline void plan_splitk(int tiles, int K, int max_split, int blocks_per_cu, int &S, int &kchunk) {
+  const int target = 256 * (blocks_per_cu > 0 ? blocks_per_cu : 2);
+  int s = tiles >= target ? 1 : target / tiles;
   const int ksteps = (K + BK - 1) / BK;
   if (s > ksteps / 4) s = ksteps / 4;   // at least 4 k-steps per split
   if (s > max_split) s = max_split;
@@ -285,6 +294,17 @@ inline void plan_splitk(int tiles, int K, int max_split, int &S, int &kchunk) {
   kchunk = per * BK;
   S = (K + kchunk - 1) / kchunk;
   if (S < 1) S = 1;
+}
+
+// resident blocks per CU of a kernel (register/LDS limited), asked once per kernel
+template <class F>
+inline int blocks_per_cu(F kernel) {
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, kThreads, 0) != hipSuccess || n < 1) {
+    (void)hipGetLastError();
+    n = 2;
+  }
+  return n;
 }
 
 }  // namespace mg
