@@ -251,6 +251,348 @@ struct TapMajorColsLoader {
   }
 };
 
+
+// ------------------------------------------------------------------ the tap-major conv kernel
+// Forward and stride-1 backward-data for channel counts that are multiples of 16: the same
+// tiling, LDS layout and MFMA schedule as mfma_gemm_kernel with both operands mn-major, but
+// with the k-loop written so that it needs almost no vector-ALU work.  On this chip a VALU
+// instruction issued while the matrix pipe is saturated costs MFMA issue time, so address
+// arithmetic in the loop is what separates 63 % from the clock-limited rate.  Here:
+//   * all global reads are buffer loads: per-thread byte offsets are loop constants, the part
+//     that changes per step (filter tap, channel block, k position) is wave-uniform and
+//     travels in the scalar offset, computed on the scalar unit;
+//   * a thread's padding test for all taps is one bit mask built before the loop; a lane
+//     whose tap falls into the padding gets an out-of-range offset, for which a buffer load
+//     returns 0 - no zero-fill, no divergent branch.
+struct TapConvParams {
+  const float *wf;      // filter re-laid as [M][K], k' = ((ch/16)*taps + tap)*16 + ch%16
+  const float *src;     // x (forward) or dy (backward-data)
+  unsigned wf_bytes, src_bytes;
+  FastDiv plane, width; // output columns per image / per row
+  int img_stride;       // elements per image of src
+  int chan_stride;      // elements per channel plane of src
+  int src_h, src_w, ph, pw, s, kW, taps;
+  int M, N, K;
+  int out_plane;        // elements per channel plane of the output
+  int64_t out_img_stride;
+};
+
+constexpr int kBufFlags = 0x00020000;           // raw buffer, 32-bit untyped data (gfx9 family)
+constexpr unsigned kOobOffset = 0x80000000u;    // beyond any tensor this path accepts (< 2 GiB)
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <int BM, int BN, int WM, int WN, bool BWD_DATA>
+__global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, float *__restrict__ out, TileGrid tg) {
+  static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
+  using ALds = MnMajorLds<BM>;
+  using BLds = MnMajorLds<BN>;
+  constexpr int PA = BM / 64;        // 16-byte filter words per thread and step
+  constexpr int KPT = BN / 16;       // gathered values per thread and step (consecutive k')
+  __shared__ __attribute__((aligned(16))) float lds_a[2][ALds::kFloats];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][BLds::kFloats];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  if (logical >= tg.total) return;
+  const int tile_n = logical / tg.tm, tile_m = logical - tile_n * tg.tm;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
+
+  // uniform bias so that every per-thread offset is non-negative and every scalar offset too
+  const int bias = BWD_DATA ? (P.taps / P.kW - 1) * P.src_w + (P.kW - 1) : P.ph * P.src_w + P.pw;
+  const __amdgpu_buffer_rsrc_t ra =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.wf), 0, static_cast<int>(P.wf_bytes), kBufFlags);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(P.src) - bias, 0, static_cast<int>(P.src_bytes + 4u * bias), kBufFlags);
+
+  // ---- filter operand: thread -> (row tid/4 + 64 s, 16-byte word tid%4); rows clamped
+  unsigned a_voff[PA];
+#pragma unroll
+  for (int s = 0; s < PA; ++s) {
+    const int row = min(m0 + (tid >> 2) + 64 * s, P.M - 1);
+    a_voff[s] = (static_cast<unsigned>(row) * P.K + 4u * (tid & 3)) * 4u;
+  }
+  // ---- gathered operand: thread -> (column tid % BN, KPT consecutive k' starting at klocal0)
+  const int klocal0 = (tid / BN) * KPT;
+  unsigned b_voff, vmask = 0;
+  {
+    const int n = n0 + tid % BN;
+    const bool col_ok = n < P.N;
+    const uint32_t nn = col_ok ? n : 0;
+    const uint32_t img = P.plane.div(nn);
+    const uint32_t p = nn - img * P.plane.d;
+    const uint32_t row = P.width.div(p);
+    const uint32_t col = p - row * P.width.d;
+    const int r0 = BWD_DATA ? static_cast<int>(row) + P.ph : static_cast<int>(row) * P.s - P.ph;
+    const int c0 = BWD_DATA ? static_cast<int>(col) + P.pw : static_cast<int>(col) * P.s - P.pw;
+    if (col_ok) {
+      for (int t = 0; t < P.taps; ++t) {
+        const int kh = t / P.kW, kw = t - kh * P.kW;
+        const int rr = BWD_DATA ? r0 - kh : r0 + kh, cc = BWD_DATA ? c0 - kw : c0 + kw;
+        if (static_cast<unsigned>(rr) < static_cast<unsigned>(P.src_h) &&
+            static_cast<unsigned>(cc) < static_cast<unsigned>(P.src_w))
+          vmask |= 1u << t;
+      }
+    }
+    // forward : src offset = thread part + (kh*W + kw)       with the bias ph*W + pw folded in
+    // bwd-data: src offset = thread part - (kh*W + kw)       with the bias (kH-1)*W + kW-1 folded in
+    const int thread_part = BWD_DATA ? r0 * P.src_w + c0 : (r0 + P.ph) * P.src_w + (c0 + P.pw);
+    b_voff = static_cast<unsigned>(static_cast<int>(img) * P.img_stride + klocal0 * P.chan_stride + thread_part) * 4u;
+  }
+
+  acc16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  u32x4 ra_regs[PA];
+  unsigned rb_regs[KPT];
+  int tap = 0, ch0 = 0;   // position of the NEXT step to load
+
+  auto load_step = [&](int step) {
+    // filter words: scalar offset = k position of the step
+    const int soff_a = step * (BK * 4);
+#pragma unroll
+    for (int s = 0; s < PA; ++s) ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[s], soff_a, 0);
+    // gathered values: scalar offset = channel block + tap displacement
+    const int kh = tap / P.kW, kw = tap - kh * P.kW;
+    const int disp = BWD_DATA ? bias - (kh * P.src_w + kw) : kh * P.src_w + kw;
+    const int soff_b = (ch0 * P.chan_stride + disp) * 4;
+    const unsigned voff = (vmask >> tap) & 1u ? b_voff : kOobOffset;
+#pragma unroll
+    for (int i = 0; i < KPT; ++i)
+      rb_regs[i] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, soff_b + i * P.chan_stride * 4, 0);
+    if (++tap == P.taps) {
+      tap = 0;
+      ch0 += BK;
+    }
+  };
+  auto store_step = [&](float *sa, float *sb) {
+#pragma unroll
+    for (int s = 0; s < PA; ++s)
+      *reinterpret_cast<u32x4 *>(sa + ((tid >> 2) + 64 * s) * ALds::kStride + 4 * (tid & 3)) = ra_regs[s];
+#pragma unroll
+    for (int q = 0; q < KPT / 4; ++q) {
+      u32x4 v = {rb_regs[4 * q], rb_regs[4 * q + 1], rb_regs[4 * q + 2], rb_regs[4 * q + 3]};
+      *reinterpret_cast<u32x4 *>(sb + (tid % BN) * BLds::kStride + klocal0 + 4 * q) = v;
+    }
+  };
+  auto mma_step = [&](const float *sa, const float *sb) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      float fa[2][4], fb[2][4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        ALds::frag(sa, wm0 + 32 * i, j, lane, fa[i]);
+        BLds::frag(sb, wn0 + 32 * i, j, lane, fb[i]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < 2; ++ni)
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
+    }
+  };
+
+  const int steps = P.K / BK;
+  load_step(0);
+  store_step(lds_a[0], lds_b[0]);
+  __syncthreads();
+  int stage = 0;
+  for (int st = 0; st < steps; ++st) {
+    const bool more = st + 1 < steps;
+    if (more) load_step(st + 1);
+    mma_step(lds_a[stage], lds_b[stage]);
+    if (more) store_step(lds_a[stage ^ 1], lds_b[stage ^ 1]);
+    __syncthreads();
+    stage ^= 1;
+  }
+
+  // epilogue (see mfma_gemm_kernel): out[img][m][p], column n = img*plane + p
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const int n = n0 + wn0 + 32 * ni + (lane & 31);
+    if (n >= P.N) continue;
+    const uint32_t img = P.plane.div(n);
+    const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+      const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = mb + 8 * (e >> 2) + (e & 3);
+        if (m < P.M) out[static_cast<int64_t>(m) * P.out_plane + coff] = acc[mi][ni][e];
+      }
+    }
+  }
+}
+
+
+// ------------------------------------------------------------------ the tap-major filter-gradient kernel
+// Backward-filter for "same" stride-1 convolutions (oH = H, oW = W) with C % 16 == 0 and
+// H*W % 16 == 0, written like conv_tap_kernel so that the k-loop does almost no vector-ALU work.
+// The reduction runs over positions k = (img, p); because the convolution is "same", the
+// gathered element of tap (dr, dc) for output position p is x[img][c][p + dr*W + dc] - linear
+// in p - so the per-thread byte offset is a loop constant and the step's (img, p0) travels in
+// the scalar offset.  A 16-wide step never straddles two images (H*W % 16 == 0).  The padding
+// test needs the column of p, kept incrementally, and one range test on the linear index.
+struct TapWgradParams {
+  const float *dy, *x;
+  unsigned dy_bytes, x_bytes;
+  int O, C, HW, W, kW, taps;
+  int ph, pw;
+  int M, N, K;           // O, C*taps, imgs*HW
+  int kchunk;            // k range per split (multiple of 16)
+};
+
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams P, float *__restrict__ part,
+                                                                  TileGrid tg) {
+  static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
+  using ALds = MnMajorLds<BM>;
+  using BLds = MnMajorLds<BN>;
+  constexpr int PA = BM / 64;
+  constexpr int KCOLS = BN / 16;     // consecutive columns (channels of one tap) per thread
+  __shared__ __attribute__((aligned(16))) float lds_a[2][ALds::kFloats];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][BLds::kFloats];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  if (logical >= tg.total) return;
+  const int per_split = tg.tm * tg.tn;
+  const int zsplit = logical / per_split;
+  const int rem = logical - zsplit * per_split;
+  const int tile_n = rem / tg.tm, tile_m = rem - tile_n * tg.tm;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
+  const int kbegin = zsplit * P.kchunk;
+  const int kend = min(P.K, kbegin + P.kchunk);
+
+  const int bias = P.ph * P.W + P.pw;
+  const __amdgpu_buffer_rsrc_t ra =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.dy), 0, static_cast<int>(P.dy_bytes), kBufFlags);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(P.x) - bias, 0, static_cast<int>(P.x_bytes + 4u * bias), kBufFlags);
+
+  // ---- dy operand: thread -> (row tid/4 + 64 s, 4 consecutive positions tid%4)
+  unsigned a_voff[PA];
+#pragma unroll
+  for (int s = 0; s < PA; ++s) {
+    const int row = min(m0 + (tid >> 2) + 64 * s, P.O - 1);
+    a_voff[s] = (static_cast<unsigned>(row) * P.HW + 4u * (tid & 3)) * 4u;
+  }
+  // ---- x operand: thread -> (position tid%16 of the step, KCOLS consecutive channels of one tap)
+  const int klocal = tid & 15;
+  const int jlocal0 = KCOLS * (tid >> 4);
+  const int j = n0 + jlocal0;
+  const bool cols_ok = j < P.N;                   // C % KCOLS == 0: all of a thread's columns or none
+  const int jj = cols_ok ? j : 0;
+  const int tap = jj / P.C, c_first = jj - tap * P.C;
+  const int kh = tap / P.kW, kw = tap - kh * P.kW;
+  const int dr = kh - P.ph, dc = kw - P.pw;
+  const int shift = dr * P.W + dc;                // x index = p + shift
+  const unsigned b_voff = static_cast<unsigned>(c_first * P.HW + klocal + shift + bias) * 4u;
+
+  acc16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int jx = 0; jx < 2; ++jx)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][jx][e] = 0.f;
+
+  // uniform position of the NEXT step to load, and this thread's column within the image row
+  int img = kbegin / P.HW, p0 = kbegin - img * P.HW;
+  int ow = (p0 + klocal) % P.W;
+
+  u32x4 ra_regs[PA];
+  unsigned rb_regs[KCOLS];
+
+  auto load_step = [&]() {
+    const int soff_a = (img * P.O * P.HW + p0) * 4;
+#pragma unroll
+    for (int s = 0; s < PA; ++s) ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[s], soff_a, 0);
+    const int p = p0 + klocal;
+    const bool ok = cols_ok && static_cast<unsigned>(p + dr * P.W) < static_cast<unsigned>(P.HW) &&
+                    static_cast<unsigned>(ow + dc) < static_cast<unsigned>(P.W);
+    const unsigned voff = ok ? b_voff : kOobOffset;
+    const int soff_b = (img * P.C * P.HW + p0) * 4;
+#pragma unroll
+    for (int i = 0; i < KCOLS; ++i)
+      rb_regs[i] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, soff_b + i * P.HW * 4, 0);
+    p0 += BK;
+    if (p0 >= P.HW) {
+      p0 = 0;
+      ++img;
+    }
+    ow += BK;                      // BK may exceed W for tiny images: reduce until in range
+    while (ow >= P.W) ow -= P.W;
+  };
+  auto store_step = [&](float *sa, float *sb) {
+#pragma unroll
+    for (int s = 0; s < PA; ++s)
+      *reinterpret_cast<u32x4 *>(sa + ((tid >> 2) + 64 * s) * ALds::kStride + 4 * (tid & 3)) = ra_regs[s];
+#pragma unroll
+    for (int i = 0; i < KCOLS; ++i)
+      reinterpret_cast<unsigned *>(sb)[(jlocal0 + i) * BLds::kStride + klocal] = rb_regs[i];
+  };
+  auto mma_step = [&](const float *sa, const float *sb) {
+#pragma unroll
+    for (int jg = 0; jg < 2; ++jg) {
+      float fa[2][4], fb[2][4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        ALds::frag(sa, wm0 + 32 * i, jg, lane, fa[i]);
+        BLds::frag(sb, wn0 + 32 * i, jg, lane, fb[i]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < 2; ++ni)
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
+    }
+  };
+
+  const int steps = (kend - kbegin) / BK;    // K and kchunk are multiples of 16
+  if (steps > 0) {
+    load_step();
+    store_step(lds_a[0], lds_b[0]);
+  }
+  __syncthreads();
+  int stage = 0;
+  for (int st = 0; st < steps; ++st) {
+    const bool more = st + 1 < steps;
+    if (more) load_step();
+    mma_step(lds_a[stage], lds_b[stage]);
+    if (more) store_step(lds_a[stage ^ 1], lds_b[stage ^ 1]);
+    __syncthreads();
+    stage ^= 1;
+  }
+
+  float *o = part + static_cast<int64_t>(zsplit) * P.M * P.N;
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const int n = n0 + wn0 + 32 * ni + (lane & 31);
+    if (n >= P.N) continue;
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+      const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = mb + 8 * (e >> 2) + (e & 3);
+        if (m < P.M) o[static_cast<int64_t>(m) * P.N + n] = acc[mi][ni][e];
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------ bwd-filter loaders, mn-major
 // A = dy: row m = output channel, k = (img, p); K contiguous inside an image.
 template <int BM>
@@ -544,9 +886,10 @@ void launch_fwd(const ConvGeo &g, const float *x, const float *w, float *y, cons
   typename BL::Params bp{x, taps, FastDiv(g.oH * g.oW), FastDiv(g.oW), static_cast<int64_t>(g.C) * g.H * g.W,
                          g.H, g.W, g.ph, g.pw, g.s, N};
   NchwCols cm{FastDiv(g.oH * g.oW), static_cast<int64_t>(g.O) * g.oH * g.oW};
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, 1);
+  const int tn = (N + BN - 1) / BN, tm = (M + BM - 1) / BM;
+  dim3 grid(grid_blocks(tm, tn, 1));
   hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, NchwCols>), grid, dim3(kThreads), 0, st, ap, bp, y,
-                     int64_t(0), static_cast<int64_t>(g.oH) * g.oW, cm, M, N, K, (K + BK - 1) / BK * BK);
+                     int64_t(0), static_cast<int64_t>(g.oH) * g.oW, cm, M, N, K, (K + BK - 1) / BK * BK, TileGrid{tm, tn, tm * tn});
 }
 
 // forward with the tap-major reduction order; wf is the filter re-laid as [O][kHW][C]
@@ -559,9 +902,10 @@ void launch_fwd_tap_major(const ConvGeo &g, const float *x, const float *wf, flo
   typename BL::Params bp{x, FastDiv(g.oH * g.oW), FastDiv(g.oW), static_cast<int64_t>(g.C) * g.H * g.W, g.H * g.W,
                          g.H, g.W, g.ph, g.pw, g.s, g.C, g.kW, g.kH * g.kW, N};
   NchwCols cm{FastDiv(g.oH * g.oW), static_cast<int64_t>(g.O) * g.oH * g.oW};
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, 1);
+  const int tn = (N + BN - 1) / BN, tm = (M + BM - 1) / BM;
+  dim3 grid(grid_blocks(tm, tn, 1));
   hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, NchwCols>), grid, dim3(kThreads), 0, st, ap, bp, y,
-                     int64_t(0), static_cast<int64_t>(g.oH) * g.oW, cm, M, N, K, K);
+                     int64_t(0), static_cast<int64_t>(g.oH) * g.oW, cm, M, N, K, K, TileGrid{tm, tn, tm * tn});
 }
 
 template <int BM, int BN, int WM, int WN>
@@ -574,9 +918,10 @@ void launch_bwd_data(const ConvGeo &g, const float *wt, const float *dy, float *
   typename BL::Params bp{dy, taps, FastDiv(g.H * g.W), FastDiv(g.W), static_cast<int64_t>(g.O) * g.oH * g.oW,
                          g.oH, g.oW, g.ph, g.pw, g.s, N};
   NchwCols cm{FastDiv(g.H * g.W), static_cast<int64_t>(g.C) * g.H * g.W};
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, 1);
+  const int tn = (N + BN - 1) / BN, tm = (M + BM - 1) / BM;
+  dim3 grid(grid_blocks(tm, tn, 1));
   hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, NchwCols>), grid, dim3(kThreads), 0, st, ap, bp, dx,
-                     int64_t(0), static_cast<int64_t>(g.H) * g.W, cm, M, N, K, (K + BK - 1) / BK * BK);
+                     int64_t(0), static_cast<int64_t>(g.H) * g.W, cm, M, N, K, (K + BK - 1) / BK * BK, TileGrid{tm, tn, tm * tn});
 }
 
 // stride-1 bwd-data with the tap-major reduction order; wt is the filter re-laid as [C][kHW][O]
@@ -589,9 +934,10 @@ void launch_bwd_data_tap_major(const ConvGeo &g, const float *wt, const float *d
   typename BL::Params bp{dy, FastDiv(g.H * g.W), FastDiv(g.W), static_cast<int64_t>(g.O) * g.oH * g.oW, g.oH * g.oW,
                          g.oH, g.oW, g.ph, g.pw, 1, g.O, g.kW, g.kH * g.kW, N};
   NchwCols cm{FastDiv(g.H * g.W), static_cast<int64_t>(g.C) * g.H * g.W};
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, 1);
+  const int tn = (N + BN - 1) / BN, tm = (M + BM - 1) / BM;
+  dim3 grid(grid_blocks(tm, tn, 1));
   hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, NchwCols>), grid, dim3(kThreads), 0, st, ap, bp, dx,
-                     int64_t(0), static_cast<int64_t>(g.H) * g.W, cm, M, N, K, K);
+                     int64_t(0), static_cast<int64_t>(g.H) * g.W, cm, M, N, K, K, TileGrid{tm, tn, tm * tn});
 }
 
 template <int BM, int BN, int WM, int WN>
@@ -614,8 +960,9 @@ int launch_bwd_filter(const ConvGeo &g, const float *x, const float *dy, float *
     TS_REQUIRE(out, "conv bwd-filter: no scratch memory for split-K");
     *ws_elems = S * mn;
   }
-  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>), dim3(tn, tm, S), dim3(kThreads), 0, st,
-                     ap, bp, out, mn, static_cast<int64_t>(N), RowMajorCols{}, M, N, K, kchunk);
+  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>), dim3(grid_blocks(tm, tn, S)),
+                     dim3(kThreads), 0, st, ap, bp, out, mn, static_cast<int64_t>(N), RowMajorCols{}, M, N, K, kchunk,
+                     TileGrid{tm, tn, tm * tn * S});
   if (S > 1)
     hipLaunchKernelGGL(splitk_fold_kernel, dim3(static_cast<unsigned>((mn + 255) / 256)), dim3(256), 0, st, out, dw,
                        mn, mn, S);
@@ -641,11 +988,103 @@ int launch_bwd_filter_tap_major(const ConvGeo &g, const float *x, const float *d
   float *part = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(S) * mn * 4));
   TS_REQUIRE(part, "conv bwd-filter: no scratch memory for split-K");
   *ws_elems = S * mn;
-  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>), dim3(tn, tm, S), dim3(kThreads), 0, st,
-                     ap, bp, part, mn, static_cast<int64_t>(N), RowMajorCols{}, M, N, K, kchunk);
+  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>), dim3(grid_blocks(tm, tn, S)),
+                     dim3(kThreads), 0, st, ap, bp, part, mn, static_cast<int64_t>(N), RowMajorCols{}, M, N, K, kchunk,
+                     TileGrid{tm, tn, tm * tn * S});
   hipLaunchKernelGGL(fold_tap_major_kernel, dim3(static_cast<unsigned>((mn + 255) / 256)), dim3(256), 0, st, part, dw,
                      g.O, g.C, g.kH * g.kW, mn, S);
   return 0;
+}
+
+// launches conv_tap_kernel; `w_relaid` is [M][K] in the tap-major order
+template <int BM, int BN, int WM, int WN, bool BWD_DATA>
+void launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, float *out, hipStream_t st) {
+  TapConvParams P;
+  const int taps = g.kH * g.kW;
+  if (BWD_DATA) {   // out = dx [imgs][C][H][W], src = dy [imgs][O][oH][oW]
+    P.M = g.C;
+    P.N = g.imgs * g.H * g.W;
+    P.K = g.O * taps;
+    P.plane = FastDiv(g.H * g.W);
+    P.width = FastDiv(g.W);
+    P.img_stride = g.O * g.oH * g.oW;
+    P.chan_stride = g.oH * g.oW;
+    P.src_h = g.oH;
+    P.src_w = g.oW;
+    P.out_plane = g.H * g.W;
+    P.out_img_stride = static_cast<int64_t>(g.C) * g.H * g.W;
+    P.src_bytes = static_cast<unsigned>(static_cast<int64_t>(g.imgs) * g.O * g.oH * g.oW * 4);
+  } else {          // out = y [imgs][O][oH][oW], src = x [imgs][C][H][W]
+    P.M = g.O;
+    P.N = g.imgs * g.oH * g.oW;
+    P.K = g.C * taps;
+    P.plane = FastDiv(g.oH * g.oW);
+    P.width = FastDiv(g.oW);
+    P.img_stride = g.C * g.H * g.W;
+    P.chan_stride = g.H * g.W;
+    P.src_h = g.H;
+    P.src_w = g.W;
+    P.out_plane = g.oH * g.oW;
+    P.out_img_stride = static_cast<int64_t>(g.O) * g.oH * g.oW;
+    P.src_bytes = static_cast<unsigned>(static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4);
+  }
+  P.wf = w_relaid;
+  P.src = src;
+  P.wf_bytes = static_cast<unsigned>(static_cast<int64_t>(P.M) * P.K * 4);
+  P.ph = g.ph;
+  P.pw = g.pw;
+  P.s = g.s;
+  P.kW = g.kW;
+  P.taps = taps;
+  const int tn = (P.N + BN - 1) / BN, tm = (P.M + BM - 1) / BM;
+  hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>), dim3(grid_blocks(tm, tn, 1)), dim3(kThreads), 0, st,
+                     P, out, TileGrid{tm, tn, tm * tn});
+}
+
+// the buffer-load path addresses with 32-bit byte offsets and a 32-tap bit mask
+inline bool tap_kernel_ok(const ConvGeo &g, int64_t src_elems, int64_t w_elems) {
+  return g.kH * g.kW <= 32 && src_elems * 4 + 4 * (static_cast<int64_t>(g.kH) * g.W + g.kW + g.ph * g.W + g.pw) < (1ll << 31) &&
+         w_elems * 4 < (1ll << 31);
+}
+
+// bwd-filter on conv_wgrad_tap_kernel ("same" stride-1 convolutions)
+template <int BM, int BN, int WM, int WN>
+int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *dw, hipStream_t st, int64_t *ws_elems) {
+  TapWgradParams P;
+  P.dy = dy;
+  P.x = x;
+  P.dy_bytes = static_cast<unsigned>(static_cast<int64_t>(g.imgs) * g.O * g.H * g.W * 4);
+  P.x_bytes = static_cast<unsigned>(static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4);
+  P.O = g.O;
+  P.C = g.C;
+  P.HW = g.H * g.W;
+  P.W = g.W;
+  P.kW = g.kW;
+  P.taps = g.kH * g.kW;
+  P.ph = g.ph;
+  P.pw = g.pw;
+  P.M = g.O;
+  P.N = g.C * g.kH * g.kW;
+  P.K = g.imgs * g.H * g.W;
+  const int tm = (P.M + BM - 1) / BM, tn = (P.N + BN - 1) / BN;
+  int S;
+  static const int occ = blocks_per_cu(conv_wgrad_tap_kernel<BM, BN, WM, WN>);
+  plan_splitk(tm * tn, P.K, 1024, occ, S, P.kchunk);
+  const int64_t mn = static_cast<int64_t>(P.M) * P.N;
+  float *part = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(S) * mn * 4));
+  TS_REQUIRE(part, "conv bwd-filter: no scratch memory for split-K");
+  *ws_elems = S * mn;
+  hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN>), dim3(grid_blocks(tm, tn, S)), dim3(kThreads), 0, st, P,
+                     part, TileGrid{tm, tn, tm * tn * S});
+  hipLaunchKernelGGL(fold_tap_major_kernel, dim3(static_cast<unsigned>((mn + 255) / 256)), dim3(256), 0, st, part, dw,
+                     g.O, g.C, g.kH * g.kW, mn, S);
+  return 0;
+}
+
+inline bool wgrad_tap_ok(const ConvGeo &g) {
+  const int64_t bytes_x = static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4, bytes_dy = static_cast<int64_t>(g.imgs) * g.O * g.H * g.W * 4;
+  return g.s == 1 && g.oH == g.H && g.oW == g.W && (g.H * g.W) % BK == 0 && g.C % BK == 0 &&
+         bytes_x + 4 * (static_cast<int64_t>(g.ph) * g.W + g.pw) < (1ll << 31) && bytes_dy < (1ll << 31);
 }
 
 int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y, int ph, int pw, int s,
@@ -661,10 +1100,16 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
       const int total = static_cast<int>(numel(w));
       hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wf, g.O, g.C,
                          g.kH * g.kW, false);
-      if (g.O <= 64)
+      if (tap_kernel_ok(g, numel(x), numel(w))) {
+        if (g.O <= 64)
+          launch_conv_tap<64, 256, 1, 4, false>(g, cf(x), wf, mf(y), st);
+        else
+          launch_conv_tap<128, 128, 2, 2, false>(g, cf(x), wf, mf(y), st);
+      } else if (g.O <= 64) {
         launch_fwd_tap_major<64, 256, 1, 4>(g, cf(x), wf, mf(y), st);
-      else
+      } else {
         launch_fwd_tap_major<128, 128, 2, 2>(g, cf(x), wf, mf(y), st);
+      }
     } else {
       const Tap *taps = tap_table(g.C, g.kH, g.kW, g.W, g.H * g.W, +1);
       TS_REQUIRE(taps, "%s: could not build the tap table", who);
@@ -690,10 +1135,16 @@ int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray 
     if (g.s == 1 && g.O % BK == 0) {
       hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
                          g.kH * g.kW, true);
-      if (g.C <= 64)
+      if (tap_kernel_ok(g, numel(dy), numel(w))) {
+        if (g.C <= 64)
+          launch_conv_tap<64, 256, 1, 4, true>(g, cf(dy), wt, mf(dx), st);
+        else
+          launch_conv_tap<128, 128, 2, 2, true>(g, cf(dy), wt, mf(dx), st);
+      } else if (g.C <= 64) {
         launch_bwd_data_tap_major<64, 256, 1, 4>(g, wt, cf(dy), mf(dx), st);
-      else
+      } else {
         launch_bwd_data_tap_major<128, 128, 2, 2>(g, wt, cf(dy), mf(dx), st);
+      }
     } else {
       // taps index dy: off = o*oH*oW (the spatial part is recomputed because of the stride test)
       const Tap *taps = tap_table(g.O, g.kH, g.kW, 0, g.oH * g.oW, 0);
@@ -718,7 +1169,12 @@ int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArra
   ProfileScope ps(p, st, numel(x) + numel(dy), numel(dw), 0);
   int rc = 0;
   if (numel(dw) > 0) {
-    if (g.C % BK == 0) {
+    if (wgrad_tap_ok(g)) {
+      if (g.O <= 64)
+        rc = launch_wgrad_tap<64, 256, 1, 4>(g, cf(x), cf(dy), mf(dw), st, &ws);
+      else
+        rc = launch_wgrad_tap<128, 128, 2, 2>(g, cf(x), cf(dy), mf(dw), st, &ws);
+    } else if (g.C % BK == 0) {
       if (g.O <= 64)
         rc = launch_bwd_filter_tap_major<64, 256, 1, 4>(g, cf(x), cf(dy), mf(dw), st, &ws);
       else
@@ -741,6 +1197,18 @@ int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArra
 }  // namespace tsplit
 
 using namespace tsplit;
+
+#ifdef EXP_TIMING
+extern "C" int ts_debug_read(unsigned long long *out, int reset) {
+  (void)hipDeviceSynchronize();
+  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(mg::g_dbg), 16 * sizeof(unsigned long long)) != hipSuccess) return -1;
+  if (reset) {
+    unsigned long long z[16] = {0};
+    (void)hipMemcpyToSymbol(HIP_SYMBOL(mg::g_dbg), z, sizeof(z));
+  }
+  return 0;
+}
+#endif
 
 extern "C" {
 

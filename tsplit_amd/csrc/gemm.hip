@@ -32,8 +32,9 @@ int launch_gemm(const float *A, int64_t lda, const float *B, int64_t ldb, float 
     TS_REQUIRE(out, "DLGpuMatrixMultiply: no scratch memory for split-K");
     *ws_elems = S * mn;
   }
-  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>), dim3(tn, tm, S), dim3(kThreads), 0, s,
-                     ap, bp, out, mn, static_cast<int64_t>(N), RowMajorCols{}, M, N, K, kchunk);
+  hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>), dim3(grid_blocks(tm, tn, S)),
+                     dim3(kThreads), 0, s, ap, bp, out, mn, static_cast<int64_t>(N), RowMajorCols{}, M, N, K, kchunk,
+                     TileGrid{tm, tn, tm * tn * S});
   if (S > 1)
     hipLaunchKernelGGL(splitk_fold_kernel, dim3(static_cast<unsigned>((mn + 255) / 256)), dim3(256), 0, s, out, C, mn,
                        mn, S);

@@ -170,13 +170,37 @@ struct RowMajorCols {   // out[m * row_stride + n]
   __device__ __forceinline__ int64_t operator()(int n) const { return n; }
 };
 
+#ifdef EXP_TIMING
+__device__ unsigned long long g_dbg[16];
+#define TS_CLK() __builtin_readcyclecounter()
+#define TS_T(i) { __builtin_amdgcn_sched_barrier(0); unsigned long long now_ = TS_CLK(); __builtin_amdgcn_sched_barrier(0); tacc[i] += now_ - tlast; tlast = now_; }
+#else
+#define TS_T(i)
+#endif
 // ------------------------------------------------------------------ the kernel
-// grid: x = N tiles, y = M tiles, z = K splits.  Split z writes to out + z * z_stride.
+// 1-D grid of grid_blocks(tm, tn, S) blocks; split z writes to out + z * z_stride.
+//
+// Block -> (tile, split) mapping.  The 8 XCDs of the chip each have their own L2 and the
+// dispatcher deals consecutive workgroup ids to them round-robin, so blocks that read the same
+// data should sit 8 ids apart.  The ids are therefore transposed (id % 8 selects a contiguous
+// eighth of the logical order) and the logical order puts the sharers next to each other: the
+// M tiles of one N tile (same gathered activations), then the N tiles, then the K splits (all
+// tiles of one split read the same k-range of both operands).
+struct TileGrid {
+  int tm, tn, total;   // M tiles, N tiles, tm * tn * S
+};
+inline unsigned grid_blocks(int tm, int tn, int S) { return static_cast<unsigned>((tm * tn * S + 7) / 8 * 8); }
+
+#ifdef EXP_WAVES4
+#define TS_OCC __attribute__((amdgpu_waves_per_eu(4, 4)))
+#else
+#define TS_OCC
+#endif
 template <int BM, int BN, int WM, int WN, class ALoader, class BLoader, class ColMap>
-__global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::Params ap, typename BLoader::Params bp,
+__global__ __launch_bounds__(kThreads) TS_OCC void mfma_gemm_kernel(typename ALoader::Params ap, typename BLoader::Params bp,
                                                              float *__restrict__ out, int64_t z_stride,
                                                              int64_t row_stride, ColMap colmap, int M, int N, int K,
-                                                             int kchunk) {
+                                                             int kchunk, TileGrid tg) {
   static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
   using ALds = typename ALoader::Lds;
   using BLds = typename BLoader::Lds;
@@ -184,9 +208,15 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::P
   __shared__ __attribute__((aligned(16))) float lds_b[2][BLds::kFloats];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  if (logical >= tg.total) return;   // padding of the grid to a multiple of 8
+  const int per_split = tg.tm * tg.tn;
+  const int zsplit = logical / per_split;
+  const int rem = logical - zsplit * per_split;
+  const int tile_n = rem / tg.tm, tile_m = rem - tile_n * tg.tm;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
-  const int kbegin = blockIdx.z * kchunk;
+  const int kbegin = zsplit * kchunk;
   const int kend = min(K, kbegin + kchunk);
 
   ALoader la;
@@ -210,15 +240,21 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::P
   }
   __syncthreads();
 
+#ifdef EXP_TIMING
+  unsigned long long tacc[5] = {0, 0, 0, 0, 0};
+  unsigned long long tlast = TS_CLK();
+#endif
   int stage = 0;
   for (int k0 = kbegin; k0 < kend; k0 += BK) {
     const bool more = k0 + BK < kend;
 #ifndef EXP_NOLOAD
     if (more) {
       la.load(k0 + BK, kend);
+      TS_T(4)
       lb.load(k0 + BK, kend);
     }
 #endif
+    TS_T(0)
     const float *sa = lds_a[stage], *sb = lds_b[stage];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -236,21 +272,30 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::P
           for (int ni = 0; ni < 2; ++ni)
             acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
     }
+    TS_T(1)
 #ifndef EXP_NOSTORE
     if (more) {
       la.store(lds_a[stage ^ 1], tid);
       lb.store(lds_b[stage ^ 1], tid);
     }
 #endif
+    TS_T(2)
 #ifndef EXP_NOBARRIER
     __syncthreads();
 #endif
+    TS_T(3)
     stage ^= 1;
   }
+#ifdef EXP_TIMING
+  if (lane == 0 && (logical % 97) == 5) {
+    for (int i = 0; i < 5; ++i) atomicAdd(&g_dbg[i + 5], tacc[i]);
+    atomicAdd(&g_dbg[4], 1ull);
+  }
+#endif
 
   // epilogue: accumulator register e of a 32x32 block holds row 8*(e/4) + 4*(lane/32) + e%4,
   // column lane%32
-  float *o = out + static_cast<int64_t>(blockIdx.z) * z_stride;
+  float *o = out + static_cast<int64_t>(zsplit) * z_stride;
 #pragma unroll
   for (int ni = 0; ni < 2; ++ni) {
     const int n = n0 + wn0 + 32 * ni + (lane & 31);
