@@ -31,11 +31,12 @@ struct Geo {
   int C;
 };
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 template <int VEC>
 struct Word;
 template <>
 struct Word<4> {
-  using T = float4;
+  using T = f32x4;
 };
 template <>
 struct Word<1> {
@@ -49,7 +50,7 @@ __device__ __forceinline__ int64_t word_addr(const Geo &g, uint32_t i, int c) {
   return (static_cast<int64_t>(n) * g.C + c) * g.wpp + j;
 }
 
-__device__ __forceinline__ void acc2(const float4 &v, float &s, float &q) {
+__device__ __forceinline__ void acc2(const f32x4 &v, float &s, float &q) {
   s += (v.x + v.y) + (v.z + v.w);
   q += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
 }
@@ -57,7 +58,7 @@ __device__ __forceinline__ void acc2(const float &v, float &s, float &q) {
   s += v;
   q += v * v;
 }
-__device__ __forceinline__ void acc_dot(const float4 &a, const float4 &b, float &s, float &d) {
+__device__ __forceinline__ void acc_dot(const f32x4 &a, const f32x4 &b, float &s, float &d) {
   s += (a.x + a.y) + (a.z + a.w);
   d += (a.x * b.x + a.y * b.y) + (a.z * b.z + a.w * b.w);
 }
@@ -65,13 +66,15 @@ __device__ __forceinline__ void acc_dot(const float &a, const float &b, float &s
   s += a;
   d += a * b;
 }
-__device__ __forceinline__ float4 axpb(const float4 &x, float a, float b) {
-  return make_float4(a * x.x + b, a * x.y + b, a * x.z + b, a * x.w + b);
+__device__ __forceinline__ f32x4 axpb(const f32x4 &x, float a, float b) {
+  const f32x4 r = {a * x.x + b, a * x.y + b, a * x.z + b, a * x.w + b};
+  return r;
 }
 __device__ __forceinline__ float axpb(const float &x, float a, float b) { return a * x + b; }
-__device__ __forceinline__ float4 lin2(const float4 &dy, const float4 &x, float k1, float k2, float k3) {
-  return make_float4(k1 * dy.x + k2 * x.x + k3, k1 * dy.y + k2 * x.y + k3, k1 * dy.z + k2 * x.z + k3,
-                     k1 * dy.w + k2 * x.w + k3);
+__device__ __forceinline__ f32x4 lin2(const f32x4 &dy, const f32x4 &x, float k1, float k2, float k3) {
+  const f32x4 r = {k1 * dy.x + k2 * x.x + k3, k1 * dy.y + k2 * x.y + k3, k1 * dy.z + k2 * x.z + k3,
+                   k1 * dy.w + k2 * x.w + k3};
+  return r;
 }
 __device__ __forceinline__ float lin2(const float &dy, const float &x, float k1, float k2, float k3) {
   return k1 * dy + k2 * x + k3;
@@ -89,15 +92,11 @@ __global__ __launch_bounds__(kThreads) void bn_stats_kernel(const float *__restr
   const W *xw = reinterpret_cast<const W *>(x);
   float sum = 0.f, sq = 0.f;
   uint32_t i = begin + threadIdx.x;
-  for (; i + 3 * kThreads < end; i += 4 * kThreads) {
-    W v0 = xw[word_addr<VEC>(g, i, c)];
-    W v1 = xw[word_addr<VEC>(g, i + kThreads, c)];
-    W v2 = xw[word_addr<VEC>(g, i + 2 * kThreads, c)];
-    W v3 = xw[word_addr<VEC>(g, i + 3 * kThreads, c)];
+  for (; i + kThreads < end; i += 2 * kThreads) {
+    const W v0 = xw[word_addr<VEC>(g, i, c)];
+    const W v1 = xw[word_addr<VEC>(g, i + kThreads, c)];
     acc2(v0, sum, sq);
     acc2(v1, sum, sq);
-    acc2(v2, sum, sq);
-    acc2(v3, sum, sq);
   }
   for (; i < end; i += kThreads) acc2(xw[word_addr<VEC>(g, i, c)], sum, sq);
   const double ds = block_sum<double, kWaves>(static_cast<double>(sum), sm);
@@ -118,13 +117,18 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(const float *__restr
                                                             float *__restrict__ save_istd) {
   using W = typename Word<VEC>::T;
   __shared__ float coef[2];
+  __shared__ double sm[kWaves];
   const int c = blockIdx.y;
+  double s = 0.0, q = 0.0;
+  for (int k = threadIdx.x; k < S; k += kThreads) {   // fixed order per thread, fixed tree: deterministic
+    s += part[(static_cast<int64_t>(c) * S + k) * 2];
+    q += part[(static_cast<int64_t>(c) * S + k) * 2 + 1];
+  }
+  if (S > 1) {
+    s = block_sum<double, kWaves>(s, sm);
+    q = block_sum<double, kWaves>(q, sm);
+  }
   if (threadIdx.x == 0) {
-    double s = 0.0, q = 0.0;
-    for (int k = 0; k < S; ++k) {
-      s += part[(static_cast<int64_t>(c) * S + k) * 2];
-      q += part[(static_cast<int64_t>(c) * S + k) * 2 + 1];
-    }
     const double mean = s * inv_m;
     double var = q * inv_m - mean * mean;
     if (var < 0.0) var = 0.0;
@@ -143,19 +147,17 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(const float *__restr
   const uint32_t end = min(begin + g.chunk, g.words);
   const W *xw = reinterpret_cast<const W *>(x);
   W *yw = reinterpret_cast<W *>(y);
+  // second and last touch of x, only touch of y: non-temporal both ways
   uint32_t i = begin + threadIdx.x;
-  for (; i + 3 * kThreads < end; i += 4 * kThreads) {
-    const int64_t a0 = word_addr<VEC>(g, i, c), a1 = word_addr<VEC>(g, i + kThreads, c),
-                  a2 = word_addr<VEC>(g, i + 2 * kThreads, c), a3 = word_addr<VEC>(g, i + 3 * kThreads, c);
-    W v0 = xw[a0], v1 = xw[a1], v2 = xw[a2], v3 = xw[a3];
-    yw[a0] = axpb(v0, a, b);
-    yw[a1] = axpb(v1, a, b);
-    yw[a2] = axpb(v2, a, b);
-    yw[a3] = axpb(v3, a, b);
+  for (; i + kThreads < end; i += 2 * kThreads) {
+    const int64_t a0 = word_addr<VEC>(g, i, c), a1 = word_addr<VEC>(g, i + kThreads, c);
+    const W v0 = __builtin_nontemporal_load(xw + a0), v1 = __builtin_nontemporal_load(xw + a1);
+    __builtin_nontemporal_store(axpb(v0, a, b), yw + a0);
+    __builtin_nontemporal_store(axpb(v1, a, b), yw + a1);
   }
   for (; i < end; i += kThreads) {
     const int64_t a0 = word_addr<VEC>(g, i, c);
-    yw[a0] = axpb(xw[a0], a, b);
+    __builtin_nontemporal_store(axpb(__builtin_nontemporal_load(xw + a0), a, b), yw + a0);
   }
 }
 
@@ -214,16 +216,23 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_dx_kernel(const float *__rest
                                                              float *__restrict__ dgamma, float *__restrict__ dbeta) {
   using W = typename Word<VEC>::T;
   __shared__ float coef[3];
+  __shared__ double sm[kWaves];
   const int c = blockIdx.y;
+  double sdy = 0.0, sdx = 0.0, sx = 0.0, sq = 0.0;
+  for (int k = threadIdx.x; k < S; k += kThreads) {
+    const double *o = part + (static_cast<int64_t>(c) * S + k) * 4;
+    sdy += o[0];
+    sdx += o[1];
+    sx += o[2];
+    sq += o[3];
+  }
+  if (S > 1) {
+    sdy = block_sum<double, kWaves>(sdy, sm);
+    sdx = block_sum<double, kWaves>(sdx, sm);
+    sx = block_sum<double, kWaves>(sx, sm);
+    sq = block_sum<double, kWaves>(sq, sm);
+  }
   if (threadIdx.x == 0) {
-    double sdy = 0.0, sdx = 0.0, sx = 0.0, sq = 0.0;
-    for (int k = 0; k < S; ++k) {
-      const double *o = part + (static_cast<int64_t>(c) * S + k) * 4;
-      sdy += o[0];
-      sdx += o[1];
-      sx += o[2];
-      sq += o[3];
-    }
     double mean, istd;
     if (save_mean && save_istd) {
       mean = static_cast<double>(save_mean[c]);
@@ -257,13 +266,15 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_dx_kernel(const float *__rest
   uint32_t i = begin + threadIdx.x;
   for (; i + kThreads < end; i += 2 * kThreads) {
     const int64_t a0 = word_addr<VEC>(g, i, c), a1 = word_addr<VEC>(g, i + kThreads, c);
-    W x0 = xw[a0], d0 = dw[a0], x1 = xw[a1], d1 = dw[a1];
-    ow[a0] = lin2(d0, x0, k1, k2, k3);
-    ow[a1] = lin2(d1, x1, k1, k2, k3);
+    const W x0 = __builtin_nontemporal_load(xw + a0), d0 = __builtin_nontemporal_load(dw + a0);
+    const W x1 = __builtin_nontemporal_load(xw + a1), d1 = __builtin_nontemporal_load(dw + a1);
+    __builtin_nontemporal_store(lin2(d0, x0, k1, k2, k3), ow + a0);
+    __builtin_nontemporal_store(lin2(d1, x1, k1, k2, k3), ow + a1);
   }
   for (; i < end; i += kThreads) {
     const int64_t a0 = word_addr<VEC>(g, i, c);
-    ow[a0] = lin2(dw[a0], xw[a0], k1, k2, k3);
+    __builtin_nontemporal_store(lin2(__builtin_nontemporal_load(dw + a0), __builtin_nontemporal_load(xw + a0), k1, k2, k3),
+                                ow + a0);
   }
 }
 
@@ -324,8 +335,8 @@ int CuDNN_DLGpuBatch_Normalization(const DLArrayHandle input_X, const DLArrayHan
   hipStream_t s = stream_of(stream_handle);
   const bool al = aligned16(input_X->data) && aligned16(output_Y->data);
   Plan st, ap;
-  TS_REQUIRE(make_plan(input_X, al, 64 * kThreads, 4096, st), "BatchNorm: unsupported shape");
-  TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 1 << 20, ap), "BatchNorm: unsupported shape");
+  TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 16384, st), "BatchNorm: unsupported shape");
+  TS_REQUIRE(make_plan(input_X, al, 4 * kThreads, 1 << 22, ap), "BatchNorm: unsupported shape");
   double *part = static_cast<double *>(scratch_get(s, 1, static_cast<size_t>(C) * st.S * 2 * sizeof(double)));
   TS_REQUIRE(part, "BatchNorm: no scratch memory");
   ProfileScope ps(p, s, numel(input_X) + 2 * C, numel(output_Y), C * st.S * 4);
@@ -364,8 +375,8 @@ int CuDNN_DLGpuBatch_Normalization_gradient(const DLArrayHandle gradient_Y, cons
   hipStream_t s = stream_of(stream_handle);
   const bool al = aligned16(input_X->data) && aligned16(gradient_Y->data) && aligned16(gradient_X->data);
   Plan rd, dxp;
-  TS_REQUIRE(make_plan(input_X, al, 32 * kThreads, 4096, rd), "BatchNorm gradient: unsupported shape");
-  TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 1 << 20, dxp), "BatchNorm gradient: unsupported shape");
+  TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 16384, rd), "BatchNorm gradient: unsupported shape");
+  TS_REQUIRE(make_plan(input_X, al, 4 * kThreads, 1 << 22, dxp), "BatchNorm gradient: unsupported shape");
   double *part = static_cast<double *>(scratch_get(s, 1, static_cast<size_t>(C) * rd.S * 4 * sizeof(double)));
   TS_REQUIRE(part, "BatchNorm gradient: no scratch memory");
   ProfileScope ps(p, s, 2 * numel(input_X) + C, numel(gradient_X) + 2 * C, C * rd.S * 8);

@@ -1,17 +1,19 @@
 // HBM-streaming elementwise kernels: graph-closure ops, Relu and the optimizer updates.
 //
-// One template serves all of them.  Every thread moves UNROLL x 16 bytes per array with
-// all loads issued before any arithmetic (so a wave keeps UNROLL dwordx4 loads per array
-// in flight), consecutive lanes touch consecutive 16-byte words, and a block covers one
-// contiguous 16 KiB span per array.  Arrays that are not 16-byte aligned (micro-tensor
-// views can start anywhere on a 4-byte boundary) take the scalar variant.
+// One template serves all of them.  Every thread moves one 16-byte word per array,
+// consecutive lanes touch consecutive words, and loads and stores are non-temporal: these
+// tensors are far larger than the caches and are touched once per kernel, and on MI355X a
+// read+write stream measured 6.5 TB/s this way against 5.7 TB/s with 4 words per thread and
+// cached accesses.  Arrays that are not 16-byte aligned (micro-tensor views can start
+// anywhere on a 4-byte boundary) take the scalar variant.
 #include "common.h"
 
 namespace tsplit {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kUnroll = 4;
+constexpr int kUnroll = 1;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 template <int N>
 struct Ptrs {
@@ -25,14 +27,14 @@ __global__ __launch_bounds__(kThreads) void ew_vec_kernel(Op op, Ptrs<Op::N> a, 
   constexpr int N = Op::N;
   const int64_t n4 = n >> 2;
   const int64_t first = (static_cast<int64_t>(blockIdx.x) * kUnroll) * kThreads + threadIdx.x;
-  float4 v[kUnroll][N];
+  f32x4 v[kUnroll][N];
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) {
     const int64_t i = first + static_cast<int64_t>(u) * kThreads;
     if (i < n4) {
 #pragma unroll
       for (int k = 0; k < N; ++k)
-        if (Op::LOAD & (1 << k)) v[u][k] = reinterpret_cast<const float4 *>(a.p[k])[i];
+        if (Op::LOAD & (1 << k)) v[u][k] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(a.p[k]) + i);
     }
   }
 #pragma unroll
@@ -51,8 +53,10 @@ __global__ __launch_bounds__(kThreads) void ew_vec_kernel(Op op, Ptrs<Op::N> a, 
       for (int j = 0; j < 4; ++j) op.apply(e[j]);
 #pragma unroll
       for (int k = 0; k < N; ++k)
-        if (Op::STORE & (1 << k))
-          reinterpret_cast<float4 *>(a.p[k])[i] = make_float4(e[0][k], e[1][k], e[2][k], e[3][k]);
+        if (Op::STORE & (1 << k)) {
+          const f32x4 r = {e[0][k], e[1][k], e[2][k], e[3][k]};
+          __builtin_nontemporal_store(r, reinterpret_cast<f32x4 *>(a.p[k]) + i);
+        }
     }
   }
   // the last (n % 4) elements

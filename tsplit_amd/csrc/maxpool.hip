@@ -15,6 +15,8 @@ namespace tsplit {
 namespace {
 
 constexpr int kThreads = 256;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 struct PoolGeo {
   int H, W, pH, pW, kH, kW, pad, stride;
@@ -75,15 +77,15 @@ __global__ __launch_bounds__(kThreads) void pool_bwd_kernel(const float *__restr
 
 // ---- 2x2 stride 2 pad 0, W % 4 == 0, H % 2 == 0, 16-byte aligned x/dx and 8-byte aligned y/dy ----
 // thread -> (plane, oh, q): input words (2oh, q) and (2oh+1, q), outputs (oh, 2q) and (oh, 2q+1)
-__global__ __launch_bounds__(kThreads) void pool2x2_fwd_kernel(const float4 *__restrict__ x, float2 *__restrict__ y,
+__global__ __launch_bounds__(kThreads) void pool2x2_fwd_kernel(const f32x4 *__restrict__ x, f32x2 *__restrict__ y,
                                                                int W4, int pH, int64_t total) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (idx >= total) return;
   const int q = static_cast<int>(idx % W4);
   const int64_t row = idx / W4;                 // plane * pH + oh
   const int64_t in = (row * 2) * W4 + q;        // (plane*H + 2*oh) * W4 + q, H = 2*pH
-  const float4 a = x[in], b = x[in + W4];
-  float2 o;
+  const f32x4 a = __builtin_nontemporal_load(x + in), b = __builtin_nontemporal_load(x + in + W4);
+  f32x2 o;
   // scan order: (0,0) (0,1) (1,0) (1,1); strict > keeps the first maximum
   float m = a.x;
   m = a.y > m ? a.y : m;
@@ -95,7 +97,7 @@ __global__ __launch_bounds__(kThreads) void pool2x2_fwd_kernel(const float4 *__r
   m = b.z > m ? b.z : m;
   m = b.w > m ? b.w : m;
   o.y = m;
-  y[idx] = o;
+  __builtin_nontemporal_store(o, y + idx);
 }
 
 __device__ __forceinline__ void route2x2(float v00, float v01, float v10, float v11, float g, float &o00, float &o01,
@@ -111,21 +113,22 @@ __device__ __forceinline__ void route2x2(float v00, float v01, float v10, float 
   o11 = k == 3 ? g : 0.f;
 }
 
-__global__ __launch_bounds__(kThreads) void pool2x2_bwd_kernel(const float4 *__restrict__ x,
-                                                               const float2 *__restrict__ dy, float4 *__restrict__ dx,
+__global__ __launch_bounds__(kThreads) void pool2x2_bwd_kernel(const f32x4 *__restrict__ x,
+                                                               const f32x2 *__restrict__ dy, f32x4 *__restrict__ dx,
                                                                int W4, int64_t total) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (idx >= total) return;
   const int q = static_cast<int>(idx % W4);
   const int64_t row = idx / W4;
   const int64_t in = (row * 2) * W4 + q;
-  const float4 a = x[in], b = x[in + W4];
-  const float2 g = dy[idx];
-  float4 oa, ob;
-  route2x2(a.x, a.y, b.x, b.y, g.x, oa.x, oa.y, ob.x, ob.y);
-  route2x2(a.z, a.w, b.z, b.w, g.y, oa.z, oa.w, ob.z, ob.w);
-  dx[in] = oa;
-  dx[in + W4] = ob;
+  const f32x4 a = __builtin_nontemporal_load(x + in), b = __builtin_nontemporal_load(x + in + W4);
+  const f32x2 g = __builtin_nontemporal_load(dy + idx);
+  float t[8];
+  route2x2(a.x, a.y, b.x, b.y, g.x, t[0], t[1], t[4], t[5]);
+  route2x2(a.z, a.w, b.z, b.w, g.y, t[2], t[3], t[6], t[7]);
+  const f32x4 oa = {t[0], t[1], t[2], t[3]}, ob = {t[4], t[5], t[6], t[7]};
+  __builtin_nontemporal_store(oa, dx + in);
+  __builtin_nontemporal_store(ob, dx + in + W4);
 }
 
 inline bool aligned8(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 7) == 0; }
@@ -167,7 +170,7 @@ int pool_forward(const char *who, const DLArray *x, DLArray *y, int64_t kH, int6
     if (fast2x2(g, x->data, y->data, nullptr)) {
       const int64_t total = planes * g.pH * (g.W / 4);
       hipLaunchKernelGGL(pool2x2_fwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
-                         dim3(kThreads), 0, s, static_cast<const float4 *>(x->data), static_cast<float2 *>(y->data),
+                         dim3(kThreads), 0, s, static_cast<const f32x4 *>(x->data), static_cast<f32x2 *>(y->data),
                          g.W / 4, g.pH, total);
     } else {
       const int64_t total = numel(y);
@@ -192,8 +195,8 @@ int pool_backward(const char *who, const DLArray *x, const DLArray *dy, DLArray 
     if (fast2x2(g, x->data, dy->data, dx->data)) {
       const int64_t total = planes * g.pH * (g.W / 4);
       hipLaunchKernelGGL(pool2x2_bwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
-                         dim3(kThreads), 0, s, static_cast<const float4 *>(x->data),
-                         static_cast<const float2 *>(dy->data), static_cast<float4 *>(dx->data), g.W / 4, total);
+                         dim3(kThreads), 0, s, static_cast<const f32x4 *>(x->data),
+                         static_cast<const f32x2 *>(dy->data), static_cast<f32x4 *>(dx->data), g.W / 4, total);
     } else {
       const int64_t total = numel(dx);
       hipLaunchKernelGGL(pool_bwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
