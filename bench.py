@@ -29,6 +29,14 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS_FP32_MFMA = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch (read + write, mean over the launches of one step) of the kernels that can
+# be the step's largest, from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
+# profiles/vgg16_b64_train_step_hbm_traffic.txt (counter units calibrated on the Relu kernel).
+TRAFFIC_BYTES_PER_LAUNCH = {
+    "conv_fwd_128x128": (165.5 + 108.6) * 1e6,
+    "conv_bwd_data_128x128": (207.2 + 98.3) * 1e6,
+    "conv_bwd_filter_128x128": (505.0 + 64.3) * 1e6,
+}
 
 
 class EventTimer(object):
@@ -94,7 +102,7 @@ def vgg_workload(batch, seed=123):
     return spec, params, x, labels, split
 
 
-def cpu_baseline(sample_batch=1, seed=123):
+def cpu_baseline(sample_batch=8, seed=123):
     """The numpy oracle (float64, as the reference's numpy path computes) on `sample_batch`
     images of the same seeded workload: one forward+backward+momentum step."""
     from oracle import nets, ops
@@ -174,7 +182,8 @@ def main():
                            "achieved": dd["rate"], "peak": PEAK_TFLOPS_FP32_MFMA if dd["unit"] == "flop" else PEAK_HBM_GBS,
                            "unit": "TFLOP/s" if dd["unit"] == "flop" else "GB/s",
                            "frac": dd["rate"] / (PEAK_TFLOPS_FP32_MFMA if dd["unit"] == "flop" else PEAK_HBM_GBS),
-                           "traffic": None, "per_launch": dd["work_per_call"], "ms_avg": dd["ms_avg"]}
+                           "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom) if split and a.batch == 64 else None,
+                           "per_launch": dd["work_per_call"], "ms_avg": dd["ms_avg"]}
         conv = [d for tag, d in k.items() if tag.startswith("conv_")]
         conv_flop, conv_ms = sum(d["work"] for d in conv), sum(d["ms_total"] for d in conv)
         out["conv_mfma_util_pct"] = 100.0 * conv_flop / (conv_ms * 1e-3) / 1e12 / PEAK_TFLOPS_FP32_MFMA

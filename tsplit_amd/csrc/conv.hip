@@ -1198,18 +1198,6 @@ int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArra
 
 using namespace tsplit;
 
-#ifdef EXP_TIMING
-extern "C" int ts_debug_read(unsigned long long *out, int reset) {
-  (void)hipDeviceSynchronize();
-  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(mg::g_dbg), 16 * sizeof(unsigned long long)) != hipSuccess) return -1;
-  if (reset) {
-    unsigned long long z[16] = {0};
-    (void)hipMemcpyToSymbol(HIP_SYMBOL(mg::g_dbg), z, sizeof(z));
-  }
-  return 0;
-}
-#endif
-
 extern "C" {
 
 int CuDNN_DLGpuConv2d(const DLArrayHandle input_x, const DLArrayHandle input_f, DLArrayHandle output,

@@ -170,13 +170,6 @@ struct RowMajorCols {   // out[m * row_stride + n]
   __device__ __forceinline__ int64_t operator()(int n) const { return n; }
 };
 
-#ifdef EXP_TIMING
-__device__ unsigned long long g_dbg[16];
-#define TS_CLK() __builtin_readcyclecounter()
-#define TS_T(i) { __builtin_amdgcn_sched_barrier(0); unsigned long long now_ = TS_CLK(); __builtin_amdgcn_sched_barrier(0); tacc[i] += now_ - tlast; tlast = now_; }
-#else
-#define TS_T(i)
-#endif
 // ------------------------------------------------------------------ the kernel
 // 1-D grid of grid_blocks(tm, tn, S) blocks; split z writes to out + z * z_stride.
 //
@@ -191,13 +184,8 @@ struct TileGrid {
 };
 inline unsigned grid_blocks(int tm, int tn, int S) { return static_cast<unsigned>((tm * tn * S + 7) / 8 * 8); }
 
-#ifdef EXP_WAVES4
-#define TS_OCC __attribute__((amdgpu_waves_per_eu(4, 4)))
-#else
-#define TS_OCC
-#endif
 template <int BM, int BN, int WM, int WN, class ALoader, class BLoader, class ColMap>
-__global__ __launch_bounds__(kThreads) TS_OCC void mfma_gemm_kernel(typename ALoader::Params ap, typename BLoader::Params bp,
+__global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::Params ap, typename BLoader::Params bp,
                                                              float *__restrict__ out, int64_t z_stride,
                                                              int64_t row_stride, ColMap colmap, int M, int N, int K,
                                                              int kchunk, TileGrid tg) {
@@ -240,21 +228,13 @@ __global__ __launch_bounds__(kThreads) TS_OCC void mfma_gemm_kernel(typename ALo
   }
   __syncthreads();
 
-#ifdef EXP_TIMING
-  unsigned long long tacc[5] = {0, 0, 0, 0, 0};
-  unsigned long long tlast = TS_CLK();
-#endif
   int stage = 0;
   for (int k0 = kbegin; k0 < kend; k0 += BK) {
     const bool more = k0 + BK < kend;
-#ifndef EXP_NOLOAD
     if (more) {
       la.load(k0 + BK, kend);
-      TS_T(4)
       lb.load(k0 + BK, kend);
     }
-#endif
-    TS_T(0)
     const float *sa = lds_a[stage], *sb = lds_b[stage];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -272,26 +252,13 @@ __global__ __launch_bounds__(kThreads) TS_OCC void mfma_gemm_kernel(typename ALo
           for (int ni = 0; ni < 2; ++ni)
             acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
     }
-    TS_T(1)
-#ifndef EXP_NOSTORE
     if (more) {
       la.store(lds_a[stage ^ 1], tid);
       lb.store(lds_b[stage ^ 1], tid);
     }
-#endif
-    TS_T(2)
-#ifndef EXP_NOBARRIER
     __syncthreads();
-#endif
-    TS_T(3)
     stage ^= 1;
   }
-#ifdef EXP_TIMING
-  if (lane == 0 && (logical % 97) == 5) {
-    for (int i = 0; i < 5; ++i) atomicAdd(&g_dbg[i + 5], tacc[i]);
-    atomicAdd(&g_dbg[4], 1ull);
-  }
-#endif
 
   // epilogue: accumulator register e of a 32x32 block holds row 8*(e/4) + 4*(lane/32) + e%4,
   // column lane%32
