@@ -281,8 +281,24 @@ constexpr int kBufFlags = 0x00020000;           // raw buffer, 32-bit untyped da
 constexpr unsigned kOobOffset = 0x80000000u;    // beyond any tensor this path accepts (< 2 GiB)
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
+// Work distribution ("stream-K"): the unit of work is one 16-wide k-step of one tile, numbered
+// tile-major.  Every block takes a contiguous range of `iters_per_block` units.  With
+// iters_per_block = k-steps per tile a block is exactly one tile (used when there are fewer
+// tiles than resident block slots).  Otherwise the grid is one full wave of resident blocks and
+// ranges cut through tiles, so that 3.06 tiles per slot cost 3.06 tile-times, not 4: a tile
+// computed by one block is stored, a tile cut in two is accumulated with float atomics into an
+// output that a small kernel zeroed before.  A range is at least one tile long, so a tile has
+// at most two contributors and 0 + a + b does not depend on their order: results stay
+// run-to-run deterministic (they do depend on where the cuts fall, i.e. on the problem shape).
+struct StreamK {
+  int ksteps;            // k-steps per tile
+  int total;             // tiles * ksteps
+  int iters_per_block;
+  int tm;                // M tiles (tile index = tile_n * tm + tile_m)
+};
+
 template <int BM, int BN, int WM, int WN, bool BWD_DATA>
-__global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, float *__restrict__ out, TileGrid tg) {
+__global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, float *__restrict__ out, StreamK sk) {
   static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
   using ALds = MnMajorLds<BM>;
   using BLds = MnMajorLds<BN>;
@@ -292,11 +308,12 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
   __shared__ __attribute__((aligned(16))) float lds_b[2][BLds::kFloats];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  if (logical >= tg.total) return;
-  const int tile_n = logical / tg.tm, tile_m = logical - tile_n * tg.tm;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
+  // consecutive workgroup ids go to different XCDs: transpose so that an XCD owns a contiguous
+  // eighth of the work (neighbouring tiles share gathered activations in its L2)
+  const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  int it = logical * sk.iters_per_block;
+  const int it_end = min(sk.total, it + sk.iters_per_block);
 
   // uniform bias so that every per-thread offset is non-negative and every scalar offset too
   const int bias = BWD_DATA ? (P.taps / P.kW - 1) * P.src_w + (P.kW - 1) : P.ph * P.src_w + P.pw;
@@ -304,134 +321,169 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.wf), 0, static_cast<int>(P.wf_bytes), kBufFlags);
   const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<float *>(P.src) - bias, 0, static_cast<int>(P.src_bytes + 4u * bias), kBufFlags);
-
-  // ---- filter operand: thread -> (row tid/4 + 64 s, 16-byte word tid%4); rows clamped
-  unsigned a_voff[PA];
-#pragma unroll
-  for (int s = 0; s < PA; ++s) {
-    const int row = min(m0 + (tid >> 2) + 64 * s, P.M - 1);
-    a_voff[s] = (static_cast<unsigned>(row) * P.K + 4u * (tid & 3)) * 4u;
-  }
-  // ---- gathered operand: thread -> (column tid % BN, KPT consecutive k' starting at klocal0)
   const int klocal0 = (tid / BN) * KPT;
-  unsigned b_voff, vmask = 0;
-  {
-    const int n = n0 + tid % BN;
-    const bool col_ok = n < P.N;
-    const uint32_t nn = col_ok ? n : 0;
-    const uint32_t img = P.plane.div(nn);
-    const uint32_t p = nn - img * P.plane.d;
-    const uint32_t row = P.width.div(p);
-    const uint32_t col = p - row * P.width.d;
-    const int r0 = BWD_DATA ? static_cast<int>(row) + P.ph : static_cast<int>(row) * P.s - P.ph;
-    const int c0 = BWD_DATA ? static_cast<int>(col) + P.pw : static_cast<int>(col) * P.s - P.pw;
-    if (col_ok) {
-      for (int t = 0; t < P.taps; ++t) {
-        const int kh = t / P.kW, kw = t - kh * P.kW;
-        const int rr = BWD_DATA ? r0 - kh : r0 + kh, cc = BWD_DATA ? c0 - kw : c0 + kw;
-        if (static_cast<unsigned>(rr) < static_cast<unsigned>(P.src_h) &&
-            static_cast<unsigned>(cc) < static_cast<unsigned>(P.src_w))
-          vmask |= 1u << t;
+
+  while (it < it_end) {
+    const int tile = it / sk.ksteps;
+    const int ks0 = it - tile * sk.ksteps;
+    const int ks1 = min(sk.ksteps, ks0 + (it_end - it));
+    it += ks1 - ks0;
+    const int tile_n = tile / sk.tm, tile_m = tile - tile_n * sk.tm;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    // ---- filter operand: thread -> (row tid/4 + 64 s, 16-byte word tid%4); rows clamped
+    unsigned a_voff[PA];
+#pragma unroll
+    for (int s = 0; s < PA; ++s) {
+      const int row = min(m0 + (tid >> 2) + 64 * s, P.M - 1);
+      a_voff[s] = (static_cast<unsigned>(row) * P.K + 4u * (tid & 3)) * 4u;
+    }
+    // ---- gathered operand: thread -> (column tid % BN, KPT consecutive k' starting at klocal0)
+    unsigned b_voff, vmask = 0;
+    {
+      const int n = n0 + tid % BN;
+      const bool col_ok = n < P.N;
+      const uint32_t nn = col_ok ? n : 0;
+      const uint32_t img = P.plane.div(nn);
+      const uint32_t p = nn - img * P.plane.d;
+      const uint32_t row = P.width.div(p);
+      const uint32_t col = p - row * P.width.d;
+      const int r0 = BWD_DATA ? static_cast<int>(row) + P.ph : static_cast<int>(row) * P.s - P.ph;
+      const int c0 = BWD_DATA ? static_cast<int>(col) + P.pw : static_cast<int>(col) * P.s - P.pw;
+      if (col_ok) {
+        for (int t = 0; t < P.taps; ++t) {
+          const int kh = t / P.kW, kw = t - kh * P.kW;
+          const int rr = BWD_DATA ? r0 - kh : r0 + kh, cc = BWD_DATA ? c0 - kw : c0 + kw;
+          if (static_cast<unsigned>(rr) < static_cast<unsigned>(P.src_h) &&
+              static_cast<unsigned>(cc) < static_cast<unsigned>(P.src_w))
+            vmask |= 1u << t;
+        }
       }
+      // forward : src offset = thread part + (kh*W + kw)       with the bias ph*W + pw folded in
+      // bwd-data: src offset = thread part - (kh*W + kw)       with the bias (kH-1)*W + kW-1 folded in
+      const int thread_part = BWD_DATA ? r0 * P.src_w + c0 : (r0 + P.ph) * P.src_w + (c0 + P.pw);
+      b_voff =
+          static_cast<unsigned>(static_cast<int>(img) * P.img_stride + klocal0 * P.chan_stride + thread_part) * 4u;
     }
-    // forward : src offset = thread part + (kh*W + kw)       with the bias ph*W + pw folded in
-    // bwd-data: src offset = thread part - (kh*W + kw)       with the bias (kH-1)*W + kW-1 folded in
-    const int thread_part = BWD_DATA ? r0 * P.src_w + c0 : (r0 + P.ph) * P.src_w + (c0 + P.pw);
-    b_voff = static_cast<unsigned>(static_cast<int>(img) * P.img_stride + klocal0 * P.chan_stride + thread_part) * 4u;
-  }
 
-  acc16 acc[2][2];
+    acc16 acc[2][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  u32x4 ra_regs[PA];
-  unsigned rb_regs[KPT];
-  int tap = 0, ch0 = 0;   // position of the NEXT step to load
+    u32x4 ra_regs[PA];
+    unsigned rb_regs[KPT];
+    // position of the NEXT step to load: step ks covers channels [16*(ks/taps), +16) of tap ks%taps
+    int tap = ks0 % P.taps, ch0 = (ks0 / P.taps) * BK;
 
-  auto load_step = [&](int step) {
-    // filter words: scalar offset = k position of the step
-    const int soff_a = step * (BK * 4);
+    auto load_step = [&](int step) {
+      // filter words: scalar offset = k position of the step
+      const int soff_a = step * (BK * 4);
 #pragma unroll
-    for (int s = 0; s < PA; ++s) ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[s], soff_a, 0);
-    // gathered values: scalar offset = channel block + tap displacement
-    const int kh = tap / P.kW, kw = tap - kh * P.kW;
-    const int disp = BWD_DATA ? bias - (kh * P.src_w + kw) : kh * P.src_w + kw;
-    const int soff_b = (ch0 * P.chan_stride + disp) * 4;
-    const unsigned voff = (vmask >> tap) & 1u ? b_voff : kOobOffset;
+      for (int s = 0; s < PA; ++s) ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[s], soff_a, 0);
+      // gathered values: scalar offset = channel block + tap displacement
+      const int kh = tap / P.kW, kw = tap - kh * P.kW;
+      const int disp = BWD_DATA ? bias - (kh * P.src_w + kw) : kh * P.src_w + kw;
+      const int soff_b = (ch0 * P.chan_stride + disp) * 4;
+      const unsigned voff = (vmask >> tap) & 1u ? b_voff : kOobOffset;
 #pragma unroll
-    for (int i = 0; i < KPT; ++i)
-      rb_regs[i] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, soff_b + i * P.chan_stride * 4, 0);
-    if (++tap == P.taps) {
-      tap = 0;
-      ch0 += BK;
-    }
-  };
-  auto store_step = [&](float *sa, float *sb) {
-#pragma unroll
-    for (int s = 0; s < PA; ++s)
-      *reinterpret_cast<u32x4 *>(sa + ((tid >> 2) + 64 * s) * ALds::kStride + 4 * (tid & 3)) = ra_regs[s];
-#pragma unroll
-    for (int q = 0; q < KPT / 4; ++q) {
-      u32x4 v = {rb_regs[4 * q], rb_regs[4 * q + 1], rb_regs[4 * q + 2], rb_regs[4 * q + 3]};
-      *reinterpret_cast<u32x4 *>(sb + (tid % BN) * BLds::kStride + klocal0 + 4 * q) = v;
-    }
-  };
-  auto mma_step = [&](const float *sa, const float *sb) {
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      float fa[2][4], fb[2][4];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        ALds::frag(sa, wm0 + 32 * i, j, lane, fa[i]);
-        BLds::frag(sb, wn0 + 32 * i, j, lane, fb[i]);
+      for (int i = 0; i < KPT; ++i)
+        rb_regs[i] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, soff_b + i * P.chan_stride * 4, 0);
+      if (++tap == P.taps) {
+        tap = 0;
+        ch0 += BK;
       }
+    };
+    auto store_step = [&](float *sa, float *sb) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
+      for (int s = 0; s < PA; ++s)
+        *reinterpret_cast<u32x4 *>(sa + ((tid >> 2) + 64 * s) * ALds::kStride + 4 * (tid & 3)) = ra_regs[s];
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi)
+      for (int q = 0; q < KPT / 4; ++q) {
+        u32x4 v = {rb_regs[4 * q], rb_regs[4 * q + 1], rb_regs[4 * q + 2], rb_regs[4 * q + 3]};
+        *reinterpret_cast<u32x4 *>(sb + (tid % BN) * BLds::kStride + klocal0 + 4 * q) = v;
+      }
+    };
+    auto mma_step = [&](const float *sa, const float *sb) {
 #pragma unroll
-          for (int ni = 0; ni < 2; ++ni)
-            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
-    }
-  };
+      for (int j = 0; j < 2; ++j) {
+        float fa[2][4], fb[2][4];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          ALds::frag(sa, wm0 + 32 * i, j, lane, fa[i]);
+          BLds::frag(sb, wn0 + 32 * i, j, lane, fb[i]);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+          for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+              acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
+      }
+    };
 
-  const int steps = P.K / BK;
-  load_step(0);
-  store_step(lds_a[0], lds_b[0]);
-  __syncthreads();
-  int stage = 0;
-  for (int st = 0; st < steps; ++st) {
-    const bool more = st + 1 < steps;
-    if (more) load_step(st + 1);
-    mma_step(lds_a[stage], lds_b[stage]);
-    if (more) store_step(lds_a[stage ^ 1], lds_b[stage ^ 1]);
+    load_step(ks0);
+    store_step(lds_a[0], lds_b[0]);
     __syncthreads();
-    stage ^= 1;
-  }
+    int stage = 0;
+    for (int st = ks0; st < ks1; ++st) {
+      const bool more = st + 1 < ks1;
+      if (more) load_step(st + 1);
+      mma_step(lds_a[stage], lds_b[stage]);
+      if (more) store_step(lds_a[stage ^ 1], lds_b[stage ^ 1]);
+      __syncthreads();   // also fences the LDS stages against the next tile of this block
+      stage ^= 1;
+    }
 
-  // epilogue (see mfma_gemm_kernel): out[img][m][p], column n = img*plane + p
+    // epilogue: accumulator register e of a 32x32 block holds row 8*(e/4) + 4*(lane/32) + e%4, column
+    // lane%32; out[img][m][p] with column n = img*plane + p
+    const bool whole = ks0 == 0 && ks1 == sk.ksteps;
 #pragma unroll
-  for (int ni = 0; ni < 2; ++ni) {
-    const int n = n0 + wn0 + 32 * ni + (lane & 31);
-    if (n >= P.N) continue;
-    const uint32_t img = P.plane.div(n);
-    const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
+    for (int ni = 0; ni < 2; ++ni) {
+      const int n = n0 + wn0 + 32 * ni + (lane & 31);
+      if (n >= P.N) continue;
+      const uint32_t img = P.plane.div(n);
+      const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
-      const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
+      for (int mi = 0; mi < 2; ++mi) {
+        const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = mb + 8 * (e >> 2) + (e & 3);
-        if (m < P.M) out[static_cast<int64_t>(m) * P.out_plane + coff] = acc[mi][ni][e];
+        for (int e = 0; e < 16; ++e) {
+          const int m = mb + 8 * (e >> 2) + (e & 3);
+          if (m < P.M) {
+            float *dst = out + static_cast<int64_t>(m) * P.out_plane + coff;
+            if (whole)
+              *dst = acc[mi][ni][e];
+            else
+              unsafeAtomicAdd(dst, acc[mi][ni][e]);
+          }
+        }
       }
     }
   }
 }
 
+// zeroes the output tiles that the stream-K ranges cut in two (block g looks at its range start)
+template <int BM, int BN>
+__global__ __launch_bounds__(kThreads) void conv_tap_zero_cut_tiles_kernel(TapConvParams P, float *__restrict__ out,
+                                                                           StreamK sk) {
+  const int start = (blockIdx.x + 1) * sk.iters_per_block;     // first unit of block g + 1
+  if (start >= sk.total || start % sk.ksteps == 0) return;       // falls on a tile boundary: nothing is cut
+  const int tile = start / sk.ksteps;
+  const int tile_n = tile / sk.tm, tile_m = tile - tile_n * sk.tm;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  for (int idx = threadIdx.x; idx < BM * BN; idx += kThreads) {
+    const int m = m0 + idx / BN, n = n0 + idx % BN;
+    if (m < P.M && n < P.N) {
+      const uint32_t img = P.plane.div(n);
+      out[static_cast<int64_t>(img) * P.out_img_stride + static_cast<int64_t>(m) * P.out_plane + (n - img * P.plane.d)] = 0.f;
+    }
+  }
+}
 
 // ------------------------------------------------------------------ the tap-major filter-gradient kernel
 // Backward-filter for "same" stride-1 convolutions (oH = H, oW = W) with C % 16 == 0 and
@@ -1037,8 +1089,23 @@ void launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, 
   P.kW = g.kW;
   P.taps = taps;
   const int tn = (P.N + BN - 1) / BN, tm = (P.M + BM - 1) / BM;
-  hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>), dim3(grid_blocks(tm, tn, 1)), dim3(kThreads), 0, st,
-                     P, out, TileGrid{tm, tn, tm * tn});
+  const int tiles = tm * tn;
+  StreamK sk;
+  sk.ksteps = P.K / BK;
+  sk.total = tiles * sk.ksteps;
+  sk.tm = tm;
+  static const int occ = blocks_per_cu(conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>);
+  const int slots = 256 * occ;
+  unsigned grid;
+  if (tiles <= slots) {          // one tile per block
+    sk.iters_per_block = sk.ksteps;
+    grid = (tiles + 7) / 8 * 8;
+  } else {                       // one full wave of blocks, equal shares of k-steps
+    grid = slots;
+    sk.iters_per_block = (sk.total + slots - 1) / slots;
+    hipLaunchKernelGGL((conv_tap_zero_cut_tiles_kernel<BM, BN>), dim3(grid), dim3(kThreads), 0, st, P, out, sk);
+  }
+  hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>), dim3(grid), dim3(kThreads), 0, st, P, out, sk);
 }
 
 // the buffer-load path addresses with 32-bit byte offsets and a 32-tap bit mask
