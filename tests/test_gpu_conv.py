@@ -27,6 +27,10 @@ CASES = [
     (2, 16, 15, 15, 24, 3, 3, 1, 1, 2),    # stride 2, odd output 8x8
     (2, 8, 7, 7, 40, 1, 1, 0, 0, 1),       # oH*oW = 49: not a multiple of 4
     (2, 6, 12, 12, 130, 5, 5, 2, 2, 1),
+    # more tiles than resident block slots: forward / backward-data take the stream-K path, where
+    # block ranges cut tiles in two and the halves meet through float atomics
+    (25, 16, 64, 64, 128, 3, 3, 1, 1, 1),  # 800 tiles of 128x128 (forward)
+    (13, 16, 128, 128, 16, 3, 3, 1, 1, 1), # 832 tiles of 64x256 (forward and backward-data)
 ]
 
 

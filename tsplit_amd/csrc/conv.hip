@@ -20,6 +20,7 @@
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <type_traits>
 #include <vector>
 
 #include "common.h"
@@ -618,15 +619,24 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
     store_step(lds_a[0], lds_b[0]);
   }
   __syncthreads();
-  int stage = 0;
-  for (int st = 0; st < steps; ++st) {
-    const bool more = st + 1 < steps;
-    if (more) load_step();
-    mma_step(lds_a[stage], lds_b[stage]);
-    if (more) store_step(lds_a[stage ^ 1], lds_b[stage ^ 1]);
-    __syncthreads();
-    stage ^= 1;
-  }
+  // A wave whose 64x64 sub-tile lies outside the matrix (ragged last N tile: 576 columns = 2.25
+  // tiles of 256) only helps with the staging and leaves the matrix pipe to other blocks.  Two
+  // copies of the loop, chosen once: a test inside the loop costs the full tiles 20 %.
+  auto k_loop = [&](auto with_mma) {
+    int stage = 0;
+    for (int st = 0; st < steps; ++st) {
+      const bool more = st + 1 < steps;
+      if (more) load_step();
+      if (decltype(with_mma)::value) mma_step(lds_a[stage], lds_b[stage]);
+      if (more) store_step(lds_a[stage ^ 1], lds_b[stage ^ 1]);
+      __syncthreads();
+      stage ^= 1;
+    }
+  };
+  if (m0 + wm0 < P.M && n0 + wn0 < P.N)
+    k_loop(std::true_type{});
+  else
+    k_loop(std::false_type{});
 
   float *o = part + static_cast<int64_t>(zsplit) * P.M * P.N;
 #pragma unroll

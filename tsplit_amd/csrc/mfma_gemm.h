@@ -23,6 +23,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 namespace tsplit {
 namespace mg {
@@ -228,37 +229,48 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::P
   }
   __syncthreads();
 
-  int stage = 0;
-  for (int k0 = kbegin; k0 < kend; k0 += BK) {
-    const bool more = k0 + BK < kend;
-    if (more) {
-      la.load(k0 + BK, kend);
-      lb.load(k0 + BK, kend);
-    }
-    const float *sa = lds_a[stage], *sb = lds_b[stage];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      float fa[2][4], fb[2][4];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        ALds::frag(sa, wm0 + 32 * i, j, lane, fa[i]);
-        BLds::frag(sb, wn0 + 32 * i, j, lane, fb[i]);
+  // A wave whose 64x64 sub-tile lies outside the matrix (ragged last tile) only helps with the
+  // staging and leaves the matrix pipe to other blocks.  Two copies of the loop, chosen once: a
+  // test inside the loop costs full tiles 20 %.
+  auto k_loop = [&](auto with_mma) {
+    int stage = 0;
+    for (int k0 = kbegin; k0 < kend; k0 += BK) {
+      const bool more = k0 + BK < kend;
+      if (more) {
+        la.load(k0 + BK, kend);
+        lb.load(k0 + BK, kend);
       }
+      if (decltype(with_mma)::value) {
+        const float *sa = lds_a[stage], *sb = lds_b[stage];
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
+        for (int j = 0; j < 2; ++j) {
+          float fa[2][4], fb[2][4];
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi)
+          for (int i = 0; i < 2; ++i) {
+            ALds::frag(sa, wm0 + 32 * i, j, lane, fa[i]);
+            BLds::frag(sb, wn0 + 32 * i, j, lane, fb[i]);
+          }
 #pragma unroll
-          for (int ni = 0; ni < 2; ++ni)
-            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
+          for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+              for (int ni = 0; ni < 2; ++ni)
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
+        }
+      }
+      if (more) {
+        la.store(lds_a[stage ^ 1], tid);
+        lb.store(lds_b[stage ^ 1], tid);
+      }
+      __syncthreads();
+      stage ^= 1;
     }
-    if (more) {
-      la.store(lds_a[stage ^ 1], tid);
-      lb.store(lds_b[stage ^ 1], tid);
-    }
-    __syncthreads();
-    stage ^= 1;
-  }
+  };
+  if (m0 + wm0 < M && n0 + wn0 < N)
+    k_loop(std::true_type{});
+  else
+    k_loop(std::false_type{});
 
   // epilogue: accumulator register e of a 32x32 block holds row 8*(e/4) + 4*(lane/32) + e%4,
   // column lane%32
