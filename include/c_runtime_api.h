@@ -112,8 +112,8 @@ int DLArrayReuseAlloc(DLContext ctx, int MEMORY_MANAGE_RULE, const index_t *inpu
 int DLArraySliceForMicroTensor(DLArrayHandle input, DLArrayHandle *output, int total_number,
                                int index, int dimension);
 
-/* ---- graph-closure elementwise ops (ref: c_runtime_api.h:115,140-141,151-152,162-163,
- *      173-174,342; impl src/ops/ArraySet.cu:9, AddElewise.cu:9, AddConst.cu:9,
+/* ---- graph-closure elementwise ops (ref: c_runtime_api.h:113,138-139,148-149,158-159,
+ *      168-169,317; impl src/ops/ArraySet.cu:9, AddElewise.cu:9, AddConst.cu:9,
  *      MultiplyElewise.cu:9, MultiplyConst.cu:9, Reshape.cu:5) ---- */
 int DLGpuArraySet(DLArrayHandle arr, float value, DLStreamHandle stream_handle, ProfilerHandle p);
 int DLGpuMatrixElementwiseAdd(const DLArrayHandle matA, const DLArrayHandle matB,
@@ -135,13 +135,13 @@ int DLGpuRelu(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle st
 int DLGpuReluGradient(const DLArrayHandle input, const DLArrayHandle in_grad, DLArrayHandle output,
                       DLStreamHandle stream_handle, ProfilerHandle p);
 
-/* ---- MatMul (ref: c_runtime_api.h:207-209; impl src/ops/MatrixMult.cu:4-72).
+/* ---- MatMul (ref: c_runtime_api.h:208-210; impl src/ops/MatrixMult.cu:4-72).
  *      Row-major 2-D C = op(A) op(B). ---- */
 int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, const DLArrayHandle matB,
                         bool transposeB, DLArrayHandle matC, DLStreamHandle stream_handle,
                         ProfilerHandle p);
 
-/* ---- Softmax / SoftmaxCrossEntropy (ref: c_runtime_api.h:272,288-294; impl
+/* ---- Softmax / SoftmaxCrossEntropy (ref: c_runtime_api.h:270,286-292; impl
  *      src/ops/Softmax.cu:24, src/ops/SoftmaxCrossEntropy.cu:44,106).  Rows = product of
  *      all but the last dimension; loss has one element = mean over rows; the gradient
  *      is (softmax(a) - b) * c[0] / a.shape[0]. ---- */
@@ -154,7 +154,7 @@ int DLGpuSoftmaxCrossEntropy_Gradient(const DLArrayHandle input_a, const DLArray
                                       DLStreamHandle stream_handle, ProfilerHandle p);
 
 /* ---- Conv2d, cross-correlation, no bias, square stride, dilation 1.
- *      `CuDNN_` symbols (ref: c_runtime_api.h:348-352; impl src/ops/CudnnConv2d.cu:6,207,410)
+ *      `CuDNN_` symbols (ref: c_runtime_api.h:323-327; impl src/ops/CudnnConv2d.cu:6,207,410)
  *      take (pad_h, pad_w, stride); they are the ones the graph ops call
  *      (python/athena/gpu_ops/Conv2d.py:116-118).  Output/gradient shapes are taken from
  *      the pre-allocated output array. ---- */
@@ -170,7 +170,7 @@ int CuDNN_DLGpuConv2d_Gradient_of_Data(const DLArrayHandle input_f, const DLArra
                                        const int padding2, const int stride,
                                        DLStreamHandle stream_handle, ProfilerHandle p);
 /*      Plain symbols: the reference header lists (padding1, padding2)
- *      (c_runtime_api.h:296-304) but its implementation and Python call sites pass ONE
+ *      (c_runtime_api.h:294-302) but its implementation and Python call sites pass ONE
  *      padding int (src/ops/Conv2d.cu:52,172,241; gpu_links/Conv2dLink.py:13-14,31-32,40-41):
  *      the implementation's signature is exported.  The caller-provided im2col workspaces
  *      are accepted and left untouched (the implicit-GEMM kernels need none). */
@@ -187,7 +187,7 @@ int DLGpuConv2d_Gradient_of_Filter(const DLArrayHandle input_x, const DLArrayHan
                                    const int stride, DLStreamHandle stream_handle,
                                    ProfilerHandle p);
 
-/* ---- BatchNorm, training mode, spatial, biased batch variance (ref: c_runtime_api.h:371-376;
+/* ---- BatchNorm, training mode, spatial, biased batch variance (ref: c_runtime_api.h:344-349;
  *      impl src/ops/CudnnBn.cu:12,212).  scale/bias/dscale/dbias/save_* hold C elements.
  *      save_mean_arr / save_var_arr may be NULL; when given, forward writes (batch mean,
  *      1/sqrt(var+eps)) and the gradient reads them instead of recomputing (the cuDNN
@@ -207,7 +207,7 @@ int CuDNN_DLGpuBatch_Normalization_gradient(const DLArrayHandle gradient_Y,
                                             DLArrayHandle save_var_arr,
                                             DLStreamHandle stream_handle, ProfilerHandle p);
 
-/* ---- MaxPool (ref: c_runtime_api.h:334-338,366-368; impl src/ops/MaxPool.cu:45,138,
+/* ---- MaxPool (ref: c_runtime_api.h:311-315,340-342; impl src/ops/MaxPool.cu:45,138,
  *      src/ops/CudnnMaxPool.cu:3,103).  Windows are clipped to the image; the maximum is the
  *      first strict maximum in row-major scan; the gradient accumulates in window order and
  *      zero-fills the rest of gradient_X itself.  Note the differing argument orders and
@@ -228,7 +228,7 @@ int CuDNN_DLGpuMax_Pooling2d_gradient(const DLArrayHandle output_Y, const DLArra
                                       const size_t padding, const size_t stride,
                                       DLStreamHandle stream_handle, ProfilerHandle p);
 
-/* ---- Concat / Slice copies (ref: c_runtime_api.h:382-384,394-396; impl
+/* ---- Concat / Slice copies (ref: c_runtime_api.h:355-357,366-368; impl
  *      src/ops/Concat.cu:22,127, src/ops/Slice.cu:30,118).  begin_pos is a host array of
  *      ndim int64. ---- */
 int DLGpuConcat(const DLArrayHandle input_x, const DLArrayHandle input_y, DLArrayHandle output,
@@ -240,7 +240,7 @@ int DLGpuSlice(const DLArrayHandle in_arr, DLArrayHandle out_arr, int64_t *begin
 int DLGpuSliceGradient(const DLArrayHandle in_arr, DLArrayHandle out_arr, int64_t *begin_pos,
                        DLStreamHandle stream_handle, ProfilerHandle p);
 
-/* ---- Optimizer updates, in place, no ProfilerHandle (ref: c_runtime_api.h:399-410; impl
+/* ---- Optimizer updates, in place, no ProfilerHandle (ref: c_runtime_api.h:371-380; impl
  *      src/ops/Optimizers.cu:9,48,87,122).  beta1t/beta2t are the host-accumulated powers. ---- */
 int SGDOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, float lr,
                        DLStreamHandle stream_handle);
@@ -251,6 +251,113 @@ int AdaGradOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, DLArra
 int AdamOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, DLArrayHandle expavg,
                         DLArrayHandle expavgsq, float lr, float beta1, float beta2, float beta1t,
                         float beta2t, float eps, DLStreamHandle stream_handle);
+
+/* ==== Operators around the core path: needed by the ResNet / Inception-v4 / Transformer
+ *      graphs of the reference's examples. ==== */
+
+/* ---- AvgPool (ref: c_runtime_api.h:305-309,329-332; impl src/ops/AvgPool.cu,
+ *      src/ops/CudnnAvgPool.cu).  Sum over the window clipped to the image divided by
+ *      kernel_H*kernel_W whatever the clipping (python/athena/gpu_ops/AvgPool.py:27-50,
+ *      139-161).  All four symbols take size_t geometry.  The `CuDNN_` gradient also
+ *      receives output_Y and input_X, which the arithmetic does not need. ---- */
+int DLGpuAvgerage_Pooling2d(const DLArrayHandle input, const size_t kernel_H,
+                            const size_t kernel_W, DLArrayHandle output, const size_t padding,
+                            const size_t stride, DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuAvgerage_Pooling2d_gradient(const DLArrayHandle gradient_Y, const size_t kernel_H,
+                                     const size_t kernel_W, DLArrayHandle gradient_X,
+                                     const size_t padding, const size_t stride,
+                                     DLStreamHandle stream_handle, ProfilerHandle p);
+int CuDNN_DLGpuAvgerage_Pooling2d(const DLArrayHandle input, const size_t kernel_H,
+                                  const size_t kernel_W, DLArrayHandle output,
+                                  const size_t padding, const size_t stride,
+                                  DLStreamHandle stream_handle, ProfilerHandle p);
+int CuDNN_DLGpuAvgerage_Pooling2d_gradient(const DLArrayHandle output_Y,
+                                           const DLArrayHandle gradient_Y,
+                                           const DLArrayHandle input_X, const size_t kernel_H,
+                                           const size_t kernel_W, DLArrayHandle gradient_X,
+                                           const size_t padding, const size_t stride,
+                                           DLStreamHandle stream_handle, ProfilerHandle p);
+
+/* ---- Broadcast / reduce (ref: c_runtime_api.h:121,129-130,319,321,442,449; impl
+ *      src/ops/Broadcast.cu:4-9 (out[i] = in[i % in_size]: new leading axes),
+ *      src/ops/ReduceSumAxisZero.cu:27,98 (sum over axis 0; the `_` variant takes a
+ *      caller workspace, which is accepted and left untouched),
+ *      src/ops/Conv2dBroadcast.cu ([C] -> [N,C,H,W]), src/ops/Conv2dReduceSum.cu
+ *      ([N,C,H,W] -> [C]), src/ops/BroadcastShape.cu:23 (add_axes: host int array of
+ *      out.ndim - in.ndim new-axis positions, or NULL for alignment from the right),
+ *      src/ops/ReduceSum.cu:3 (axes: host int array; out holds the kept elements, with or
+ *      without the reduced axes as extent-1 axes)).  The last two have no ProfilerHandle. ---- */
+int DLGpuBroadcastTo(const DLArrayHandle input, DLArrayHandle output,
+                     DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuReduceSumAxisZero(const DLArrayHandle input, DLArrayHandle output,
+                           DLStreamHandle stream_handle, ProfilerHandle p);
+int _DLGpuReduceSumAxisZero(const DLArrayHandle input, DLArrayHandle output,
+                            DLArrayHandle arr_workspace, DLStreamHandle stream_handle,
+                            ProfilerHandle p);
+int DLGpuConv2d_broadcast_to(const DLArrayHandle input_x, DLArrayHandle output_y,
+                             DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuConv2d_reduce_sum(const DLArrayHandle input_x, DLArrayHandle output_y,
+                           DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuBroadcastShape(const DLArrayHandle in_arr, DLArrayHandle out_arr, int *add_axes,
+                        DLStreamHandle stream_handle);
+int DLGpuReduceSum(const DLArrayHandle in_arr, DLArrayHandle out_arr, int *axes, int num_ax,
+                   DLStreamHandle stream_handle);
+
+/* ---- Pad, 4-D, mode 0 (CONSTANT) only (ref: c_runtime_api.h:351,353; impl
+ *      src/ops/Pad.cu:23,76).  paddings: host array of pad_len ints, (before, after) pairs
+ *      for the LAST pad_len/2 axes.  Unpadded leading axes are copied whole, as np.pad does
+ *      (python/athena/gpu_ops/Pad.py:194-196); the reference's kernel keeps only their last
+ *      index (src/ops/Pad.cu:29-31), which is not followed.  Modes 1/2 fail. ---- */
+int DLGpuPad(const DLArrayHandle input_X, DLArrayHandle output_Y, int *paddings, int pad_len,
+             size_t mode, float constant_values, DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuPad_gradient(const DLArrayHandle output_gradient_Y, DLArrayHandle input_gradient_X,
+                      int *paddings, int pad_len, size_t mode, DLStreamHandle stream_handle,
+                      ProfilerHandle p);
+
+/* ---- Transpose (ref: c_runtime_api.h:360; impl src/ops/Transpose.cu).  perm: host array
+ *      of ndim ints, output axis d is input axis perm[d]. ---- */
+int DLGpuTranspose(const DLArrayHandle input, DLArrayHandle output, int *perm,
+                   DLStreamHandle stream_handle, ProfilerHandle p);
+
+/* ---- BatchMatMul (ref: c_runtime_api.h:445-447; impl src/ops/BatchMatrixMult.cu).
+ *      Row-major C[..., n, m] = op(A[...]) op(B[...]) for every leading index; no
+ *      ProfilerHandle. ---- */
+int DLGpuBatchMatrixMultiply(const DLArrayHandle matA, bool transposeA, const DLArrayHandle matB,
+                             bool transposeB, DLArrayHandle matC, DLStreamHandle stream_handle);
+
+/* ---- OneHot / Where / Embedding (ref: c_runtime_api.h:443,444,280-284; impl
+ *      src/ops/OneHot.cu:16, src/ops/Where.cu:10, src/ops/EmbeddingLookup.cu:14,67).
+ *      ids are float32 holding integers.  The embedding symbols honour ids as the numpy
+ *      branch does (python/athena/gpu_ops/EmbeddingLookUp.py:41-42); the reference's CUDA
+ *      kernels use the row number instead (src/ops/EmbeddingLookup.cu:6-7,59-60).  The
+ *      gradient zero-fills input_grad and scatter-adds; an id outside the table fails. ---- */
+int DLGpuOneHot(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle);
+int DLGpuWhere(const DLArrayHandle cond, const DLArrayHandle arr1, const DLArrayHandle arr2,
+               DLArrayHandle output, DLStreamHandle stream_handle);
+int DLGpuEmbeddingLookUp(const DLArrayHandle input, const DLArrayHandle ids, DLArrayHandle output,
+                         DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuEmbeddingLookUp_Gradient(const DLArrayHandle output_grad, const DLArrayHandle ids,
+                                  DLArrayHandle input_grad, DLStreamHandle stream_handle,
+                                  ProfilerHandle p);
+
+/* ---- Elementwise math (ref: c_runtime_api.h:178-179,188-189,197,218,226,252,260; impl
+ *      src/ops/DivideElewise.cu:6, DivideConst.cu:6 (val / input), Opposite.cu:6, Sqrt.cu:6,46,
+ *      Tanh.cu:6, Sigmoid.cu:6) ---- */
+int DLGpuMatrixElementwiseDivide(const DLArrayHandle matA, const DLArrayHandle matB,
+                                 DLArrayHandle output, DLStreamHandle stream_handle,
+                                 ProfilerHandle p);
+int DLGpuMatrixDivConst(float val, const DLArrayHandle input, DLArrayHandle output,
+                        DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuOpposite(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle,
+                  ProfilerHandle p);
+int DLGpuSqrt(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle,
+              ProfilerHandle p);
+int DLGpuReciprocalSqrt(const DLArrayHandle input, DLArrayHandle output,
+                        DLStreamHandle stream_handle, ProfilerHandle p);
+int DLGpuTanh(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle,
+              ProfilerHandle p);
+int DLGpuSigmoid(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle,
+                 ProfilerHandle p);
 
 #ifdef __cplusplus
 } /* extern "C" */

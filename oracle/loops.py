@@ -147,3 +147,157 @@ def max_pool_grad_loops(x, dy, kH, kW, pad, stride):
                                 hm, wm = i, j
                     dx[n, c, hm, wm] += dy[n, c, h, w]
     return dx
+
+
+def avg_pool_loops(x, kH, kW, pad, stride):
+    """gpu_ops/AvgPool.py:27-50."""
+    N, C, H, W = x.shape
+    pH, pW = _out(H, kH, pad, stride), _out(W, kW, pad, stride)
+    y = np.zeros((N, C, pH, pW), dtype=np.float64)
+    for n in range(N):
+        for c in range(C):
+            for h in range(pH):
+                for w in range(pW):
+                    hs, ws = h * stride - pad, w * stride - pad
+                    he, we = min(hs + kH, H), min(ws + kW, W)
+                    hs, ws = max(hs, 0), max(ws, 0)
+                    for i in range(hs, he):
+                        for j in range(ws, we):
+                            y[n, c, h, w] += x[n, c, i, j]
+                    y[n, c, h, w] /= kH * kW
+    return y
+
+
+def avg_pool_grad_loops(dy, x_shape, kH, kW, pad, stride):
+    """gpu_ops/AvgPool.py:139-161."""
+    N, C, H, W = x_shape
+    pH, pW = dy.shape[2], dy.shape[3]
+    dx = np.zeros(x_shape, dtype=np.float64)
+    for n in range(N):
+        for c in range(C):
+            for h in range(pH):
+                for w in range(pW):
+                    hs, ws = h * stride - pad, w * stride - pad
+                    he, we = min(hs + kH, H), min(ws + kW, W)
+                    hs, ws = max(hs, 0), max(ws, 0)
+                    for i in range(hs, he):
+                        for j in range(ws, we):
+                            dx[n, c, i, j] += dy[n, c, h, w] / (kH * kW)
+    return dx
+
+
+def broadcast_flat_loops(x, out_shape):
+    """src/ops/Broadcast.cu:4-9: out[id] = in[id % in_size]."""
+    flat = np.asarray(x).reshape(-1)
+    out = np.empty(int(np.prod(out_shape)), dtype=flat.dtype)
+    for i in range(out.size):
+        out[i] = flat[i % flat.size]
+    return out.reshape(out_shape)
+
+
+def broadcast_shape_loops(x, out_shape, add_axes=None):
+    """src/ops/BroadcastShape.cu:4-63: host builds in_dims (1 where an axis is new or
+    broadcast), the kernel walks the output index and skips axes of extent 1."""
+    x = np.asarray(x)
+    nd = len(out_shape)
+    diff = nd - x.ndim
+    in_dims = [0] * nd
+    if add_axes is None:
+        for i in range(nd):
+            in_dims[i] = 1 if i < diff else x.shape[i - diff]
+    else:
+        for a in add_axes[:diff]:
+            in_dims[a] = 1
+        o = 0
+        for i in range(x.ndim):
+            while in_dims[o] == 1:
+                o += 1
+            in_dims[o] = x.shape[i]
+            o += 1
+    strides = [int(np.prod(out_shape[i + 1:])) for i in range(nd)]
+    flat = x.reshape(-1)
+    out = np.empty(int(np.prod(out_shape)), dtype=x.dtype)
+    for o_ind in range(out.size):
+        i_ind, t = 0, o_ind
+        for i in range(nd):
+            i_ind *= in_dims[i]
+            q = t // strides[i]
+            if in_dims[i] > 1:
+                i_ind += q
+            t %= strides[i]
+        out[o_ind] = flat[i_ind]
+    return out.reshape(out_shape)
+
+
+def pad_loops(x, paddings, constant):
+    """src/ops/Pad.cu:4-18 with np.pad's treatment of the unpadded leading axes
+    (gpu_ops/Pad.py:194-196): each output element is either the shifted input element
+    or the constant."""
+    full = [(0, 0)] * (x.ndim - len(paddings)) + [tuple(p) for p in paddings]
+    out_shape = tuple(x.shape[i] + full[i][0] + full[i][1] for i in range(x.ndim))
+    out = np.empty(out_shape, dtype=x.dtype)
+    for idx in np.ndindex(*out_shape):
+        src = tuple(idx[i] - full[i][0] for i in range(x.ndim))
+        inside = all(0 <= src[i] < x.shape[i] for i in range(x.ndim))
+        out[idx] = x[src] if inside else constant
+    return out
+
+
+def transpose_loops(x, perm):
+    """src/ops/Transpose.cu:3-17: out[o] = in[sum_d coord_d(o) * in_stride[perm[d]]]."""
+    out_shape = tuple(x.shape[p] for p in perm)
+    out = np.empty(out_shape, dtype=x.dtype)
+    for idx in np.ndindex(*out_shape):
+        src = [0] * x.ndim
+        for d, p in enumerate(perm):
+            src[p] = idx[d]
+        out[idx] = x[tuple(src)]
+    return out
+
+
+def batch_matmul_loops(A, transA, B, transB):
+    """One 2-D product per leading index (src/ops/BatchMatrixMult.cu: strided batched GEMM)."""
+    lead = A.shape[:-2]
+    A2 = A.reshape((-1,) + A.shape[-2:]).astype(np.float64)
+    B2 = B.reshape((-1,) + B.shape[-2:]).astype(np.float64)
+    outs = []
+    for b in range(A2.shape[0]):
+        a = A2[b].T if transA else A2[b]
+        bb = B2[b].T if transB else B2[b]
+        n, k = a.shape
+        m = bb.shape[1]
+        c = np.zeros((n, m))
+        for i in range(n):
+            for j in range(m):
+                s = 0.0
+                for t in range(k):
+                    s += a[i, t] * bb[t, j]
+                c[i, j] = s
+        outs.append(c)
+    return np.stack(outs).reshape(lead + outs[0].shape)
+
+
+def one_hot_loops(ids, num_classes):
+    """src/ops/OneHot.cu:3-14: out[ind] = float(ind % last) == ids[ind / last]."""
+    flat = np.asarray(ids, dtype=np.float32).reshape(-1)
+    out = np.zeros(flat.size * num_classes, dtype=np.float32)
+    for ind in range(out.size):
+        out[ind] = 1.0 if np.float32(ind % num_classes) == flat[ind // num_classes] else 0.0
+    return out.reshape(np.shape(ids) + (num_classes,))
+
+
+def embedding_loops(table, ids):
+    flat = np.asarray(ids).reshape(-1)
+    out = np.empty((flat.size, table.shape[1]), dtype=table.dtype)
+    for r in range(flat.size):
+        out[r] = table[int(flat[r])]
+    return out.reshape(np.shape(ids) + (table.shape[1],))
+
+
+def embedding_grad_loops(dy, ids, table_shape):
+    flat = np.asarray(ids).reshape(-1)
+    d2 = dy.reshape(flat.size, table_shape[1]).astype(np.float64)
+    g = np.zeros(table_shape, dtype=np.float64)
+    for r in range(flat.size):
+        g[int(flat[r])] += d2[r]
+    return g

@@ -35,6 +35,13 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
   softmax / softmax_ce / softmax_ce_grad           pinned: closed forms, invariants
   sgd / momentum / adagrad / adam                  pinned: hand-computed 3-step vectors
   split / concat / slice                           pinned: integer index arithmetic
+  avg_pool / avg_pool_grad                         pinned: literal loops, depthwise
+      correlation with a constant filter, adjoint identity
+  broadcast_* / reduce_* / pad / transpose / one_hot / where / embedding_*
+                                                   pinned: literal loops on small shapes
+  batch_matmul                                     pinned: per-batch matmul loops
+  sqrt / rsqrt / sigmoid / tanh / opposite / div_const / divide
+                                                   pinned: inverse-function identities
 """
 import numpy as np
 
@@ -415,3 +422,180 @@ def array_set(shape, value):
 
 def reshape(a, shape):
     return np.asarray(a, F32).reshape(shape)
+
+
+# --------------------------------------------------------------------------
+# AvgPool  (reference: gpu_ops/AvgPool.py:27-50 fwd, :139-161 bwd)
+# --------------------------------------------------------------------------
+def avg_pool(x, kH, kW, pad=0, stride=1, dtype=np.float64):
+    """Sum over the window clipped to the image, divided by kH*kW whatever the
+    clipping (padding counts as zeros in the mean)."""
+    x = _f(x, dtype)
+    N, C, H, W = x.shape
+    pH, pW = conv_out_size(H, kH, pad, stride), conv_out_size(W, kW, pad, stride)
+    xp = np.zeros((N, C, H + 2 * pad + kH, W + 2 * pad + kW), dtype=dtype)   # slack for floor-sized outputs
+    xp[:, :, pad:pad + H, pad:pad + W] = x
+    y = np.zeros((N, C, pH, pW), dtype=dtype)
+    for i in range(kH):
+        for j in range(kW):
+            y += xp[:, :, i:i + (pH - 1) * stride + 1:stride, j:j + (pW - 1) * stride + 1:stride]
+    return y / (kH * kW)
+
+
+def avg_pool_grad(dy, x_shape, kH, kW, pad=0, stride=1, dtype=np.float64):
+    """Every in-image element of a window receives dy/(kH*kW)."""
+    dy = _f(dy, dtype)
+    N, C, H, W = x_shape
+    pH, pW = dy.shape[2], dy.shape[3]
+    dxp = np.zeros((N, C, H + 2 * pad + kH, W + 2 * pad + kW), dtype=dtype)
+    g = dy / (kH * kW)
+    for i in range(kH):
+        for j in range(kW):
+            dxp[:, :, i:i + (pH - 1) * stride + 1:stride, j:j + (pW - 1) * stride + 1:stride] += g
+    return dxp[:, :, pad:pad + H, pad:pad + W].copy()
+
+
+# --------------------------------------------------------------------------
+# Broadcast / reduce  (reference: gpu_ops/Broadcast.py:59, ReduceSumAxisZero.py:55,
+# Conv2dBroadcast.py:54-55, Conv2dReduceSum.py:48, BroadcastShape.py:52-56,
+# ReduceSum.py:58-64)
+# --------------------------------------------------------------------------
+def broadcast_to(x, shape, dtype=np.float64):
+    """numpy broadcasting of x against `shape` (new leading axes)."""
+    return np.broadcast_to(_f(x, dtype), shape).copy()
+
+
+def reduce_sum_axis_zero(x, dtype=np.float64):
+    return np.sum(_f(x, dtype), axis=0)
+
+
+def conv2d_broadcast_to(bias, shape, dtype=np.float64):
+    """bias [C] -> [N,C,H,W] with out[n,c,h,w] = bias[c] (src/ops/Conv2dBroadcast.cu:4-10)."""
+    b = _f(bias, dtype)
+    assert b.shape == (shape[1],)
+    return np.broadcast_to(b.reshape(1, -1, 1, 1), shape).copy()
+
+
+def conv2d_reduce_sum(x, dtype=np.float64):
+    return np.sum(_f(x, dtype), axis=(0, 2, 3))
+
+
+def broadcast_shape(x, shape, add_axes=None, dtype=np.float64):
+    """With add_axes: x's axes are placed at the positions of `shape` not listed in
+    add_axes, the listed ones are new; without: numpy alignment from the right
+    (src/ops/BroadcastShape.cu:23-63)."""
+    x = _f(x, dtype)
+    if add_axes:
+        in_shape = list(shape)
+        for a in add_axes:
+            in_shape[a] = 1
+        rest = [i for i in range(len(shape)) if i not in set(add_axes)]
+        assert len(rest) == x.ndim
+        for i, a in enumerate(rest):
+            in_shape[a] = x.shape[i]
+        x = x.reshape(in_shape)
+    return np.broadcast_to(x, shape).copy()
+
+
+def reduce_sum(x, axes, keepdims=False, dtype=np.float64):
+    return np.sum(_f(x, dtype), axis=tuple(axes), keepdims=keepdims)
+
+
+# --------------------------------------------------------------------------
+# Pad  (reference: gpu_ops/Pad.py:194-203; CONSTANT mode, paddings for the last
+# len(paddings) axes of a 4-D tensor: gpu_ops/Pad.py:73-80)
+# --------------------------------------------------------------------------
+def _full_paddings(paddings, ndim=4):
+    paddings = [tuple(p) for p in paddings]
+    return [(0, 0)] * (ndim - len(paddings)) + paddings
+
+
+def pad(x, paddings, constant=0.0, dtype=np.float64):
+    x = _f(x, dtype)
+    return np.pad(x, _full_paddings(paddings, x.ndim), mode="constant", constant_values=(constant, constant))
+
+
+def pad_grad(dy, paddings, dtype=np.float64):
+    dy = _f(dy, dtype)
+    sl = tuple(slice(lo, dy.shape[i] - hi) for i, (lo, hi) in enumerate(_full_paddings(paddings, dy.ndim)))
+    return dy[sl].copy()
+
+
+# --------------------------------------------------------------------------
+# BatchMatMul / Transpose  (reference: gpu_ops/BatchMatrixMult.py:50-75, Transpose.py:55)
+# --------------------------------------------------------------------------
+def batch_matmul(A, transA, B, transB, dtype=np.float64):
+    A, B = _f(A, dtype), _f(B, dtype)
+    if transA:
+        A = np.swapaxes(A, -1, -2)
+    if transB:
+        B = np.swapaxes(B, -1, -2)
+    return np.matmul(A, B)
+
+
+def transpose(x, perm):
+    return np.ascontiguousarray(np.transpose(np.asarray(x, dtype=F32), perm))
+
+
+# --------------------------------------------------------------------------
+# OneHot / Where / Embedding  (reference: gpu_ops/OneHot.py:44-46, Where.py:44,
+# EmbeddingLookUp.py:41-42)
+# --------------------------------------------------------------------------
+def one_hot(ids, num_classes):
+    ids = np.asarray(ids, dtype=F32)
+    return (ids[..., None] == np.arange(num_classes, dtype=F32)).astype(F32)
+
+
+def where(cond, a, b):
+    return np.where(np.asarray(cond, dtype=F32) != 0, np.asarray(a, dtype=F32), np.asarray(b, dtype=F32))
+
+
+def embedding_lookup(table, ids):
+    """out[..., :] = table[int(ids[...]), :].  The numpy branch is followed; the CUDA
+    kernel of the reference ignores ids (src/ops/EmbeddingLookup.cu:6-7 uses the row
+    number instead), which cannot be what a lookup means."""
+    table = np.asarray(table, dtype=F32)
+    idx = np.asarray(ids, dtype=F32).astype(np.int64)
+    return table[idx.reshape(-1)].reshape(idx.shape + (table.shape[1],))
+
+
+def embedding_lookup_grad(dy, ids, table_shape, dtype=np.float64):
+    """Scatter-add of the output gradient rows into a zeroed table gradient
+    (src/ops/EmbeddingLookup.cu:56-65 with ids honoured)."""
+    dy = _f(dy, dtype)
+    idx = np.asarray(ids, dtype=F32).astype(np.int64).reshape(-1)
+    g = np.zeros(table_shape, dtype=dtype)
+    np.add.at(g, idx, dy.reshape(-1, table_shape[1]))
+    return g
+
+
+# --------------------------------------------------------------------------
+# Elementwise math  (reference: gpu_ops/Sqrt.py, Sigmoid.py, Tanh.py, Opposite.py,
+# Division.py; src/ops/DivideConst.cu:6 divides the constant BY the tensor)
+# --------------------------------------------------------------------------
+def sqrt(x, dtype=np.float64):
+    return np.sqrt(_f(x, dtype))
+
+
+def rsqrt(x, dtype=np.float64):
+    return 1.0 / np.sqrt(_f(x, dtype))
+
+
+def sigmoid(x, dtype=np.float64):
+    return 1.0 / (1.0 + np.exp(-_f(x, dtype)))
+
+
+def tanh(x, dtype=np.float64):
+    return np.tanh(_f(x, dtype))
+
+
+def opposite(x, dtype=np.float64):
+    return -_f(x, dtype)
+
+
+def div_const(c, x, dtype=np.float64):
+    return dtype(F32(c)) / _f(x, dtype)
+
+
+def divide(a, b, dtype=np.float64):
+    return _f(a, dtype) / _f(b, dtype)

@@ -1,4 +1,5 @@
-// HBM-streaming elementwise kernels: graph-closure ops, Relu and the optimizer updates.
+// HBM-streaming elementwise kernels: graph-closure ops, Relu, elementwise math, Where and
+// the optimizer updates.
 //
 // One template serves all of them.  Every thread moves one 16-byte word per array,
 // consecutive lanes touch consecutive words, and loads and stores are non-temporal: these
@@ -150,6 +151,39 @@ struct ReluGradOp {   // out = (sign(x)+1)*0.5*dy ; arrays: out, x, dy
     v[0] = (sgn + 1.f) * 0.5f * v[2];
   }
 };
+struct DivOp {    // out = a / b
+  static constexpr int N = 3, LOAD = 6, STORE = 1;
+  __device__ void apply(float (&v)[3]) const { v[0] = v[1] / v[2]; }
+};
+struct DivConstOp {   // out = c / a  (src/ops/DivideConst.cu:6)
+  static constexpr int N = 2, LOAD = 2, STORE = 1;
+  float c;
+  __device__ void apply(float (&v)[2]) const { v[0] = c / v[1]; }
+};
+struct NegOp {
+  static constexpr int N = 2, LOAD = 2, STORE = 1;
+  __device__ void apply(float (&v)[2]) const { v[0] = -v[1]; }
+};
+struct SqrtOp {
+  static constexpr int N = 2, LOAD = 2, STORE = 1;
+  __device__ void apply(float (&v)[2]) const { v[0] = sqrtf(v[1]); }
+};
+struct RsqrtOp {  // correctly rounded quotient rather than the approximate rsqrt instruction
+  static constexpr int N = 2, LOAD = 2, STORE = 1;
+  __device__ void apply(float (&v)[2]) const { v[0] = 1.f / sqrtf(v[1]); }
+};
+struct TanhOp {
+  static constexpr int N = 2, LOAD = 2, STORE = 1;
+  __device__ void apply(float (&v)[2]) const { v[0] = tanhf(v[1]); }
+};
+struct SigmoidOp {   // 1/(1+1/exp(x)) (src/ops/Sigmoid.cu:6); saturates to 0 and 1 without NaN
+  static constexpr int N = 2, LOAD = 2, STORE = 1;
+  __device__ void apply(float (&v)[2]) const { v[0] = 1.f / (1.f + expf(-v[1])); }
+};
+struct WhereOp {     // out = cond != 0 ? a : b ; arrays: out, cond, a, b
+  static constexpr int N = 4, LOAD = 14, STORE = 1;
+  __device__ void apply(float (&v)[4]) const { v[0] = v[1] != 0.f ? v[2] : v[3]; }
+};
 // optimizers: arrays param, grad, state...; evaluation order of src/ops/Optimizers.cu
 struct SgdOp {
   static constexpr int N = 2, LOAD = 3, STORE = 1;
@@ -290,6 +324,59 @@ int DLGpuReluGradient(const DLArrayHandle input, const DLArrayHandle in_grad, DL
   const int64_t n = numel(output);
   ProfileScope ps(p, s, 2 * n, n, 0);
   launch(ReluGradOp{}, Ptrs<3>{{fp(output), fp(input), fp(in_grad)}}, n, s);
+  return ps.finish();
+}
+
+#define UNARY_ENTRY(symbol, OP)                                                                                      \
+  int symbol(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle, ProfilerHandle p) {     \
+    TS_REQUIRE(input && output, #symbol ": NULL array");                                                             \
+    SAME_SIZE(input, output, #symbol);                                                                               \
+    hipStream_t s = stream_of(stream_handle);                                                                        \
+    const int64_t n = numel(output);                                                                                 \
+    ProfileScope ps(p, s, n, n, 0);                                                                                  \
+    launch(OP{}, Ptrs<2>{{fp(output), fp(input)}}, n, s);                                                            \
+    return ps.finish();                                                                                              \
+  }
+
+UNARY_ENTRY(DLGpuOpposite, NegOp)
+UNARY_ENTRY(DLGpuSqrt, SqrtOp)
+UNARY_ENTRY(DLGpuReciprocalSqrt, RsqrtOp)
+UNARY_ENTRY(DLGpuTanh, TanhOp)
+UNARY_ENTRY(DLGpuSigmoid, SigmoidOp)
+#undef UNARY_ENTRY
+
+int DLGpuMatrixElementwiseDivide(const DLArrayHandle matA, const DLArrayHandle matB, DLArrayHandle output,
+                                 DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(matA && matB && output, "DLGpuMatrixElementwiseDivide: NULL array");
+  SAME_SIZE(matA, output, "DLGpuMatrixElementwiseDivide");
+  SAME_SIZE(matB, output, "DLGpuMatrixElementwiseDivide");
+  hipStream_t s = stream_of(stream_handle);
+  const int64_t n = numel(output);
+  ProfileScope ps(p, s, 2 * n, n, 0);
+  launch(DivOp{}, Ptrs<3>{{fp(output), fp(matA), fp(matB)}}, n, s);
+  return ps.finish();
+}
+
+int DLGpuMatrixDivConst(float val, const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle,
+                        ProfilerHandle p) {
+  TS_REQUIRE(input && output, "DLGpuMatrixDivConst: NULL array");
+  SAME_SIZE(input, output, "DLGpuMatrixDivConst");
+  hipStream_t s = stream_of(stream_handle);
+  const int64_t n = numel(output);
+  ProfileScope ps(p, s, n, n, 0);
+  launch(DivConstOp{val}, Ptrs<2>{{fp(output), fp(input)}}, n, s);
+  return ps.finish();
+}
+
+int DLGpuWhere(const DLArrayHandle cond, const DLArrayHandle arr1, const DLArrayHandle arr2, DLArrayHandle output,
+               DLStreamHandle stream_handle) {
+  TS_REQUIRE(cond && arr1 && arr2 && output, "DLGpuWhere: NULL array");
+  SAME_SIZE(cond, output, "DLGpuWhere");
+  SAME_SIZE(arr1, output, "DLGpuWhere");
+  SAME_SIZE(arr2, output, "DLGpuWhere");
+  hipStream_t s = stream_of(stream_handle);
+  ProfileScope ps(nullptr, s, 0, 0, 0);
+  launch(WhereOp{}, Ptrs<4>{{fp(output), fp(cond), fp(arr1), fp(arr2)}}, numel(output), s);
   return ps.finish();
 }
 

@@ -10,7 +10,7 @@ namespace tsplit {
 
 struct FastDiv {
   uint32_t d, m, s1, s2;
-  __host__ __device__ explicit FastDiv(uint32_t div = 1) : d(div) {
+  __host__ __device__ FastDiv(uint32_t div = 1) : d(div) {
     uint32_t l = 0;
     while ((1ull << l) < div) ++l;
     m = static_cast<uint32_t>(((1ull << 32) * ((1ull << l) - div)) / div + 1);

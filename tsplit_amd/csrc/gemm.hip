@@ -1,11 +1,14 @@
-// DLGpuMatrixMultiply: row-major 2-D C = op(A) op(B) on the fp32 MFMA tile engine.
+// DLGpuMatrixMultiply and DLGpuBatchMatrixMultiply: row-major C = op(A) op(B) on the fp32 MFMA
+// tile engine.
 //
 // The four transpose combinations only change which loader stages each operand (a
 // transposed operand is simply one whose other index is contiguous); nothing is ever
 // transposed in memory.  Skinny problems (M <= 64, the fully-connected layers at batch 64)
 // use 64x256 tiles; when the tile count cannot fill 256 CUs the K range is split across
 // blocks and folded by a second deterministic kernel (the 64x25088x4096 layer streams a
-// 392 MiB weight matrix and needs every CU pulling on HBM).
+// 392 MiB weight matrix and needs every CU pulling on HBM).  The batched form runs every
+// leading index as one more grid dimension of the same kernel (no split-K: attention-sized
+// batches already give thousands of tiles); narrow outputs (N <= 64) use 256x64 tiles.
 #include "common.h"
 #include "mfma_gemm.h"
 
@@ -48,6 +51,30 @@ int dispatch_tile(const float *A, int64_t lda, const float *B, int64_t ldb, floa
   return launch_gemm<128, 128, 2, 2, TA, TB>(A, lda, B, ldb, C, M, N, K, s, ws);
 }
 
+template <int BM, int BN, int WM, int WN, bool TA, bool TB>
+int launch_batched(const float *A, int64_t lda, int64_t sa, const float *B, int64_t ldb, int64_t sb, float *C, int batch,
+                   int M, int N, int K, hipStream_t s) {
+  using AL = typename std::conditional<TA, MnContigLoader<BM>, KContigLoader<BM>>::type;
+  using BL = typename std::conditional<TB, KContigLoader<BN>, MnContigLoader<BN>>::type;
+  typename AL::Params ap{A, lda, M, lda % 4 == 0 && sa % 4 == 0 && aligned16(A)};
+  typename BL::Params bp{B, ldb, N, ldb % 4 == 0 && sb % 4 == 0 && aligned16(B)};
+  const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+  const int64_t blocks = static_cast<int64_t>(tm) * tn * batch;
+  TS_REQUIRE(blocks < (1ll << 31) - 8, "DLGpuBatchMatrixMultiply: too many tiles");
+  hipLaunchKernelGGL((mfma_batched_gemm_kernel<BM, BN, WM, WN, AL, BL>), dim3(grid_blocks(tm, tn, batch)),
+                     dim3(kThreads), 0, s, ap, bp, C, sa, sb, static_cast<int64_t>(M) * N, M, N, K,
+                     TileGrid{tm, tn, tm * tn * batch});
+  return 0;
+}
+
+template <bool TA, bool TB>
+int dispatch_batched(const float *A, int64_t lda, int64_t sa, const float *B, int64_t ldb, int64_t sb, float *C,
+                     int batch, int M, int N, int K, hipStream_t s) {
+  if (M <= 64) return launch_batched<64, 256, 1, 4, TA, TB>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
+  if (N <= 64) return launch_batched<256, 64, 4, 1, TA, TB>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
+  return launch_batched<128, 128, 2, 2, TA, TB>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
+}
+
 }  // namespace
 }  // namespace tsplit
 
@@ -81,6 +108,43 @@ extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, co
     if (transposeA && transposeB) rc = dispatch_tile<true, true>(A, lda, B, ldb, C, m, n, k, s, &ws);
   }
   if (p) p->workspace_memory = mib(ws);
+  if (rc) return rc;
+  return ps.finish();
+}
+
+extern "C" int DLGpuBatchMatrixMultiply(const DLArrayHandle matA, bool transposeA, const DLArrayHandle matB,
+                                        bool transposeB, DLArrayHandle matC, DLStreamHandle stream_handle) {
+  TS_REQUIRE(matA && matB && matC, "DLGpuBatchMatrixMultiply: NULL array");
+  const int nd = matC->ndim;
+  TS_REQUIRE(nd >= 2 && matA->ndim == nd && matB->ndim == nd, "DLGpuBatchMatrixMultiply: ranks must agree and be >= 2");
+  int64_t batch = 1;
+  for (int d = 0; d < nd - 2; ++d) {
+    TS_REQUIRE(matA->shape[d] == matC->shape[d] && matB->shape[d] == matC->shape[d],
+               "DLGpuBatchMatrixMultiply: leading axis %d differs between the operands", d);
+    batch *= matC->shape[d];
+  }
+  const int64_t a0 = matA->shape[nd - 2], a1 = matA->shape[nd - 1], b0 = matB->shape[nd - 2], b1 = matB->shape[nd - 1];
+  const int64_t M = matC->shape[nd - 2], N = matC->shape[nd - 1];
+  const int64_t K = transposeA ? a0 : a1, Am = transposeA ? a1 : a0;
+  const int64_t Bk = transposeB ? b1 : b0, Bn = transposeB ? b0 : b1;
+  TS_REQUIRE(Am == M && Bn == N && Bk == K,
+             "DLGpuBatchMatrixMultiply: shapes do not conform: op(A) %lldx%lld, op(B) %lldx%lld, C %lldx%lld", (long long)Am,
+             (long long)K, (long long)Bk, (long long)Bn, (long long)M, (long long)N);
+  TS_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) - 64 && batch < (1ll << 31),
+             "DLGpuBatchMatrixMultiply: dimension too large");
+  hipStream_t s = stream_of(stream_handle);
+  ProfileScope ps(nullptr, s, 0, 0, 0);
+  int rc = 0;
+  if (M > 0 && N > 0 && batch > 0) {
+    const float *A = static_cast<const float *>(matA->data), *B = static_cast<const float *>(matB->data);
+    float *C = static_cast<float *>(matC->data);
+    const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K), b = static_cast<int>(batch);
+    const int64_t sa = a0 * a1, sb = b0 * b1;
+    if (!transposeA && !transposeB) rc = dispatch_batched<false, false>(A, a1, sa, B, b1, sb, C, b, m, n, k, s);
+    if (!transposeA && transposeB) rc = dispatch_batched<false, true>(A, a1, sa, B, b1, sb, C, b, m, n, k, s);
+    if (transposeA && !transposeB) rc = dispatch_batched<true, false>(A, a1, sa, B, b1, sb, C, b, m, n, k, s);
+    if (transposeA && transposeB) rc = dispatch_batched<true, true>(A, a1, sa, B, b1, sb, C, b, m, n, k, s);
+  }
   if (rc) return rc;
   return ps.finish();
 }

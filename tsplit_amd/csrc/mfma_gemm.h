@@ -185,11 +185,11 @@ struct TileGrid {
 };
 inline unsigned grid_blocks(int tm, int tn, int S) { return static_cast<unsigned>((tm * tn * S + 7) / 8 * 8); }
 
+// One block's tile: out[m0.., n0..] (+)= A[m0.., kbegin..kend) B[kbegin..kend), n0..].
 template <int BM, int BN, int WM, int WN, class ALoader, class BLoader, class ColMap>
-__global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::Params ap, typename BLoader::Params bp,
-                                                             float *__restrict__ out, int64_t z_stride,
-                                                             int64_t row_stride, ColMap colmap, int M, int N, int K,
-                                                             int kchunk, TileGrid tg) {
+__device__ __forceinline__ void mfma_gemm_tile(const typename ALoader::Params &ap, const typename BLoader::Params &bp,
+                                               float *__restrict__ o, int64_t row_stride, const ColMap &colmap, int M,
+                                               int N, int m0, int n0, int kbegin, int kend) {
   static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
   using ALds = typename ALoader::Lds;
   using BLds = typename BLoader::Lds;
@@ -197,16 +197,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::P
   __shared__ __attribute__((aligned(16))) float lds_b[2][BLds::kFloats];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  if (logical >= tg.total) return;   // padding of the grid to a multiple of 8
-  const int per_split = tg.tm * tg.tn;
-  const int zsplit = logical / per_split;
-  const int rem = logical - zsplit * per_split;
-  const int tile_n = rem / tg.tm, tile_m = rem - tile_n * tg.tm;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
-  const int kbegin = zsplit * kchunk;
-  const int kend = min(K, kbegin + kchunk);
 
   ALoader la;
   BLoader lb;
@@ -274,7 +265,6 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::P
 
   // epilogue: accumulator register e of a 32x32 block holds row 8*(e/4) + 4*(lane/32) + e%4,
   // column lane%32
-  float *o = out + static_cast<int64_t>(zsplit) * z_stride;
 #pragma unroll
   for (int ni = 0; ni < 2; ++ni) {
     const int n = n0 + wn0 + 32 * ni + (lane & 31);
@@ -290,6 +280,49 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::P
       }
     }
   }
+}
+
+// block id -> (z, tile_m, tile_n) in the XCD-aware order described above; false for the blocks
+// that only pad the grid to a multiple of 8
+__device__ __forceinline__ bool block_tile(const TileGrid &tg, int &z, int &tile_m, int &tile_n) {
+  const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  if (logical >= tg.total) return false;
+  const int per_split = tg.tm * tg.tn;
+  z = logical / per_split;
+  const int rem = logical - z * per_split;
+  tile_n = rem / tg.tm;
+  tile_m = rem - tile_n * tg.tm;
+  return true;
+}
+
+// split-K GEMM: split z covers k in [z*kchunk, (z+1)*kchunk) and writes to out + z * z_stride
+template <int BM, int BN, int WM, int WN, class ALoader, class BLoader, class ColMap>
+__global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(typename ALoader::Params ap, typename BLoader::Params bp,
+                                                             float *__restrict__ out, int64_t z_stride,
+                                                             int64_t row_stride, ColMap colmap, int M, int N, int K,
+                                                             int kchunk, TileGrid tg) {
+  int z, tile_m, tile_n;
+  if (!block_tile(tg, z, tile_m, tile_n)) return;
+  const int kbegin = z * kchunk;
+  mfma_gemm_tile<BM, BN, WM, WN, ALoader, BLoader, ColMap>(ap, bp, out + static_cast<int64_t>(z) * z_stride, row_stride,
+                                                           colmap, M, N, tile_m * BM, tile_n * BN, kbegin,
+                                                           min(K, kbegin + kchunk));
+}
+
+// batched GEMM: z is the batch index; operands and output advance by their batch strides
+template <int BM, int BN, int WM, int WN, class ALoader, class BLoader>
+__global__ __launch_bounds__(kThreads) void mfma_batched_gemm_kernel(typename ALoader::Params ap,
+                                                                     typename BLoader::Params bp,
+                                                                     float *__restrict__ out, int64_t a_zstride,
+                                                                     int64_t b_zstride, int64_t c_zstride, int M, int N,
+                                                                     int K, TileGrid tg) {
+  int z, tile_m, tile_n;
+  if (!block_tile(tg, z, tile_m, tile_n)) return;
+  ap.p += static_cast<int64_t>(z) * a_zstride;
+  bp.p += static_cast<int64_t>(z) * b_zstride;
+  mfma_gemm_tile<BM, BN, WM, WN, ALoader, BLoader, RowMajorCols>(ap, bp, out + static_cast<int64_t>(z) * c_zstride,
+                                                                 static_cast<int64_t>(N), RowMajorCols{}, M, N,
+                                                                 tile_m * BM, tile_n * BN, 0, K);
 }
 
 // out[i] = sum_z part[z * stride + i], z ascending (deterministic split-K fold)

@@ -20,6 +20,12 @@ __all__ = [
     "max_pooling2d", "max_pooling2d_gradient", "CuDNN_max_pooling2d", "CuDNN_max_pooling2d_gradient",
     "concat", "concat_gradient", "matrix_slice", "matrix_slice_gradient",
     "sgd_update", "momentum_update", "adagrad_update", "adam_update",
+    "average_pooling2d", "average_pooling2d_gradient", "CuDNN_average_pooling2d",
+    "CuDNN_average_pooling2d_gradient", "broadcast_to", "reduce_sum_axis_zero", "_reduce_sum_axis_zero",
+    "conv2d_broadcast_to", "conv2d_reduce_sum", "broadcast_shape", "reduce_sum", "pad", "pad_gradient",
+    "matrix_transpose", "batch_matrix_multiply", "one_hot", "where", "embedding_lookup",
+    "embedding_lookup_gradient", "matrix_elementwise_divide", "matrix_elementwise_divide_const",
+    "matrix_opposite", "matrix_sqrt", "matrix_rsqrt", "tanh", "sigmoid",
 ]
 
 
@@ -219,3 +225,142 @@ def adam_update(param, grad, expavg, expavgsq, lr, beta1, beta2, beta1t, beta2t,
     check_call(_LIB.AdamOptimizerUpdate(_h(param), _h(grad), _h(expavg), _h(expavgsq), ctypes.c_float(lr),
                                         ctypes.c_float(beta1), ctypes.c_float(beta2), ctypes.c_float(beta1t),
                                         ctypes.c_float(beta2t), ctypes.c_float(eps), _s(stream)))
+
+
+# ---- AvgPool (gpu_links/AvgPoolLink.py:8,15; gpu_links/CudnnAvgPoolLink.py:8,15) ----
+def average_pooling2d(in_arr, kernel_H, kernel_W, pooled_layer, padding=0, stride=1, stream=None, profiler=None):
+    check_call(_LIB.DLGpuAvgerage_Pooling2d(_h(in_arr), ctypes.c_size_t(kernel_H), ctypes.c_size_t(kernel_W),
+                                            _h(pooled_layer), ctypes.c_size_t(padding), ctypes.c_size_t(stride),
+                                            _s(stream), _p(profiler)))
+
+
+def average_pooling2d_gradient(in_gradient_y, kernel_H, kernel_W, out_gradient_x, padding=0, stride=1,
+                               stream=None, profiler=None):
+    check_call(_LIB.DLGpuAvgerage_Pooling2d_gradient(
+        _h(in_gradient_y), ctypes.c_size_t(kernel_H), ctypes.c_size_t(kernel_W), _h(out_gradient_x),
+        ctypes.c_size_t(padding), ctypes.c_size_t(stride), _s(stream), _p(profiler)))
+
+
+def CuDNN_average_pooling2d(in_arr, kernel_H, kernel_W, pooled_layer, padding=0, stride=1, stream=None,
+                            profiler=None):
+    check_call(_LIB.CuDNN_DLGpuAvgerage_Pooling2d(
+        _h(in_arr), ctypes.c_size_t(kernel_H), ctypes.c_size_t(kernel_W), _h(pooled_layer),
+        ctypes.c_size_t(padding), ctypes.c_size_t(stride), _s(stream), _p(profiler)))
+
+
+def CuDNN_average_pooling2d_gradient(in_arr_y, in_gradient_y, in_arr_x, kernel_H, kernel_W, out_gradient_x,
+                                     padding=0, stride=1, stream=None, profiler=None):
+    check_call(_LIB.CuDNN_DLGpuAvgerage_Pooling2d_gradient(
+        _h(in_arr_y), _h(in_gradient_y), _h(in_arr_x), ctypes.c_size_t(kernel_H), ctypes.c_size_t(kernel_W),
+        _h(out_gradient_x), ctypes.c_size_t(padding), ctypes.c_size_t(stride), _s(stream), _p(profiler)))
+
+
+# ---- Broadcast / reduce (gpu_links/BroadcastLink.py:8, ReduceSumAxisZeroLink.py:7,15,
+#      Conv2dBroadcastLink.py:8, Conv2dReduceSumLink.py:8, BroadcastShapeLink.py:8, ReduceSumLink.py:7) ----
+def broadcast_to(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuBroadcastTo(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def reduce_sum_axis_zero(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuReduceSumAxisZero(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def _reduce_sum_axis_zero(in_arr, out_arr, workspace_arr, stream=None, profiler=None):
+    check_call(_LIB._DLGpuReduceSumAxisZero(_h(in_arr), _h(out_arr), _h(workspace_arr), _s(stream), _p(profiler)))
+
+
+def conv2d_broadcast_to(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuConv2d_broadcast_to(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def conv2d_reduce_sum(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuConv2d_reduce_sum(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def broadcast_shape(in_arr, out_arr, add_axes=None, stream=None):
+    pointer = (ctypes.c_int * len(add_axes))(*list(add_axes)) if add_axes else None
+    check_call(_LIB.DLGpuBroadcastShape(_h(in_arr), _h(out_arr), pointer, _s(stream)))
+
+
+def reduce_sum(in_arr, out_arr, axes, stream=None):
+    pointer = (ctypes.c_int * len(axes))(*list(axes))
+    check_call(_LIB.DLGpuReduceSum(_h(in_arr), _h(out_arr), pointer, ctypes.c_int(len(axes)), _s(stream)))
+
+
+# ---- Pad (gpu_links/PadLink.py:8,30): paddings is a list of (before, after) pairs for the last axes ----
+_PAD_MODES = {"CONSTANT": 0, "REFLECT": 1, "SYMMETRIC": 2}
+
+
+def _pad_args(paddings, mode):
+    flat = [int(v) for pair in paddings for v in pair]
+    assert mode in _PAD_MODES
+    return (ctypes.c_int * len(flat))(*flat), len(flat), ctypes.c_size_t(_PAD_MODES[mode])
+
+
+def pad(in_arr, out_arr, paddings, mode="CONSTANT", constant_values=0, stream=None, profiler=None):
+    arr, n, m = _pad_args(paddings, mode)
+    check_call(_LIB.DLGpuPad(_h(in_arr), _h(out_arr), arr, n, m, ctypes.c_float(constant_values),
+                             _s(stream), _p(profiler)))
+
+
+def pad_gradient(out_grad_arr, in_grad_arr, paddings, mode="CONSTANT", stream=None, profiler=None):
+    arr, n, m = _pad_args(paddings, mode)
+    check_call(_LIB.DLGpuPad_gradient(_h(out_grad_arr), _h(in_grad_arr), arr, n, m, _s(stream), _p(profiler)))
+
+
+# ---- Transpose / BatchMatMul (gpu_links/MatrixTransLink.py:8, BatchMatrixMultLink.py:7) ----
+def matrix_transpose(in_mat, out_mat, perm, stream=None, profiler=None):
+    pointer = (ctypes.c_int * len(perm))(*list(perm))
+    check_call(_LIB.DLGpuTranspose(_h(in_mat), _h(out_mat), pointer, _s(stream), _p(profiler)))
+
+
+def batch_matrix_multiply(matA, transA, matB, transB, matC, stream=None):
+    check_call(_LIB.DLGpuBatchMatrixMultiply(_h(matA), ctypes.c_bool(bool(transA)), _h(matB),
+                                             ctypes.c_bool(bool(transB)), _h(matC), _s(stream)))
+
+
+# ---- OneHot / Where / Embedding (gpu_links/OneHotLink.py:8, WhereLink.py:8, EmbeddingLookUpLink.py:8,15) ----
+def one_hot(in_arr, out_arr, stream=None):
+    check_call(_LIB.DLGpuOneHot(_h(in_arr), _h(out_arr), _s(stream)))
+
+
+def where(cond, arr1, arr2, out_arr, stream=None):
+    check_call(_LIB.DLGpuWhere(_h(cond), _h(arr1), _h(arr2), _h(out_arr), _s(stream)))
+
+
+def embedding_lookup(in_mat, ids, out_mat, stream=None, profiler=None):
+    check_call(_LIB.DLGpuEmbeddingLookUp(_h(in_mat), _h(ids), _h(out_mat), _s(stream), _p(profiler)))
+
+
+def embedding_lookup_gradient(grad_out, ids, grad_in, stream=None, profiler=None):
+    check_call(_LIB.DLGpuEmbeddingLookUp_Gradient(_h(grad_out), _h(ids), _h(grad_in), _s(stream), _p(profiler)))
+
+
+# ---- Elementwise math (gpu_links/MatrixDivideLink.py:7, MatrixDivideConstLink.py:7, OppositeLink.py:8,
+#      MatrixSqrtLink.py:8, MatrixRsqrtLink.py:8, TanhLink.py:8, SigmoidLink.py:7) ----
+def matrix_elementwise_divide(matA, matB, matC, stream=None, profiler=None):
+    check_call(_LIB.DLGpuMatrixElementwiseDivide(_h(matA), _h(matB), _h(matC), _s(stream), _p(profiler)))
+
+
+def matrix_elementwise_divide_const(val, in_mat, out_mat, stream=None, profiler=None):
+    check_call(_LIB.DLGpuMatrixDivConst(ctypes.c_float(val), _h(in_mat), _h(out_mat), _s(stream), _p(profiler)))
+
+
+def matrix_opposite(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuOpposite(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def matrix_sqrt(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuSqrt(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def matrix_rsqrt(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuReciprocalSqrt(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def tanh(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuTanh(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+def sigmoid(in_arr, out_arr, stream=None, profiler=None):
+    check_call(_LIB.DLGpuSigmoid(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
