@@ -16,7 +16,6 @@ Prints ONE JSON line.  Besides the contract fields it carries
   cpu_baseline  the numpy CPU oracle timed on this host on a bounded sample of the workload
 """
 import argparse
-import ctypes
 import json
 import os
 import sys
@@ -37,56 +36,6 @@ TRAFFIC_BYTES_PER_LAUNCH = {
     "conv_bwd_data_128x128": (207.2 + 98.3) * 1e6,
     "conv_bwd_filter_128x128": (505.0 + 64.3) * 1e6,
 }
-
-
-class EventTimer(object):
-    """Brackets every operator call with a pair of HIP events on the compute stream; elapsed
-    times are read after the final synchronisation, so nothing blocks inside the step."""
-
-    def __init__(self, ctx):
-        from tsplit_amd.stream import create_event_handle
-        self._mk = lambda: create_event_handle(ctx)
-        self._hip = ctypes.CDLL("libamdhip64.so")
-        self._pool, self._used, self.spans = [], 0, []
-        self.enabled = False
-
-    def _ev(self):
-        if self._used == len(self._pool):
-            self._pool.append(self._mk())
-        self._used += 1
-        return self._pool[self._used - 1]
-
-    def begin(self, stream):
-        if self.enabled:
-            self._a = self._ev()
-            self._a.record(stream)
-
-    def end(self, stream, tag, work, unit):
-        if self.enabled:
-            b = self._ev()
-            b.record(stream)
-            self.spans.append((tag, work, unit, self._a, b))
-
-    def collect(self):
-        """-> {tag: dict(calls, ms_total, ms_avg, work_per_call, unit, rate)} ; rate in TFLOP/s or GB/s"""
-        out = {}
-        ms = ctypes.c_float(0)
-        for tag, work, unit, a, b in self.spans:
-            ea = ctypes.cast(a.handle.contents.handle, ctypes.POINTER(ctypes.c_void_p))[0]
-            eb = ctypes.cast(b.handle.contents.handle, ctypes.POINTER(ctypes.c_void_p))[0]
-            rc = self._hip.hipEventElapsedTime(ctypes.byref(ms), ctypes.c_void_p(ea), ctypes.c_void_p(eb))
-            if rc != 0:
-                raise RuntimeError("hipEventElapsedTime failed: %d" % rc)
-            d = out.setdefault(tag, {"calls": 0, "ms_total": 0.0, "work": 0.0, "unit": unit})
-            d["calls"] += 1
-            d["ms_total"] += ms.value
-            d["work"] += work
-        for d in out.values():
-            d["ms_avg"] = d["ms_total"] / d["calls"]
-            d["work_per_call"] = d["work"] / d["calls"]
-            sec = d["ms_total"] * 1e-3
-            d["rate"] = d["work"] / sec / (1e12 if d["unit"] == "flop" else 1e9) if sec > 0 else 0.0
-        return out
 
 
 def vgg_workload(batch, seed=123):
@@ -138,6 +87,7 @@ def main():
                  "The one-GPU figure is the whole-job throughput.")
 
     from tsplit_amd import ndarray, trainer
+    from tsplit_amd.timing import EventTimer
     ctx = ndarray.gpu(0)
     spec, params, x, labels, split = vgg_workload(a.batch)
     if a.no_split:

@@ -183,6 +183,12 @@ POOL_CASES = [
     ((2, 3, 8, 8), 3, 3, 1, 2),          # floors
     ((2, 2, 9, 11), 3, 3, 0, 2),         # Inception pool
     ((1, 2, 6, 7), 2, 3, 0, 1),          # overlapping, non-square
+    ((2, 3, 9, 10), 3, 3, 1, 1),         # 3x3 stride 1: nine windows over an element
+    ((2, 3, 9, 10), 2, 2, 0, 1),         # 2x2 stride 1
+    ((2, 3, 9, 10), 2, 2, 1, 2),         # 2x2 stride 2 with padding
+    ((1, 2, 12, 12), 3, 3, 0, 3),        # 3x3 stride 3: disjoint windows
+    ((1, 2, 11, 9), 2, 2, 0, 3),         # gaps between windows
+    ((4, 16, 57, 57), 3, 3, 1, 2),       # larger overlapping case
 ]
 
 

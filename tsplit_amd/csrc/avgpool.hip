@@ -7,7 +7,10 @@
 // plane, lanes striding over the plane and a shuffle reduction, so that reads stay
 // coalesced.  Backward is a gather: one thread per input element sums the dy of the windows
 // that contain it in ascending window order and divides once; no atomics, no zero-fill pass.
+#include <algorithm>
+
 #include "common.h"
+#include "fastdiv.h"
 #include "reduce.h"
 
 namespace tsplit {
@@ -18,24 +21,59 @@ constexpr int kThreads = 256;
 struct AvgGeo {
   int H, W, pH, pW, kH, kW, pad, stride;
   float area;
+  FastDiv div_pw, div_ph, div_w, div_h, div_stride;
 };
 
+// idx -> (plane, row, col) for rows of `w` elements and planes of `h` rows; 32-bit fast path
+__device__ __forceinline__ void split3(int64_t idx, int64_t total, const FastDiv &w, const FastDiv &h, int64_t &plane,
+                                       int &row, int &col) {
+  if (total < (1ll << 32)) {
+    const uint32_t i = static_cast<uint32_t>(idx);
+    const uint32_t t = w.div(i);
+    col = static_cast<int>(i - t * w.d);
+    const uint32_t pl = h.div(t);
+    row = static_cast<int>(t - pl * h.d);
+    plane = pl;
+  } else {
+    col = static_cast<int>(idx % w.d);
+    const int64_t t = idx / w.d;
+    row = static_cast<int>(t % h.d);
+    plane = t / h.d;
+  }
+}
+
+// K: compile-time square window (all taps are fetched with predicated loads issued together),
+// or 0 for run-time window sizes (a loop over the clipped window).
+template <int K>
 __global__ __launch_bounds__(kThreads) void avg_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, AvgGeo g,
                                                            int64_t total) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (idx >= total) return;
-  const int ow = static_cast<int>(idx % g.pW);
-  const int64_t t = idx / g.pW;
-  const int oh = static_cast<int>(t % g.pH);
-  const int64_t nc = t / g.pH;
+  int ow, oh;
+  int64_t nc;
+  split3(idx, total, g.div_pw, g.div_ph, nc, oh, ow);
   const float *plane = x + nc * g.H * g.W;
-  int hs = oh * g.stride - g.pad, ws = ow * g.stride - g.pad;
-  const int he = min(hs + g.kH, g.H), we = min(ws + g.kW, g.W);
-  hs = max(hs, 0);
-  ws = max(ws, 0);
+  const int h0 = oh * g.stride - g.pad, w0 = ow * g.stride - g.pad;
   float acc = 0.f;
-  for (int i = hs; i < he; ++i)
-    for (int j = ws; j < we; ++j) acc += plane[i * g.W + j];
+  if (K > 0) {
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+      const int ih = h0 + i;
+      const bool row_ok = static_cast<unsigned>(ih) < static_cast<unsigned>(g.H);
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        const int iw = w0 + j;
+        const bool ok = row_ok && static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
+        const float v = ok ? plane[ih * g.W + iw] : 0.f;
+        acc += v;
+      }
+    }
+  } else {
+    const int he = min(h0 + g.kH, g.H), we = min(w0 + g.kW, g.W);
+    const int hs = max(h0, 0), ws = max(w0, 0);
+    for (int i = hs; i < he; ++i)
+      for (int j = ws; j < we; ++j) acc += plane[i * g.W + j];
+  }
   y[idx] = acc / g.area;
 }
 
@@ -52,23 +90,39 @@ __global__ __launch_bounds__(kThreads) void avg_global_kernel(const float *__res
   if (lane == 0) y[plane] = acc / area;
 }
 
+// NW: compile-time bound on the windows per axis that can contain one element, ceil(k / stride)
+// (predicated loads issued together), or 0 for a run-time loop.
+template <int NW>
 __global__ __launch_bounds__(kThreads) void avg_bwd_kernel(const float *__restrict__ dy, float *__restrict__ dx, AvgGeo g,
                                                            int64_t total) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (idx >= total) return;
-  const int w = static_cast<int>(idx % g.W);
-  const int64_t t = idx / g.W;
-  const int h = static_cast<int>(t % g.H);
-  const int64_t nc = t / g.H;
+  int w, h;
+  int64_t nc;
+  split3(idx, total, g.div_w, g.div_h, nc, h, w);
   const float *dplane = dy + nc * g.pH * g.pW;
-  // windows oh with oh*s - pad <= h < oh*s - pad + kH
-  const int oh_lo = max(0, (h + g.pad - g.kH + g.stride) / g.stride);
-  const int oh_hi = min(g.pH - 1, (h + g.pad) / g.stride);
-  const int ow_lo = max(0, (w + g.pad - g.kW + g.stride) / g.stride);
-  const int ow_hi = min(g.pW - 1, (w + g.pad) / g.stride);
+  // windows oh with oh*s - pad <= h < oh*s - pad + kH, i.e. ceil((h + pad - kH + 1) / s) <= oh <= (h + pad) / s
+  const int th = h + g.pad - g.kH + g.stride, tw = w + g.pad - g.kW + g.stride;
+  const int oh_lo = th > 0 ? static_cast<int>(g.div_stride.div(th)) : 0;
+  const int oh_hi = min(g.pH - 1, static_cast<int>(g.div_stride.div(h + g.pad)));
+  const int ow_lo = tw > 0 ? static_cast<int>(g.div_stride.div(tw)) : 0;
+  const int ow_hi = min(g.pW - 1, static_cast<int>(g.div_stride.div(w + g.pad)));
   float acc = 0.f;
-  for (int oh = oh_lo; oh <= oh_hi; ++oh)
-    for (int ow = ow_lo; ow <= ow_hi; ++ow) acc += dplane[oh * g.pW + ow];
+  if (NW > 0) {
+#pragma unroll
+    for (int a = 0; a < NW; ++a) {
+      const int oh = oh_lo + a;
+#pragma unroll
+      for (int b = 0; b < NW; ++b) {
+        const int ow = ow_lo + b;
+        const float v = (oh <= oh_hi && ow <= ow_hi) ? dplane[oh * g.pW + ow] : 0.f;
+        acc += v;
+      }
+    }
+  } else {
+    for (int oh = oh_lo; oh <= oh_hi; ++oh)
+      for (int ow = ow_lo; ow <= ow_hi; ++ow) acc += dplane[oh * g.pW + ow];
+  }
   dx[idx] = acc / g.area;
 }
 
@@ -91,6 +145,11 @@ int check_geo(const char *who, const DLArray *x, const DLArray *y, size_t kH, si
   g.pad = static_cast<int>(pad);
   g.stride = static_cast<int>(stride);
   g.area = static_cast<float>(kH * kW);
+  g.div_pw = FastDiv(static_cast<uint32_t>(g.pW > 0 ? g.pW : 1));
+  g.div_ph = FastDiv(static_cast<uint32_t>(g.pH > 0 ? g.pH : 1));
+  g.div_w = FastDiv(static_cast<uint32_t>(g.W > 0 ? g.W : 1));
+  g.div_h = FastDiv(static_cast<uint32_t>(g.H > 0 ? g.H : 1));
+  g.div_stride = FastDiv(static_cast<uint32_t>(g.stride));
   TS_REQUIRE(g.H + 2 * g.pad >= g.kH && g.W + 2 * g.pad >= g.kW, "%s: kernel larger than the padded image", who);
   const int eh = (g.H + 2 * g.pad - g.kH) / g.stride + 1, ew = (g.W + 2 * g.pad - g.kW) / g.stride + 1;
   TS_REQUIRE(g.pH == eh && g.pW == ew, "%s: output is %dx%d, expected %dx%d", who, g.pH, g.pW, eh, ew);
@@ -111,8 +170,16 @@ int avg_forward(const char *who, const DLArray *x, DLArray *y, size_t kH, size_t
                          dim3(kThreads), 0, s, static_cast<const float *>(x->data), static_cast<float *>(y->data),
                          g.H * g.W, g.area, total);
     } else {
-      hipLaunchKernelGGL(avg_fwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)), dim3(kThreads),
-                         0, s, static_cast<const float *>(x->data), static_cast<float *>(y->data), g, total);
+      const dim3 grid(static_cast<unsigned>((total + kThreads - 1) / kThreads)), block(kThreads);
+      const float *xp = static_cast<const float *>(x->data);
+      float *yp = static_cast<float *>(y->data);
+      const int k = g.kH == g.kW ? g.kH : 0;
+      if (k == 2)
+        hipLaunchKernelGGL(avg_fwd_kernel<2>, grid, block, 0, s, xp, yp, g, total);
+      else if (k == 3)
+        hipLaunchKernelGGL(avg_fwd_kernel<3>, grid, block, 0, s, xp, yp, g, total);
+      else
+        hipLaunchKernelGGL(avg_fwd_kernel<0>, grid, block, 0, s, xp, yp, g, total);
     }
   }
   return ps.finish();
@@ -125,9 +192,20 @@ int avg_backward(const char *who, const DLArray *dy, DLArray *dx, size_t kH, siz
   hipStream_t s = stream_of(sh);
   ProfileScope ps(p, s, numel(dy), numel(dx), 0);
   const int64_t total = numel(dx);
-  if (total > 0)
-    hipLaunchKernelGGL(avg_bwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)), dim3(kThreads), 0,
-                       s, static_cast<const float *>(dy->data), static_cast<float *>(dx->data), g, total);
+  if (total > 0) {
+    const dim3 grid(static_cast<unsigned>((total + kThreads - 1) / kThreads)), block(kThreads);
+    const float *dyp = static_cast<const float *>(dy->data);
+    float *dxp = static_cast<float *>(dx->data);
+    const int nw = (std::max(g.kH, g.kW) + g.stride - 1) / g.stride;   // windows per axis over one element
+    if (nw == 1)
+      hipLaunchKernelGGL(avg_bwd_kernel<1>, grid, block, 0, s, dyp, dxp, g, total);
+    else if (nw == 2)
+      hipLaunchKernelGGL(avg_bwd_kernel<2>, grid, block, 0, s, dyp, dxp, g, total);
+    else if (nw == 3)
+      hipLaunchKernelGGL(avg_bwd_kernel<3>, grid, block, 0, s, dyp, dxp, g, total);
+    else
+      hipLaunchKernelGGL(avg_bwd_kernel<0>, grid, block, 0, s, dyp, dxp, g, total);
+  }
   return ps.finish();
 }
 

@@ -3,13 +3,16 @@
 // Semantics (src/ops/MaxPool.cu:3-43, python/athena/gpu_ops/MaxPool.py:8-68): the window is
 // clipped to the image, the maximum is the first strict maximum in row-major scan order.
 // The backward pass is a gather: one thread per input element looks at the (at most
-// ceil(k/s)^2) windows that contain it, recomputes each window's argmax and adds that
-// window's dy when the argmax is this element -- in ascending window order, which is the
-// accumulation order of the reference's scatter loop, without atomics and without a
-// separate zero-fill pass (every dx element is written exactly once).
+// ceil(k/s)^2) windows that contain it and adds a window's dy when the window's argmax is
+// this element -- in ascending window order, which is the accumulation order of the
+// reference's scatter loop, without atomics and without a separate zero-fill pass (every dx
+// element is written exactly once).  Non-overlapping windows recompute their argmax in the
+// same kernel; overlapping 2x2 / 3x3 windows take their argmax from a first pass that stores
+// one index per window in scratch.
 // The 2x2 / stride 2 / no padding case (every VGG pool) has a vectorised path: a thread
 // owns two adjacent windows, i.e. one 16-byte word from each of two input rows.
 #include "common.h"
+#include "fastdiv.h"
 
 namespace tsplit {
 namespace {
@@ -20,13 +23,62 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 struct PoolGeo {
   int H, W, pH, pW, kH, kW, pad, stride;
+  FastDiv div_pw, div_ph, div_w, div_h, div_stride;
 };
 
+// idx -> (plane, row, col) for rows of `w` elements and planes of `h` rows; 32-bit fast path
+__device__ __forceinline__ void split3(int64_t idx, int64_t total, const FastDiv &w, const FastDiv &h, int64_t &plane,
+                                       int &row, int &col) {
+  if (total < (1ll << 32)) {
+    const uint32_t i = static_cast<uint32_t>(idx);
+    const uint32_t t = w.div(i);
+    col = static_cast<int>(i - t * w.d);
+    const uint32_t pl = h.div(t);
+    row = static_cast<int>(t - pl * h.d);
+    plane = pl;
+  } else {
+    col = static_cast<int>(idx % w.d);
+    const int64_t t = idx / w.d;
+    row = static_cast<int>(t % h.d);
+    plane = t / h.d;
+  }
+}
+
+// Flat index (h*W + w) of the first strict maximum of window (oh, ow) in row-major scan order.
+// K: compile-time square window -- every tap is fetched with a predicated load, so the loads
+// issue together -- or 0 for run-time window sizes (a loop over the clipped window).
+template <int K>
 __device__ __forceinline__ int window_argmax(const float *__restrict__ plane, const PoolGeo &g, int oh, int ow) {
-  int hs = oh * g.stride - g.pad, ws = ow * g.stride - g.pad;
-  const int he = min(hs + g.kH, g.H), we = min(ws + g.kW, g.W);
-  hs = max(hs, 0);
-  ws = max(ws, 0);
+  const int h0 = oh * g.stride - g.pad, w0 = ow * g.stride - g.pad;
+  if (K > 0) {
+    constexpr int KK = K > 0 ? K : 1;
+    float v[KK][KK];
+    bool ok[KK][KK];
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+      const int ih = h0 + i;
+      const bool row_ok = static_cast<unsigned>(ih) < static_cast<unsigned>(g.H);
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        const int iw = w0 + j;
+        ok[i][j] = row_ok && static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
+        v[i][j] = ok[i][j] ? plane[ih * g.W + iw] : 0.f;
+      }
+    }
+    int best = -1;
+    float bv = 0.f;
+#pragma unroll
+    for (int i = 0; i < K; ++i)
+#pragma unroll
+      for (int j = 0; j < K; ++j)
+        if (ok[i][j] && (best < 0 || v[i][j] > bv)) {
+          bv = v[i][j];
+          best = (h0 + i) * g.W + w0 + j;
+        }
+    return best;   // >= 0: padding is smaller than the window, so one tap is always inside
+  }
+  const int he = min(h0 + g.kH, g.H), we = min(w0 + g.kW, g.W);
+  const int hs = max(h0, 0), ws = max(w0, 0);
   int best = hs * g.W + ws;
   float bv = plane[best];
   for (int i = hs; i < he; ++i)
@@ -40,38 +92,103 @@ __device__ __forceinline__ int window_argmax(const float *__restrict__ plane, co
   return best;
 }
 
+template <int K>
 __global__ __launch_bounds__(kThreads) void pool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
                                                             PoolGeo g, int64_t total) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (idx >= total) return;
-  const int ow = static_cast<int>(idx % g.pW);
-  const int64_t t = idx / g.pW;
-  const int oh = static_cast<int>(t % g.pH);
-  const int64_t nc = t / g.pH;
+  int ow, oh;
+  int64_t nc;
+  split3(idx, total, g.div_pw, g.div_ph, nc, oh, ow);
   const float *plane = x + nc * g.H * g.W;
-  y[idx] = plane[window_argmax(plane, g, oh, ow)];
+  y[idx] = plane[window_argmax<K>(plane, g, oh, ow)];
 }
 
+// NW: compile-time bound on the windows per axis that can contain one element (ceil(k / stride)),
+// 0 for a run-time loop.
+template <int K, int NW>
 __global__ __launch_bounds__(kThreads) void pool_bwd_kernel(const float *__restrict__ x, const float *__restrict__ dy,
                                                             float *__restrict__ dx, PoolGeo g, int64_t total) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (idx >= total) return;
-  const int w = static_cast<int>(idx % g.W);
-  const int64_t t = idx / g.W;
-  const int h = static_cast<int>(t % g.H);
-  const int64_t nc = t / g.H;
+  int w, h;
+  int64_t nc;
+  split3(idx, total, g.div_w, g.div_h, nc, h, w);
   const float *plane = x + nc * g.H * g.W;
   const float *dplane = dy + nc * g.pH * g.pW;
-  // windows oh with oh*s - pad <= h < oh*s - pad + kH
-  const int oh_lo = max(0, (h + g.pad - g.kH + g.stride) / g.stride);   // ceil((h+pad-kH+1)/s) for the non-negative case
-  const int oh_hi = min(g.pH - 1, (h + g.pad) / g.stride);
-  const int ow_lo = max(0, (w + g.pad - g.kW + g.stride) / g.stride);
-  const int ow_hi = min(g.pW - 1, (w + g.pad) / g.stride);
+  // windows oh with oh*s - pad <= h < oh*s - pad + kH, i.e. ceil((h + pad - kH + 1) / s) <= oh <= (h + pad) / s
+  const int th = h + g.pad - g.kH + g.stride, tw = w + g.pad - g.kW + g.stride;
+  const int oh_lo = th > 0 ? static_cast<int>(g.div_stride.div(th)) : 0;
+  const int oh_hi = min(g.pH - 1, static_cast<int>(g.div_stride.div(h + g.pad)));
+  const int ow_lo = tw > 0 ? static_cast<int>(g.div_stride.div(tw)) : 0;
+  const int ow_hi = min(g.pW - 1, static_cast<int>(g.div_stride.div(w + g.pad)));
   const int me = h * g.W + w;
   float acc = 0.f;
-  for (int oh = oh_lo; oh <= oh_hi; ++oh)
-    for (int ow = ow_lo; ow <= ow_hi; ++ow)
-      if (window_argmax(plane, g, oh, ow) == me) acc += dplane[oh * g.pW + ow];
+  if (NW > 0) {
+#pragma unroll
+    for (int a = 0; a < NW; ++a) {
+#pragma unroll
+      for (int b = 0; b < NW; ++b) {
+        // a window beyond the last one is replaced by the last one and its result discarded
+        const int oh = min(oh_lo + a, oh_hi), ow = min(ow_lo + b, ow_hi);
+        const bool live = oh_lo + a <= oh_hi && ow_lo + b <= ow_hi;
+        const bool mine = window_argmax<K>(plane, g, oh, ow) == me;
+        const float gy = dplane[oh * g.pW + ow];
+        if (live && mine) acc += gy;
+      }
+    }
+  } else {
+    for (int oh = oh_lo; oh <= oh_hi; ++oh)
+      for (int ow = ow_lo; ow <= ow_hi; ++ow)
+        if (window_argmax<K>(plane, g, oh, ow) == me) acc += dplane[oh * g.pW + ow];
+  }
+  dx[idx] = acc;
+}
+
+// Two-pass backward for overlapping windows: the argmax of every window is computed once into
+// scratch (one thread per window), then every input element compares its own flat index with
+// the stored argmax of the at most NW x NW windows over it.
+template <int K>
+__global__ __launch_bounds__(kThreads) void pool_argmax_kernel(const float *__restrict__ x, int *__restrict__ arg,
+                                                               PoolGeo g, int64_t total) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx >= total) return;
+  int ow, oh;
+  int64_t nc;
+  split3(idx, total, g.div_pw, g.div_ph, nc, oh, ow);
+  arg[idx] = window_argmax<K>(x + nc * g.H * g.W, g, oh, ow);
+}
+
+template <int NW>
+__global__ __launch_bounds__(kThreads) void pool_bwd_from_argmax_kernel(const int *__restrict__ arg,
+                                                                        const float *__restrict__ dy,
+                                                                        float *__restrict__ dx, PoolGeo g,
+                                                                        int64_t total) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx >= total) return;
+  int w, h;
+  int64_t nc;
+  split3(idx, total, g.div_w, g.div_h, nc, h, w);
+  const int64_t wbase = nc * g.pH * g.pW;
+  const int th = h + g.pad - g.kH + g.stride, tw = w + g.pad - g.kW + g.stride;
+  const int oh_lo = th > 0 ? static_cast<int>(g.div_stride.div(th)) : 0;
+  const int oh_hi = min(g.pH - 1, static_cast<int>(g.div_stride.div(h + g.pad)));
+  const int ow_lo = tw > 0 ? static_cast<int>(g.div_stride.div(tw)) : 0;
+  const int ow_hi = min(g.pW - 1, static_cast<int>(g.div_stride.div(w + g.pad)));
+  const int me = h * g.W + w;
+  float acc = 0.f;
+#pragma unroll
+  for (int a = 0; a < NW; ++a) {
+#pragma unroll
+    for (int b = 0; b < NW; ++b) {
+      const int oh = min(oh_lo + a, oh_hi), ow = min(ow_lo + b, ow_hi);
+      const bool live = oh_lo + a <= oh_hi && ow_lo + b <= ow_hi;
+      const int64_t wi = wbase + oh * g.pW + ow;
+      const int am = arg[wi];
+      const float gy = dy[wi];
+      if (live && am == me) acc += gy;
+    }
+  }
   dx[idx] = acc;
 }
 
@@ -148,6 +265,11 @@ int check_geo(const char *who, const DLArray *x, const DLArray *y, int64_t kH, i
   g.kW = static_cast<int>(kW);
   g.pad = static_cast<int>(pad);
   g.stride = static_cast<int>(stride);
+  g.div_pw = FastDiv(static_cast<uint32_t>(g.pW > 0 ? g.pW : 1));
+  g.div_ph = FastDiv(static_cast<uint32_t>(g.pH > 0 ? g.pH : 1));
+  g.div_w = FastDiv(static_cast<uint32_t>(g.W > 0 ? g.W : 1));
+  g.div_h = FastDiv(static_cast<uint32_t>(g.H > 0 ? g.H : 1));
+  g.div_stride = FastDiv(static_cast<uint32_t>(g.stride));
   TS_REQUIRE(g.H + 2 * g.pad >= g.kH && g.W + 2 * g.pad >= g.kW, "%s: kernel larger than the padded image", who);
   const int eh = (g.H + 2 * g.pad - g.kH) / g.stride + 1, ew = (g.W + 2 * g.pad - g.kW) / g.stride + 1;
   TS_REQUIRE(g.pH == eh && g.pW == ew, "%s: output is %dx%d, expected %dx%d", who, g.pH, g.pW, eh, ew);
@@ -174,9 +296,16 @@ int pool_forward(const char *who, const DLArray *x, DLArray *y, int64_t kH, int6
                          g.W / 4, g.pH, total);
     } else {
       const int64_t total = numel(y);
-      hipLaunchKernelGGL(pool_fwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
-                         dim3(kThreads), 0, s, static_cast<const float *>(x->data), static_cast<float *>(y->data), g,
-                         total);
+      const dim3 grid(static_cast<unsigned>((total + kThreads - 1) / kThreads)), block(kThreads);
+      const float *xp = static_cast<const float *>(x->data);
+      float *yp = static_cast<float *>(y->data);
+      const int k = g.kH == g.kW ? g.kH : 0;
+      if (k == 2)
+        hipLaunchKernelGGL(pool_fwd_kernel<2>, grid, block, 0, s, xp, yp, g, total);
+      else if (k == 3)
+        hipLaunchKernelGGL(pool_fwd_kernel<3>, grid, block, 0, s, xp, yp, g, total);
+      else
+        hipLaunchKernelGGL(pool_fwd_kernel<0>, grid, block, 0, s, xp, yp, g, total);
     }
   }
   return ps.finish();
@@ -199,9 +328,32 @@ int pool_backward(const char *who, const DLArray *x, const DLArray *dy, DLArray 
                          static_cast<const f32x2 *>(dy->data), static_cast<f32x4 *>(dx->data), g.W / 4, total);
     } else {
       const int64_t total = numel(dx);
-      hipLaunchKernelGGL(pool_bwd_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
-                         dim3(kThreads), 0, s, static_cast<const float *>(x->data),
-                         static_cast<const float *>(dy->data), static_cast<float *>(dx->data), g, total);
+      const dim3 grid(static_cast<unsigned>((total + kThreads - 1) / kThreads)), block(kThreads);
+      const float *xp = static_cast<const float *>(x->data), *dyp = static_cast<const float *>(dy->data);
+      float *dxp = static_cast<float *>(dx->data);
+      const int k = g.kH == g.kW ? g.kH : 0;
+      const int nw = k > 0 ? (k + g.stride - 1) / g.stride : 0;   // windows per axis over one element
+      const int64_t windows = numel(dy);
+      int *arg = nullptr;
+      if ((k == 2 || k == 3) && (nw == 2 || nw == 3) && windows > 0) {
+        arg = static_cast<int *>(scratch_get(s, 5, static_cast<size_t>(windows) * sizeof(int)));
+        TS_REQUIRE(arg, "%s: out of device memory for %lld window indices", who, (long long)windows);
+        if (p) p->workspace_memory = mib(windows);
+        const dim3 wgrid(static_cast<unsigned>((windows + kThreads - 1) / kThreads));
+        if (k == 2)
+          hipLaunchKernelGGL(pool_argmax_kernel<2>, wgrid, block, 0, s, xp, arg, g, windows);
+        else
+          hipLaunchKernelGGL(pool_argmax_kernel<3>, wgrid, block, 0, s, xp, arg, g, windows);
+        if (nw == 2)
+          hipLaunchKernelGGL(pool_bwd_from_argmax_kernel<2>, grid, block, 0, s, arg, dyp, dxp, g, total);
+        else
+          hipLaunchKernelGGL(pool_bwd_from_argmax_kernel<3>, grid, block, 0, s, arg, dyp, dxp, g, total);
+      } else if (k == 3 && nw == 1)
+        hipLaunchKernelGGL((pool_bwd_kernel<3, 1>), grid, block, 0, s, xp, dyp, dxp, g, total);
+      else if (k == 2 && nw == 1)
+        hipLaunchKernelGGL((pool_bwd_kernel<2, 1>), grid, block, 0, s, xp, dyp, dxp, g, total);
+      else
+        hipLaunchKernelGGL((pool_bwd_kernel<0, 0>), grid, block, 0, s, xp, dyp, dxp, g, total);
     }
   }
   return ps.finish();

@@ -2,9 +2,9 @@
 //
 // The axes of the input are split into kept and reduced ones (each list collapsed,
 // nd_index.h).  Two kernels cover every pattern:
-//   - columns: the innermost input axis is kept.  A thread owns one output element (or one
-//     16-byte word of them) and walks the reduced index space; neighbouring lanes read
-//     neighbouring addresses on every step.
+//   - columns: the innermost input axis is kept.  A block owns 64 output elements (or 64
+//     16-byte words of them) and four row-lanes share the walk over the reduced index space;
+//     neighbouring lanes read neighbouring addresses on every step.
 //   - rows: the innermost input axis is reduced.  A group of 64 or 256 threads owns one
 //     output element, strides over the reduced index space (16-byte words along the
 //     innermost axis where possible) and finishes with a shuffle / LDS reduction.
@@ -59,54 +59,72 @@ __device__ __forceinline__ int64_t reduced_offset(const ReduceGeo &g, uint32_t r
   return off;
 }
 
-// VEC outputs per thread; dst[output][slice]
+// A block is 64 output units (VEC outputs each) wide and 4 row-lanes deep: row-lane ry adds
+// the reduced indices r0 + ry, r0 + ry + 4, ... of the block's slice; the four partial sums
+// are combined through LDS in a fixed order.  dst[slice][output].
+constexpr int kColsWide = 64, kRowLanes = kThreads / kColsWide;
 template <int VEC>
 __global__ __launch_bounds__(kThreads) void reduce_cols_kernel(const float *__restrict__ in, float *__restrict__ dst,
                                                                ReduceGeo g) {
-  const uint32_t o = blockIdx.x * kThreads + threadIdx.x;
-  if (o >= g.outputs) return;
-  const float *p = in + kept_offset(g, o, VEC);
-  const uint32_t r0 = blockIdx.y * g.chunk, r1 = min(r0 + g.chunk, g.rtotal);
+  __shared__ float sm[kRowLanes - 1][kColsWide][VEC];
+  const int cx = threadIdx.x % kColsWide, ry = threadIdx.x / kColsWide;
+  const uint32_t o = blockIdx.x * kColsWide + cx;
+  const bool live = o < g.outputs;
   float acc[VEC] = {};
-  if (g.nr == 1) {
-    const int64_t st = g.rstride[0];
-    const float *q = p + static_cast<int64_t>(r0) * st;
-    for (uint32_t r = r0; r < r1; ++r, q += st) {
-      if (VEC == 4) {
-        const f32x4 v = *reinterpret_cast<const f32x4 *>(q);
-        acc[0] += v.x;
-        acc[1 % VEC] += v.y;
-        acc[2 % VEC] += v.z;
-        acc[3 % VEC] += v.w;
-      } else {
-        acc[0] += *q;
+  if (live) {
+    const float *p = in + kept_offset(g, o, VEC);
+    const uint32_t r0 = blockIdx.y * g.chunk, r1 = min(r0 + g.chunk, g.rtotal);
+    if (g.nr == 1) {
+      const int64_t st = g.rstride[0] * kRowLanes;
+      const float *q = p + static_cast<int64_t>(r0 + ry) * g.rstride[0];
+#pragma unroll 8
+      for (uint32_t r = r0 + ry; r < r1; r += kRowLanes, q += st) {
+        if (VEC == 4) {
+          const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(q));
+          acc[0] += v.x;
+          acc[1 % VEC] += v.y;
+          acc[2 % VEC] += v.z;
+          acc[3 % VEC] += v.w;
+        } else {
+          acc[0] += __builtin_nontemporal_load(q);
+        }
       }
-    }
-  } else {
-    for (uint32_t r = r0; r < r1; ++r) {
-      const float *q = p + reduced_offset(g, r, 1);
-      if (VEC == 4) {
-        const f32x4 v = *reinterpret_cast<const f32x4 *>(q);
-        acc[0] += v.x;
-        acc[1 % VEC] += v.y;
-        acc[2 % VEC] += v.z;
-        acc[3 % VEC] += v.w;
-      } else {
-        acc[0] += *q;
+    } else {
+#pragma unroll 4
+      for (uint32_t r = r0 + ry; r < r1; r += kRowLanes) {
+        const float *q = p + reduced_offset(g, r, 1);
+        if (VEC == 4) {
+          const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(q));
+          acc[0] += v.x;
+          acc[1 % VEC] += v.y;
+          acc[2 % VEC] += v.z;
+          acc[3 % VEC] += v.w;
+        } else {
+          acc[0] += __builtin_nontemporal_load(q);
+        }
       }
     }
   }
-  if (gridDim.y == 1) {
-    float *d = dst + static_cast<int64_t>(o) * VEC;
+  if (ry > 0) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) sm[ry - 1][cx][j] = acc[j];
+  }
+  __syncthreads();
+  if (ry == 0 && live) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      float t = acc[j];
+#pragma unroll
+      for (int l = 0; l < kRowLanes - 1; ++l) t += sm[l][cx][j];
+      acc[j] = t;
+    }
+    float *d = dst + (static_cast<int64_t>(blockIdx.y) * g.outputs + o) * VEC;
     if (VEC == 4) {
       const f32x4 r = {acc[0], acc[1 % VEC], acc[2 % VEC], acc[3 % VEC]};
       *reinterpret_cast<f32x4 *>(d) = r;
     } else {
       d[0] = acc[0];
     }
-  } else {
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) dst[(static_cast<int64_t>(o) * VEC + j) * gridDim.y + blockIdx.y] = acc[j];
   }
 }
 
@@ -138,21 +156,28 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_kernel(const float *__re
   } else {
     acc = block_sum<float, kThreads / kWave>(acc, smem);
   }
-  if (live && lane == 0) dst[static_cast<int64_t>(o) * gridDim.y + blockIdx.y] = acc;
+  if (live && lane == 0) dst[static_cast<int64_t>(blockIdx.y) * g.outputs + o] = acc;
 }
 
-// out[o] = sum of part[o][0..slices), G threads per output; the order of additions is fixed
-template <int G>
+// out[o] = sum over slices of part[slice][o]: 64 outputs x 4 slice-lanes per block, slice-lane l
+// adds slices l, l + 4, ...; the four sums are combined through LDS in a fixed order.
 __global__ __launch_bounds__(kThreads) void fold_slices_kernel(const float *__restrict__ part, float *__restrict__ out,
                                                                uint32_t outputs, int slices) {
-  const uint32_t o = (blockIdx.x * kThreads + threadIdx.x) / G;
-  if (o >= outputs) return;            // whole groups leave together
-  const int lane = threadIdx.x % G;
-  const float *p = part + static_cast<int64_t>(o) * slices;
+  __shared__ float sm[kRowLanes - 1][kColsWide];
+  const int cx = threadIdx.x % kColsWide, ry = threadIdx.x / kColsWide;
+  const uint32_t o = blockIdx.x * kColsWide + cx;
   float acc = 0.f;
-  for (int s = lane; s < slices; s += G) acc += p[s];
-  if (G == kWave) acc = wave_sum(acc);
-  if (lane == 0) out[o] = acc;
+  if (o < outputs) {
+#pragma unroll 8
+    for (int s = ry; s < slices; s += kRowLanes) acc += part[static_cast<int64_t>(s) * outputs + o];
+  }
+  if (ry > 0) sm[ry - 1][cx] = acc;
+  __syncthreads();
+  if (ry == 0 && o < outputs) {
+#pragma unroll
+    for (int l = 0; l < kRowLanes - 1; ++l) acc += sm[l][cx];
+    out[o] = acc;
+  }
 }
 
 __global__ __launch_bounds__(kThreads) void copy_kernel(const float *__restrict__ in, float *__restrict__ out, int64_t n) {
@@ -174,7 +199,7 @@ int reduce_sum(const char *who, const float *in, float *out, Axis *kept, int nk,
   if (outputs == 0) return 0;
   TS_REQUIRE(outputs < (1ll << 31) && rtotal < (1ll << 31), "%s: more than 2^31 kept or reduced elements", who);
   if (rtotal == 0) {   // empty sums
-    hipLaunchKernelGGL(fold_slices_kernel<1>, dim3(static_cast<unsigned>((outputs + kThreads - 1) / kThreads)),
+    hipLaunchKernelGGL(fold_slices_kernel, dim3(static_cast<unsigned>((outputs + kColsWide - 1) / kColsWide)),
                        dim3(kThreads), 0, s, in, out, static_cast<uint32_t>(outputs), 0);
     return 0;
   }
@@ -213,13 +238,22 @@ int reduce_sum(const char *who, const float *in, float *out, Axis *kept, int nk,
   g.rtotal = static_cast<uint32_t>(r_units);
   int group = 1;
   if (rows) group = r_units >= 2048 ? kThreads : kWave;
-  // slices: enough threads for the chip, at least `min_chunk` reduced indices per thread group
-  const int64_t min_chunk = rows ? static_cast<int64_t>(group) * 8 : 32;
-  int64_t slices = (kTargetThreads + out_units * group - 1) / (out_units * group);
-  slices = std::min<int64_t>(slices, (r_units + min_chunk - 1) / min_chunk);
-  slices = std::max<int64_t>(1, std::min<int64_t>(slices, 1024));
-  int64_t chunk = (r_units + slices - 1) / slices;
-  if (rows) chunk = (chunk + group - 1) / group * group;
+  // slices: enough blocks for the chip while every thread still has a few loads to overlap
+  int64_t slices, chunk;
+  if (rows) {
+    const int64_t min_chunk = static_cast<int64_t>(group) * 8;
+    slices = (kTargetThreads + out_units * group - 1) / (out_units * group);
+    slices = std::min<int64_t>(slices, (r_units + min_chunk - 1) / min_chunk);
+    slices = std::max<int64_t>(1, std::min<int64_t>(slices, 1024));
+    chunk = (r_units + slices - 1) / slices;
+    chunk = (chunk + group - 1) / group * group;
+  } else {
+    const int64_t out_blocks = (out_units + kColsWide - 1) / kColsWide, min_chunk = 8 * kRowLanes;
+    slices = (kTargetThreads / kThreads + out_blocks - 1) / out_blocks;
+    slices = std::min<int64_t>(slices, (r_units + min_chunk - 1) / min_chunk);
+    slices = std::max<int64_t>(1, std::min<int64_t>(slices, 1024));
+    chunk = (r_units + slices - 1) / slices;
+  }
   slices = (r_units + chunk - 1) / chunk;
   g.chunk = static_cast<uint32_t>(chunk);
   float *dst = out;
@@ -242,18 +276,14 @@ int reduce_sum(const char *who, const float *in, float *out, Axis *kept, int nk,
         hipLaunchKernelGGL((reduce_rows_kernel<kThreads, 1>), grid, dim3(kThreads), 0, s, in, dst, g);
     }
   } else {
-    const dim3 grid(static_cast<unsigned>((out_units + kThreads - 1) / kThreads), static_cast<unsigned>(slices));
+    const dim3 grid(static_cast<unsigned>((out_units + kColsWide - 1) / kColsWide), static_cast<unsigned>(slices));
     if (vec)
       hipLaunchKernelGGL(reduce_cols_kernel<4>, grid, dim3(kThreads), 0, s, in, dst, g);
     else
       hipLaunchKernelGGL(reduce_cols_kernel<1>, grid, dim3(kThreads), 0, s, in, dst, g);
   }
-  if (slices > 16)
-    hipLaunchKernelGGL(fold_slices_kernel<kWave>,
-                       dim3(static_cast<unsigned>((outputs * kWave + kThreads - 1) / kThreads)), dim3(kThreads), 0, s, dst,
-                       out, static_cast<uint32_t>(outputs), static_cast<int>(slices));
-  else if (slices > 1)
-    hipLaunchKernelGGL(fold_slices_kernel<1>, dim3(static_cast<unsigned>((outputs + kThreads - 1) / kThreads)),
+  if (slices > 1)
+    hipLaunchKernelGGL(fold_slices_kernel, dim3(static_cast<unsigned>((outputs + kColsWide - 1) / kColsWide)),
                        dim3(kThreads), 0, s, dst, out, static_cast<uint32_t>(outputs), static_cast<int>(slices));
   return 0;
 }
