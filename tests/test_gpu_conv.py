@@ -31,6 +31,11 @@ CASES = [
     # block ranges cut tiles in two and the halves meet through float atomics
     (25, 16, 64, 64, 128, 3, 3, 1, 1, 1),  # 800 tiles of 128x128 (forward)
     (13, 16, 128, 128, 16, 3, 3, 1, 1, 1), # 832 tiles of 64x256 (forward and backward-data)
+    # at most 32 filter columns (C*kH*kW): backward-filter takes the few-columns kernel
+    (4, 3, 64, 64, 64, 3, 3, 1, 1, 1),     # several K slices, folded
+    (3, 1, 19, 23, 100, 5, 5, 2, 2, 1),    # 25 columns, two row tiles, ragged K (oH*oW odd)
+    (2, 2, 20, 20, 33, 4, 4, 1, 1, 2),     # exactly 32 columns, stride 2
+    (1, 3, 5, 5, 7, 3, 3, 1, 1, 1),        # K = 25: one partial step
 ]
 
 

@@ -1158,6 +1158,236 @@ int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *d
   return 0;
 }
 
+// ------------------------------------------------------------------ bwd-filter, few columns
+// dw[O, N] with N = C*kH*kW <= 32 (the first layer of an image network: 3 input channels).  The
+// 64x64-per-wave tiling would spend 7/8 of its MFMAs on padding, and the reduction
+// (K = imgs*oH*oW, hundreds of thousands) is what has to be streamed: dy is read exactly
+// once.  A block owns 64 rows x 32 columns and a slice of K; steps are 32 k wide; the four
+// waves split every step's k four ways (8 k each = 4 MFMAs per 32x32 block), so the whole
+// block advances one step per barrier, and their accumulators are added through LDS at the
+// end.  Slice sums go to scratch and are folded in slice order.
+constexpr int NK = 32;                 // k per step
+constexpr int kNStride = NK + 4;       // LDS row stride (floats), keeps 16-byte alignment
+constexpr int kNarrowCols = 32;
+struct NarrowWgradParams {
+  const float *dy, *x;
+  const Tap *taps;
+  FastDiv plane, width;    // oH*oW, oW
+  int64_t img_stride;      // C*H*W
+  int O, N, K, H, W, ph, pw, s, steps_per_slice;
+  bool vec;                // oH*oW % 4 == 0 and dy 16-byte aligned
+};
+
+__global__ __launch_bounds__(kThreads) void conv_wgrad_narrow_kernel(NarrowWgradParams P, float *__restrict__ part) {
+  constexpr int kAFloats = 64 * kNStride, kBFloats = kNarrowCols * kNStride;
+  __shared__ __attribute__((aligned(16))) float lds_all[2 * kAFloats + 2 * kBFloats];
+  float(*lds_a)[kAFloats] = reinterpret_cast<float(*)[kAFloats]>(lds_all);
+  float(*lds_b)[kBFloats] = reinterpret_cast<float(*)[kBFloats]>(lds_all + 2 * kAFloats);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m0 = blockIdx.y * 64;
+  const int kbegin = blockIdx.x * P.steps_per_slice * NK;
+  const int kend = min(P.K, kbegin + P.steps_per_slice * NK);
+
+  // A (dy rows): thread -> rows tid/8 and tid/8 + 32, k quad tid%8
+  const int arow = tid >> 3, akq = tid & 7;
+  // B (gathered x): thread -> k = tid%32, columns tid/32 + 8*i
+  const int bk = tid & 31, bcol = tid >> 5;
+  int toff[4];
+  short tkh[4], tkw[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int j = bcol + 8 * i;
+    if (j < P.N) {
+      const Tap t = P.taps[j];
+      toff[i] = t.off;
+      tkh[i] = t.kh;
+      tkw[i] = t.kw;
+    } else {
+      toff[i] = 0;
+      tkh[i] = -20000;   // fails the range test for any row
+      tkw[i] = 0;
+    }
+  }
+  float4 ra[2];
+  float rb[4];
+  auto dy_one = [&](int k, int row) -> float {
+    if (k >= kend) return 0.f;
+    const uint32_t img = P.plane.div(k);
+    const uint32_t px = k - img * P.plane.d;
+    return P.dy[(static_cast<int64_t>(img) * P.O + row) * P.plane.d + px];
+  };
+  auto load = [&](int k0) {
+    {
+      const int k = k0 + 4 * akq;
+      const uint32_t img = P.plane.div(k);
+      const uint32_t px = k - img * P.plane.d;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int row = m0 + arow + 32 * h;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (row < P.O) {
+          if (P.vec && k + 3 < kend) {
+            v = *reinterpret_cast<const float4 *>(P.dy + (static_cast<int64_t>(img) * P.O + row) * P.plane.d + px);
+          } else {
+            v.x = dy_one(k, row);
+            v.y = dy_one(k + 1, row);
+            v.z = dy_one(k + 2, row);
+            v.w = dy_one(k + 3, row);
+          }
+        }
+        ra[h] = v;
+      }
+    }
+    {
+      const int k = k0 + bk;
+      const bool k_ok = k < kend;
+      const uint32_t kk = k_ok ? k : 0;
+      const uint32_t img = P.plane.div(kk);
+      const uint32_t px = kk - img * P.plane.d;
+      const uint32_t oh = P.width.div(px);
+      const uint32_t ow = px - oh * P.width.d;
+      const int r0 = static_cast<int>(oh) * P.s - P.ph, c0 = static_cast<int>(ow) * P.s - P.pw;
+      const float *base = P.x + static_cast<int64_t>(img) * P.img_stride + static_cast<int64_t>(r0) * P.W + c0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int rr = r0 + tkh[i], cc = c0 + tkw[i];
+        float v = 0.f;
+        if (k_ok && static_cast<unsigned>(rr) < static_cast<unsigned>(P.H) &&
+            static_cast<unsigned>(cc) < static_cast<unsigned>(P.W))
+          v = base[toff[i]];
+        rb[i] = v;
+      }
+    }
+  };
+  auto store = [&](int stage) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      *reinterpret_cast<float4 *>(&lds_a[stage][(arow + 32 * h) * kNStride + 4 * akq]) = ra[h];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds_b[stage][(bcol + 8 * i) * kNStride + bk] = rb[i];
+  };
+
+  acc16 acc[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+
+  if (kbegin < kend) {
+    load(kbegin);
+    store(0);
+  }
+  __syncthreads();
+  int stage = 0;
+  for (int k0 = kbegin; k0 < kend; k0 += NK) {
+    const bool more = k0 + NK < kend;
+    if (more) load(k0 + NK);
+    // this wave's 8 k of the step: lanes 0-31 supply k = 8*wave + e, lanes 32-63 k = 8*wave + 4 + e
+    const int kofs = 8 * wave + 4 * (lane >> 5);
+    const float4 fb = *reinterpret_cast<const float4 *>(&lds_b[stage][(lane & 31) * kNStride + kofs]);
+    const float4 fa0 = *reinterpret_cast<const float4 *>(&lds_a[stage][(lane & 31) * kNStride + kofs]);
+    const float4 fa1 = *reinterpret_cast<const float4 *>(&lds_a[stage][(32 + (lane & 31)) * kNStride + kofs]);
+    acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa0.x, fb.x, acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa1.x, fb.x, acc[1], 0, 0, 0);
+    acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa0.y, fb.y, acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa1.y, fb.y, acc[1], 0, 0, 0);
+    acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa0.z, fb.z, acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa1.z, fb.z, acc[1], 0, 0, 0);
+    acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa0.w, fb.w, acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa1.w, fb.w, acc[1], 0, 0, 0);
+    if (more) store(stage ^ 1);
+    __syncthreads();
+    stage ^= 1;
+  }
+
+  // add the four waves' accumulators: waves 1-3 park theirs in LDS (the staging buffers are
+  // free now: the loop ended with a barrier), wave 0 adds them to its own in a fixed order and
+  // writes the block's 64 x N slice sum.  red[wave - 1][row][col], row stride 33.
+  float *red = lds_all;
+  static_assert(3 * 64 * 33 <= 2 * kAFloats + 2 * kBFloats, "reduction buffer fits in the staging LDS");
+  if (wave > 0) {
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = 32 * mi + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+        red[((wave - 1) * 64 + row) * 33 + (lane & 31)] = acc[mi][e];
+      }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    float *o = part + static_cast<int64_t>(blockIdx.x) * P.O * P.N;
+    const int col = lane & 31;
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = 32 * mi + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+        const float v = ((acc[mi][e] + red[row * 33 + col]) + red[(64 + row) * 33 + col]) + red[(128 + row) * 33 + col];
+        if (m0 + row < P.O && col < P.N) o[static_cast<int64_t>(m0 + row) * P.N + col] = v;
+      }
+  }
+}
+
+// out[i] = sum over slices of part[slice][i]: 64 outputs x 4 slice-lanes per block, slice-lane l
+// adds slices l, l + 4, ... and the four sums are combined through LDS in a fixed order.
+__global__ __launch_bounds__(kThreads) void fold_many_slices_kernel(const float *__restrict__ part,
+                                                                    float *__restrict__ out, int n, int slices) {
+  __shared__ float sm[3][64];
+  const int cx = threadIdx.x & 63, ry = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + cx;
+  float acc = 0.f;
+  if (i < n) {
+#pragma unroll 8
+    for (int s = ry; s < slices; s += 4) acc += part[static_cast<int64_t>(s) * n + i];
+  }
+  if (ry > 0) sm[ry - 1][cx] = acc;
+  __syncthreads();
+  if (ry == 0 && i < n) out[i] = ((acc + sm[0][cx]) + sm[1][cx]) + sm[2][cx];
+}
+
+inline bool wgrad_narrow_ok(const ConvGeo &g) {
+  return g.C * g.kH * g.kW <= kNarrowCols && static_cast<int64_t>(g.imgs) * g.oH * g.oW < (1ll << 31) - 64;
+}
+
+int launch_wgrad_narrow(const ConvGeo &g, const float *x, const float *dy, float *dw, hipStream_t st,
+                        int64_t *ws_elems) {
+  NarrowWgradParams P;
+  P.dy = dy;
+  P.x = x;
+  P.taps = tap_table(g.C, g.kH, g.kW, g.W, g.H * g.W, +1);
+  TS_REQUIRE(P.taps, "conv bwd-filter: could not build the tap table");
+  P.plane = FastDiv(g.oH * g.oW);
+  P.width = FastDiv(g.oW);
+  P.img_stride = static_cast<int64_t>(g.C) * g.H * g.W;
+  P.O = g.O;
+  P.N = g.C * g.kH * g.kW;
+  P.K = g.imgs * g.oH * g.oW;
+  P.H = g.H;
+  P.W = g.W;
+  P.ph = g.ph;
+  P.pw = g.pw;
+  P.s = g.s;
+  P.vec = (g.oH * g.oW) % 4 == 0 && aligned16(dy);
+  const int tm = (g.O + 63) / 64;
+  const int steps = (P.K + NK - 1) / NK;
+  // about four blocks per CU, at least 8 steps each
+  int slices = std::max(1, std::min(1024 / tm, steps / 8));
+  P.steps_per_slice = (steps + slices - 1) / slices;
+  slices = (steps + P.steps_per_slice - 1) / P.steps_per_slice;
+  const int mn = g.O * P.N;
+  float *part = dw;
+  if (slices > 1) {
+    part = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(slices) * mn * 4));
+    TS_REQUIRE(part, "conv bwd-filter: no scratch memory for split-K");
+    *ws_elems = static_cast<int64_t>(slices) * mn;
+  }
+  hipLaunchKernelGGL(conv_wgrad_narrow_kernel, dim3(slices, tm), dim3(kThreads), 0, st, P, part);
+  if (slices > 1)
+    hipLaunchKernelGGL(fold_many_slices_kernel, dim3((mn + 63) / 64), dim3(kThreads), 0, st, part, dw, mn, slices);
+  return 0;
+}
+
 inline bool wgrad_tap_ok(const ConvGeo &g) {
   const int64_t bytes_x = static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4, bytes_dy = static_cast<int64_t>(g.imgs) * g.O * g.H * g.W * 4;
   return g.s == 1 && g.oH == g.H && g.oW == g.W && (g.H * g.W) % BK == 0 && g.C % BK == 0 &&
@@ -1246,7 +1476,9 @@ int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArra
   ProfileScope ps(p, st, numel(x) + numel(dy), numel(dw), 0);
   int rc = 0;
   if (numel(dw) > 0) {
-    if (wgrad_tap_ok(g)) {
+    if (wgrad_narrow_ok(g)) {
+      rc = launch_wgrad_narrow(g, cf(x), cf(dy), mf(dw), st, &ws);
+    } else if (wgrad_tap_ok(g)) {
       if (g.O <= 64)
         rc = launch_wgrad_tap<64, 256, 1, 4>(g, cf(x), cf(dy), mf(dw), st, &ws);
       else
