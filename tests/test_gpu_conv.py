@@ -27,10 +27,14 @@ CASES = [
     (2, 16, 15, 15, 24, 3, 3, 1, 1, 2),    # stride 2, odd output 8x8
     (2, 8, 7, 7, 40, 1, 1, 0, 0, 1),       # oH*oW = 49: not a multiple of 4
     (2, 6, 12, 12, 130, 5, 5, 2, 2, 1),
-    # more tiles than resident block slots: forward / backward-data take the stream-K path, where
-    # block ranges cut tiles in two and the halves meet through float atomics
+    # forward / backward-data cut the k-steps of all tiles into equal ranges, one per resident
+    # block; the pieces of a cut tile are assembled by a second kernel
     (25, 16, 64, 64, 128, 3, 3, 1, 1, 1),  # 800 tiles of 128x128 (forward)
     (13, 16, 128, 128, 16, 3, 3, 1, 1, 1), # 832 tiles of 64x256 (forward and backward-data)
+    # fewer tiles than resident blocks: every tile is cut into many pieces
+    (8, 512, 14, 14, 256, 3, 3, 1, 1, 1),  # 26 tiles of 128x128, 288 k-steps each
+    (8, 512, 28, 28, 64, 3, 3, 1, 1, 1),   # forward on 64x256 tiles
+    (8, 64, 28, 28, 512, 3, 3, 1, 1, 1),   # backward-data on 64x256 tiles
     # at most 32 filter columns (C*kH*kW): backward-filter takes the few-columns kernel
     (4, 3, 64, 64, 64, 3, 3, 1, 1, 1),     # several K slices, folded
     (3, 1, 19, 23, 100, 5, 5, 2, 2, 1),    # 25 columns, two row tiles, ragged K (oH*oW odd)

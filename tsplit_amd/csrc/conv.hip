@@ -283,14 +283,18 @@ constexpr unsigned kOobOffset = 0x80000000u;    // beyond any tensor this path a
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // Work distribution ("stream-K"): the unit of work is one 16-wide k-step of one tile, numbered
-// tile-major.  Every block takes a contiguous range of `iters_per_block` units.  With
-// iters_per_block = k-steps per tile a block is exactly one tile (used when there are fewer
-// tiles than resident block slots).  Otherwise the grid is one full wave of resident blocks and
-// ranges cut through tiles, so that 3.06 tiles per slot cost 3.06 tile-times, not 4: a tile
-// computed by one block is stored, a tile cut in two is accumulated with float atomics into an
-// output that a small kernel zeroed before.  A range is at least one tile long, so a tile has
-// at most two contributors and 0 + a + b does not depend on their order: results stay
-// run-to-run deterministic (they do depend on where the cuts fall, i.e. on the problem shape).
+// tile-major.  Every block takes a contiguous range of `iters_per_block` units and the grid is
+// one full wave of resident blocks, so that 3.06 tiles per slot cost 3.06 tile-times, not 4,
+// and 392 tiles on 768 slots keep every slot busy.  A tile computed by one block is stored
+// directly.  Cut tiles are completed in one of two ways, both independent of scheduling:
+//   - ranges at least one tile long (more tiles than slots): a tile has at most two
+//     contributors, which add with float atomics into an output that a small kernel zeroed
+//     before; 0 + a + b does not depend on the order;
+//   - shorter ranges (fewer tiles than slots): every block parks the accumulators of its (at
+//     most two) partial pieces in scratch -- slot 0 for a piece that is the first segment of
+//     its range, slot 1 for a partial last segment -- and a second kernel adds the pieces of
+//     each tile in ascending block order and writes the tile.
+// Results do depend on where the cuts fall, i.e. on the problem shape.
 struct StreamK {
   int ksteps;            // k-steps per tile
   int total;             // tiles * ksteps
@@ -299,7 +303,8 @@ struct StreamK {
 };
 
 template <int BM, int BN, int WM, int WN, bool BWD_DATA>
-__global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, float *__restrict__ out, StreamK sk) {
+__global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, float *__restrict__ out,
+                                                            float *__restrict__ pieces, StreamK sk) {
   static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
   using ALds = MnMajorLds<BM>;
   using BLds = MnMajorLds<BN>;
@@ -313,7 +318,8 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
   // consecutive workgroup ids go to different XCDs: transpose so that an XCD owns a contiguous
   // eighth of the work (neighbouring tiles share gathered activations in its L2)
   const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  int it = logical * sk.iters_per_block;
+  const int it_begin = logical * sk.iters_per_block;
+  int it = it_begin;
   const int it_end = min(sk.total, it + sk.iters_per_block);
 
   // uniform bias so that every per-thread offset is non-negative and every scalar offset too
@@ -443,26 +449,92 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
     // epilogue: accumulator register e of a 32x32 block holds row 8*(e/4) + 4*(lane/32) + e%4, column
     // lane%32; out[img][m][p] with column n = img*plane + p
     const bool whole = ks0 == 0 && ks1 == sk.ksteps;
+    if (whole) {
 #pragma unroll
-    for (int ni = 0; ni < 2; ++ni) {
-      const int n = n0 + wn0 + 32 * ni + (lane & 31);
-      if (n >= P.N) continue;
-      const uint32_t img = P.plane.div(n);
-      const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
+      for (int ni = 0; ni < 2; ++ni) {
+        const int n = n0 + wn0 + 32 * ni + (lane & 31);
+        if (n >= P.N) continue;
+        const uint32_t img = P.plane.div(n);
+        const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi) {
-        const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
+        for (int mi = 0; mi < 2; ++mi) {
+          const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int m = mb + 8 * (e >> 2) + (e & 3);
-          if (m < P.M) {
-            float *dst = out + static_cast<int64_t>(m) * P.out_plane + coff;
-            if (whole)
-              *dst = acc[mi][ni][e];
-            else
-              unsafeAtomicAdd(dst, acc[mi][ni][e]);
+          for (int e = 0; e < 16; ++e) {
+            const int m = mb + 8 * (e >> 2) + (e & 3);
+            if (m < P.M) out[static_cast<int64_t>(m) * P.out_plane + coff] = acc[mi][ni][e];
           }
         }
+      }
+    } else if (pieces == nullptr) {
+      // ranges are at least one tile long: a cut tile has exactly two contributors, which add into
+      // an output zeroed beforehand (0 + a + b does not depend on the order)
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) {
+        const int n = n0 + wn0 + 32 * ni + (lane & 31);
+        if (n >= P.N) continue;
+        const uint32_t img = P.plane.div(n);
+        const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) {
+          const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int m = mb + 8 * (e >> 2) + (e & 3);
+            if (m < P.M) unsafeAtomicAdd(out + static_cast<int64_t>(m) * P.out_plane + coff, acc[mi][ni][e]);
+          }
+        }
+      }
+    } else {
+      // a piece of a tile cut more than once: registers go to scratch as they are, [register][thread]
+      const int slot = (it - (ks1 - ks0)) == it_begin ? 0 : 1;
+      float *pc = pieces + (static_cast<int64_t>(logical) * 2 + slot) * (BM * BN) + tid;
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) pc[((mi * 2 + ni) * 16 + e) * kThreads] = acc[mi][ni][e];
+    }
+  }
+}
+
+// Assembles the tiles that block ranges cut into pieces: block = tile; adds the pieces in
+// ascending block order and stores the tile.  Thread and register layout are those of
+// conv_tap_kernel's epilogue.
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvParams P, float *__restrict__ out,
+                                                                     const float *__restrict__ pieces, StreamK sk) {
+  const int tile = blockIdx.x;
+  const int first = tile * sk.ksteps, last = first + sk.ksteps - 1;
+  const int b0 = first / sk.iters_per_block, b1 = last / sk.iters_per_block;
+  if (b0 == b1) return;   // computed and stored by one block
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
+  const int tile_n = tile / sk.tm, tile_m = tile - tile_n * sk.tm;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  float acc[64];
+#pragma unroll
+  for (int r = 0; r < 64; ++r) acc[r] = 0.f;
+  for (int b = b0; b <= b1; ++b) {
+    const int slot = b * sk.iters_per_block >= first ? 0 : 1;
+    const float *pc = pieces + (static_cast<int64_t>(b) * 2 + slot) * (BM * BN) + tid;
+#pragma unroll
+    for (int r = 0; r < 64; ++r) acc[r] += pc[r * kThreads];
+  }
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const int n = n0 + wn0 + 32 * ni + (lane & 31);
+    if (n >= P.N) continue;
+    const uint32_t img = P.plane.div(n);
+    const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+      const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = mb + 8 * (e >> 2) + (e & 3);
+        if (m < P.M) out[static_cast<int64_t>(m) * P.out_plane + coff] = acc[(mi * 2 + ni) * 16 + e];
       }
     }
   }
@@ -1060,7 +1132,7 @@ int launch_bwd_filter_tap_major(const ConvGeo &g, const float *x, const float *d
 
 // launches conv_tap_kernel; `w_relaid` is [M][K] in the tap-major order
 template <int BM, int BN, int WM, int WN, bool BWD_DATA>
-void launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, float *out, hipStream_t st) {
+int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, float *out, hipStream_t st) {
   TapConvParams P;
   const int taps = g.kH * g.kW;
   if (BWD_DATA) {   // out = dx [imgs][C][H][W], src = dy [imgs][O][oH][oW]
@@ -1107,15 +1179,30 @@ void launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, 
   static const int occ = blocks_per_cu(conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>);
   const int slots = 256 * occ;
   unsigned grid;
-  if (tiles <= slots) {          // one tile per block
+  float *pieces = nullptr;
+  bool zero_cut = false;
+  if (tiles % slots == 0 || sk.total < slots * 8) {
+    // whole tiles fill whole waves of blocks, or there is too little work to cut: one tile per block
     sk.iters_per_block = sk.ksteps;
     grid = (tiles + 7) / 8 * 8;
   } else {                       // one full wave of blocks, equal shares of k-steps
     grid = slots;
     sk.iters_per_block = (sk.total + slots - 1) / slots;
-    hipLaunchKernelGGL((conv_tap_zero_cut_tiles_kernel<BM, BN>), dim3(grid), dim3(kThreads), 0, st, P, out, sk);
+    if (sk.iters_per_block >= sk.ksteps) {
+      zero_cut = true;           // at most two contributors per tile: atomics onto zeroed tiles
+    } else {
+      pieces = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(grid) * 2 * BM * BN * sizeof(float)));
+      TS_REQUIRE(pieces, "conv: no scratch memory for the pieces of cut tiles");
+    }
   }
-  hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>), dim3(grid), dim3(kThreads), 0, st, P, out, sk);
+  if (zero_cut)
+    hipLaunchKernelGGL((conv_tap_zero_cut_tiles_kernel<BM, BN>), dim3(grid), dim3(kThreads), 0, st, P, out, sk);
+  hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>), dim3(grid), dim3(kThreads), 0, st, P, out, pieces,
+                     sk);
+  if (pieces)
+    hipLaunchKernelGGL((conv_tap_assemble_kernel<BM, BN, WM, WN>), dim3(tiles), dim3(kThreads), 0, st, P, out, pieces,
+                       sk);
+  return 0;
 }
 
 // the buffer-load path addresses with 32-bit byte offsets and a 32-tap bit mask
@@ -1408,10 +1495,9 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
       hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wf, g.O, g.C,
                          g.kH * g.kW, false);
       if (tap_kernel_ok(g, numel(x), numel(w))) {
-        if (g.O <= 64)
-          launch_conv_tap<64, 256, 1, 4, false>(g, cf(x), wf, mf(y), st);
-        else
-          launch_conv_tap<128, 128, 2, 2, false>(g, cf(x), wf, mf(y), st);
+        const int rc = g.O <= 64 ? launch_conv_tap<64, 256, 1, 4, false>(g, cf(x), wf, mf(y), st)
+                                 : launch_conv_tap<128, 128, 2, 2, false>(g, cf(x), wf, mf(y), st);
+        if (rc) return rc;
       } else if (g.O <= 64) {
         launch_fwd_tap_major<64, 256, 1, 4>(g, cf(x), wf, mf(y), st);
       } else {
@@ -1443,10 +1529,9 @@ int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray 
       hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
                          g.kH * g.kW, true);
       if (tap_kernel_ok(g, numel(dy), numel(w))) {
-        if (g.C <= 64)
-          launch_conv_tap<64, 256, 1, 4, true>(g, cf(dy), wt, mf(dx), st);
-        else
-          launch_conv_tap<128, 128, 2, 2, true>(g, cf(dy), wt, mf(dx), st);
+        const int rc = g.C <= 64 ? launch_conv_tap<64, 256, 1, 4, true>(g, cf(dy), wt, mf(dx), st)
+                                 : launch_conv_tap<128, 128, 2, 2, true>(g, cf(dy), wt, mf(dx), st);
+        if (rc) return rc;
       } else if (g.C <= 64) {
         launch_bwd_data_tap_major<64, 256, 1, 4>(g, wt, cf(dy), mf(dx), st);
       } else {
