@@ -1,0 +1,89 @@
+"""Whole-graph parity for the branched example networks (BASELINE configs 3-5 at reduced
+size): the same builder code (tsplit_amd/workloads.py) runs on a tape over the C ABI and on a
+tape over the numpy oracle; loss, logits and every parameter gradient are compared, then a few
+SGD steps.  Tolerances: loss 1e-3 relative; logits and gradients 2e-3 of their largest entry
+(the conv / matmul bar; these graphs chain tens of them)."""
+import numpy as np
+import pytest
+
+from oracle_backend import OracleBackend
+from util import assert_close, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(build, seed, steps=3, lr=0.05):
+    """build(tape, binder) -> (loss, logits).  Returns the per-step losses of both backends
+    after checking the first step in detail."""
+    from tsplit_amd import graph, workloads
+    store_g, store_o = workloads.ParamStore(seed), workloads.ParamStore(seed)
+    losses = {"gpu": [], "oracle": []}
+    for step in range(steps):
+        results = {}
+        for tag, backend, store in (("gpu", graph.GpuBackend(), store_g), ("oracle", OracleBackend(), store_o)):
+            t = graph.Tape(backend)
+            b = workloads.Binder(t, store)
+            loss, logits = build(t, b)
+            t.backward(loss)
+            results[tag] = (float(backend.to_numpy(loss.value).reshape(-1)[0]), backend.to_numpy(logits.value), b.grads())
+            b.sgd_step(lr)
+            b.pull()
+            losses[tag].append(results[tag][0])
+        (lg, yg, gg), (lo, yo, go) = results["gpu"], results["oracle"]
+        assert np.isfinite(lg) and abs(lg - lo) <= 1e-3 * abs(lo), (step, lg, lo)
+        if step == 0:
+            assert_close(yg, yo, 2e-3, "logits")
+            assert list(gg) == list(go) and len(gg) > 0
+            worst = max((max_rel_err(gg[k].reshape(go[k].shape), go[k]), k) for k in go)
+            assert worst[0] <= 2e-3, "gradient of %s off by %.3e" % (worst[1], worst[0])
+            # every trainable parameter received a gradient
+            assert set(gg) == {k for k, tr in store_g.trainable.items() if tr}
+    return losses
+
+
+def _onehot(rng, n, classes):
+    y = np.zeros((n, classes), np.float32)
+    y[np.arange(n), rng.randint(0, classes, n)] = 1
+    return y
+
+
+def test_resnet_bottleneck_graph(rng):
+    """Stem 7x7/2 + 3x3/2 max pool, two bottleneck stages (2 and 2 blocks, the second with the
+    stride-2 projection shortcut), global average pool, FC: the ResNet-50 topology, shortened."""
+    from tsplit_amd import workloads
+    x = rng.normal(size=(4, 3, 32, 32)).astype(np.float32)
+    y = _onehot(rng, 4, 10)
+
+    def build(t, b):
+        return workloads.resnet(t, b, b.input(x), b.input(y), blocks=(2, 2), base=8, classes=10)
+    losses = _both(build, seed=5)
+    assert losses["gpu"][-1] < losses["gpu"][0]
+
+
+def test_inception_v4_graph(rng):
+    """Stem, one Inception-A, Reduction-A, one Inception-B (1x7 / 7x1), Reduction-B, one
+    Inception-C (1x3 / 3x1), global average pool, FC + bias, at 1/8 of the channel widths."""
+    from tsplit_amd import workloads
+    x = rng.normal(size=(3, 3, 107, 107)).astype(np.float32)     # 11x11 / 5x5 / 2x2 planes in the A / B / C blocks
+    y = _onehot(rng, 3, 10)
+
+    def build(t, b):
+        return workloads.inception_v4(t, b, b.input(x), b.input(y), n_a=1, n_b=1, n_c=1, div=8, classes=10)
+    _both(build, seed=6, steps=2, lr=0.01)
+
+
+def test_transformer_graph(rng):
+    """Encoder-decoder, 1+1 blocks (three attention layers, two feed-forward layers), 4 heads, padding and causal masks, shared embedding /
+    logits table, label smoothing; token id 0 occurs so that the padding paths are taken."""
+    from tsplit_amd import workloads
+    cfg = workloads.TransformerConfig(batch=3, len1=10, len2=8, d_model=32, heads=4, d_ff=64, blocks=1, vocab=50,
+                                      mask_value=-1.0, embed_std=0.05, pos_amplitude=0.2)
+    xs = rng.randint(0, cfg.vocab, size=(cfg.batch, cfg.len1)).astype(np.float32)
+    ys_in = rng.randint(0, cfg.vocab, size=(cfg.batch, cfg.len2)).astype(np.float32)
+    ys_out = rng.randint(0, cfg.vocab, size=(cfg.batch, cfg.len2)).astype(np.float32)
+    xs[:, -2:] = 0
+    ys_in[:, -1] = 0
+
+    def build(t, b):
+        return workloads.transformer(t, b, cfg, b.input(xs), b.input(ys_in), b.input(ys_out))
+    _both(build, seed=7, steps=3, lr=0.01)

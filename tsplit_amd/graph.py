@@ -1,0 +1,457 @@
+"""A small reverse-mode tape over the operator library, for graphs with branches.
+
+The reference builds such graphs with `ad.<op>_op` nodes and differentiates them with
+`ad.gradients` (python/athena/gpu_ops/executor.py:160-196); each node's `compute` calls one
+`gpu_links` function and its `gradient` names the nodes of the backward pass.  This tape does
+the same work eagerly: every method below runs one forward operator and records the calls of
+the backward operators the reference's `gradient` would schedule (cited per method).  It
+exists so that the residual, multi-branch and attention graphs of the reference's examples
+can be run through the C ABI; `trainer.py` remains the harness of the sequential nets.
+
+The arithmetic comes from a backend object.  `GpuBackend` (below) maps every primitive onto
+`gpu_links`; the tests plug in a numpy backend with the same methods to check whole graphs.
+"""
+import numpy as np
+
+from . import gpu_links as L
+from . import ndarray
+
+
+class Var(object):
+    """A value on the tape: backend array, shape, accumulated gradient."""
+    __slots__ = ["value", "shape", "grad", "needs_grad", "name"]
+
+    def __init__(self, value, shape, needs_grad, name=None):
+        self.value, self.shape, self.grad, self.needs_grad, self.name = value, tuple(shape), None, needs_grad, name
+
+
+def _prod(shape):
+    n = 1
+    for s in shape:
+        n *= int(s)
+    return n
+
+
+def conv_out(size, k, pad, stride):
+    return (size + 2 * pad - k) // stride + 1
+
+
+class GpuBackend(object):
+    """Primitives on device arrays, one `gpu_links` call each (plus the output allocation)."""
+
+    def __init__(self, ctx=None, stream=None):
+        self.ctx = ctx or ndarray.gpu(0)
+        self.stream = stream
+
+    # ---- storage
+    def from_numpy(self, a):
+        return ndarray.array(np.ascontiguousarray(a, dtype=np.float32), self.ctx)
+
+    def to_numpy(self, x):
+        return x.asnumpy()
+
+    def empty(self, shape):
+        return ndarray.empty(tuple(int(s) for s in shape), self.ctx)
+
+    def reshape(self, x, shape):
+        out = self.empty(shape)
+        L.array_reshape(x, out, self.stream)
+        return out
+
+    # ---- contractions
+    def conv2d(self, x, w, xs, ws, ph, pw, s):
+        y = self.empty((xs[0], ws[0], conv_out(xs[2], ws[2], ph, s), conv_out(xs[3], ws[3], pw, s)))
+        L.CuDNN_conv2d(x, w, y, ph, pw, s, self.stream)
+        return y
+
+    def conv2d_grad_data(self, w, dy, xs, ph, pw, s):
+        dx = self.empty(xs)
+        L.CuDNN_conv2d_gradient_of_data(w, dy, dx, ph, pw, s, self.stream)
+        return dx
+
+    def conv2d_grad_filter(self, x, dy, ws, ph, pw, s):
+        dw = self.empty(ws)
+        L.CuDNN_conv2d_gradient_of_filter(x, dy, dw, ph, pw, s, self.stream)
+        return dw
+
+    def matmul(self, a, ta, b, tb, out_shape):
+        c = self.empty(out_shape)
+        L.matrix_multiply(a, ta, b, tb, c, self.stream)
+        return c
+
+    def batch_matmul(self, a, ta, b, tb, out_shape):
+        c = self.empty(out_shape)
+        L.batch_matrix_multiply(a, ta, b, tb, c, self.stream)
+        return c
+
+    # ---- normalisation, activations, pooling
+    def bn(self, x, gamma, beta, xs, eps):
+        y = self.empty(xs)
+        L.CuDNN_Batch_Normalization(x, gamma, beta, y, None, None, 0.99, eps, self.stream)
+        return y
+
+    def bn_grad(self, dy, x, gamma, xs, eps):
+        dx, dg, db = self.empty(xs), self.empty((1, xs[1], 1, 1)), self.empty((1, xs[1], 1, 1))
+        L.CuDNN_Batch_Normalization_gradient(dy, x, gamma, dx, dg, db, None, None, eps, self.stream)
+        return dx, dg, db
+
+    def relu(self, x, shape):
+        y = self.empty(shape)
+        L.relu(x, y, self.stream)
+        return y
+
+    def relu_grad(self, x, dy, shape):
+        dx = self.empty(shape)
+        L.relu_gradient(x, dy, dx, self.stream)
+        return dx
+
+    def max_pool(self, x, xs, k, pad, s):
+        y = self.empty((xs[0], xs[1], conv_out(xs[2], k, pad, s), conv_out(xs[3], k, pad, s)))
+        L.CuDNN_max_pooling2d(x, k, k, y, pad, s, self.stream)
+        return y
+
+    def max_pool_grad(self, x, y, dy, xs, k, pad, s):
+        dx = self.empty(xs)
+        L.CuDNN_max_pooling2d_gradient(y, dy, x, k, k, dx, pad, s, self.stream)
+        return dx
+
+    def avg_pool(self, x, xs, k, pad, s):
+        y = self.empty((xs[0], xs[1], conv_out(xs[2], k, pad, s), conv_out(xs[3], k, pad, s)))
+        L.CuDNN_average_pooling2d(x, k, k, y, pad, s, self.stream)
+        return y
+
+    def avg_pool_grad(self, x, y, dy, xs, k, pad, s):
+        dx = self.empty(xs)
+        L.CuDNN_average_pooling2d_gradient(y, dy, x, k, k, dx, pad, s, self.stream)
+        return dx
+
+    # ---- elementwise, broadcast, reduce, layout
+    def add(self, a, b, shape):
+        c = self.empty(shape)
+        L.matrix_elementwise_add(a, b, c, self.stream)
+        return c
+
+    def mul_const(self, a, c, shape):
+        out = self.empty(shape)
+        L.matrix_elementwise_multiply_by_const(a, c, out, self.stream)
+        return out
+
+    def add_const(self, a, c, shape):
+        out = self.empty(shape)
+        L.matrix_elementwise_add_by_const(a, c, out, self.stream)
+        return out
+
+    def broadcast_shape(self, x, out_shape):
+        out = self.empty(out_shape)
+        L.broadcast_shape(x, out, None, self.stream)
+        return out
+
+    def reduce_sum(self, x, axes, out_shape):
+        out = self.empty(out_shape)
+        L.reduce_sum(x, out, axes, self.stream)
+        return out
+
+    def broadcast_to(self, x, out_shape):
+        out = self.empty(out_shape)
+        L.broadcast_to(x, out, self.stream)
+        return out
+
+    def reduce_sum_axis_zero(self, x, out_shape):
+        out = self.empty(out_shape)
+        L.reduce_sum_axis_zero(x, out, self.stream)
+        return out
+
+    def concat(self, a, b, out_shape, axis):
+        out = self.empty(out_shape)
+        L.concat(a, b, out, axis, self.stream)
+        return out
+
+    def concat_grad(self, dout, in_shape, axis, idx):
+        g = self.empty(in_shape)
+        L.concat_gradient(dout, g, axis, idx, self.stream)
+        return g
+
+    def transpose(self, x, perm, out_shape):
+        out = self.empty(out_shape)
+        L.matrix_transpose(x, out, perm, self.stream)
+        return out
+
+    def where(self, cond, a, b, shape):
+        out = self.empty(shape)
+        L.where(cond, a, b, out, self.stream)
+        return out
+
+    def one_hot(self, ids, out_shape):
+        out = self.empty(out_shape)
+        L.one_hot(ids, out, self.stream)
+        return out
+
+    def embedding(self, table, ids, out_shape):
+        out = self.empty(out_shape)
+        L.embedding_lookup(table, ids, out, self.stream)
+        return out
+
+    def embedding_grad(self, dy, ids, table_shape):
+        g = self.empty(table_shape)
+        L.embedding_lookup_gradient(dy, ids, g, self.stream)
+        return g
+
+    def zeros(self, shape):
+        out = self.empty(shape)
+        L.array_set(out, 0.0, self.stream)
+        return out
+
+    # ---- loss, update
+    def softmax_ce(self, logits, labels):
+        loss = self.empty((1,))
+        L.softmax_cross_entropy(logits, labels, loss, self.stream)
+        return loss
+
+    def softmax_ce_grad(self, logits, labels, shape):
+        one = self.empty((1,))
+        L.array_set(one, 1.0, self.stream)
+        g = self.empty(shape)
+        L.softmax_cross_entropy_gradient(logits, labels, one, g, self.stream)
+        return g
+
+    def sgd(self, p, g, lr):
+        L.sgd_update(p, g, lr, self.stream)
+
+    def sync(self):
+        if self.stream:
+            self.stream.sync()
+        else:
+            ndarray.empty((1,), self.ctx).asnumpy()
+
+
+class Tape(object):
+    def __init__(self, backend):
+        self.b = backend
+        self._nodes = []     # (output Var, backward closure)
+
+    # ---- leaves
+    def param(self, value, shape, name=None):
+        return Var(value, shape, True, name)
+
+    def const(self, value, shape, name=None):
+        return Var(value, shape, False, name)
+
+    def _out(self, value, shape, inputs, backward):
+        v = Var(value, shape, any(i.needs_grad for i in inputs))
+        if v.needs_grad:
+            self._nodes.append((v, backward))
+        return v
+
+    def _acc(self, var, g):
+        if not var.needs_grad:
+            return
+        var.grad = g if var.grad is None else self.b.add(var.grad, g, var.shape)
+
+    # ---- operators (reference gradient rules cited)
+    def conv2d(self, x, w, ph, pw, stride):
+        """gpu_ops/Conv2d.py:100-118 (compute), :120 (gradient: a data-gradient and a filter-gradient node)."""
+        y = self.b.conv2d(x.value, w.value, x.shape, w.shape, ph, pw, stride)
+        ys = (x.shape[0], w.shape[0], conv_out(x.shape[2], w.shape[2], ph, stride), conv_out(x.shape[3], w.shape[3], pw, stride))
+
+        def back(g):
+            if w.needs_grad:
+                self._acc(w, self.b.conv2d_grad_filter(x.value, g, w.shape, ph, pw, stride))
+            if x.needs_grad:
+                self._acc(x, self.b.conv2d_grad_data(w.value, g, x.shape, ph, pw, stride))
+        return self._out(y, ys, [x, w], back)
+
+    def batch_norm(self, x, gamma, beta, eps=0.01):
+        """gpu_ops/BatchNorm.py:54-83 (compute), :166-227 (gradient node; statistics recomputed, no
+        saved arrays); gamma / beta receive their gradients as in gpu_ops/BatchNorm2.py:104-114."""
+        y = self.b.bn(x.value, gamma.value, beta.value, x.shape, eps)
+
+        def back(g):
+            dx, dg, db = self.b.bn_grad(g, x.value, gamma.value, x.shape, eps)
+            self._acc(x, dx)
+            self._acc(gamma, dg)
+            self._acc(beta, db)
+        return self._out(y, x.shape, [x, gamma, beta], back)
+
+    def relu(self, x):
+        """gpu_ops/Relu.py:51,117."""
+        y = self.b.relu(x.value, x.shape)
+        return self._out(y, x.shape, [x], lambda g: self._acc(x, self.b.relu_grad(x.value, g, x.shape)))
+
+    def max_pool(self, x, k, pad, stride):
+        """gpu_ops/MaxPool.py:119 (compute), :146 (gradient)."""
+        y = self.b.max_pool(x.value, x.shape, k, pad, stride)
+        ys = (x.shape[0], x.shape[1], conv_out(x.shape[2], k, pad, stride), conv_out(x.shape[3], k, pad, stride))
+        return self._out(y, ys, [x], lambda g: self._acc(x, self.b.max_pool_grad(x.value, y, g, x.shape, k, pad, stride)))
+
+    def avg_pool(self, x, k, pad, stride):
+        """gpu_ops/AvgPool.py:78 (compute), :103-104 (gradient)."""
+        y = self.b.avg_pool(x.value, x.shape, k, pad, stride)
+        ys = (x.shape[0], x.shape[1], conv_out(x.shape[2], k, pad, stride), conv_out(x.shape[3], k, pad, stride))
+        return self._out(y, ys, [x], lambda g: self._acc(x, self.b.avg_pool_grad(x.value, y, g, x.shape, k, pad, stride)))
+
+    def add(self, a, b):
+        """gpu_ops/AddElewise.py:54 (compute), :95 (gradient: both inputs receive the output gradient)."""
+        assert a.shape == b.shape, (a.shape, b.shape)
+        y = self.b.add(a.value, b.value, a.shape)
+
+        def back(g):
+            self._acc(a, g)
+            self._acc(b, g)
+        return self._out(y, a.shape, [a, b], back)
+
+    def scale(self, a, c):
+        """gpu_ops/MultiplyConst.py:45 (compute), :63 (gradient: the output gradient times the constant)."""
+        y = self.b.mul_const(a.value, c, a.shape)
+        return self._out(y, a.shape, [a], lambda g: self._acc(a, self.b.mul_const(g, c, a.shape)))
+
+    def shift(self, a, c):
+        y = self.b.add_const(a.value, c, a.shape)
+        return self._out(y, a.shape, [a], lambda g: self._acc(a, g))
+
+    def reshape(self, a, shape):
+        """gpu_ops/Reshape.py:42 (compute: a copy), :61 (gradient: reshaped back)."""
+        shape = list(shape)
+        if -1 in shape:
+            known = _prod([s for s in shape if s != -1])
+            shape[shape.index(-1)] = _prod(a.shape) // known
+        shape = tuple(shape)
+        y = self.b.reshape(a.value, shape)
+        return self._out(y, shape, [a], lambda g: self._acc(a, self.b.reshape(g, a.shape)))
+
+    def concat(self, a, b, axis):
+        """gpu_ops/Concat.py:47-60 (compute), :65 (gradient: two concat_gradient nodes, idx 0 and 1)."""
+        shape = list(a.shape)
+        shape[axis] += b.shape[axis]
+        shape = tuple(shape)
+        y = self.b.concat(a.value, b.value, shape, axis)
+
+        def back(g):
+            if a.needs_grad:
+                self._acc(a, self.b.concat_grad(g, a.shape, axis, 0))
+            if b.needs_grad:
+                self._acc(b, self.b.concat_grad(g, b.shape, axis, 1))
+        return self._out(y, shape, [a, b], back)
+
+    def matmul(self, a, b, trans_a=False, trans_b=False):
+        """gpu_ops/MatrixMult.py:57-86 (compute), :95-124 (gradient)."""
+        m = a.shape[1] if trans_a else a.shape[0]
+        n = b.shape[0] if trans_b else b.shape[1]
+        y = self.b.matmul(a.value, trans_a, b.value, trans_b, (m, n))
+
+        def back(g):
+            if a.needs_grad:
+                if not trans_a:
+                    ga = self.b.matmul(g, False, b.value, not trans_b, a.shape)
+                else:
+                    ga = self.b.matmul(b.value, trans_b, g, True, a.shape)
+                self._acc(a, ga)
+            if b.needs_grad:
+                if not trans_b:
+                    gb = self.b.matmul(a.value, not trans_a, g, False, b.shape)
+                else:
+                    gb = self.b.matmul(g, True, a.value, trans_a, b.shape)
+                self._acc(b, gb)
+        return self._out(y, (m, n), [a, b], back)
+
+    def batch_matmul(self, a, b, trans_a=False, trans_b=False):
+        """gpu_ops/BatchMatrixMult.py:49-75 (compute), :77 (gradient: the four transpose cases)."""
+        lead = a.shape[:-2]
+        m = a.shape[-1] if trans_a else a.shape[-2]
+        n = b.shape[-2] if trans_b else b.shape[-1]
+        ys = tuple(lead) + (m, n)
+        y = self.b.batch_matmul(a.value, trans_a, b.value, trans_b, ys)
+
+        def back(g):
+            if a.needs_grad:
+                if not trans_a:
+                    ga = self.b.batch_matmul(g, False, b.value, not trans_b, a.shape)
+                else:
+                    ga = self.b.batch_matmul(b.value, trans_b, g, True, a.shape)
+                self._acc(a, ga)
+            if b.needs_grad:
+                if not trans_b:
+                    gb = self.b.batch_matmul(a.value, not trans_a, g, False, b.shape)
+                else:
+                    gb = self.b.batch_matmul(g, True, a.value, trans_a, b.shape)
+                self._acc(b, gb)
+        return self._out(y, ys, [a, b], back)
+
+    def add_bias(self, x, bias):
+        """x [rows, cols] + broadcast(bias [cols]) (gpu_ops/Broadcast.py:45-59, gradient :65 =
+        reduce_sum_axis_zero)."""
+        bb = self.b.broadcast_to(bias.value, x.shape)
+        y = self.b.add(x.value, bb, x.shape)
+
+        def back(g):
+            self._acc(x, g)
+            if bias.needs_grad:
+                self._acc(bias, self.b.reduce_sum_axis_zero(g, bias.shape))
+        return self._out(y, x.shape, [x, bias], back)
+
+    def broadcast_like(self, x, shape):
+        """gpu_ops/BroadcastTF.py:46-58 (numpy alignment from the right); gradient = reduce_sum
+        over the broadcast axes (gpu_ops/BroadcastShape.py:61)."""
+        shape = tuple(shape)
+        y = self.b.broadcast_shape(x.value, shape)
+        diff = len(shape) - len(x.shape)
+        axes = [d for d in range(len(shape)) if d < diff or (x.shape[d - diff] == 1 and shape[d] != 1)]
+
+        def back(g):
+            if axes:
+                self._acc(x, self.b.reduce_sum(g, axes, x.shape))
+            else:
+                self._acc(x, g)
+        return self._out(y, shape, [x], back)
+
+    def transpose(self, x, perm):
+        """gpu_ops/Transpose.py:44-58 (compute), :60 (gradient: the inverse permutation)."""
+        perm = list(perm)
+        ys = tuple(x.shape[p] for p in perm)
+        y = self.b.transpose(x.value, perm, ys)
+        inv = [0] * len(perm)
+        for i, p in enumerate(perm):
+            inv[p] = i
+        return self._out(y, ys, [x], lambda g: self._acc(x, self.b.transpose(g, inv, x.shape)))
+
+    def where(self, cond, a, b):
+        """gpu_ops/Where.py:41-48 (compute), :50-55 (gradient: where(cond, g, 0) and where(cond, 0, g))."""
+        y = self.b.where(cond.value, a.value, b.value, a.shape)
+
+        def back(g):
+            z = self.b.zeros(a.shape)
+            if a.needs_grad:
+                self._acc(a, self.b.where(cond.value, g, z, a.shape))
+            if b.needs_grad:
+                self._acc(b, self.b.where(cond.value, z, g, a.shape))
+        return self._out(y, a.shape, [a, b], back)
+
+    def one_hot(self, ids, classes):
+        """gpu_ops/OneHot.py:44-46; no gradient."""
+        ys = tuple(ids.shape) + (classes,)
+        return Var(self.b.one_hot(ids.value, ys), ys, False)
+
+    def embedding(self, table, ids):
+        """gpu_ops/EmbeddingLookUp.py:41-42, gradient :48-49."""
+        ys = tuple(ids.shape) + (table.shape[1],)
+        y = self.b.embedding(table.value, ids.value, ys)
+        return self._out(y, ys, [table], lambda g: self._acc(table, self.b.embedding_grad(g, ids.value, table.shape)))
+
+    def softmax_ce(self, logits, labels):
+        """gpu_ops/SoftmaxCrossEntropy.py:46-67 (compute), :73 and :134-135 (gradient) with an adjoint of one."""
+        assert len(logits.shape) == 2
+        loss = self.b.softmax_ce(logits.value, labels.value)
+        return self._out(loss, (1,), [logits],
+                         lambda g: self._acc(logits, self.b.softmax_ce_grad(logits.value, labels.value, logits.shape)))
+
+    # ---- reverse sweep
+    def backward(self, loss):
+        """Runs the recorded backward operators in reverse order; the loss adjoint is one
+        (gpu_ops/executor.py:175), folded into softmax_ce's gradient."""
+        loss.grad = True
+        for v, back in reversed(self._nodes):
+            if v.grad is None:
+                continue
+            back(v.grad)
+            if v is not loss:
+                v.grad = None      # interior gradients are dropped as soon as they are consumed
+        self._nodes = []
