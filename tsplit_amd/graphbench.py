@@ -1,0 +1,101 @@
+"""Times one training step (forward, backward, SGD) of the branched example networks at the
+sizes of the reference's benchmark configurations, on one MI355X through the C ABI.
+
+    python -m tsplit_amd.graphbench --net resnet50|inception_v4|transformer [--steps 5] [--warmup 2]
+
+Prints one JSON object: samples/s, ms/step, final loss, operator calls per step.  Synthetic
+seeded inputs; parameters as in workloads.py.  (The headline benchmark of this repository is
+bench.py; this sweep only shows the other configurations running at their real shapes.)
+"""
+import argparse
+import json
+import time
+
+import numpy as np
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--net", default="resnet50", choices=["resnet50", "inception_v4", "transformer"])
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--batch", type=int, default=0)
+    ap.add_argument("--lr", type=float, default=1e-4)
+    a = ap.parse_args()
+    from . import graph, ndarray, stream, workloads
+    ctx = ndarray.gpu(0)
+    st = stream.create_stream_handle(ctx)
+    backend = graph.GpuBackend(ctx, st)
+    rng = np.random.RandomState(123)
+    store = workloads.ParamStore(123)
+    calls = [0]
+
+    if a.net == "resnet50":
+        n = a.batch or 64
+        x = rng.standard_normal((n, 3, 224, 224)).astype(np.float32)
+        y = np.zeros((n, 1000), np.float32)
+        y[np.arange(n), rng.randint(0, 1000, n)] = 1
+
+        def build(t, b, cache):
+            return workloads.resnet(t, b, cache["x"], cache["y"])
+        inputs = {"x": x, "y": y}
+        desc = "ResNet-50, fp32 NCHW, batch %d, 3x224x224, 1000 classes" % n
+    elif a.net == "inception_v4":
+        n = a.batch or 32
+        x = rng.standard_normal((n, 3, 299, 299)).astype(np.float32)
+        y = np.zeros((n, 1000), np.float32)
+        y[np.arange(n), rng.randint(0, 1000, n)] = 1
+
+        def build(t, b, cache):
+            return workloads.inception_v4(t, b, cache["x"], cache["y"])
+        inputs = {"x": x, "y": y}
+        desc = "Inception-v4, fp32 NCHW, batch %d, 3x299x299, 1000 classes" % n
+    else:
+        n = a.batch or 32
+        # no softmax in this graph: masked scores are set to 0 and values are kept small so that twelve
+        # blocks stay finite
+        cfg = workloads.TransformerConfig(batch=n, mask_value=0.0, embed_std=0.0002, pos_amplitude=0.003)
+        inputs = {"xs": rng.randint(1, cfg.vocab, size=(n, cfg.len1)).astype(np.float32),
+                  "yi": rng.randint(1, cfg.vocab, size=(n, cfg.len2)).astype(np.float32),
+                  "yo": rng.randint(1, cfg.vocab, size=(n, cfg.len2)).astype(np.float32)}
+
+        def build(t, b, cache):
+            return workloads.transformer(t, b, cfg, cache["xs"], cache["yi"], cache["yo"])
+        desc = "Transformer 6+6 blocks, d_model 512, 8 heads, FFN 2048, length 256, batch %d, vocab 32000" % n
+
+    binder = None
+    dev_inputs = None
+    loss_val = float("nan")
+
+    def one_step():
+        nonlocal binder, dev_inputs
+        t = graph.Tape(backend)
+        if binder is None:
+            binder = workloads.Binder(t, store)
+            dev_inputs = {k: binder.input(v) for k, v in inputs.items()}      # resident before timing
+        else:
+            binder.t, binder._n = t, 0
+            for v in binder.vars.values():
+                v.grad = None
+        loss, _ = build(t, binder, dev_inputs)
+        calls[0] = len(t._nodes)
+        t.backward(loss)
+        binder.sgd_step(a.lr)
+        return loss
+
+    for _ in range(a.warmup):
+        one_step()
+    backend.sync()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        loss = one_step()
+    backend.sync()
+    dt = time.perf_counter() - t0
+    loss_val = float(loss.value.asnumpy()[0])
+    print(json.dumps({"net": a.net, "workload": desc, "samples_per_s": n * a.steps / dt, "ms_per_step": dt / a.steps * 1e3,
+                      "steps": a.steps, "warmup": a.warmup, "final_loss": loss_val, "forward_ops_per_step": calls[0],
+                      "dtype": "f32", "data": "synthetic"}))
+
+
+if __name__ == "__main__":
+    main()
