@@ -35,6 +35,14 @@ CASES = [
     (8, 512, 14, 14, 256, 3, 3, 1, 1, 1),  # 26 tiles of 128x128, 288 k-steps each
     (8, 512, 28, 28, 64, 3, 3, 1, 1, 1),   # forward on 64x256 tiles
     (8, 64, 28, 28, 512, 3, 3, 1, 1, 1),   # backward-data on 64x256 tiles
+    # strided convolutions: backward-data runs one GEMM per stride phase
+    (2, 32, 14, 14, 48, 1, 1, 0, 0, 2),    # 1x1 stride 2 (ResNet shortcut): three of four phases are zero
+    (2, 24, 15, 15, 40, 3, 3, 1, 1, 2),    # 3x3 stride 2 pad 1, odd input
+    (2, 16, 17, 17, 20, 3, 3, 0, 0, 2),    # 3x3 stride 2 valid (Inception reductions)
+    (1, 8, 23, 19, 12, 7, 7, 3, 3, 2),     # 7x7 stride 2 pad 3 (ResNet stem), non-square
+    (2, 8, 20, 20, 12, 5, 5, 2, 2, 3),     # stride 3
+    (1, 70, 12, 12, 130, 3, 3, 1, 1, 2),   # 128x128 tiles, ragged
+    (1, 4, 9, 9, 6, 2, 2, 0, 0, 3),        # stride larger than the filter: some inputs get no gradient
     # at most 32 filter columns (C*kH*kW): backward-filter takes the few-columns kernel
     (4, 3, 64, 64, 64, 3, 3, 1, 1, 1),     # several K slices, folded
     (3, 1, 19, 23, 100, 5, 5, 2, 2, 1),    # 25 columns, two row tiles, ragged K (oH*oW odd)

@@ -499,13 +499,15 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
   }
 }
 
-// Assembles the tiles that block ranges cut into pieces: block = tile; adds the pieces in
-// ascending block order and stores the tile.  Thread and register layout are those of
+// Assembles the tiles that block ranges cut into pieces.  Four blocks per tile, one per 32x32
+// accumulator block of every wave (registers 16q .. 16q+15): each adds the pieces in ascending
+// block order and stores its share of the tile.  Thread and register layout are those of
 // conv_tap_kernel's epilogue.
 template <int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvParams P, float *__restrict__ out,
                                                                      const float *__restrict__ pieces, StreamK sk) {
-  const int tile = blockIdx.x;
+  const int tile = blockIdx.x >> 2, q = blockIdx.x & 3;
+  const int mi = q >> 1, ni = q & 1;
   const int first = tile * sk.ksteps, last = first + sk.ksteps - 1;
   const int b0 = first / sk.iters_per_block, b1 = last / sk.iters_per_block;
   if (b0 == b1) return;   // computed and stored by one block
@@ -513,30 +515,24 @@ __global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvPara
   const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
   const int tile_n = tile / sk.tm, tile_m = tile - tile_n * sk.tm;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  float acc[64];
+  float acc[16];
 #pragma unroll
-  for (int r = 0; r < 64; ++r) acc[r] = 0.f;
+  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
   for (int b = b0; b <= b1; ++b) {
     const int slot = b * sk.iters_per_block >= first ? 0 : 1;
-    const float *pc = pieces + (static_cast<int64_t>(b) * 2 + slot) * (BM * BN) + tid;
+    const float *pc = pieces + (static_cast<int64_t>(b) * 2 + slot) * (BM * BN) + (q * 16) * kThreads + tid;
 #pragma unroll
-    for (int r = 0; r < 64; ++r) acc[r] += pc[r * kThreads];
+    for (int e = 0; e < 16; ++e) acc[e] += __builtin_nontemporal_load(pc + e * kThreads);
   }
+  const int n = n0 + wn0 + 32 * ni + (lane & 31);
+  if (n >= P.N) return;
+  const uint32_t img = P.plane.div(n);
+  const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
+  const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
 #pragma unroll
-  for (int ni = 0; ni < 2; ++ni) {
-    const int n = n0 + wn0 + 32 * ni + (lane & 31);
-    if (n >= P.N) continue;
-    const uint32_t img = P.plane.div(n);
-    const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
-#pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
-      const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = mb + 8 * (e >> 2) + (e & 3);
-        if (m < P.M) out[static_cast<int64_t>(m) * P.out_plane + coff] = acc[(mi * 2 + ni) * 16 + e];
-      }
-    }
+  for (int e = 0; e < 16; ++e) {
+    const int m = mb + 8 * (e >> 2) + (e & 3);
+    if (m < P.M) out[static_cast<int64_t>(m) * P.out_plane + coff] = acc[e];
   }
 }
 
@@ -1058,6 +1054,149 @@ void launch_bwd_data(const ConvGeo &g, const float *wt, const float *dy, float *
                      int64_t(0), static_cast<int64_t>(g.H) * g.W, cm, M, N, K, (K + BK - 1) / BK * BK, TileGrid{tm, tn, tm * tn});
 }
 
+// ------------------------------------------------------------------ strided bwd-data by phases
+// With stride s an input position (h, w) only receives the taps kh = (h + ph) mod s (mod s),
+// kw likewise: 1 - 1/s^2 of the taps of the plain formulation multiply nothing.  The positions
+// are therefore split into s*s phases (a, b) = ((h + ph) mod s, (w + pw) mod s).  Within a
+// phase, h = a' + s*i and the tap kh = a + s*u reads dy row i + (a' + ph - kh)/s: a stride-1
+// correlation of dy with the sub-filter {kh = a (mod s)} x {kw = b (mod s)}, whose outputs are
+// scattered with stride s.  Each phase is one GEMM with K = O * |taps of the phase| and
+// N = imgs * Hp * Wp on the forward gather loader; phases without taps (a 1x1 filter with
+// stride 2 has one phase with a tap and three without) are zero-filled.
+struct PhaseCols {   // column n = (img, i, j) of a phase -> img*img_stride + (a + s*i)*W + (b + s*j)
+  FastDiv plane, width;
+  int64_t img_stride;
+  int a, b, s, W;
+  __device__ __forceinline__ int64_t operator()(int n) const {
+    const uint32_t img = plane.div(n);
+    const uint32_t p = n - img * plane.d;
+    const uint32_t i = width.div(p);
+    const uint32_t j = p - i * width.d;
+    return static_cast<int64_t>(img) * img_stride + static_cast<int64_t>(a + s * static_cast<int>(i)) * W + (b + s * static_cast<int>(j));
+  }
+};
+
+struct PhasePlan {
+  const Tap *taps = nullptr;   // device table of the phase's (o, u, v) in order
+  int nu = 0, nv = 0;          // taps of the phase along each axis
+  int a0 = 0, b0 = 0;          // first input row / column of the phase
+  int hp = 0, wp = 0;          // positions of the phase along each axis
+  int shift_r = 0, shift_c = 0;   // the loader's padding: dy row = i - shift_r + tap.kh
+};
+
+struct PhaseKey {
+  int O, kH, kW, oH, oW, H, W, ph, pw, s, a, b;
+  bool operator<(const PhaseKey &o) const {
+    return std::tie(O, kH, kW, oH, oW, H, W, ph, pw, s, a, b) <
+           std::tie(o.O, o.kH, o.kW, o.oH, o.oW, o.H, o.W, o.ph, o.pw, o.s, o.a, o.b);
+  }
+};
+std::map<PhaseKey, PhasePlan> g_phase_plans;
+
+// floor division for possibly negative numerators
+inline int floor_div(int x, int d) { return x >= 0 ? x / d : -((-x + d - 1) / d); }
+
+bool phase_plan(const ConvGeo &g, int a, int b, PhasePlan &out) {
+  std::lock_guard<std::mutex> lk(g_taps_mu);
+  const PhaseKey key{g.O, g.kH, g.kW, g.oH, g.oW, g.H, g.W, g.ph, g.pw, g.s, a, b};
+  auto it = g_phase_plans.find(key);
+  if (it != g_phase_plans.end()) {
+    out = it->second;
+    return true;
+  }
+  PhasePlan pl;
+  const int s = g.s;
+  pl.a0 = ((a - g.ph) % s + s) % s;
+  pl.b0 = ((b - g.pw) % s + s) % s;
+  pl.hp = pl.a0 < g.H ? (g.H - pl.a0 + s - 1) / s : 0;
+  pl.wp = pl.b0 < g.W ? (g.W - pl.b0 + s - 1) / s : 0;
+  pl.nu = a < g.kH ? (g.kH - a + s - 1) / s : 0;
+  pl.nv = b < g.kW ? (g.kW - b + s - 1) / s : 0;
+  if (pl.nu > 0 && pl.nv > 0 && pl.hp > 0 && pl.wp > 0) {
+    // dy row of tap u for position i: i + dr(u), dr(u) = (a0 + ph - (a + s*u)) / s (exact); the
+    // smallest dr belongs to the last tap
+    pl.shift_r = -floor_div(pl.a0 + g.ph - (a + s * (pl.nu - 1)), s);
+    pl.shift_c = -floor_div(pl.b0 + g.pw - (b + s * (pl.nv - 1)), s);
+    std::vector<Tap> h(static_cast<size_t>(g.O) * pl.nu * pl.nv);
+    size_t i = 0;
+    for (int o = 0; o < g.O; ++o)
+      for (int u = 0; u < pl.nu; ++u)
+        for (int v = 0; v < pl.nv; ++v, ++i) {
+          const int dr = floor_div(pl.a0 + g.ph - (a + s * u), s), dc = floor_div(pl.b0 + g.pw - (b + s * v), s);
+          h[i].kh = static_cast<short>(dr + pl.shift_r);   // >= 0
+          h[i].kw = static_cast<short>(dc + pl.shift_c);
+          h[i].off = o * g.oH * g.oW + h[i].kh * g.oW + h[i].kw;
+        }
+    Tap *d = nullptr;
+    if (hipMalloc(&d, h.size() * sizeof(Tap)) != hipSuccess) return false;
+    if (hipMemcpy(d, h.data(), h.size() * sizeof(Tap), hipMemcpyHostToDevice) != hipSuccess) return false;
+    pl.taps = d;
+  }
+  g_phase_plans[key] = pl;
+  out = pl;
+  return true;
+}
+
+// sub-filter of a phase: out[c][(o, u, v)] = w[o][c][a + s*u][b + s*v]
+__global__ __launch_bounds__(256) void filter_phase_kernel(const float *__restrict__ w, float *__restrict__ out, int O,
+                                                           int C, int kH, int kW, int a, int b, int s, int nu, int nv) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  const int kp = O * nu * nv;
+  if (idx >= C * kp) return;
+  const int c = idx / kp;
+  int r = idx - c * kp;
+  const int o = r / (nu * nv);
+  r -= o * nu * nv;
+  const int u = r / nv, v = r - u * nv;
+  out[idx] = w[((o * C + c) * kH + (a + s * u)) * kW + (b + s * v)];
+}
+
+__global__ __launch_bounds__(256) void zero_fill_kernel(float *__restrict__ p, int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < n) p[i] = 0.f;
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_bwd_data_phases(const ConvGeo &g, const float *w, const float *dy, float *dx, float *wscratch,
+                           hipStream_t st) {
+  using AL = KContigLoader<BM>;
+  using BL = GatherColsLoader<BN, false>;
+  const int s = g.s;
+  PhasePlan plans[64];
+  TS_REQUIRE(s * s <= 64, "conv bwd-data: stride %d not supported", s);
+  bool any_empty = false;
+  for (int a = 0; a < s; ++a)
+    for (int b = 0; b < s; ++b) {
+      PhasePlan &pl = plans[a * s + b];
+      TS_REQUIRE(phase_plan(g, a, b, pl), "conv bwd-data: could not build a phase table");
+      if (pl.hp > 0 && pl.wp > 0 && (pl.nu == 0 || pl.nv == 0)) any_empty = true;
+    }
+  if (any_empty) {
+    const int64_t n = static_cast<int64_t>(g.imgs) * g.C * g.H * g.W;
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, dx, n);
+  }
+  int64_t woff = 0;
+  for (int a = 0; a < s; ++a)
+    for (int b = 0; b < s; ++b) {
+      const PhasePlan &pl = plans[a * s + b];
+      if (!pl.taps) continue;
+      const int K = g.O * pl.nu * pl.nv, N = g.imgs * pl.hp * pl.wp, M = g.C;
+      float *wp = wscratch + woff;          // every phase uses its own part of the re-laid filter
+      woff += static_cast<int64_t>(M) * K;
+      hipLaunchKernelGGL(filter_phase_kernel, dim3((M * K + 255) / 256), dim3(256), 0, st, w, wp, g.O, g.C, g.kH, g.kW,
+                         a, b, s, pl.nu, pl.nv);
+      typename AL::Params ap{wp, K, M, K % 4 == 0 && aligned16(wp)};
+      typename BL::Params bp{dy, pl.taps, FastDiv(pl.hp * pl.wp), FastDiv(pl.wp), static_cast<int64_t>(g.O) * g.oH * g.oW,
+                             g.oH, g.oW, pl.shift_r, pl.shift_c, 1, N};
+      PhaseCols cm{FastDiv(pl.hp * pl.wp), FastDiv(pl.wp), static_cast<int64_t>(g.C) * g.H * g.W, pl.a0, pl.b0, s, g.W};
+      const int tn = (N + BN - 1) / BN, tm = (M + BM - 1) / BM;
+      hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, PhaseCols>), dim3(grid_blocks(tm, tn, 1)),
+                         dim3(kThreads), 0, st, ap, bp, dx, int64_t(0), static_cast<int64_t>(g.H) * g.W, cm, M, N, K,
+                         (K + BK - 1) / BK * BK, TileGrid{tm, tn, tm * tn});
+    }
+  return 0;
+}
+
 // stride-1 bwd-data with the tap-major reduction order; wt is the filter re-laid as [C][kHW][O]
 template <int BM, int BN, int WM, int WN>
 void launch_bwd_data_tap_major(const ConvGeo &g, const float *wt, const float *dy, float *dx, hipStream_t st) {
@@ -1200,7 +1339,7 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
   hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>), dim3(grid), dim3(kThreads), 0, st, P, out, pieces,
                      sk);
   if (pieces)
-    hipLaunchKernelGGL((conv_tap_assemble_kernel<BM, BN, WM, WN>), dim3(tiles), dim3(kThreads), 0, st, P, out, pieces,
+    hipLaunchKernelGGL((conv_tap_assemble_kernel<BM, BN, WM, WN>), dim3(tiles * 4), dim3(kThreads), 0, st, P, out, pieces,
                        sk);
   return 0;
 }
@@ -1538,15 +1677,22 @@ int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray 
         launch_bwd_data_tap_major<128, 128, 2, 2>(g, wt, cf(dy), mf(dx), st);
       }
     } else {
-      // taps index dy: off = o*oH*oW (the spatial part is recomputed because of the stride test)
-      const Tap *taps = tap_table(g.O, g.kH, g.kW, 0, g.oH * g.oW, 0);
-      TS_REQUIRE(taps, "%s: could not build the tap table", who);
-      hipLaunchKernelGGL(filter_oc_swap_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
-                         g.kH * g.kW);
-      if (g.C <= 64)
-        launch_bwd_data<64, 256, 1, 4>(g, wt, cf(dy), mf(dx), taps, st);
-      else
-        launch_bwd_data<128, 128, 2, 2>(g, wt, cf(dy), mf(dx), taps, st);
+      if (g.s > 1) {
+        // the sub-filters of all phases together hold every filter element once
+        const int rc = g.C <= 64 ? launch_bwd_data_phases<64, 256, 1, 4>(g, cf(w), cf(dy), mf(dx), wt, st)
+                                 : launch_bwd_data_phases<128, 128, 2, 2>(g, cf(w), cf(dy), mf(dx), wt, st);
+        if (rc) return rc;
+      } else {
+        // taps index dy: off = o*oH*oW (the spatial part is recomputed because of the stride test)
+        const Tap *taps = tap_table(g.O, g.kH, g.kW, 0, g.oH * g.oW, 0);
+        TS_REQUIRE(taps, "%s: could not build the tap table", who);
+        hipLaunchKernelGGL(filter_oc_swap_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
+                           g.kH * g.kW);
+        if (g.C <= 64)
+          launch_bwd_data<64, 256, 1, 4>(g, wt, cf(dy), mf(dx), taps, st);
+        else
+          launch_bwd_data<128, 128, 2, 2>(g, wt, cf(dy), mf(dx), taps, st);
+      }
     }
   }
   return ps.finish();
