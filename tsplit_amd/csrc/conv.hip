@@ -964,16 +964,28 @@ __global__ __launch_bounds__(256) void filter_tap_major_kernel(const float *__re
 
 // split-K fold for the tap-major bwd-filter: part[z][o][tap][c] summed over z (ascending, so the
 // result does not depend on scheduling) and written as dw[o][c][tap]
+// A block folds 64 outputs with 4 slice-lanes each (lane l adds slices l, l + 4, ...), combined
+// through LDS in a fixed order.
 __global__ __launch_bounds__(256) void fold_tap_major_kernel(const float *__restrict__ part, float *__restrict__ dw,
                                                              int O, int C, int kHW, int64_t stride, int S) {
-  const int idx = blockIdx.x * 256 + threadIdx.x;     // index into one partial: (o*kHW + tap)*C + c
-  if (idx >= O * C * kHW) return;
-  float acc = part[idx];
-  for (int z = 1; z < S; ++z) acc += part[z * stride + idx];
-  const int c = idx % C;
-  const int t = idx / C;
-  const int tap = t % kHW, o = t / kHW;
-  dw[(o * C + c) * kHW + tap] = acc;
+  __shared__ float sm[3][64];
+  const int cx = threadIdx.x & 63, ry = threadIdx.x >> 6;
+  const int idx = blockIdx.x * 64 + cx;                // index into one partial: (o*kHW + tap)*C + c
+  const bool live = idx < O * C * kHW;
+  float acc = 0.f;
+  if (live) {
+#pragma unroll 4
+    for (int z = ry; z < S; z += 4) acc += part[z * stride + idx];
+  }
+  if (ry > 0) sm[ry - 1][cx] = acc;
+  __syncthreads();
+  if (ry == 0 && live) {
+    acc = ((acc + sm[0][cx]) + sm[1][cx]) + sm[2][cx];
+    const int c = idx % C;
+    const int t = idx / C;
+    const int tap = t % kHW, o = t / kHW;
+    dw[(o * C + c) * kHW + tap] = acc;
+  }
 }
 
 // ------------------------------------------------------------------ host side
@@ -1264,7 +1276,7 @@ int launch_bwd_filter_tap_major(const ConvGeo &g, const float *x, const float *d
   hipLaunchKernelGGL((mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>), dim3(grid_blocks(tm, tn, S)),
                      dim3(kThreads), 0, st, ap, bp, part, mn, static_cast<int64_t>(N), RowMajorCols{}, M, N, K, kchunk,
                      TileGrid{tm, tn, tm * tn * S});
-  hipLaunchKernelGGL(fold_tap_major_kernel, dim3(static_cast<unsigned>((mn + 255) / 256)), dim3(256), 0, st, part, dw,
+  hipLaunchKernelGGL(fold_tap_major_kernel, dim3(static_cast<unsigned>((mn + 63) / 64)), dim3(256), 0, st, part, dw,
                      g.O, g.C, g.kH * g.kW, mn, S);
   return 0;
 }
@@ -1379,7 +1391,7 @@ int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *d
   *ws_elems = S * mn;
   hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN>), dim3(grid_blocks(tm, tn, S)), dim3(kThreads), 0, st, P,
                      part, TileGrid{tm, tn, tm * tn * S});
-  hipLaunchKernelGGL(fold_tap_major_kernel, dim3(static_cast<unsigned>((mn + 255) / 256)), dim3(256), 0, st, part, dw,
+  hipLaunchKernelGGL(fold_tap_major_kernel, dim3(static_cast<unsigned>((mn + 63) / 64)), dim3(256), 0, st, part, dw,
                      g.O, g.C, g.kH * g.kW, mn, S);
   return 0;
 }
