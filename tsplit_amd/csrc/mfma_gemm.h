@@ -343,7 +343,7 @@ inline void plan_splitk(int tiles, int K, int max_split, int blocks_per_cu, int 
   const int target = 256 * (blocks_per_cu > 0 ? blocks_per_cu : 2);
   int s = tiles >= target ? 1 : target / tiles;
   const int ksteps = (K + BK - 1) / BK;
-  if (s > ksteps / 4) s = ksteps / 4;   // at least 4 k-steps per split
+  if (s > ksteps / 16) s = ksteps / 16;   // at least 16 k-steps per split: shorter ones are all prologue and epilogue
   if (s > max_split) s = max_split;
   if (s < 1) s = 1;
   int per = (ksteps + s - 1) / s;

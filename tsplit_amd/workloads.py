@@ -52,6 +52,7 @@ class Binder(object):
     def __init__(self, tape, store):
         self.t, self.store, self.vars = tape, store, collections.OrderedDict()
         self._n = 0
+        self._consts = {}
 
     def unique(self, prefix):
         self._n += 1
@@ -67,6 +68,14 @@ class Binder(object):
     def input(self, array):
         a = np.ascontiguousarray(array, dtype=np.float32)
         return self.t.const(self.t.b.from_numpy(a), a.shape)
+
+    def constant(self, key, make):
+        """A constant tensor built and uploaded once per binder: make() -> numpy array."""
+        if key not in self._consts:
+            a = np.ascontiguousarray(make(), dtype=np.float32)
+            self._consts[key] = (self.t.b.from_numpy(a), a.shape)
+        value, shape = self._consts[key]
+        return self.t.const(value, shape)
 
     def grads(self):
         """name -> numpy gradient of every trainable parameter that received one."""
@@ -226,7 +235,7 @@ def _dense(t, b, x, fan_in, fan_out, relu=False):
 
 
 def _const_full(t, b, value, shape):
-    one = b.input(np.full((1,), value, np.float32))
+    one = b.constant(("scalar", float(value)), lambda: np.full((1,), value, np.float32))
     return t.broadcast_like(one, shape)
 
 
@@ -251,7 +260,7 @@ def _attention(t, b, cfg, queries, keys, values, mask_ids, causal):
         m = t.reshape(m, (N, 1, 1, tk))
         scores = t.add(scores, t.broadcast_like(m, scores.shape))
     if causal:
-        tril = b.input(np.tril(np.ones((tq, tk), np.float32)))
+        tril = b.constant(("tril", tq, tk), lambda: np.tril(np.ones((tq, tk), np.float32)))
         future = t.broadcast_like(tril, scores.shape)
         scores = t.where(future, scores, _const_full(t, b, cfg.mask_value, scores.shape))
     ctx = t.batch_matmul(scores, v)                                                     # [N,h,tq,dh]
@@ -268,12 +277,15 @@ def _ffn(t, b, cfg, x):
 
 def _positions(t, b, ids, length, d, amplitude):
     """examples/transformer.py:189-212: sinusoids, zeroed where the token id is 0."""
-    pos = np.array([[p / np.power(10000.0, (i & -2) / float(d)) for i in range(d)] for p in range(length)])
-    pos[:, 0::2] = np.sin(pos[:, 0::2])
-    pos[:, 1::2] = np.cos(pos[:, 1::2])
     n = ids.shape[0]
-    enc = b.input(np.tile((amplitude * pos[None]).astype(np.float32), (n, 1, 1)))
-    zeros = b.input(np.zeros((n, length, d), np.float32))
+
+    def table():
+        pos = np.array([[p / np.power(10000.0, (i & -2) / float(d)) for i in range(d)] for p in range(length)])
+        pos[:, 0::2] = np.sin(pos[:, 0::2])
+        pos[:, 1::2] = np.cos(pos[:, 1::2])
+        return np.tile((amplitude * pos[None]).astype(np.float32), (n, 1, 1))
+    enc = b.constant(("pos", n, length, d, float(amplitude)), table)
+    zeros = b.constant(("zeros", n, length, d), lambda: np.zeros((n, length, d), np.float32))
     cond = t.broadcast_like(t.reshape(ids, (n, length, 1)), (n, length, d))
     return t.where(cond, enc, zeros)
 
