@@ -62,27 +62,37 @@ int current_or(int dev) {
 // ---------------------------------------------------------------- host memory
 // Host tensors are pinned when a device is present (the reference's GPU build does the
 // same: src/common/cpu_device_api.cc:30-36) so that stream copies really are asynchronous;
-// on a machine without a device they are plain aligned memory.
+// on a machine without a device they are plain aligned memory.  With MEMORY_MANAGE_RULE != 0
+// they come from a pool of pinned slabs (same best-fit core as the device pool): pinning costs
+// hundreds of microseconds per call, and an executor that swaps tensors out and in allocates a
+// host buffer per tensor and step.  Rule 0 pins and unpins per tensor.
 std::set<void *> g_pinned;
 
-void *host_alloc(size_t bytes) {
+bool have_device() {
+  static const bool yes = [] {
+    int n = 0;
+    const bool ok = hipGetDeviceCount(&n) == hipSuccess && n > 0;
+    if (!ok) (void)hipGetLastError();
+    return ok;
+  }();
+  return yes;
+}
+
+void *host_raw_alloc(size_t bytes) {
   if (bytes == 0) bytes = 4;
   void *p = nullptr;
-  int n = 0;
-  if (hipGetDeviceCount(&n) == hipSuccess && n > 0) {
+  if (have_device()) {
     if (hipHostMalloc(&p, bytes, hipHostMallocDefault) == hipSuccess) {
       g_pinned.insert(p);
       return p;
     }
-    (void)hipGetLastError();
-  } else {
     (void)hipGetLastError();
   }
   if (posix_memalign(&p, 256, bytes) != 0) return nullptr;
   return p;
 }
 
-void host_free(void *p) {
+void host_raw_free(void *p) {
   auto it = g_pinned.find(p);
   if (it != g_pinned.end()) {
     g_pinned.erase(it);
@@ -92,11 +102,33 @@ void host_free(void *p) {
   }
 }
 
+void *host_slab_alloc(size_t bytes, void *) { return host_raw_alloc(bytes); }
+void host_slab_release(void *p, void *) { host_raw_free(p); }
+size_t host_slab_available(void *) { return ~size_t(0) >> 1; }
+
+BinnedPool *host_pool() {
+  static BinnedPool *pool = new BinnedPool(PoolBacking{host_slab_alloc, host_slab_release, host_slab_available, nullptr},
+                                           env_bytes("TSPLIT_HOST_POOL_SLAB_BYTES", 256ull << 20),
+                                           env_bytes("TSPLIT_HOST_POOL_LIMIT_BYTES", ~size_t(0)));
+  return pool;
+}
+
+void *host_alloc(size_t bytes, int rule) { return rule != 0 ? host_pool()->Malloc(bytes) : host_raw_alloc(bytes); }
+
+void host_free(void *p, int rule) {
+  if (rule != 0 && host_pool()->Free(p)) return;
+  host_raw_free(p);
+}
+
 size_t byte_size(const DLArray *a) { return static_cast<size_t>(numel(a)) * 4; }
 
 void *data_alloc(DLContext ctx, size_t bytes, int rule) {
   std::lock_guard<std::mutex> lk(g_mu);
-  if (ctx.device_type == kCPU) return host_alloc(bytes);
+  if (ctx.device_type == kCPU) {
+    void *hp = host_alloc(bytes, rule);
+    if (!hp) throw std::runtime_error("out of host memory");
+    return hp;
+  }
   if (ctx.device_type != kGPU) throw std::runtime_error("unknown device type");
   current_or(ctx.device_id);
   void *p = nullptr;
@@ -116,7 +148,7 @@ void data_free(DLContext ctx, void *p, int rule) {
   if (!p) return;
   std::lock_guard<std::mutex> lk(g_mu);
   if (ctx.device_type == kCPU) {
-    host_free(p);
+    host_free(p, rule);
     return;
   }
   current_or(ctx.device_id);
