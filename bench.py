@@ -81,6 +81,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-split", action="store_true")
     ap.add_argument("--no-events", action="store_true", help="time the steps without per-launch events")
+    ap.add_argument("--fused", action="store_true",
+                    help="run every BatchNorm+Relu pair through the fused symbols (outside the reference's ABI)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build is single-GPU by design (no collectives, no sharding); run with --gpus 1. "
@@ -93,7 +95,8 @@ def main():
     if a.no_split:
         split = {}
     timer = None if a.no_events else EventTimer(ctx)
-    t = trainer.Trainer(spec, params, x.shape, 1000, ctx, optimizer=("momentum", 1e-4, 0.9), split=split, timer=timer)
+    t = trainer.Trainer(spec, params, x.shape, 1000, ctx, optimizer=("momentum", 1e-4, 0.9), split=split, timer=timer,
+                        fuse_bn_relu=a.fused)
     gx, gy = ndarray.array(x, ctx), ndarray.array(labels, ctx)      # resident before timing
     for _ in range(a.warmup):
         t.step(gx, gy)
@@ -114,8 +117,9 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "VGG-16 training step (fwd+bwd+momentum SGD), fp32 NCHW, batch %d, 3x224x224, "
-                               "1000 classes, He init, %s" % (a.batch, "4 batch micro-tensors on the 4 largest conv layers"
-                                                              if split else "no micro-tensor split"),
+                               "1000 classes, He init, %s%s" % (a.batch, "4 batch micro-tensors on the 4 largest conv layers"
+                                                                if split else "no micro-tensor split",
+                                                                ", BatchNorm+Relu pairs fused" if a.fused else ""),
                    "global_batch": a.batch, "final_loss": loss},
     }
     if timer:

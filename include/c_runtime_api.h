@@ -359,6 +359,25 @@ int DLGpuTanh(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle st
 int DLGpuSigmoid(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle,
                  ProfilerHandle p);
 
+/* ---- Fused BatchNorm + Relu.  NO counterpart in the reference (its ABI has one symbol per graph
+ *      node); for hosts that know the Relu follows the BatchNorm and want to skip its two passes
+ *      over the activation.  Forward: output_Y = max(BN(input_X), 0); both save arrays are
+ *      required and receive (batch mean, 1/sqrt(var+eps)).  Gradient: gradient_Y is the gradient
+ *      behind the Relu; it is gated with the reference's Relu derivative (sign(z)+1)/2 of
+ *      z = BN(input_X), rebuilt from input_X, bn_scale, bn_bias and the saved statistics of the
+ *      fused forward call, then the BatchNorm gradient is taken.  Results equal the two-call
+ *      sequence (same float expressions). ---- */
+int TSplit_BatchNormRelu(const DLArrayHandle input_X, const DLArrayHandle bn_scale,
+                         const DLArrayHandle bn_bias, DLArrayHandle output_Y, float eps,
+                         DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                         DLStreamHandle stream_handle, ProfilerHandle p);
+int TSplit_BatchNormRelu_gradient(const DLArrayHandle gradient_Y, const DLArrayHandle input_X,
+                                  const DLArrayHandle bn_scale, const DLArrayHandle bn_bias,
+                                  DLArrayHandle gradient_X, DLArrayHandle gradient_bn_scale,
+                                  DLArrayHandle gradient_bn_bias, float eps,
+                                  DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                                  DLStreamHandle stream_handle, ProfilerHandle p);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

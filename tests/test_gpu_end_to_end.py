@@ -44,8 +44,8 @@ def _small_convnet():
             ("flatten",), ("fc", "f1", 16 * 4 * 4, 32), ("fc", "f2", 32, 10)]
 
 
-@pytest.mark.parametrize("split", [None, {0: 4, 3: 4}, {3: 3}])
-def test_convnet_momentum_tracks_oracle_with_and_without_split(split):
+@pytest.mark.parametrize("split,fuse", [(None, False), ({0: 4, 3: 4}, False), ({3: 3}, False), (None, True), ({0: 4, 3: 4}, True)])
+def test_convnet_momentum_tracks_oracle_with_and_without_split(split, fuse):
     from tsplit_amd import ndarray, trainer
     rng = np.random.RandomState(7)
     spec = _small_convnet()
@@ -54,7 +54,8 @@ def test_convnet_momentum_tracks_oracle_with_and_without_split(split):
     params = trainer.init_params(spec, seed=5)
     ref_losses, ref_params = nets.train(spec, params, X, Y, steps=6, lr=0.05, momentum=0.9)
     ctx = ndarray.gpu(0)
-    t = trainer.Trainer(spec, params, X.shape, 10, ctx, optimizer=("momentum", 0.05, 0.9), split=split)
+    t = trainer.Trainer(spec, params, X.shape, 10, ctx, optimizer=("momentum", 0.05, 0.9), split=split,
+                        fuse_bn_relu=fuse)
     gx, gy = ndarray.array(X, ctx), ndarray.array(Y, ctx)
     losses = []
     for _ in range(6):

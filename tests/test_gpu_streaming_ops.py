@@ -292,3 +292,47 @@ def test_pool_and_profiler_and_events(ts, rng):
     back.async_d2h(dev, ts.stream, dev.gpu2cpu_event)
     dev.gpu2cpu_event.sync()
     np.testing.assert_array_equal(back.asnumpy(), host.asnumpy())
+
+
+@pytest.mark.parametrize("shape", [(4, 8, 6, 6), (3, 5, 7, 9), (16, 64, 56, 56)])
+def test_fused_batchnorm_relu_equals_the_two_call_sequence(ts, shape, rng):
+    """The fused symbols have no counterpart in the reference; their contract is to reproduce
+    BatchNorm followed by Relu (and the reverse sweep) exactly, and through them the oracle."""
+    C = shape[1]
+    x = rng.normal(size=shape).astype(np.float32)
+    gamma = (1 + 0.1 * rng.normal(size=(1, C, 1, 1))).astype(np.float32)
+    beta = (0.1 * rng.normal(size=(1, C, 1, 1))).astype(np.float32)
+    dy = rng.normal(size=shape).astype(np.float32)
+    L, s = ts.links, ts.stream
+    gx, gg, gb, gdy = ts.arr(x), ts.arr(gamma), ts.arr(beta), ts.arr(dy)
+    # two calls per direction
+    sm, sv = ts.empty((1, C, 1, 1)), ts.empty((1, C, 1, 1))
+    y_bn, y = ts.empty(shape), ts.empty(shape)
+    L.CuDNN_Batch_Normalization(gx, gg, gb, y_bn, sm, sv, 0.99, 0.01, s)
+    L.relu(y_bn, y, s)
+    d_bn, dx, dg, db = ts.empty(shape), ts.empty(shape), ts.empty((1, C, 1, 1)), ts.empty((1, C, 1, 1))
+    L.relu_gradient(y_bn, gdy, d_bn, s)
+    L.CuDNN_Batch_Normalization_gradient(d_bn, gx, gg, dx, dg, db, sm, sv, 0.01, s)
+    # one call per direction
+    fm, fv = ts.empty((1, C, 1, 1)), ts.empty((1, C, 1, 1))
+    fy, fdx, fdg, fdb = ts.empty(shape), ts.empty(shape), ts.empty((1, C, 1, 1)), ts.empty((1, C, 1, 1))
+    L.batch_norm_relu(gx, gg, gb, fy, fm, fv, 0.01, s)
+    L.batch_norm_relu_gradient(gdy, gx, gg, gb, fdx, fdg, fdb, fm, fv, 0.01, s)
+    ref_y = O.relu(O.batchnorm_forward(x, gamma, beta, 0.01)[0])
+    assert_close(fy.asnumpy(), ref_y, TOL, "bn+relu")
+    assert_close(fy.asnumpy(), y.asnumpy(), 1e-6, "fused vs two calls, forward")
+    # the Relu gate is discontinuous at 0: compare where the pre-activation is clearly off zero
+    z = O.batchnorm_forward(x, gamma, beta, 0.01)[0]
+    g = O.relu_grad(z, dy)
+    rdx, rdg, rdb = O.batchnorm_backward(g, x, gamma, 0.01)
+    assert_close(fdx.asnumpy(), rdx, 5e-4, "bn+relu dx")
+    assert_close(fdg.asnumpy().ravel(), rdg.ravel(), 5e-4, "bn+relu dgamma")
+    assert_close(fdb.asnumpy().ravel(), rdb.ravel(), 5e-4, "bn+relu dbeta")
+    assert_close(fdx.asnumpy(), dx.asnumpy(), 5e-4, "fused vs two calls, dx")
+    np.testing.assert_allclose(fm.asnumpy(), sm.asnumpy(), rtol=1e-6)
+
+
+def test_fused_batchnorm_relu_needs_saved_statistics(ts):
+    x, g, b, y = ts.empty((2, 3, 4, 4)), ts.empty((1, 3, 1, 1)), ts.empty((1, 3, 1, 1)), ts.empty((2, 3, 4, 4))
+    with pytest.raises(Exception):
+        ts.links.batch_norm_relu(x, g, b, y, None, None, 0.01, ts.stream)

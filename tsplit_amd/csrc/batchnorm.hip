@@ -6,6 +6,8 @@
 //             [apply]  every block folds the partials of its channel, then y = a*x + b
 //   backward: [reduce] partial (sum dy, sum dy*x, sum x, sum x^2)   -> scratch (double)
 //             [dx]     folds them, then dx = k1*dy + k2*x + k3; split 0 writes dgamma/dbeta
+// Fused forms (TSplit_BatchNormRelu*): the apply pass stores max(a*x + b, 0) and the backward
+// passes gate dy with relu'(a*x + b) recomputed from x, so the Relu costs no pass of its own.
 // Threads walk a per-channel virtual index (in 16-byte words when H*W % 4 == 0) that is
 // mapped to (plane, offset) with a multiply-shift division, so consecutive lanes read
 // consecutive words of one plane.  Per-thread accumulation is float32 over a few hundred
@@ -71,6 +73,23 @@ __device__ __forceinline__ f32x4 axpb(const f32x4 &x, float a, float b) {
   return r;
 }
 __device__ __forceinline__ float axpb(const float &x, float a, float b) { return a * x + b; }
+// Relu and its reference gradient factor (sign(z)+1)/2 (0.5 at z == 0)
+__device__ __forceinline__ float relu1(float z) { return fmaxf(z, 0.f); }
+__device__ __forceinline__ f32x4 relu_w(const f32x4 &z) {
+  const f32x4 r = {relu1(z.x), relu1(z.y), relu1(z.z), relu1(z.w)};
+  return r;
+}
+__device__ __forceinline__ float relu_w(const float &z) { return relu1(z); }
+__device__ __forceinline__ float gate1(float z) { return z > 0.f ? 1.f : (z < 0.f ? 0.f : 0.5f); }
+// dy * relu'(a*x + b)
+__device__ __forceinline__ f32x4 gated(const f32x4 &dy, const f32x4 &x, float a, float b) {
+  const f32x4 r = {dy.x * gate1(a * x.x + b), dy.y * gate1(a * x.y + b), dy.z * gate1(a * x.z + b),
+                   dy.w * gate1(a * x.w + b)};
+  return r;
+}
+__device__ __forceinline__ float gated(const float &dy, const float &x, float a, float b) {
+  return dy * gate1(a * x + b);
+}
 __device__ __forceinline__ f32x4 lin2(const f32x4 &dy, const f32x4 &x, float k1, float k2, float k3) {
   const f32x4 r = {k1 * dy.x + k2 * x.x + k3, k1 * dy.y + k2 * x.y + k3, k1 * dy.z + k2 * x.z + k3,
                    k1 * dy.w + k2 * x.w + k3};
@@ -108,7 +127,7 @@ __global__ __launch_bounds__(kThreads) void bn_stats_kernel(const float *__restr
   }
 }
 
-template <int VEC>
+template <int VEC, bool RELU>
 __global__ __launch_bounds__(kThreads) void bn_apply_kernel(const float *__restrict__ x, float *__restrict__ y,
                                                             const float *__restrict__ gamma,
                                                             const float *__restrict__ beta,
@@ -132,10 +151,17 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(const float *__restr
     const double mean = s * inv_m;
     double var = q * inv_m - mean * mean;
     if (var < 0.0) var = 0.0;
-    const double istd = 1.0 / sqrt(var + static_cast<double>(eps));
+    double istd = 1.0 / sqrt(var + static_cast<double>(eps));
+    double mean_used = mean;
+    if (RELU) {
+      // the fused backward pass rebuilds a and b from the saved float statistics and must see
+      // the same sign of a*x + b: derive the coefficients from the rounded values here too
+      mean_used = static_cast<double>(static_cast<float>(mean));
+      istd = static_cast<double>(static_cast<float>(istd));
+    }
     const double a = static_cast<double>(gamma[c]) * istd;
     coef[0] = static_cast<float>(a);
-    coef[1] = static_cast<float>(static_cast<double>(beta[c]) - mean * a);
+    coef[1] = static_cast<float>(static_cast<double>(beta[c]) - mean_used * a);
     if (blockIdx.x == 0) {
       if (save_mean) save_mean[c] = static_cast<float>(mean);
       if (save_istd) save_istd[c] = static_cast<float>(istd);
@@ -152,23 +178,37 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(const float *__restr
   for (; i + kThreads < end; i += 2 * kThreads) {
     const int64_t a0 = word_addr<VEC>(g, i, c), a1 = word_addr<VEC>(g, i + kThreads, c);
     const W v0 = __builtin_nontemporal_load(xw + a0), v1 = __builtin_nontemporal_load(xw + a1);
-    __builtin_nontemporal_store(axpb(v0, a, b), yw + a0);
-    __builtin_nontemporal_store(axpb(v1, a, b), yw + a1);
+    __builtin_nontemporal_store(RELU ? relu_w(axpb(v0, a, b)) : axpb(v0, a, b), yw + a0);
+    __builtin_nontemporal_store(RELU ? relu_w(axpb(v1, a, b)) : axpb(v1, a, b), yw + a1);
   }
   for (; i < end; i += kThreads) {
     const int64_t a0 = word_addr<VEC>(g, i, c);
-    __builtin_nontemporal_store(axpb(__builtin_nontemporal_load(xw + a0), a, b), yw + a0);
+    const W z = axpb(__builtin_nontemporal_load(xw + a0), a, b);
+    __builtin_nontemporal_store(RELU ? relu_w(z) : z, yw + a0);
   }
 }
 
 // partials per block: sum dy, sum dy*x, sum x, sum x^2
-template <int VEC, bool STATS>
+// RELU: dy is the gradient behind a fused Relu; it is gated with relu'(a*x + b), a and b rebuilt
+// from the saved statistics (gamma, beta, save_mean, save_istd must be given).
+template <int VEC, bool STATS, bool RELU>
 __global__ __launch_bounds__(kThreads) void bn_bwd_reduce_kernel(const float *__restrict__ dy,
                                                                  const float *__restrict__ x,
-                                                                 double *__restrict__ part, Geo g, int S) {
+                                                                 double *__restrict__ part, Geo g, int S,
+                                                                 const float *__restrict__ gamma,
+                                                                 const float *__restrict__ beta,
+                                                                 const float *__restrict__ save_mean,
+                                                                 const float *__restrict__ save_istd) {
   using W = typename Word<VEC>::T;
   __shared__ double sm[kWaves];
   const int c = blockIdx.y, s = blockIdx.x;
+  float ga = 0.f, gb = 0.f;
+  if (RELU) {
+    // the same float expressions as the forward pass, so that the sign of a*x + b is the same
+    const double a = static_cast<double>(gamma[c]) * static_cast<double>(save_istd[c]);
+    ga = static_cast<float>(a);
+    gb = static_cast<float>(static_cast<double>(beta[c]) - static_cast<double>(save_mean[c]) * a);
+  }
   const uint32_t begin = s * g.chunk;
   const uint32_t end = min(begin + g.chunk, g.words);
   const W *xw = reinterpret_cast<const W *>(x);
@@ -178,6 +218,10 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_reduce_kernel(const float *__
   for (; i + kThreads < end; i += 2 * kThreads) {
     const int64_t a0 = word_addr<VEC>(g, i, c), a1 = word_addr<VEC>(g, i + kThreads, c);
     W x0 = xw[a0], d0 = dw[a0], x1 = xw[a1], d1 = dw[a1];
+    if (RELU) {
+      d0 = gated(d0, x0, ga, gb);
+      d1 = gated(d1, x1, ga, gb);
+    }
     acc_dot(d0, x0, sdy, sdx);
     acc_dot(d1, x1, sdy, sdx);
     if (STATS) {
@@ -188,6 +232,7 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_reduce_kernel(const float *__
   for (; i < end; i += kThreads) {
     const int64_t a0 = word_addr<VEC>(g, i, c);
     W x0 = xw[a0], d0 = dw[a0];
+    if (RELU) d0 = gated(d0, x0, ga, gb);
     acc_dot(d0, x0, sdy, sdx);
     if (STATS) acc2(x0, sx, sq);
   }
@@ -207,15 +252,16 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_reduce_kernel(const float *__
   }
 }
 
-template <int VEC>
+template <int VEC, bool RELU>
 __global__ __launch_bounds__(kThreads) void bn_bwd_dx_kernel(const float *__restrict__ dy, const float *__restrict__ x,
                                                              float *__restrict__ dx, const float *__restrict__ gamma,
                                                              const double *__restrict__ part, int S, Geo g, float eps,
                                                              double inv_m, const float *__restrict__ save_mean,
                                                              const float *__restrict__ save_istd,
-                                                             float *__restrict__ dgamma, float *__restrict__ dbeta) {
+                                                             float *__restrict__ dgamma, float *__restrict__ dbeta,
+                                                             const float *__restrict__ beta) {
   using W = typename Word<VEC>::T;
-  __shared__ float coef[3];
+  __shared__ float coef[5];
   __shared__ double sm[kWaves];
   const int c = blockIdx.y;
   double sdy = 0.0, sdx = 0.0, sx = 0.0, sq = 0.0;
@@ -251,6 +297,10 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_dx_kernel(const float *__rest
     coef[0] = static_cast<float>(k1);
     coef[1] = static_cast<float>(k2);
     coef[2] = static_cast<float>(k3);
+    if (RELU) {
+      coef[3] = static_cast<float>(k1);   // a = gamma * istd
+      coef[4] = static_cast<float>(static_cast<double>(beta[c]) - mean * k1);
+    }
     if (blockIdx.x == 0) {
       if (dgamma) dgamma[c] = static_cast<float>(dscale);
       if (dbeta) dbeta[c] = static_cast<float>(dbias);
@@ -258,6 +308,7 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_dx_kernel(const float *__rest
   }
   __syncthreads();
   const float k1 = coef[0], k2 = coef[1], k3 = coef[2];
+  const float ga = RELU ? coef[3] : 0.f, gb = RELU ? coef[4] : 0.f;
   const uint32_t begin = blockIdx.x * g.chunk;
   const uint32_t end = min(begin + g.chunk, g.words);
   const W *xw = reinterpret_cast<const W *>(x);
@@ -268,13 +319,13 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_dx_kernel(const float *__rest
     const int64_t a0 = word_addr<VEC>(g, i, c), a1 = word_addr<VEC>(g, i + kThreads, c);
     const W x0 = __builtin_nontemporal_load(xw + a0), d0 = __builtin_nontemporal_load(dw + a0);
     const W x1 = __builtin_nontemporal_load(xw + a1), d1 = __builtin_nontemporal_load(dw + a1);
-    __builtin_nontemporal_store(lin2(d0, x0, k1, k2, k3), ow + a0);
-    __builtin_nontemporal_store(lin2(d1, x1, k1, k2, k3), ow + a1);
+    __builtin_nontemporal_store(lin2(RELU ? gated(d0, x0, ga, gb) : d0, x0, k1, k2, k3), ow + a0);
+    __builtin_nontemporal_store(lin2(RELU ? gated(d1, x1, ga, gb) : d1, x1, k1, k2, k3), ow + a1);
   }
   for (; i < end; i += kThreads) {
     const int64_t a0 = word_addr<VEC>(g, i, c);
-    __builtin_nontemporal_store(lin2(__builtin_nontemporal_load(dw + a0), __builtin_nontemporal_load(xw + a0), k1, k2, k3),
-                                ow + a0);
+    const W x0 = __builtin_nontemporal_load(xw + a0), d0 = __builtin_nontemporal_load(dw + a0);
+    __builtin_nontemporal_store(lin2(RELU ? gated(d0, x0, ga, gb) : d0, x0, k1, k2, k3), ow + a0);
   }
 }
 
@@ -320,39 +371,120 @@ using namespace tsplit;
 
 extern "C" {
 
-int CuDNN_DLGpuBatch_Normalization(const DLArrayHandle input_X, const DLArrayHandle bn_scale,
-                                   const DLArrayHandle bn_bias, DLArrayHandle output_Y, float momentum, float eps,
-                                   DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
-                                   DLStreamHandle stream_handle, ProfilerHandle p) {
-  (void)momentum;
-  TS_REQUIRE(input_X && bn_scale && bn_bias && output_Y, "BatchNorm: NULL array");
-  TS_REQUIRE(input_X->ndim == 4 && output_Y->ndim == 4, "BatchNorm: input and output must be 4-D NCHW");
-  TS_REQUIRE(numel(input_X) == numel(output_Y), "BatchNorm: input/output sizes differ");
+static int bn_forward(const char *who, bool relu, const DLArrayHandle input_X, const DLArrayHandle bn_scale,
+                      const DLArrayHandle bn_bias, DLArrayHandle output_Y, float eps, DLArrayHandle save_mean_arr,
+                      DLArrayHandle save_var_arr, DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(input_X && bn_scale && bn_bias && output_Y, "%s: NULL array", who);
+  TS_REQUIRE(input_X->ndim == 4 && output_Y->ndim == 4, "%s: input and output must be 4-D NCHW", who);
+  TS_REQUIRE(numel(input_X) == numel(output_Y), "%s: input/output sizes differ", who);
   const int64_t C = input_X->shape[1];
-  TS_REQUIRE(numel(bn_scale) == C && numel(bn_bias) == C, "BatchNorm: scale/bias must hold C=%lld elements", (long long)C);
-  TS_REQUIRE(!save_mean_arr || numel(save_mean_arr) == C, "BatchNorm: save_mean must hold C elements");
-  TS_REQUIRE(!save_var_arr || numel(save_var_arr) == C, "BatchNorm: save_var must hold C elements");
+  TS_REQUIRE(numel(bn_scale) == C && numel(bn_bias) == C, "%s: scale/bias must hold C=%lld elements", who, (long long)C);
+  TS_REQUIRE(!save_mean_arr || numel(save_mean_arr) == C, "%s: save_mean must hold C elements", who);
+  TS_REQUIRE(!save_var_arr || numel(save_var_arr) == C, "%s: save_var must hold C elements", who);
+  TS_REQUIRE(!relu || (save_mean_arr && save_var_arr), "%s: the fused form needs both save arrays", who);
   hipStream_t s = stream_of(stream_handle);
   const bool al = aligned16(input_X->data) && aligned16(output_Y->data);
   Plan st, ap;
-  TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 16384, st), "BatchNorm: unsupported shape");
-  TS_REQUIRE(make_plan(input_X, al, 4 * kThreads, 1 << 22, ap), "BatchNorm: unsupported shape");
+  TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 16384, st), "%s: unsupported shape", who);
+  TS_REQUIRE(make_plan(input_X, al, 4 * kThreads, 1 << 22, ap), "%s: unsupported shape", who);
   double *part = static_cast<double *>(scratch_get(s, 1, static_cast<size_t>(C) * st.S * 2 * sizeof(double)));
-  TS_REQUIRE(part, "BatchNorm: no scratch memory");
+  TS_REQUIRE(part, "%s: no scratch memory", who);
   ProfileScope ps(p, s, numel(input_X) + 2 * C, numel(output_Y), C * st.S * 4);
   const double inv_m = 1.0 / static_cast<double>(st.m);
   float *sm = save_mean_arr ? mf(save_mean_arr) : nullptr;
   float *sv = save_var_arr ? mf(save_var_arr) : nullptr;
   dim3 gs(st.S, static_cast<unsigned>(C)), ga(ap.S, static_cast<unsigned>(C));
+#define BN_APPLY(V, R)                                                                                              \
+  hipLaunchKernelGGL((bn_apply_kernel<V, R>), ga, dim3(kThreads), 0, s, cf(input_X), mf(output_Y), cf(bn_scale),    \
+                     cf(bn_bias), part, st.S, ap.g, eps, inv_m, sm, sv)
   if (st.vec == 4) {
     hipLaunchKernelGGL(bn_stats_kernel<4>, gs, dim3(kThreads), 0, s, cf(input_X), part, st.g, st.S);
-    hipLaunchKernelGGL(bn_apply_kernel<4>, ga, dim3(kThreads), 0, s, cf(input_X), mf(output_Y), cf(bn_scale),
-                       cf(bn_bias), part, st.S, ap.g, eps, inv_m, sm, sv);
+    if (relu)
+      BN_APPLY(4, true);
+    else
+      BN_APPLY(4, false);
   } else {
     hipLaunchKernelGGL(bn_stats_kernel<1>, gs, dim3(kThreads), 0, s, cf(input_X), part, st.g, st.S);
-    hipLaunchKernelGGL(bn_apply_kernel<1>, ga, dim3(kThreads), 0, s, cf(input_X), mf(output_Y), cf(bn_scale),
-                       cf(bn_bias), part, st.S, ap.g, eps, inv_m, sm, sv);
+    if (relu)
+      BN_APPLY(1, true);
+    else
+      BN_APPLY(1, false);
   }
+#undef BN_APPLY
+  return ps.finish();
+}
+
+int CuDNN_DLGpuBatch_Normalization(const DLArrayHandle input_X, const DLArrayHandle bn_scale,
+                                   const DLArrayHandle bn_bias, DLArrayHandle output_Y, float momentum, float eps,
+                                   DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                                   DLStreamHandle stream_handle, ProfilerHandle p) {
+  (void)momentum;
+  return bn_forward("BatchNorm", false, input_X, bn_scale, bn_bias, output_Y, eps, save_mean_arr, save_var_arr,
+                    stream_handle, p);
+}
+
+int TSplit_BatchNormRelu(const DLArrayHandle input_X, const DLArrayHandle bn_scale, const DLArrayHandle bn_bias,
+                         DLArrayHandle output_Y, float eps, DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                         DLStreamHandle stream_handle, ProfilerHandle p) {
+  return bn_forward("TSplit_BatchNormRelu", true, input_X, bn_scale, bn_bias, output_Y, eps, save_mean_arr,
+                    save_var_arr, stream_handle, p);
+}
+
+static int bn_backward(const char *who, bool relu, const DLArrayHandle gradient_Y, const DLArrayHandle input_X,
+                       const DLArrayHandle bn_scale, const DLArrayHandle bn_bias, DLArrayHandle gradient_X,
+                       DLArrayHandle gradient_bn_scale, DLArrayHandle gradient_bn_bias, float eps,
+                       DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr, DLStreamHandle stream_handle,
+                       ProfilerHandle p) {
+  TS_REQUIRE(gradient_Y && input_X && bn_scale && gradient_X, "%s: NULL array", who);
+  TS_REQUIRE(input_X->ndim == 4, "%s: input must be 4-D NCHW", who);
+  TS_REQUIRE(numel(input_X) == numel(gradient_Y) && numel(input_X) == numel(gradient_X), "%s: x, dy, dx sizes differ", who);
+  const int64_t C = input_X->shape[1];
+  TS_REQUIRE(numel(bn_scale) == C, "%s: scale must hold C elements", who);
+  TS_REQUIRE(!gradient_bn_scale || numel(gradient_bn_scale) == C, "%s: dscale must hold C elements", who);
+  TS_REQUIRE(!gradient_bn_bias || numel(gradient_bn_bias) == C, "%s: dbias must hold C elements", who);
+  const bool saved = save_mean_arr && save_var_arr;
+  TS_REQUIRE(!saved || (numel(save_mean_arr) == C && numel(save_var_arr) == C),
+             "%s: saved statistics must hold C elements", who);
+  TS_REQUIRE(!relu || (saved && bn_bias && numel(bn_bias) == C),
+             "%s: the fused form needs the bias and the statistics saved by the fused forward call", who);
+  hipStream_t s = stream_of(stream_handle);
+  const bool al = aligned16(input_X->data) && aligned16(gradient_Y->data) && aligned16(gradient_X->data);
+  Plan rd, dxp;
+  TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 16384, rd), "%s: unsupported shape", who);
+  TS_REQUIRE(make_plan(input_X, al, 4 * kThreads, 1 << 22, dxp), "%s: unsupported shape", who);
+  double *part = static_cast<double *>(scratch_get(s, 1, static_cast<size_t>(C) * rd.S * 4 * sizeof(double)));
+  TS_REQUIRE(part, "%s: no scratch memory", who);
+  ProfileScope ps(p, s, 2 * numel(input_X) + C, numel(gradient_X) + 2 * C, C * rd.S * 8);
+  const double inv_m = 1.0 / static_cast<double>(rd.m);
+  const float *sm = saved ? cf(save_mean_arr) : nullptr;
+  const float *sv = saved ? cf(save_var_arr) : nullptr;
+  const float *bias = bn_bias ? cf(bn_bias) : nullptr;
+  float *dg = gradient_bn_scale ? mf(gradient_bn_scale) : nullptr;
+  float *db = gradient_bn_bias ? mf(gradient_bn_bias) : nullptr;
+  dim3 gr(rd.S, static_cast<unsigned>(C)), gd(dxp.S, static_cast<unsigned>(C));
+#define BN_BWD(V, ST, R)                                                                                            \
+  do {                                                                                                              \
+    hipLaunchKernelGGL((bn_bwd_reduce_kernel<V, ST, R>), gr, dim3(kThreads), 0, s, cf(gradient_Y), cf(input_X),     \
+                       part, rd.g, rd.S, cf(bn_scale), bias, sm, sv);                                               \
+    hipLaunchKernelGGL((bn_bwd_dx_kernel<V, R>), gd, dim3(kThreads), 0, s, cf(gradient_Y), cf(input_X),             \
+                       mf(gradient_X), cf(bn_scale), part, rd.S, dxp.g, eps, inv_m, sm, sv, dg, db, bias);          \
+  } while (0)
+  if (rd.vec == 4) {
+    if (relu)
+      BN_BWD(4, false, true);
+    else if (saved)
+      BN_BWD(4, false, false);
+    else
+      BN_BWD(4, true, false);
+  } else {
+    if (relu)
+      BN_BWD(1, false, true);
+    else if (saved)
+      BN_BWD(1, false, false);
+    else
+      BN_BWD(1, true, false);
+  }
+#undef BN_BWD
   return ps.finish();
 }
 
@@ -361,48 +493,17 @@ int CuDNN_DLGpuBatch_Normalization_gradient(const DLArrayHandle gradient_Y, cons
                                             DLArrayHandle gradient_bn_scale, DLArrayHandle gradient_bn_bias,
                                             float eps, DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
                                             DLStreamHandle stream_handle, ProfilerHandle p) {
-  TS_REQUIRE(gradient_Y && input_X && bn_scale && gradient_X, "BatchNorm gradient: NULL array");
-  TS_REQUIRE(input_X->ndim == 4, "BatchNorm gradient: input must be 4-D NCHW");
-  TS_REQUIRE(numel(input_X) == numel(gradient_Y) && numel(input_X) == numel(gradient_X),
-             "BatchNorm gradient: x, dy, dx sizes differ");
-  const int64_t C = input_X->shape[1];
-  TS_REQUIRE(numel(bn_scale) == C, "BatchNorm gradient: scale must hold C elements");
-  TS_REQUIRE(!gradient_bn_scale || numel(gradient_bn_scale) == C, "BatchNorm gradient: dscale must hold C elements");
-  TS_REQUIRE(!gradient_bn_bias || numel(gradient_bn_bias) == C, "BatchNorm gradient: dbias must hold C elements");
-  const bool saved = save_mean_arr && save_var_arr;
-  TS_REQUIRE(!saved || (numel(save_mean_arr) == C && numel(save_var_arr) == C),
-             "BatchNorm gradient: saved statistics must hold C elements");
-  hipStream_t s = stream_of(stream_handle);
-  const bool al = aligned16(input_X->data) && aligned16(gradient_Y->data) && aligned16(gradient_X->data);
-  Plan rd, dxp;
-  TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 16384, rd), "BatchNorm gradient: unsupported shape");
-  TS_REQUIRE(make_plan(input_X, al, 4 * kThreads, 1 << 22, dxp), "BatchNorm gradient: unsupported shape");
-  double *part = static_cast<double *>(scratch_get(s, 1, static_cast<size_t>(C) * rd.S * 4 * sizeof(double)));
-  TS_REQUIRE(part, "BatchNorm gradient: no scratch memory");
-  ProfileScope ps(p, s, 2 * numel(input_X) + C, numel(gradient_X) + 2 * C, C * rd.S * 8);
-  const double inv_m = 1.0 / static_cast<double>(rd.m);
-  const float *sm = saved ? cf(save_mean_arr) : nullptr;
-  const float *sv = saved ? cf(save_var_arr) : nullptr;
-  float *dg = gradient_bn_scale ? mf(gradient_bn_scale) : nullptr;
-  float *db = gradient_bn_bias ? mf(gradient_bn_bias) : nullptr;
-  dim3 gr(rd.S, static_cast<unsigned>(C)), gd(dxp.S, static_cast<unsigned>(C));
-#define BN_BWD(V)                                                                                                   \
-  do {                                                                                                              \
-    if (saved)                                                                                                      \
-      hipLaunchKernelGGL((bn_bwd_reduce_kernel<V, false>), gr, dim3(kThreads), 0, s, cf(gradient_Y), cf(input_X),   \
-                         part, rd.g, rd.S);                                                                         \
-    else                                                                                                            \
-      hipLaunchKernelGGL((bn_bwd_reduce_kernel<V, true>), gr, dim3(kThreads), 0, s, cf(gradient_Y), cf(input_X),    \
-                         part, rd.g, rd.S);                                                                         \
-    hipLaunchKernelGGL(bn_bwd_dx_kernel<V>, gd, dim3(kThreads), 0, s, cf(gradient_Y), cf(input_X), mf(gradient_X),  \
-                       cf(bn_scale), part, rd.S, dxp.g, eps, inv_m, sm, sv, dg, db);                                \
-  } while (0)
-  if (rd.vec == 4)
-    BN_BWD(4);
-  else
-    BN_BWD(1);
-#undef BN_BWD
-  return ps.finish();
+  return bn_backward("BatchNorm gradient", false, gradient_Y, input_X, bn_scale, nullptr, gradient_X, gradient_bn_scale,
+                     gradient_bn_bias, eps, save_mean_arr, save_var_arr, stream_handle, p);
+}
+
+int TSplit_BatchNormRelu_gradient(const DLArrayHandle gradient_Y, const DLArrayHandle input_X,
+                                  const DLArrayHandle bn_scale, const DLArrayHandle bn_bias, DLArrayHandle gradient_X,
+                                  DLArrayHandle gradient_bn_scale, DLArrayHandle gradient_bn_bias, float eps,
+                                  DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                                  DLStreamHandle stream_handle, ProfilerHandle p) {
+  return bn_backward("TSplit_BatchNormRelu_gradient", true, gradient_Y, input_X, bn_scale, bn_bias, gradient_X,
+                     gradient_bn_scale, gradient_bn_bias, eps, save_mean_arr, save_var_arr, stream_handle, p);
 }
 
 }  // extern "C"

@@ -26,6 +26,7 @@ __all__ = [
     "matrix_transpose", "batch_matrix_multiply", "one_hot", "where", "embedding_lookup",
     "embedding_lookup_gradient", "matrix_elementwise_divide", "matrix_elementwise_divide_const",
     "matrix_opposite", "matrix_sqrt", "matrix_rsqrt", "tanh", "sigmoid",
+    "batch_norm_relu", "batch_norm_relu_gradient",
 ]
 
 
@@ -364,3 +365,18 @@ def tanh(in_arr, out_arr, stream=None, profiler=None):
 
 def sigmoid(in_arr, out_arr, stream=None, profiler=None):
     check_call(_LIB.DLGpuSigmoid(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
+
+
+# ---- Fused BatchNorm + Relu (no counterpart in the reference's gpu_links) ----
+def batch_norm_relu(in_arr, bn_scale_arr, bn_bias_arr, out_arr, save_mean, save_var, eps=0.01, stream=None,
+                    profiler=None):
+    check_call(_LIB.TSplit_BatchNormRelu(_h(in_arr), _h(bn_scale_arr), _h(bn_bias_arr), _h(out_arr),
+                                         ctypes.c_float(eps), _h(save_mean), _h(save_var), _s(stream), _p(profiler)))
+
+
+def batch_norm_relu_gradient(in_gradient_y, in_arr_x, in_bn_scale, in_bn_bias, out_gradient_x, out_gradient_bn_scale,
+                             out_gradient_bn_bias, saved_mean, saved_var, eps=0.01, stream=None, profiler=None):
+    check_call(_LIB.TSplit_BatchNormRelu_gradient(
+        _h(in_gradient_y), _h(in_arr_x), _h(in_bn_scale), _h(in_bn_bias), _h(out_gradient_x),
+        _h(out_gradient_bn_scale), _h(out_gradient_bn_bias), ctypes.c_float(eps), _h(saved_mean), _h(saved_var),
+        _s(stream), _p(profiler)))

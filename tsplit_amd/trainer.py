@@ -108,8 +108,14 @@ def _out_shape(layer, s):
 
 class Trainer(object):
     def __init__(self, spec, params, input_shape, num_classes, ctx=None, optimizer=("sgd", 0.1),
-                 split=None, bn_eps=0.01, timer=None):
+                 split=None, bn_eps=0.01, timer=None, fuse_bn_relu=False):
         self.spec = list(spec)
+        # with fuse_bn_relu a ("bn", ...) layer directly followed by ("relu",) runs as ONE fused call
+        # in each direction (symbols outside the reference's ABI); the Relu layer's own arrays are
+        # then never touched: the fused output and input gradient live in the BN layer's slots
+        self.fused = set()
+        if fuse_bn_relu:
+            self.fused = {li for li, l in enumerate(self.spec[:-1]) if l[0] == "bn" and self.spec[li + 1][0] == "relu"}
         # optional per-call timing hook: timer.begin(stream) / timer.end(stream, tag, work, unit)
         self.timer = timer
         self.ctx = ctx if ctx is not None else ndarray.gpu(0)
@@ -132,8 +138,9 @@ class Trainer(object):
         for li, layer in enumerate(self.spec):
             s = _out_shape(layer, s)
             self.shapes.append(s)
-            self.acts.append(ndarray.empty(s, self.ctx))
-            self.dacts.append(ndarray.empty(s, self.ctx))
+            unused = li in self.fused          # the BN output of a fused pair never exists
+            self.acts.append(None if unused else ndarray.empty(s, self.ctx))
+            self.dacts.append(None if unused else ndarray.empty(s, self.ctx))
             if layer[0] == "bn":
                 c = layer[2]
                 self.saved[li] = (ndarray.empty((1, c, 1, 1), self.ctx), ndarray.empty((1, c, 1, 1), self.ctx))
@@ -185,11 +192,19 @@ class Trainer(object):
                 pairs = list(zip(a.sTensor, out.sTensor)) if li in self.split else [(a, out)]
                 for xa, ya in pairs:
                     self._run(tag, 2.0 * n(ya.shape) * cin * k * k, "flop", L.CuDNN_conv2d, xa, w, ya, pad, pad, stride)
+            elif kind == "bn" and li in self.fused:
+                name = layer[1]
+                sm, sv = self.saved[li]
+                # writes the Relu layer's output directly
+                self._run("bn_relu_fwd", 8.0 * n(a.shape), "byte", L.batch_norm_relu, a, self.params[name + "_scale"],
+                          self.params[name + "_bias"], self.acts[li + 2], sm, sv, self.eps)
             elif kind == "bn":
                 name = layer[1]
                 sm, sv = self.saved[li]
                 self._run("bn_fwd", 8.0 * n(a.shape), "byte", L.CuDNN_Batch_Normalization, a,
                           self.params[name + "_scale"], self.params[name + "_bias"], out, sm, sv, 0.99, self.eps)
+            elif kind == "relu" and li - 1 in self.fused:
+                pass
             elif kind == "relu":
                 self._run("relu_fwd", 8.0 * n(a.shape), "byte", L.relu, a, out)
             elif kind == "maxpool":
@@ -234,12 +249,21 @@ class Trainer(object):
                     for ga, gi in zip(gs, gis):
                         self._run("conv_bwd_data_" + self._tile(cin), 2.0 * n(ga.shape) * cin * k * k, "flop",
                                   L.CuDNN_conv2d_gradient_of_data, w, ga, gi, pad, pad, stride)
+            elif kind == "bn" and li in self.fused:
+                name = layer[1]
+                sm, sv = self.saved[li]
+                # consumes the gradient behind the Relu layer
+                self._run("bn_relu_bwd", 12.0 * n(a.shape), "byte", L.batch_norm_relu_gradient, self.dacts[li + 2], a,
+                          self.params[name + "_scale"], self.params[name + "_bias"], g_in,
+                          self.grads[name + "_scale"], self.grads[name + "_bias"], sm, sv, self.eps)
             elif kind == "bn":
                 name = layer[1]
                 sm, sv = self.saved[li]
                 self._run("bn_bwd", 12.0 * n(a.shape), "byte", L.CuDNN_Batch_Normalization_gradient, g_out, a,
                           self.params[name + "_scale"], g_in, self.grads[name + "_scale"],
                           self.grads[name + "_bias"], sm, sv, self.eps)
+            elif kind == "relu" and li - 1 in self.fused:
+                pass
             elif kind == "relu":
                 self._run("relu_bwd", 12.0 * n(a.shape), "byte", L.relu_gradient, a, g_out, g_in)
             elif kind == "maxpool":
