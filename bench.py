@@ -14,6 +14,8 @@ Prints ONE JSON line.  Besides the contract fields it carries
                 recorded on the compute stream around every launch inside the timed region
   kernels       the same figures for every operator class (TFLOP/s or GB/s)
   cpu_baseline  the numpy CPU oracle timed on this host on a bounded sample of the workload
+  cpu_baseline_onednn  the same sample through PyTorch-CPU's bundled oneDNN (a library figure
+                beside the oracle's; the reference's own dnnl build cannot be compiled here)
 """
 import argparse
 import json
@@ -70,6 +72,57 @@ def cpu_baseline(sample_batch=8, seed=123):
     return {"value": sample_batch / dt, "unit": "samples/s", "cores": int(cores), "kind": "port",
             "sample": "one VGG-16 fwd+bwd+momentum step on %d of the 64 seeded images, numpy oracle in float64 "
                       "(%.1f s, loss %.4f)" % (sample_batch, dt, loss)}
+
+
+def cpu_baseline_onednn(sample_batch=8, seed=123):
+    """The same step on the same seeded sample through oneDNN as bundled with PyTorch-CPU
+    (conv / batch-norm / pooling / matmul primitives, fp32, all host cores): the closest
+    available stand-in for the reference's dnnl CPU operator build (src/dnnl_ops), whose
+    oneDNN 1.x sources cannot be compiled against the library versions on this machine.
+    Returns None when torch is not importable."""
+    try:
+        import torch
+        import torch.nn.functional as F
+    except Exception:
+        return None
+    spec, params, x, labels, _ = vgg_workload(sample_batch, seed)
+    torch.set_num_threads(os.cpu_count() or 1)
+    P = {k: torch.tensor(v, requires_grad=True) for k, v in params.items()}
+    vel = {k: torch.zeros_like(v) for k, v in P.items()}
+    xt, yt = torch.tensor(x), torch.tensor(labels)
+
+    def step():
+        h = xt
+        for layer in spec:
+            kind = layer[0]
+            if kind == "conv":
+                h = F.conv2d(h, P[layer[1] + "_weight"], padding=layer[5], stride=layer[6])
+            elif kind == "bn":
+                h = F.batch_norm(h, None, None, P[layer[1] + "_scale"].reshape(-1), P[layer[1] + "_bias"].reshape(-1),
+                                 training=True, eps=0.01)
+            elif kind == "relu":
+                h = F.relu(h)
+            elif kind == "maxpool":
+                h = F.max_pool2d(h, layer[1], layer[3], layer[2])
+            elif kind == "flatten":
+                h = h.reshape(h.shape[0], -1)
+            elif kind == "fc":
+                h = h @ P[layer[1] + "_weight"]
+        loss = -(yt * F.log_softmax(h, dim=1)).sum(dim=1).mean()
+        loss.backward()
+        with torch.no_grad():
+            for k, p in P.items():
+                vel[k].mul_(0.9).sub_(p.grad, alpha=0.01)
+                p.add_(vel[k])
+                p.grad = None
+        return float(loss.detach())
+    step()                       # warm-up: primitive creation, allocator
+    t0 = time.perf_counter()
+    loss = step()
+    dt = time.perf_counter() - t0
+    return {"value": sample_batch / dt, "unit": "samples/s", "cores": int(torch.get_num_threads()), "kind": "library",
+            "sample": "one VGG-16 fwd+bwd+momentum step on %d of the 64 seeded images, PyTorch-CPU %s with its "
+                      "bundled oneDNN, fp32 (%.2f s, loss %.4f)" % (sample_batch, torch.__version__, dt, loss)}
 
 
 def main():
@@ -144,6 +197,9 @@ def main():
         out["kernels"] = kernels
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+        onednn = cpu_baseline_onednn()
+        if onednn:
+            out["cpu_baseline_onednn"] = onednn
     print(json.dumps(out))
 
 
