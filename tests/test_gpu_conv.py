@@ -48,6 +48,12 @@ CASES = [
     (3, 1, 19, 23, 100, 5, 5, 2, 2, 1),    # 25 columns, two row tiles, ragged K (oH*oW odd)
     (2, 2, 20, 20, 33, 4, 4, 1, 1, 2),     # exactly 32 columns, stride 2
     (1, 3, 5, 5, 7, 3, 3, 1, 1, 1),        # K = 25: one partial step
+    # "same" stride-1 filters with H*W a multiple of 4 but not of 16: the tap-major backward-filter
+    # kernel pads each image's positions to a multiple of 16
+    (3, 16, 6, 6, 20, 3, 3, 1, 1, 1),      # 36 positions, image rows shorter than one k-step
+    (2, 16, 2, 2, 8, 3, 3, 1, 1, 1),       # 4 positions
+    (2, 32, 10, 14, 24, 1, 7, 0, 3, 1),    # 140 positions, 1x7 filter
+    (5, 48, 14, 14, 72, 3, 3, 1, 1, 1),    # 196 positions, odd image count
 ]
 
 

@@ -567,11 +567,14 @@ struct TapWgradParams {
   unsigned dy_bytes, x_bytes;
   int O, C, HW, W, kW, taps;
   int ph, pw;
-  int M, N, K;           // O, C*taps, imgs*HW
+  int M, N, K;           // O, C*taps, imgs*HWp
   int kchunk;            // k range per split (multiple of 16)
+  int HWp;               // HW rounded up to a multiple of 16: the reduction runs over imgs*HWp positions
 };
 
-template <int BM, int BN, int WM, int WN>
+// TAIL: H*W is a multiple of 4 but not of 16.  Every image's positions are padded to HWp; the
+// padded ones read as zeros (one more compare per operand and step).
+template <int BM, int BN, int WM, int WN, bool TAIL>
 __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams P, float *__restrict__ part,
                                                                   TileGrid tg) {
   static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
@@ -628,18 +631,22 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
       for (int e = 0; e < 16; ++e) acc[i][jx][e] = 0.f;
 
   // uniform position of the NEXT step to load, and this thread's column within the image row
-  int img = kbegin / P.HW, p0 = kbegin - img * P.HW;
+  int img = kbegin / P.HWp, p0 = kbegin - img * P.HWp;
   int ow = (p0 + klocal) % P.W;
+  const int ow_first = klocal % P.W;   // column of this thread's position in the first step of an image
 
   u32x4 ra_regs[PA];
   unsigned rb_regs[KCOLS];
 
   auto load_step = [&]() {
     const int soff_a = (img * P.O * P.HW + p0) * 4;
+    const bool word_ok = !TAIL || p0 + 4 * (tid & 3) < P.HW;     // H*W % 4 == 0: a word is all in or all out
 #pragma unroll
-    for (int s = 0; s < PA; ++s) ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[s], soff_a, 0);
+    for (int s = 0; s < PA; ++s)
+      ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, word_ok ? a_voff[s] : kOobOffset, soff_a, 0);
     const int p = p0 + klocal;
-    const bool ok = cols_ok && static_cast<unsigned>(p + dr * P.W) < static_cast<unsigned>(P.HW) &&
+    const bool ok = cols_ok && (!TAIL || p < P.HW) &&
+                    static_cast<unsigned>(p + dr * P.W) < static_cast<unsigned>(P.HW) &&
                     static_cast<unsigned>(ow + dc) < static_cast<unsigned>(P.W);
     const unsigned voff = ok ? b_voff : kOobOffset;
     const int soff_b = (img * P.C * P.HW + p0) * 4;
@@ -647,12 +654,13 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
     for (int i = 0; i < KCOLS; ++i)
       rb_regs[i] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, soff_b + i * P.HW * 4, 0);
     p0 += BK;
-    if (p0 >= P.HW) {
-      p0 = 0;
-      ++img;
-    }
     ow += BK;                      // BK may exceed W for tiny images: reduce until in range
     while (ow >= P.W) ow -= P.W;
+    if (p0 >= P.HWp) {
+      p0 = 0;
+      ++img;
+      if (TAIL) ow = ow_first;     // positions do not continue across the padded tail
+    }
   };
   auto store_step = [&](float *sa, float *sb) {
 #pragma unroll
@@ -1380,17 +1388,23 @@ int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *d
   P.pw = g.pw;
   P.M = g.O;
   P.N = g.C * g.kH * g.kW;
-  P.K = g.imgs * g.H * g.W;
+  P.HWp = (P.HW + BK - 1) / BK * BK;
+  P.K = g.imgs * P.HWp;
+  const bool tail = P.HWp != P.HW;
   const int tm = (P.M + BM - 1) / BM, tn = (P.N + BN - 1) / BN;
   int S;
-  static const int occ = blocks_per_cu(conv_wgrad_tap_kernel<BM, BN, WM, WN>);
+  static const int occ = blocks_per_cu(conv_wgrad_tap_kernel<BM, BN, WM, WN, false>);
   plan_splitk(tm * tn, P.K, 1024, occ, S, P.kchunk);
   const int64_t mn = static_cast<int64_t>(P.M) * P.N;
   float *part = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(S) * mn * 4));
   TS_REQUIRE(part, "conv bwd-filter: no scratch memory for split-K");
   *ws_elems = S * mn;
-  hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN>), dim3(grid_blocks(tm, tn, S)), dim3(kThreads), 0, st, P,
-                     part, TileGrid{tm, tn, tm * tn * S});
+  if (tail)
+    hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN, true>), dim3(grid_blocks(tm, tn, S)), dim3(kThreads), 0,
+                       st, P, part, TileGrid{tm, tn, tm * tn * S});
+  else
+    hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN, false>), dim3(grid_blocks(tm, tn, S)), dim3(kThreads), 0,
+                       st, P, part, TileGrid{tm, tn, tm * tn * S});
   hipLaunchKernelGGL(fold_tap_major_kernel, dim3(static_cast<unsigned>((mn + 63) / 64)), dim3(256), 0, st, part, dw,
                      g.O, g.C, g.kH * g.kW, mn, S);
   return 0;
@@ -1628,7 +1642,7 @@ int launch_wgrad_narrow(const ConvGeo &g, const float *x, const float *dy, float
 
 inline bool wgrad_tap_ok(const ConvGeo &g) {
   const int64_t bytes_x = static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4, bytes_dy = static_cast<int64_t>(g.imgs) * g.O * g.H * g.W * 4;
-  return g.s == 1 && g.oH == g.H && g.oW == g.W && (g.H * g.W) % BK == 0 && g.C % BK == 0 &&
+  return g.s == 1 && g.oH == g.H && g.oW == g.W && (g.H * g.W) % 4 == 0 && g.C % BK == 0 &&
          bytes_x + 4 * (static_cast<int64_t>(g.ph) * g.W + g.pw) < (1ll << 31) && bytes_dy < (1ll << 31);
 }
 
