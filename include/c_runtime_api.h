@@ -359,6 +359,36 @@ int DLGpuTanh(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle st
 int DLGpuSigmoid(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle,
                  ProfilerHandle p);
 
+/* ---- Dropout (ref: c_runtime_api.h:334-338; impl src/ops/CudnnDropout.cu:4-77, :79-151).
+ *      `dropout` is the probability of zeroing an element, survivors are scaled by
+ *      1/(1-dropout) (cuDNN's meaning of the argument).  The generator is re-seeded with the
+ *      reference's constant before every call (CudnnDropout.cu:33,41), so equal element counts
+ *      give equal masks.  With first_time == 1 the forward call allocates the reserve space (one
+ *      bit per element) from the device pool and stores its byte size and address through the two
+ *      pointers; later forward calls and the gradient reuse it.  Which elements are dropped is
+ *      this library's generator (Philox-4x32-10), not cuDNN's.  In the gradient call output_Y is
+ *      the incoming gradient and input_X receives the result. ---- */
+int CuDNN_DLGpuDropout(const DLArrayHandle input_X, const float dropout, DLArrayHandle output_Y,
+                       int *reserve_size, void **reserve_space, int first_time,
+                       DLStreamHandle stream_handle, ProfilerHandle p);
+int CuDNN_DLGpuDropout_gradient(const DLArrayHandle output_Y, const float dropout,
+                                DLArrayHandle input_X, int *reserve_size, void **reserve_space,
+                                DLStreamHandle stream_handle, ProfilerHandle p);
+
+/* ---- CSR sparse x dense products (ref: c_runtime_api.h:362-364; impl
+ *      src/ops/CuSparseCsrmv.cu:3-64, src/ops/CuSparseCsrmm.cu:34-114).  data: fp32 values
+ *      [nnz]; row: int32 row pointers [nrow+1]; col: int32 column indices [nnz], zero based
+ *      (python/athena/ndarray.py:445-455).  Csrmv: output = A input, or A^T input.  Csrmm:
+ *      matC = op(A) op(matB), dense operands row-major, all four transpose combinations. ---- */
+int CuSparse_DLGpuCsrmv(const DLArrayHandle data_handle, const DLArrayHandle row_handle,
+                        const DLArrayHandle col_handle, int nrow, int ncol, bool transpose,
+                        const DLArrayHandle input_handle, DLArrayHandle output_handle,
+                        DLStreamHandle stream_handle, ProfilerHandle p);
+int CuSparse_DLGpuCsrmm(const DLArrayHandle data_handle, const DLArrayHandle row_handle,
+                        const DLArrayHandle col_handle, int nrow, int ncol, bool transposeA,
+                        const DLArrayHandle matB, bool transposeB, DLArrayHandle matC,
+                        DLStreamHandle stream_handle, ProfilerHandle p);
+
 /* ---- Fused BatchNorm + Relu.  NO counterpart in the reference (its ABI has one symbol per graph
  *      node); for hosts that know the Relu follows the BatchNorm and want to skip its two passes
  *      over the activation.  Forward: output_Y = max(BN(input_X), 0); both save arrays are

@@ -301,3 +301,33 @@ def embedding_grad_loops(dy, ids, table_shape):
     for r in range(flat.size):
         g[int(flat[r])] += d2[r]
     return g
+
+
+def csrmv_loops(data, indptr, indices, nrow, ncol, trans, x):
+    """Row-by-row walk of the CSR arrays: y = A x, or y = A^T x (gpu_ops/CuSparse.py:55-58)."""
+    y = np.zeros(ncol if trans else nrow, dtype=np.float64)
+    for i in range(nrow):
+        for j in range(int(indptr[i]), int(indptr[i + 1])):
+            if trans:
+                y[int(indices[j])] += float(data[j]) * float(x[i])
+            else:
+                y[i] += float(data[j]) * float(x[int(indices[j])])
+    return y
+
+
+def csrmm_loops(data, indptr, indices, nrow, ncol, transA, B, transB):
+    """C = op(A) op(B) entry by entry (gpu_ops/CuSparse.py:150-163)."""
+    Bm = np.asarray(B, dtype=np.float64)
+    if transB:
+        Bm = Bm.T
+    n = Bm.shape[1]
+    C = np.zeros((ncol if transA else nrow, n), dtype=np.float64)
+    for i in range(nrow):
+        for j in range(int(indptr[i]), int(indptr[i + 1])):
+            c = int(indices[j])
+            for t in range(n):
+                if transA:
+                    C[c, t] += float(data[j]) * Bm[i, t]
+                else:
+                    C[i, t] += float(data[j]) * Bm[c, t]
+    return C

@@ -42,6 +42,17 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
   batch_matmul                                     pinned: per-batch matmul loops
   sqrt / rsqrt / sigmoid / tanh / opposite / div_const / divide
                                                    pinned: inverse-function identities
+  csrmv / csrmm                                    pinned: scipy.sparse products are the
+      reference's CPU path; checked against dense float64 products and literal loops
+  reduce_sum_axis_zero (workspace form)            same function as reduce_sum_axis_zero
+  dropout / dropout_grad                           arithmetic pinned (kept elements scaled
+      by 1/(1-p), dropped ones exactly 0, the gradient reuses the forward mask, the mask
+      repeats from call to call because the reference re-seeds before every call);
+      philox4x32_10 pinned by the published Random123 known-answer vectors.
+      WHICH elements are dropped: PARITY UNPINNED.  The reference's GPU mask comes from
+      cuDNN's generator (src/ops/CudnnDropout.cu:33-60, closed source, unversioned) and its
+      CPU paths use libc rand() (src/dnnl_ops/Dropout.cpp:17-31) or numpy's global
+      generator (gpu_ops/Dropout.py:64-67); no reference test or fixture fixes a mask.
 """
 import numpy as np
 
@@ -599,3 +610,81 @@ def div_const(c, x, dtype=np.float64):
 
 def divide(a, b, dtype=np.float64):
     return _f(a, dtype) / _f(b, dtype)
+
+
+# --------------------------------------------------------------------------
+# Sparse products  (reference: gpu_ops/CuSparse.py:52-59 csrmv, :147-163 csrmm; the GPU
+# symbols take the three CSR arrays, src/ops/CuSparseCsrmv.cu:3-47, CuSparseCsrmm.cu:34-96)
+# --------------------------------------------------------------------------
+def _csr(data, indptr, indices, nrow, ncol, dtype):
+    import scipy.sparse
+    return scipy.sparse.csr_matrix((_f(data, dtype), np.asarray(indices, dtype=np.int32),
+                                    np.asarray(indptr, dtype=np.int32)), shape=(nrow, ncol))
+
+
+def csrmv(data, indptr, indices, nrow, ncol, trans, x, dtype=np.float64):
+    """y = A x, or A^T x when `trans` (gpu_ops/CuSparse.py:55-58)."""
+    A = _csr(data, indptr, indices, nrow, ncol, dtype)
+    return (A.T if trans else A).dot(_f(x, dtype))
+
+
+def csrmm(data, indptr, indices, nrow, ncol, transA, B, transB, dtype=np.float64):
+    """C = op(A) op(B), all dense operands row-major (gpu_ops/CuSparse.py:150-163)."""
+    A = _csr(data, indptr, indices, nrow, ncol, dtype)
+    Bm = _f(B, dtype)
+    return (A.T if transA else A).dot(Bm.T if transB else Bm)
+
+
+# --------------------------------------------------------------------------
+# Dropout  (reference GPU symbol: src/ops/CudnnDropout.cu:4-77 forward, :79-151 gradient)
+# --------------------------------------------------------------------------
+DROPOUT_SEED = 19260817          # src/ops/CudnnDropout.cu:33 (set again before every call)
+
+_PHILOX_M0, _PHILOX_M1 = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57)
+_PHILOX_W0, _PHILOX_W1 = 0x9E3779B9, 0xBB67AE85
+_MASK32 = np.uint64(0xFFFFFFFF)
+
+
+def philox4x32_10(c0, c1, c2, c3, k0, k1):
+    """Philox-4x32 with 10 rounds (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3",
+    SC'11).  Counters are uint32 arrays (or scalars), the key two uint32 scalars; returns the four
+    output words as uint32 arrays."""
+    c = [np.asarray(v, dtype=np.uint64) for v in (c0, c1, c2, c3)]
+    k0, k1 = int(k0) & 0xFFFFFFFF, int(k1) & 0xFFFFFFFF
+    for _ in range(10):
+        p0 = _PHILOX_M0 * c[0]
+        p1 = _PHILOX_M1 * c[2]
+        c = [(p1 >> np.uint64(32)) ^ c[1] ^ np.uint64(k0), p1 & _MASK32,
+             (p0 >> np.uint64(32)) ^ c[3] ^ np.uint64(k1), p0 & _MASK32]
+        k0, k1 = (k0 + _PHILOX_W0) & 0xFFFFFFFF, (k1 + _PHILOX_W1) & 0xFFFFFFFF
+    return [v.astype(np.uint32) for v in c]
+
+
+def dropout_mask(n, dropout, seed=DROPOUT_SEED):
+    """keep[i] for i < n.  Element i takes word i%4 of philox4x32_10(counter=(i//4,0,0,0),
+    key=(seed low, seed high)) and is kept iff word >= floor(dropout * 2^32): a fraction
+    `dropout` of the words lies below the threshold."""
+    groups = (n + 3) // 4
+    idx = np.arange(groups, dtype=np.uint64)
+    zero = np.zeros(groups, dtype=np.uint64)
+    words = philox4x32_10(idx & _MASK32, idx >> np.uint64(32), zero, zero, seed & 0xFFFFFFFF, seed >> 32)
+    flat = np.stack(words, axis=1).reshape(-1)[:n].astype(np.uint64)
+    threshold = np.uint64(min(int(float(np.float32(dropout)) * 4294967296.0), 1 << 32))
+    return flat >= threshold
+
+
+def dropout(x, dropout, dtype=np.float64):
+    """-> (y, keep).  cuDNN semantics of the GPU symbol: each element is zeroed with probability
+    `dropout`, the others are multiplied by 1/(1-dropout) (src/ops/CudnnDropout.cu:41,58-60)."""
+    xv = _f(x, dtype)
+    keep = dropout_mask(xv.size, dropout).reshape(xv.shape)
+    with np.errstate(divide="ignore", invalid="ignore"):       # dropout == 1: nothing is kept
+        scale = F32(1.0) / (F32(1.0) - F32(dropout))
+        return np.where(keep, xv * dtype(scale), dtype(0)), keep
+
+
+def dropout_grad(dy, dropout, keep, dtype=np.float64):
+    """dx = dy * keep / (1-dropout) with the forward call's mask (src/ops/CudnnDropout.cu:130-132)."""
+    with np.errstate(divide="ignore", invalid="ignore"):
+        scale = F32(1.0) / (F32(1.0) - F32(dropout))
+        return np.where(keep, _f(dy, dtype) * dtype(scale), dtype(0))

@@ -183,6 +183,16 @@ std::map<ScratchKey, ScratchBuf> g_scratch;
 
 }  // namespace
 
+// Pool memory for an operator that must hand a buffer to its caller (dropout's reserve space);
+// nullptr when the device has none left.
+void *device_pool_alloc(int device_id, size_t bytes) {
+  try {
+    return data_alloc(DLContext{device_id, kGPU}, bytes, 1);
+  } catch (const std::exception &) {
+    return nullptr;
+  }
+}
+
 void *scratch_get(hipStream_t stream, int slot, size_t bytes) {
   std::lock_guard<std::mutex> lk(g_mu);
   ScratchBuf &b = g_scratch[ScratchKey{stream, slot}];

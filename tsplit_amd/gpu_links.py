@@ -27,6 +27,7 @@ __all__ = [
     "embedding_lookup_gradient", "matrix_elementwise_divide", "matrix_elementwise_divide_const",
     "matrix_opposite", "matrix_sqrt", "matrix_rsqrt", "tanh", "sigmoid",
     "batch_norm_relu", "batch_norm_relu_gradient",
+    "CuDNN_Dropout", "CuDNN_Dropout_gradient", "CuSparse_Csrmv", "CuSparse_Csrmm",
 ]
 
 
@@ -335,6 +336,37 @@ def embedding_lookup(in_mat, ids, out_mat, stream=None, profiler=None):
 
 def embedding_lookup_gradient(grad_out, ids, grad_in, stream=None, profiler=None):
     check_call(_LIB.DLGpuEmbeddingLookUp_Gradient(_h(grad_out), _h(ids), _h(grad_in), _s(stream), _p(profiler)))
+
+
+# ---- Dropout (gpu_links/CudnnDropoutLink.py:8,15).  reserve_size is a ctypes.c_int and
+#      reserve_space a ctypes.c_void_p owned by the caller (one pair per dropout node); the first
+#      forward call (firstTime == 1) fills both. ----
+def CuDNN_Dropout(in_arr, dropout, out_arr, reserve_size, reserve_space, firstTime, stream=None, profiler=None):
+    check_call(_LIB.CuDNN_DLGpuDropout(_h(in_arr), ctypes.c_float(dropout), _h(out_arr), ctypes.byref(reserve_size),
+                                       ctypes.byref(reserve_space), ctypes.c_int(firstTime), _s(stream),
+                                       _p(profiler)))
+
+
+def CuDNN_Dropout_gradient(in_gradient_y, dropout, out_gradient_x, reserve_size, reserve_space, stream=None,
+                           profiler=None):
+    check_call(_LIB.CuDNN_DLGpuDropout_gradient(_h(in_gradient_y), ctypes.c_float(dropout), _h(out_gradient_x),
+                                                ctypes.byref(reserve_size), ctypes.byref(reserve_space),
+                                                _s(stream), _p(profiler)))
+
+
+# ---- CSR sparse products (gpu_links/CuSparseLink.py:7,13) ----
+def CuSparse_Csrmv(mat, trans, in_arr, out_arr, stream=None, profiler=None):
+    assert isinstance(mat, _nd.ND_Sparse_Array)
+    check_call(_LIB.CuSparse_DLGpuCsrmv(_h(mat.data), _h(mat.row), _h(mat.col), ctypes.c_int(mat.nrow),
+                                        ctypes.c_int(mat.ncol), ctypes.c_bool(bool(trans)), _h(in_arr), _h(out_arr),
+                                        _s(stream), _p(profiler)))
+
+
+def CuSparse_Csrmm(matA, transA, matB, transB, matC, stream=None, profiler=None):
+    assert isinstance(matA, _nd.ND_Sparse_Array)
+    check_call(_LIB.CuSparse_DLGpuCsrmm(_h(matA.data), _h(matA.row), _h(matA.col), ctypes.c_int(matA.nrow),
+                                        ctypes.c_int(matA.ncol), ctypes.c_bool(bool(transA)), _h(matB),
+                                        ctypes.c_bool(bool(transB)), _h(matC), _s(stream), _p(profiler)))
 
 
 # ---- Elementwise math (gpu_links/MatrixDivideLink.py:7, MatrixDivideConstLink.py:7, OppositeLink.py:8,

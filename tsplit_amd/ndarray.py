@@ -153,9 +153,15 @@ class NDArray(object):
             raise TypeError("type %s not supported" % str(type(value)))
 
     def _sync_copyfrom(self, source_array, data_type=np.float32):
+        """Synchronous copy from a numpy array.  data_type np.int32 stores the 32-bit integers
+        as they are (the index arrays of a sparse matrix, python/athena/ndarray.py:198-219)."""
         source_array = np.ascontiguousarray(source_array, dtype=data_type)
         if source_array.shape != self.shape:
             raise ValueError("array shape do not match the shape of NDArray")
+        if source_array.dtype == np.int32:
+            source_array = source_array.view(np.float32)
+        elif source_array.dtype != np.float32:
+            raise TypeError("only float32 and int32 elements are stored, not %s" % source_array.dtype)
         src, shape = NDArray._numpyasarray(source_array)
         check_call(_LIB.DLArrayCopyFromTo(ctypes.byref(src), self.handle, None))
         _ = shape
@@ -218,6 +224,49 @@ def empty(shape, ctx=cpu(0)):
     check_call(_LIB.DLArrayAlloc(cshape, ctypes.c_int64(len(cshape)), ctx, ctypes.byref(handle),
                                  ctypes.c_int(MEMORY_MANAGE_RULE)))
     return NDArray(handle)
+
+
+class ND_Sparse_Array(object):
+    """CSR matrix on a device: values, row pointers and column indices as three 1-D arrays
+    (python/athena/ndarray.py:412-425)."""
+    __slots__ = ["data", "row", "col", "nrow", "ncol"]
+
+    def __init__(self, data, row, col, nrow, ncol):
+        self.data = data
+        self.row = row
+        self.col = col
+        self.nrow = nrow
+        self.ncol = ncol
+
+    @property
+    def shape(self):
+        return (self.nrow, self.ncol)
+
+
+def sparse_array(values, indices, shape, ctx=cpu(0)):
+    """CSR copy on `ctx` of the matrix with `values` at `indices` = (rows, cols); entries
+    with equal coordinates are summed and every row's columns come out ascending, as
+    scipy.sparse.csr_matrix builds them (python/athena/ndarray.py:428-455)."""
+    assert len(shape) == len(indices) == 2
+    assert len(values) == len(indices[0]) == len(indices[1])
+    rows = np.asarray(indices[0], dtype=np.int64)
+    cols = np.asarray(indices[1], dtype=np.int64)
+    vals = np.asarray(values, dtype=np.float32)
+    assert rows.size == 0 or (rows.min() >= 0 and rows.max() < shape[0] and cols.min() >= 0 and cols.max() < shape[1])
+    key = rows * int(shape[1]) + cols
+    uniq, inverse = np.unique(key, return_inverse=True)
+    summed = np.zeros(uniq.shape, dtype=np.float32)
+    np.add.at(summed, inverse, vals)
+    urows, ucols = uniq // int(shape[1]), uniq % int(shape[1])
+    indptr = np.zeros(int(shape[0]) + 1, dtype=np.int32)
+    np.cumsum(np.bincount(urows, minlength=int(shape[0])), out=indptr[1:])
+    values_ret = empty(summed.shape, ctx)
+    values_ret._sync_copyfrom(summed)
+    row_ret = empty(indptr.shape, ctx)
+    row_ret._sync_copyfrom(indptr, np.int32)
+    col_ret = empty(ucols.shape, ctx)
+    col_ret._sync_copyfrom(ucols, np.int32)
+    return ND_Sparse_Array(values_ret, row_ret, col_ret, int(shape[0]), int(shape[1]))
 
 
 def numpyasdlarrayhandle(data):

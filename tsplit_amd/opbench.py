@@ -19,8 +19,9 @@ PEAK_GBS = 8000.0
 PEAK_TFLOPS = 157.3
 
 
-def _cases(L, A, E):
-    """-> list of (name, work, unit, launch) ; A(shape) = random device array, E(shape) = empty one."""
+def _cases(L, A, E, S):
+    """-> list of (name, work, unit, launch) ; A(shape) = random device array, E(shape) = empty one,
+    S(nrow, ncol, per_row) = random CSR matrix with per_row entries in every row."""
     c = []
 
     def add(name, work, unit, fn):
@@ -104,6 +105,24 @@ def _cases(L, A, E):
     add("opposite", 8 * ne, "byte", lambda s: L.matrix_opposite(xa, xo, s))
     add("div_const", 8 * ne, "byte", lambda s: L.matrix_elementwise_divide_const(2.0, xa, xo, s))
     add("divide", 12 * ne, "byte", lambda s: L.matrix_elementwise_divide(xa, xb, xo, s))
+    # dropout on the same activation: 8 B/element of values plus one mask bit
+    import ctypes
+    rsize, rspace = ctypes.c_int(0), ctypes.c_void_p(0)
+    L.CuDNN_Dropout(xa, 0.1, xo, rsize, rspace, 1, None)
+    add("dropout_fwd", 8.125 * ne, "byte", lambda s: L.CuDNN_Dropout(xa, 0.1, xo, rsize, rspace, 0, s))
+    add("dropout_bwd", 8.125 * ne, "byte", lambda s: L.CuDNN_Dropout_gradient(xa, 0.1, xo, rsize, rspace, s))
+    # CSR products on a graph-like matrix: 2^20 rows, 16 entries per row, 64 feature columns
+    nr, per, nf = 1 << 20, 16, 64
+    sp = S(nr, nr, per)
+    xv, yv = A((nr,)), E((nr,))
+    bm, cm = A((nr, nf)), E((nr, nf))
+    csr_bytes = 8 * nr * per + 4 * (nr + 1)
+    add("csrmv/1M_rows_16_per_row", csr_bytes + 8 * nr, "byte", lambda s: L.CuSparse_Csrmv(sp, False, xv, yv, s))
+    add("csrmv_trans/1M_rows_16_per_row", csr_bytes + 8 * nr, "byte", lambda s: L.CuSparse_Csrmv(sp, True, xv, yv, s))
+    add("csrmm/1M_rows_16_per_row_64_cols", csr_bytes + 8 * nr * nf, "byte",
+        lambda s: L.CuSparse_Csrmm(sp, False, bm, False, cm, s))
+    add("csrmm_transA/1M_rows_16_per_row_64_cols", csr_bytes + 8 * nr * nf, "byte",
+        lambda s: L.CuSparse_Csrmm(sp, True, bm, False, cm, s))
     return c
 
 
@@ -131,9 +150,19 @@ def main():
     def E(shape):
         return ndarray.empty(shape, ctx)
 
+    def S(nrow, ncol, per_row):
+        cols = np.sort(rng.randint(0, ncol, size=(nrow, per_row)), axis=1).astype(np.int32).reshape(-1)
+        ptr = (np.arange(nrow + 1, dtype=np.int64) * per_row).astype(np.int32)
+        vals = rng.standard_normal(size=nrow * per_row).astype(np.float32)
+        d, r, c = ndarray.empty(vals.shape, ctx), ndarray.empty(ptr.shape, ctx), ndarray.empty(cols.shape, ctx)
+        d._sync_copyfrom(vals)
+        r._sync_copyfrom(ptr, np.int32)
+        c._sync_copyfrom(cols, np.int32)
+        return ndarray.ND_Sparse_Array(d, r, c, nrow, ncol)
+
     timer = EventTimer(ctx)
     rows = []
-    for name, work, unit, fn in _cases(L, A, E):
+    for name, work, unit, fn in _cases(L, A, E, S):
         if a.filter and a.filter not in name:
             continue
         fn(st)
