@@ -295,11 +295,23 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 //     its range, slot 1 for a partial last segment -- and a second kernel adds the pieces of
 //     each tile in ascending block order and writes the tile.
 // Results do depend on where the cuts fall, i.e. on the problem shape.
+// The tiles of one M row (tile_m fixed) form a chain of tn * ksteps k-steps, cut into equal
+// ranges for the blocks of that row; block `logical` works on row logical % tm, range
+// logical / tm.  Blocks with consecutive ids therefore sit on the tm tiles that share one set
+// of gathered columns, at the same k-step at about the same time, in one XCD: the gathered
+// operand comes from HBM once and from that XCD's L2 for the other tm - 1 tiles.
+// A row's first whole_waves * ranges tiles are taken whole, one per block and wave of blocks:
+// all blocks of an XCD then walk k together and share each step's filter words in its L2 as
+// well.  Only the rest of the chain (between one and two tiles per block, or everything when
+// there are fewer tiles than blocks) is cut into equal ranges.
 struct StreamK {
   int ksteps;            // k-steps per tile
-  int total;             // tiles * ksteps
+  int total;             // k-steps of the cut part of one M row's chain
   int iters_per_block;
   int tm;                // M tiles (tile index = tile_n * tm + tile_m)
+  int ranges;            // blocks per M row
+  int whole_waves;       // tiles every block takes whole before its range of the cut part
+  int cut_first;         // tile_n of the first tile of the cut part (= whole_waves * ranges)
 };
 
 template <int BM, int BN, int WM, int WN, bool BWD_DATA>
@@ -318,7 +330,8 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
   // consecutive workgroup ids go to different XCDs: transpose so that an XCD owns a contiguous
   // eighth of the work (neighbouring tiles share gathered activations in its L2)
   const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  const int it_begin = logical * sk.iters_per_block;
+  const int range = logical / sk.tm, tile_m = logical - range * sk.tm;
+  const int it_begin = range * sk.iters_per_block;
   int it = it_begin;
   const int it_end = min(sk.total, it + sk.iters_per_block);
 
@@ -330,12 +343,21 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
       const_cast<float *>(P.src) - bias, 0, static_cast<int>(P.src_bytes + 4u * bias), kBufFlags);
   const int klocal0 = (tid / BN) * KPT;
 
-  while (it < it_end) {
-    const int tile = it / sk.ksteps;
-    const int ks0 = it - tile * sk.ksteps;
-    const int ks1 = min(sk.ksteps, ks0 + (it_end - it));
-    it += ks1 - ks0;
-    const int tile_n = tile / sk.tm, tile_m = tile - tile_n * sk.tm;
+  int wave_no = 0;
+  while (wave_no < sk.whole_waves || it < it_end) {
+    int tile_n, ks0, ks1;
+    if (wave_no < sk.whole_waves) {
+      tile_n = wave_no * sk.ranges + range;
+      ks0 = 0;
+      ks1 = sk.ksteps;
+      ++wave_no;
+    } else {
+      const int t = it / sk.ksteps;
+      tile_n = sk.cut_first + t;
+      ks0 = it - t * sk.ksteps;
+      ks1 = min(sk.ksteps, ks0 + (it_end - it));
+      it += ks1 - ks0;
+    }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     // ---- filter operand: thread -> (row tid/4 + 64 s, 16-byte word tid%4); rows clamped
@@ -508,19 +530,21 @@ __global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvPara
                                                                      const float *__restrict__ pieces, StreamK sk) {
   const int tile = blockIdx.x >> 2, q = blockIdx.x & 3;
   const int mi = q >> 1, ni = q & 1;
-  const int first = tile * sk.ksteps, last = first + sk.ksteps - 1;
+  const int t = tile / sk.tm, tile_m = tile - t * sk.tm;                  // t: tile of the cut part
+  const int tile_n = sk.cut_first + t;
+  const int first = t * sk.ksteps, last = first + sk.ksteps - 1;          // within the cut part of row tile_m
   const int b0 = first / sk.iters_per_block, b1 = last / sk.iters_per_block;
   if (b0 == b1) return;   // computed and stored by one block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
-  const int tile_n = tile / sk.tm, tile_m = tile - tile_n * sk.tm;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   float acc[16];
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[e] = 0.f;
   for (int b = b0; b <= b1; ++b) {
     const int slot = b * sk.iters_per_block >= first ? 0 : 1;
-    const float *pc = pieces + (static_cast<int64_t>(b) * 2 + slot) * (BM * BN) + (q * 16) * kThreads + tid;
+    const float *pc =
+        pieces + (static_cast<int64_t>(b * sk.tm + tile_m) * 2 + slot) * (BM * BN) + (q * 16) * kThreads + tid;
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] += __builtin_nontemporal_load(pc + e * kThreads);
   }
@@ -540,10 +564,10 @@ __global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvPara
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void conv_tap_zero_cut_tiles_kernel(TapConvParams P, float *__restrict__ out,
                                                                            StreamK sk) {
-  const int start = (blockIdx.x + 1) * sk.iters_per_block;     // first unit of block g + 1
+  const int range = blockIdx.x / sk.tm, tile_m = blockIdx.x - range * sk.tm;
+  const int start = (range + 1) * sk.iters_per_block;            // first k-step of the next range of this row
   if (start >= sk.total || start % sk.ksteps == 0) return;       // falls on a tile boundary: nothing is cut
-  const int tile = start / sk.ksteps;
-  const int tile_n = tile / sk.tm, tile_m = tile - tile_n * sk.tm;
+  const int tile_n = sk.cut_first + start / sk.ksteps;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   for (int idx = threadIdx.x; idx < BM * BN; idx += kThreads) {
     const int m = m0 + idx / BN, n = n0 + idx % BN;
@@ -1333,21 +1357,34 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
   const int tiles = tm * tn;
   StreamK sk;
   sk.ksteps = P.K / BK;
-  sk.total = tiles * sk.ksteps;
+  sk.total = tn * sk.ksteps;
   sk.tm = tm;
   static const int occ = blocks_per_cu(conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>);
   const int slots = 256 * occ;
   unsigned grid;
   float *pieces = nullptr;
   bool zero_cut = false;
-  if (tiles % slots == 0 || sk.total < slots * 8) {
+  sk.whole_waves = 0;
+  sk.cut_first = 0;
+  int cut_tiles = tiles;         // tiles the assemble kernel looks at
+  if (tiles % slots == 0 || static_cast<int64_t>(tiles) * sk.ksteps < slots * 8) {
     // whole tiles fill whole waves of blocks, or there is too little work to cut: one tile per block
     sk.iters_per_block = sk.ksteps;
+    sk.ranges = tn;
     grid = (tiles + 7) / 8 * 8;
-  } else {                       // one full wave of blocks, equal shares of k-steps
-    grid = slots;
-    sk.iters_per_block = (sk.total + slots - 1) / slots;
-    if (sk.iters_per_block >= sk.ksteps) {
+  } else {                       // one full wave of blocks
+    // ranges per row: a multiple of 8, so that the tm blocks of one range share an XCD
+    sk.ranges = std::max(8, slots / tm / 8 * 8);
+    grid = static_cast<unsigned>(sk.ranges) * tm;
+    const int full = tn / sk.ranges;
+    sk.whole_waves = tn % sk.ranges == 0 ? full : std::max(0, full - 1);
+    sk.cut_first = sk.whole_waves * sk.ranges;
+    sk.total = (tn - sk.cut_first) * sk.ksteps;
+    cut_tiles = (tn - sk.cut_first) * tm;
+    sk.iters_per_block = std::max(1, (sk.total + sk.ranges - 1) / sk.ranges);
+    if (sk.total == 0) {
+      // whole waves cover every row exactly: nothing is cut
+    } else if (sk.iters_per_block >= sk.ksteps) {
       zero_cut = true;           // at most two contributors per tile: atomics onto zeroed tiles
     } else {
       pieces = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(grid) * 2 * BM * BN * sizeof(float)));
@@ -1359,8 +1396,8 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
   hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>), dim3(grid), dim3(kThreads), 0, st, P, out, pieces,
                      sk);
   if (pieces)
-    hipLaunchKernelGGL((conv_tap_assemble_kernel<BM, BN, WM, WN>), dim3(tiles * 4), dim3(kThreads), 0, st, P, out, pieces,
-                       sk);
+    hipLaunchKernelGGL((conv_tap_assemble_kernel<BM, BN, WM, WN>), dim3(cut_tiles * 4), dim3(kThreads), 0, st, P, out,
+                       pieces, sk);
   return 0;
 }
 
