@@ -34,9 +34,9 @@ PEAK_HBM_GBS = 8000.0
 # be the step's largest, from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
 # profiles/vgg16_b64_train_step_hbm_traffic.txt (counter units calibrated on the Relu kernel).
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "conv_fwd_128x128": (165.5 + 108.6) * 1e6,
-    "conv_bwd_data_128x128": (207.2 + 98.3) * 1e6,
-    "conv_bwd_filter_128x128": (505.0 + 64.3) * 1e6,
+    "conv_fwd_128x128": (469.0 + 139.4) * 1e6,
+    "conv_bwd_data_128x128": (653.7 + 129.7) * 1e6,
+    "conv_bwd_filter_128x128": (498.0 + 64.2) * 1e6,
 }
 
 
