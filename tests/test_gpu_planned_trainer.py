@@ -1,0 +1,100 @@
+"""The budgeted executor against the plain one on the GPU: same losses step by step, measured
+peak within the budget, tensors really leaving and coming back."""
+import numpy as np
+import pytest
+
+from tsplit_amd import planner, trainer
+
+pytestmark = pytest.mark.gpu
+
+SPEC = [("conv", "c1", 3, 16, 3, 1, 1), ("bn", "c1_bn", 16), ("relu",),
+        ("conv", "c2", 16, 16, 3, 1, 1), ("bn", "c2_bn", 16), ("relu",), ("maxpool", 2, 0, 2),
+        ("conv", "c3", 16, 32, 3, 1, 1), ("bn", "c3_bn", 32), ("relu",),
+        ("conv", "c4", 32, 32, 3, 1, 1), ("bn", "c4_bn", 32), ("relu",), ("maxpool", 2, 0, 2),
+        ("flatten",), ("fc", "f1", 32 * 8 * 8, 64), ("fc", "f2", 64, 10)]
+IN = (12, 3, 32, 32)
+OPT = ("momentum", 0.01, 0.9)
+
+
+def _data(rng):
+    x = rng.standard_normal(size=IN).astype(np.float32)
+    labels = np.zeros((IN[0], 10), np.float32)
+    labels[np.arange(IN[0]), rng.randint(0, 10, IN[0])] = 1.0
+    return x, labels
+
+
+def _plain_losses(spec_fused, steps, rng_seed=5):
+    from tsplit_amd import ndarray
+    rng = np.random.RandomState(rng_seed)
+    params = trainer.init_params(SPEC, seed=3)
+    t = trainer.Trainer(SPEC, params, IN, 10, optimizer=OPT, fuse_bn_relu=spec_fused)
+    x, labels = _data(rng)
+    gx, gl = ndarray.array(x, t.ctx), ndarray.array(labels, t.ctx)
+    out = []
+    for _ in range(steps):
+        t.step(gx, gl)
+        out.append(t.loss_value())
+    return out, {k: v.asnumpy() for k, v in t.params.items()}
+
+
+def _planned(spec, budget_frac, steps, piece_bytes=64 << 10, rng_seed=5):
+    from tsplit_amd import ndarray
+    from tsplit_amd.planned_trainer import PlannedTrainer, make_plan
+    rng = np.random.RandomState(rng_seed)
+    params = trainer.init_params(SPEC, seed=3)
+    free = make_plan(spec, IN, 10, None, OPT)
+    budget = None
+    if budget_frac is not None:
+        shapes = planner.layer_shapes(spec, IN)
+        floor, _ = planner.simulate(spec, shapes, range(1, len(spec)), free.fixed_bytes)
+        budget = int(floor + budget_frac * (free.peak_bytes - floor))
+    plan = make_plan(spec, IN, 10, budget, OPT, piece_bytes=piece_bytes)
+    t = PlannedTrainer(spec, params, IN, 10, plan, optimizer=OPT)
+    x, labels = _data(rng)
+    gx, gl = ndarray.array(x, t.ctx), ndarray.array(labels, t.ctx)
+    out = []
+    for _ in range(steps):
+        t.step(gx, gl)
+        out.append(t.loss_value())
+    return out, {k: v.asnumpy() for k, v in t.params.items()}, t, plan, free
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_unlimited_budget_equals_plain_trainer(fused):
+    spec = planner.fuse_spec(SPEC) if fused else SPEC
+    want, wp = _plain_losses(fused, 4)
+    got, gp, t, plan, _ = _planned(spec, None, 4)
+    assert not plan.swap
+    assert got == want                                  # same kernels on the same data: bit for bit
+    for k in wp:
+        assert np.array_equal(gp[k], wp[k]), k
+    # without a budget releases are not waited for, so the executor may hold a little more
+    assert t.peak >= plan.peak_bytes
+    assert t.live == plan.fixed_bytes - 4 * IN[0] * 10        # between steps: everything but the caller's labels
+    # with exactly the replayed peak as budget the run must fit: the replay and the executor
+    # agree to the byte
+    got2, _, t2, plan2, _ = _planned(spec, 1.0, 4)
+    assert not plan2.swap and plan2.budget_bytes == plan.peak_bytes
+    assert t2.peak == plan.peak_bytes and got2 == want
+
+
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("frac", [0.6, 0.1])
+def test_budget_is_met_and_results_do_not_change(fused, frac):
+    spec = planner.fuse_spec(SPEC) if fused else SPEC
+    want, wp = _plain_losses(fused, 4)
+    got, gp, t, plan, free = _planned(spec, frac, 4)
+    assert plan.swap and plan.budget_bytes < free.peak_bytes
+    assert t.peak <= plan.budget_bytes
+    # swapping moves bytes, it does not change them; split convolutions may round differently
+    np.testing.assert_allclose(got, want, rtol=2e-5)
+    for k in wp:
+        np.testing.assert_allclose(gp[k], wp[k], rtol=1e-4, atol=2e-5, err_msg=k)
+    if not plan.split:
+        assert got == want
+
+
+def test_impossible_budget_is_refused():
+    from tsplit_amd.planned_trainer import make_plan
+    with pytest.raises(ValueError, match="cannot be met"):
+        make_plan(SPEC, IN, 10, 64 << 10, OPT)

@@ -1,0 +1,88 @@
+"""Host-side checks of the memory planner: the allocation replay, the greedy choice and the
+layer-list fusion.  No GPU work."""
+import numpy as np
+import pytest
+
+from tsplit_amd import planner, trainer
+
+SMALL = [("conv", "c1", 3, 8, 3, 1, 1), ("bn", "c1_bn", 8), ("relu",), ("conv", "c2", 8, 8, 3, 1, 1), ("bn", "c2_bn", 8),
+         ("relu",), ("maxpool", 2, 0, 2), ("flatten",), ("fc", "f1", 8 * 8 * 8, 10)]
+IN = (4, 3, 16, 16)
+
+
+def test_fuse_spec_merges_bn_relu_pairs_only():
+    f = planner.fuse_spec(SMALL)
+    assert [l[0] for l in f] == ["conv", "bnrelu", "conv", "bnrelu", "maxpool", "flatten", "fc"]
+    assert f[1] == ("bnrelu", "c1_bn", 8)
+    assert planner.fuse_spec([("bn", "x", 4), ("maxpool", 2, 0, 2), ("relu",)]) == [("bn", "x", 4), ("maxpool", 2, 0, 2), ("relu",)]
+    assert planner.layer_shapes(f, IN)[-1] == (4, 10)
+
+
+def test_simulate_without_swapping_holds_every_activation_at_the_turn():
+    shapes = planner.layer_shapes(SMALL, IN)
+    size = planner.tensor_bytes(shapes)
+    peak, events = planner.simulate(SMALL, shapes, (), fixed_bytes=1000)
+    # last backward layer (fc): all activations + logits gradient + the fc input gradient
+    turn = [e for e in events if e[0] == "bwd" and e[1] == len(SMALL) - 1][0]
+    assert turn[2] == 1000 + sum(size) + size[-1] + size[-2]
+    assert peak == max(e[2] for e in events) >= turn[2]
+    # forward residency grows by one tensor per layer
+    fwd = [e[2] for e in events if e[0] == "fwd"]
+    assert fwd == [1000 + sum(size[:i + 2]) for i in range(len(SMALL))]
+
+
+def test_swapping_lowers_the_peak_and_in_place_gradients_cost_nothing():
+    shapes = planner.layer_shapes(SMALL, IN)
+    size = planner.tensor_bytes(shapes)
+    base, _ = planner.simulate(SMALL, shapes, ())
+    less, events = planner.simulate(SMALL, shapes, (1, 2, 3), prefetch=1)
+    assert less < base
+    # while layer 5 runs backward (Relu, in place) tensors 1..3 are away and one gradient is live
+    e5 = [e for e in events if e[0] == "bwd" and e[1] == 5][0]
+    assert not ({1, 2, 3} & set(e5[3])) and {4, 5, 6} <= set(e5[3])
+    assert e5[2] == sum(size[j] for j in e5[3]) + size[6]
+    # one layer ahead: tensor 3 is back while layer 4 runs backward
+    e4 = [e for e in events if e[0] == "bwd" and e[1] == 4][0]
+    assert 3 in e4[3] and 2 not in e4[3]
+
+
+def test_plan_meets_budgets_and_swaps_more_as_they_shrink():
+    fixed = 4096
+    free = planner.plan_memory(SMALL, IN, None, fixed)
+    assert not free.swap and not free.split
+    shapes = planner.layer_shapes(SMALL, IN)
+    floor, _ = planner.simulate(SMALL, shapes, range(1, len(SMALL)), fixed)     # everything that may leave has left
+    assert floor < free.peak_bytes
+    prev = set()
+    for frac in (0.9, 0.5, 0.0):
+        budget = int(floor + frac * (free.peak_bytes - floor))
+        p = planner.plan_memory(SMALL, IN, budget, fixed, piece_bytes=2048)
+        assert p.peak_bytes <= budget
+        assert 0 not in p.swap and len(SMALL) not in p.swap
+        assert len(p.swap) >= len(prev)
+        prev = set(p.swap)
+        for li, k in p.split.items():
+            assert SMALL[li][0] == "conv" and li in p.swap and 1 < k <= IN[0]
+    d = p.describe()
+    assert d["swap"] == sorted(p.swap) and d["budget_GiB"] == budget / planner.GiB
+
+
+def test_plan_raises_when_nothing_more_can_leave():
+    with pytest.raises(ValueError, match="cannot be met"):
+        planner.plan_memory(SMALL, IN, 1024, 0)
+
+
+def test_vgg16_batch64_numbers():
+    """The unplanned peak of VGG-16 b64: 3 x 527.8 MiB of parameter-sized arrays plus 39 conv-block
+    tensors, pools, FC activations, and two gradients at the widest point."""
+    spec = trainer.vgg16_spec(1000, 224)
+    shapes = planner.layer_shapes(spec, (64, 3, 224, 224))
+    size = planner.tensor_bytes(shapes)
+    conv_out = sum(size[i + 1] for i, l in enumerate(spec) if l[0] == "conv")
+    assert conv_out == 4 * 867041280                     # 867.0 M conv-output elements per step
+    fused = planner.fuse_spec(spec)
+    p_plain = planner.plan_memory(spec, (64, 3, 224, 224), None, 0)
+    p_fused = planner.plan_memory(fused, (64, 3, 224, 224), None, 0)
+    assert p_plain.peak_bytes - p_fused.peak_bytes == conv_out    # the BatchNorm outputs never exist
+    tight = planner.plan_memory(fused, (64, 3, 224, 224), 6 << 30, 1660 << 20)
+    assert tight.peak_bytes <= 6 << 30 and tight.swap

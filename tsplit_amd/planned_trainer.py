@@ -1,0 +1,329 @@
+"""Executor for sequential conv nets under a device-memory budget.
+
+Runs the same operator sequence as `tsplit_amd.trainer.Trainer` (one GPU symbol per graph
+node, filter gradients before data gradients, one optimizer call per parameter), but holds
+tensors only while the schedule of `tsplit_amd.planner` needs them:
+
+  * activations are allocated when their producer runs and released after their last backward
+    use; gradients live for two layers; Relu / BatchNorm gradients are written in place;
+  * the tensors the plan marks leave for pinned host memory after their forward use, in batch
+    micro-tensors on a copy stream (DLArrayCopyFromTo + DLEventRecord / DLEventSync, as the
+    reference's swapping executors do: python/athena/gpu_ops/vdnnExecutor.py:202-330), and come
+    back `prefetch` layers before the backward sweep needs them; a convolution whose input was
+    swapped starts each backward micro-op as soon as that micro-tensor has arrived;
+  * device memory is handed back to the pool only after the GPU has finished with it (an event
+    per release), so a buffer re-used by a copy-in can never still be read by a queued kernel.
+
+The budget covers what this executor allocates: parameters, gradients, optimizer state, the
+batch, activations and activation gradients.  The operator library's own scratch (split-K
+partials, re-laid filters, BatchNorm partial sums: tens of MB) is outside it.
+"""
+import collections
+
+import numpy as np
+
+from . import gpu_links as L
+from . import ndarray
+from .planner import IN_PLACE_BACKWARD, layer_shapes
+from .stream import create_event_handle, create_stream_handle
+from .trainer import param_shapes
+
+
+def fixed_bytes(spec, input_shape, num_classes, optimizer, split=()):
+    """Bytes the executor holds for the whole run: parameters, their gradients, optimizer state,
+    BatchNorm statistics, the per-piece filter gradients of split convolutions, loss and seed, and
+    the caller's labels (the batch itself is tensor 0 of the planner's replay)."""
+    shapes = param_shapes(spec)
+    params = sum(4 * int(np.prod(s)) for s in shapes.values())
+    total = params * (3 if optimizer[0] == "momentum" else 2)
+    total += sum(2 * 4 * l[2] for l in spec if l[0] in ("bn", "bnrelu"))
+    total += sum(4 * int(np.prod(shapes[spec[li][1] + "_weight"])) for li in split)
+    total += 8 + 4 * input_shape[0] * num_classes
+    return total
+
+
+def make_plan(spec, input_shape, num_classes, budget_bytes, optimizer=("sgd", 0.1), **kw):
+    """Plan for `spec` under `budget_bytes` (None: no limit), with the executor's own fixed
+    allocations accounted for."""
+    from .planner import plan_memory
+    split = ()
+    for _ in range(4):
+        plan = plan_memory(spec, input_shape, budget_bytes, fixed_bytes(spec, input_shape, num_classes, optimizer, split),
+                           **kw)
+        if set(plan.split) == set(split):
+            return plan
+        split = tuple(plan.split)
+    return plan
+
+
+class PlannedTrainer(object):
+    def __init__(self, spec, params, input_shape, num_classes, plan, ctx=None, optimizer=("sgd", 0.1), bn_eps=0.01):
+        self.spec = list(spec)
+        self.plan = plan
+        self.prefetch = plan.prefetch
+        self.ctx = ctx if ctx is not None else ndarray.gpu(0)
+        self.host_ctx = ndarray.cpu(0)
+        self.stream = create_stream_handle(self.ctx)
+        self.out_stream = create_stream_handle(self.ctx)     # device -> host copies
+        self.in_stream = create_stream_handle(self.ctx)      # host -> device copies
+        self.optimizer = optimizer
+        self.eps = bn_eps
+        self.shapes = layer_shapes(self.spec, input_shape)
+        assert self.shapes[-1] == (input_shape[0], num_classes), (self.shapes[-1], num_classes)
+        self.nl = len(self.spec)
+        self.budget = plan.budget_bytes
+        self.live = 0
+        self.peak = 0
+        self.pending = collections.deque()     # (array, bytes, [events]) released, GPU maybe not done
+        self.stall_events = 0
+        # parameters, gradients, optimizer state, per-layer saved statistics: fixed for the run
+        self.params = {k: self._own(ndarray.array(v, self.ctx)) for k, v in params.items()}
+        self.grads = {k: self._own(ndarray.empty(v.shape, self.ctx)) for k, v in params.items()}
+        self.state = {}
+        if optimizer[0] == "momentum":
+            self.state = {k: self._own(ndarray.array(np.zeros(v.shape, np.float32), self.ctx)) for k, v in params.items()}
+        self.saved = {}
+        for li, layer in enumerate(self.spec):
+            if layer[0] in ("bn", "bnrelu"):
+                c = layer[2]
+                self.saved[li] = (self._own(ndarray.empty((1, c, 1, 1), self.ctx)),
+                                  self._own(ndarray.empty((1, c, 1, 1), self.ctx)))
+        # per-piece filter gradient of the split convolutions, summed into the layer's gradient
+        self.dw_piece = {li: self._own(ndarray.empty(param_shapes([self.spec[li]])[self.spec[li][1] + "_weight"], self.ctx))
+                         for li in plan.split}
+        self.loss = self._own(ndarray.empty((1,), self.ctx))
+        self.ones = self._own(ndarray.empty((1,), self.ctx))
+        L.array_set(self.ones, 1.0, self.stream)
+        self.host = {j: ndarray.empty(self.shapes[j], self.host_ctx) for j in plan.swap}     # pinned
+        self.acts = [None] * (self.nl + 1)
+        self.in_events = {}                    # tensor -> list of per-piece copy-in events
+        self.away = set()                      # tensors whose device copy is released
+
+    # ------------------------------------------------------------------ memory accounting
+    @staticmethod
+    def _bytes(arr):
+        return 4 * int(np.prod(arr.shape))
+
+    def _own(self, arr):
+        self.live += self._bytes(arr)
+        self.peak = max(self.peak, self.live)
+        return arr
+
+    def _reap(self, need=0, force=False):
+        """Hand finished releases back to the pool; wait for as many as `need` more bytes take
+        (all of them with `force`)."""
+        while self.pending:
+            arr, nbytes, events = self.pending[0]
+            done = all(e.query() for e in events)
+            if not done:
+                if not force and (self.budget is None or self.live + need <= self.budget):
+                    return
+                self.stall_events += 0 if force else 1
+                for e in events:
+                    e.sync()
+            self.pending.popleft()
+            if isinstance(arr, tuple):         # a swapped tensor keeps its struct: drop the data only
+                arr[0].delete_itself()
+                arr[0].sTensor = []
+            self.live -= nbytes
+
+    def _alloc(self, shape, reuse=None):
+        nbytes = 4 * int(np.prod(shape))
+        self._reap(nbytes)
+        if self.budget is not None and self.live + nbytes > self.budget:
+            raise MemoryError("budget of %d bytes: %d live, %d more needed" % (self.budget, self.live, nbytes))
+        if reuse is not None:
+            reuse.malloc_itself()
+            arr = reuse
+        else:
+            arr = ndarray.empty(shape, self.ctx)
+        self.live += nbytes
+        self.peak = max(self.peak, self.live)
+        return arr
+
+    def _release(self, arr, extra_events=(), keep_struct=False):
+        """The host is done with `arr`; the pool gets it once the compute stream has passed this point."""
+        ev = create_event_handle(self.ctx)
+        ev.record(self.stream)
+        self.pending.append(((arr,) if keep_struct else arr, self._bytes(arr), [ev] + list(extra_events)))
+
+    # ------------------------------------------------------------------ swapping
+    def _pieces(self, arr, li):
+        k = self.plan.split.get(li, 1)
+        if k == 1:
+            return [arr]
+        if not arr.sTensor or arr.split_number != k:
+            arr.sTensor = []
+            arr.split_tensor(k)
+        return arr.sTensor
+
+    def _swap_out(self, j, produced_event):
+        """Tensor j is complete once `produced_event` has passed; copy it out piece by piece."""
+        produced_event.sync()
+        dev, host = self.acts[j], self.host[j]
+        for d, h in zip(self._pieces(dev, j), self._pieces(host, j)):
+            h.async_d2h(d, self.out_stream)
+        done = create_event_handle(self.ctx)
+        done.record(self.out_stream)
+        return done
+
+    def _swap_in(self, j):
+        if j not in self.away:
+            return
+        self.away.discard(j)
+        dev = self._alloc(self.shapes[j], reuse=self.acts[j])
+        events = []
+        for d, h in zip(self._pieces(dev, j), self._pieces(self.host[j], j)):
+            d.async_h2d(h, self.in_stream)
+            ev = create_event_handle(self.ctx)
+            ev.record(self.in_stream)
+            events.append(ev)
+        self.in_events[j] = events
+
+    def _arrived(self, j, piece=None):
+        events = self.in_events.get(j)
+        if not events:
+            return
+        if piece is None:
+            for e in events:
+                e.sync()
+            del self.in_events[j]
+        else:
+            events[piece].sync()
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, x, labels):
+        self.acts[0] = x
+        produced = None                       # event after the layer that produced the current input
+        for li, layer in enumerate(self.spec):
+            a = self.acts[li]
+            out = self.acts[li + 1] = self._alloc(self.shapes[li + 1])
+            kind = layer[0]
+            if kind == "conv":
+                _, name, cin, cout, k, pad, stride = layer
+                w = self.params[name + "_weight"]
+                for xa, ya in zip(self._pieces(a, li), self._pieces(out, li)):
+                    L.CuDNN_conv2d(xa, w, ya, pad, pad, stride, self.stream)
+            elif kind == "bnrelu":
+                sm, sv = self.saved[li]
+                L.batch_norm_relu(a, self.params[layer[1] + "_scale"], self.params[layer[1] + "_bias"], out, sm, sv,
+                                  self.eps, self.stream)
+            elif kind == "bn":
+                sm, sv = self.saved[li]
+                L.CuDNN_Batch_Normalization(a, self.params[layer[1] + "_scale"], self.params[layer[1] + "_bias"], out,
+                                            sm, sv, 0.99, self.eps, self.stream)
+            elif kind == "relu":
+                L.relu(a, out, self.stream)
+            elif kind == "maxpool":
+                _, k, pad, stride = layer
+                L.CuDNN_max_pooling2d(a, k, k, out, pad, stride, self.stream)
+            elif kind == "flatten":
+                L.array_reshape(a, out, self.stream)
+            elif kind == "fc":
+                L.matrix_multiply(a, False, self.params[layer[1] + "_weight"], False, out, self.stream)
+            else:
+                raise ValueError(kind)
+            after = create_event_handle(self.ctx)
+            after.record(self.stream)
+            if li in self.plan.swap:
+                copied = self._swap_out(li, produced)
+                self._release(a, [copied], keep_struct=True)
+                self.away.add(li)
+            produced = after
+        L.softmax_cross_entropy(self.acts[-1], labels, self.loss, self.stream)
+        return self.loss
+
+    # ------------------------------------------------------------------ backward
+    def backward(self, labels):
+        self._reap(force=True)                 # every tensor that left has really left
+        g_out = self._alloc(self.shapes[-1])
+        L.softmax_cross_entropy_gradient(self.acts[-1], labels, self.ones, g_out, self.stream)
+        for li in range(self.nl - 1, -1, -1):
+            layer = self.spec[li]
+            kind = layer[0]
+            # copy-in: this layer's input now if it is still away, the next `prefetch` ones ahead of time
+            for j in range(li, max(0, li - self.prefetch) - 1, -1):
+                if j >= 1:
+                    self._swap_in(j)
+            a, y = self.acts[li], self.acts[li + 1]
+            first = li == 0
+            in_place = kind in IN_PLACE_BACKWARD
+            g_in = None if first else g_out if in_place else self._alloc(self.shapes[li])
+            if kind == "conv":
+                _, name, cin, cout, k, pad, stride = layer
+                w, dw = self.params[name + "_weight"], self.grads[name + "_weight"]
+                xs, gs = self._pieces(a, li), self._pieces(g_out, li)
+                for i, (xa, ga) in enumerate(zip(xs, gs)):
+                    self._arrived(li, i if len(xs) > 1 else None)
+                    if i == 0:
+                        L.CuDNN_conv2d_gradient_of_filter(xa, ga, dw, pad, pad, stride, self.stream)
+                    else:
+                        piece = self.dw_piece[li]
+                        L.CuDNN_conv2d_gradient_of_filter(xa, ga, piece, pad, pad, stride, self.stream)
+                        L.matrix_elementwise_add(dw, piece, dw, self.stream)
+                self.in_events.pop(li, None)
+                if not first:
+                    for ga, gi in zip(gs, self._pieces(g_in, li)):
+                        L.CuDNN_conv2d_gradient_of_data(w, ga, gi, pad, pad, stride, self.stream)
+            else:
+                self._arrived(li)
+                if kind == "bnrelu":
+                    sm, sv = self.saved[li]
+                    name = layer[1]
+                    L.batch_norm_relu_gradient(g_out, a, self.params[name + "_scale"], self.params[name + "_bias"], g_in,
+                                               self.grads[name + "_scale"], self.grads[name + "_bias"], sm, sv, self.eps,
+                                               self.stream)
+                elif kind == "bn":
+                    sm, sv = self.saved[li]
+                    name = layer[1]
+                    L.CuDNN_Batch_Normalization_gradient(g_out, a, self.params[name + "_scale"], g_in,
+                                                         self.grads[name + "_scale"], self.grads[name + "_bias"], sm, sv,
+                                                         self.eps, self.stream)
+                elif kind == "relu":
+                    L.relu_gradient(a, g_out, g_in, self.stream)
+                elif kind == "maxpool":
+                    _, k, pad, stride = layer
+                    L.CuDNN_max_pooling2d_gradient(y, g_out, a, k, k, g_in, pad, stride, self.stream)
+                elif kind == "flatten":
+                    L.array_reshape(g_out, g_in, self.stream)
+                elif kind == "fc":
+                    w = self.params[layer[1] + "_weight"]
+                    L.matrix_multiply(a, True, g_out, False, self.grads[layer[1] + "_weight"], self.stream)
+                    if not first:
+                        L.matrix_multiply(g_out, False, w, True, g_in, self.stream)
+            # the layer's output and output gradient are dead now
+            self._release(y)
+            self.acts[li + 1] = None
+            if not in_place or first:
+                self._release(g_out)
+            g_out = g_in
+        self.acts[0] = None
+
+    # ------------------------------------------------------------------ update / step
+    def update(self):
+        for name, p in self.params.items():
+            g = self.grads[name]
+            if self.optimizer[0] == "sgd":
+                L.sgd_update(p, g, self.optimizer[1], self.stream)
+            elif self.optimizer[0] == "momentum":
+                L.momentum_update(p, g, self.state[name], self.optimizer[1], self.optimizer[2], False, self.stream)
+            else:
+                raise ValueError(self.optimizer[0])
+
+    def step(self, x, labels):
+        self.live += self._bytes(x) + self._bytes(labels)      # the caller's batch counts against the budget
+        self.peak = max(self.peak, self.live)
+        self.forward(x, labels)
+        self.backward(labels)
+        self.update()
+        self.stream.sync()
+        self._reap(force=True)                                  # everything queued has finished by now
+        self.live -= self._bytes(x) + self._bytes(labels)
+        return self.loss
+
+    def sync(self):
+        self.stream.sync()
+
+    def loss_value(self):
+        self.sync()
+        return float(self.loss.asnumpy()[0])

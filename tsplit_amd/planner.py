@@ -1,0 +1,239 @@
+"""Memory planner for the sequential-net trainer: which saved activations leave the device
+between their forward and backward use, and in how many batch micro-tensors the layers around
+them run, so that a training step fits a device-memory budget.
+
+The reference ships the primitives for this (batch micro-tensor views, DLArrayReuseAlloc, the
+swap copies and events: src/common/c_runtime_api.cc:164-271, python/athena/ndarray.py:221-243,
+351-409) and the tensor-granularity policies built on them (python/athena/gpu_ops/
+vdnnExecutor.py:202-330), but not the planner that chooses splits; this module is that planner
+for the layer lists of `tsplit_amd.trainer`.
+
+Model.  Tensor j is the input of layer j (tensor 0 is the batch, tensor L the logits).  Every
+tensor is needed again in the backward sweep (by the layer that consumed it, and a max-pool's
+output also by the pool itself).  A BatchNorm directly followed by a Relu may be merged into one
+"bnrelu" layer (`fuse_spec`), which runs on the fused entry points and never materialises the
+BatchNorm output.  The executor (`tsplit_amd.planned_trainer`) follows this
+schedule, which `simulate` replays byte for byte:
+
+  forward  of layer i : allocate tensor i+1, run; then a swapped tensor i starts leaving
+                        (it left the compute stream's hands) and is released once its copy is done
+  backward of layer i : tensor i must be resident (a swapped one was re-allocated and its
+                        copy-in started while layer i+1 ran backward: one layer ahead);
+                        allocate the input gradient unless the layer writes it in place
+                        (Relu, BatchNorm: elementwise in the gradient); run; release tensor
+                        i+1 and the output gradient
+
+Choice.  Greedy: while the replayed peak exceeds the budget, take the moment of the peak and,
+among the tensors resident but idle then, swap the one that adds the least estimated step
+time per byte it frees.  The estimate (`step_ms`) walks the same schedule with a cost model:
+layer times from measured rates, one copy at a time per link direction, the sweep waiting
+where a copy has not finished - so a tensor whose transfer hides behind a long convolution is
+cheap, and a run of neighbouring small tensors that would queue on the link is not.  Layers
+whose input is swapped run in micro-tensors of at most `piece_bytes`, so that a backward
+micro-op starts as soon as its own piece has arrived.
+"""
+import numpy as np
+
+GiB = float(1 << 30)
+
+
+class CostModel(object):
+    """Rates measured on one MI355X with this library (fp32): contractions, streaming
+    kernels on the bytes they move, and the pinned-host link each way."""
+
+    def __init__(self, conv_tflops=110.0, conv_tflops_narrow=90.0, matmul_tflops=65.0, stream_gbs=5500.0,
+                 link_gbs=55.0):
+        self.conv_tflops = conv_tflops
+        self.conv_tflops_narrow = conv_tflops_narrow
+        self.matmul_tflops = matmul_tflops
+        self.stream_gbs = stream_gbs
+        self.link_gbs = link_gbs
+
+    def copy_ms(self, nbytes):
+        return nbytes / (self.link_gbs * 1e9) * 1e3
+
+    def layer_ms(self, layer, in_shape, out_shape, backward, first=False):
+        """Estimated time of one layer's forward (or backward) sweep."""
+        n_in, n_out = float(np.prod(in_shape)), float(np.prod(out_shape))
+        kind = layer[0]
+        if kind == "conv":
+            _, _, cin, cout, k, _, _ = layer
+            flop = 2.0 * n_out * cin * k * k
+            rate = self.conv_tflops if min(cin, cout) > 64 else self.conv_tflops_narrow
+            passes = (1 if first else 2) if backward else 1
+            return passes * flop / (rate * 1e12) * 1e3
+        if kind == "fc":
+            flop = 2.0 * in_shape[0] * layer[2] * layer[3]
+            return (2 if backward and not first else 1) * flop / (self.matmul_tflops * 1e12) * 1e3
+        moved = {"bn": (20.0 if backward else 12.0) * n_in, "relu": (12.0 if backward else 8.0) * n_in,
+                 "bnrelu": (20.0 if backward else 12.0) * n_in,
+                 "maxpool": 4.0 * ((2 * n_in + n_out) if backward else (n_in + n_out)),
+                 "flatten": 0.0}[kind]
+        return moved / (self.stream_gbs * 1e9) * 1e3
+
+
+IN_PLACE_BACKWARD = ("relu", "bn", "bnrelu")   # the input gradient may overwrite the output gradient
+
+
+class MemoryPlan(object):
+    def __init__(self, swap, split, peak_bytes, est_step_ms, est_free_step_ms, fixed_bytes, budget_bytes, prefetch):
+        self.swap = frozenset(swap)          # tensor indices that leave the device after their forward use
+        self.split = dict(split)             # layer index -> batch micro-tensors
+        self.prefetch = prefetch             # layers of lead a copy-in gets over the backward sweep
+        self.peak_bytes = peak_bytes
+        self.est_step_ms = est_step_ms             # cost-model step time with this plan ...
+        self.est_free_step_ms = est_free_step_ms   # ... and with nothing swapped
+        self.fixed_bytes = fixed_bytes
+        self.budget_bytes = budget_bytes
+
+    def describe(self):
+        return {"swap": sorted(self.swap), "split": {int(k): int(v) for k, v in sorted(self.split.items())},
+                "prefetch": self.prefetch, "peak_GiB": self.peak_bytes / GiB, "est_step_ms": self.est_step_ms,
+                "est_free_step_ms": self.est_free_step_ms,
+                "fixed_GiB": self.fixed_bytes / GiB,
+                "budget_GiB": None if self.budget_bytes is None else self.budget_bytes / GiB}
+
+
+def fuse_spec(spec):
+    """("bn", name, C), ("relu",) -> ("bnrelu", name, C)."""
+    out, i = [], 0
+    while i < len(spec):
+        if spec[i][0] == "bn" and i + 1 < len(spec) and spec[i + 1][0] == "relu":
+            out.append(("bnrelu",) + tuple(spec[i][1:]))
+            i += 2
+        else:
+            out.append(spec[i])
+            i += 1
+    return out
+
+
+def layer_shapes(spec, input_shape):
+    from .trainer import _out_shape
+    shapes = [tuple(input_shape)]
+    for layer in spec:
+        shapes.append(_out_shape(layer, shapes[-1]))
+    return shapes
+
+
+def tensor_bytes(shapes):
+    return [4 * int(np.prod(s)) for s in shapes]
+
+
+def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3):
+    """Replays the executor's allocation schedule.  Returns (peak_bytes, events) where events is
+    a list of (phase, layer, resident_bytes, resident_tensor_indices, busy_tensor_indices)."""
+    L = len(spec)
+    size = tensor_bytes(shapes)
+    swap = set(swap)
+    resident = set([0])
+    grad_bytes = 0
+    events = []
+
+    def note(phase, li):
+        events.append((phase, li, fixed_bytes + sum(size[j] for j in resident) + grad_bytes, frozenset(resident),
+                       frozenset((li, li + 1))))
+
+    for li in range(L):
+        resident.add(li + 1)
+        note("fwd", li)
+        if li in swap:
+            resident.discard(li)
+    g_out = size[L]                    # the loss gradient has the logits' size
+    for li in range(L - 1, -1, -1):
+        # the layer's own input must be there; copy-in of the next `prefetch` layers down starts now
+        for j in range(li, max(0, li - prefetch) - 1, -1):
+            if j >= 1 and j in swap:
+                resident.add(j)
+        in_place = spec[li][0] in IN_PLACE_BACKWARD
+        g_in = 0 if li == 0 else g_out if in_place else size[li]
+        grad_bytes = g_out if (li == 0 or in_place) else g_out + g_in
+        note("bwd", li)
+        resident.discard(li + 1)
+        g_out = g_in
+        grad_bytes = g_out
+    peak = max(e[2] for e in events)
+    return peak, events
+
+
+def step_ms(spec, shapes, swap, cost, prefetch=3):
+    """Estimated step time under the replayed schedule: one compute stream, one copy-out and one
+    copy-in stream (each link direction carries one copy at a time, in issue order).  A swapped
+    tensor starts leaving when its consumer starts and the sweep waits for it when that consumer
+    ends (the release point of the replay); a copy-in is issued `prefetch` layers ahead and the
+    layer that needs the tensor waits for its arrival."""
+    L = len(spec)
+    size = tensor_bytes(shapes)
+    swap = set(swap)
+    t = out_free = 0.0
+    for li in range(L):
+        t0 = t
+        t += cost.layer_ms(spec[li], shapes[li], shapes[li + 1], False)
+        if li in swap:
+            out_free = max(out_free, t0) + cost.copy_ms(size[li])
+            t = max(t, out_free)
+    in_free, arrival = 0.0, {}
+    for li in range(L - 1, -1, -1):
+        for j in range(li, max(0, li - prefetch) - 1, -1):
+            if j >= 1 and j in swap and j not in arrival:
+                in_free = max(in_free, t) + cost.copy_ms(size[j])
+                arrival[j] = in_free
+        t = max(t, arrival.get(li, 0.0)) + cost.layer_ms(spec[li], shapes[li], shapes[li + 1], True, first=li == 0)
+    return t
+
+
+def plan_memory(spec, input_shape, budget_bytes=None, fixed_bytes=0, cost=None, piece_bytes=128 << 20, prefetch=3):
+    """-> MemoryPlan for `spec` (already fused, if fusion is wanted).  Raises ValueError when
+    even swapping every idle tensor does not fit the budget."""
+    cost = cost or CostModel()
+    shapes = layer_shapes(spec, input_shape)
+    batch = shapes[0][0]
+    size = tensor_bytes(shapes)
+    L = len(spec)
+    swap = set()
+    free_ms = now_ms = step_ms(spec, shapes, swap, cost, prefetch)
+    while True:
+        peak, events = simulate(spec, shapes, swap, fixed_bytes, prefetch)
+        if budget_bytes is None or peak <= budget_bytes:
+            break
+        # moments at the peak; candidates = resident, idle, not yet swapped, neither batch nor logits
+        candidates = set()
+        for phase, li, total, resident, busy in events:
+            if total < peak:
+                continue
+            for j in resident - busy - swap:
+                if j == 0 or j >= L:
+                    continue
+                if phase == "bwd" and li - prefetch <= j < li:
+                    continue            # on its way back in at that moment
+                candidates.add(j)
+        best = None
+        for j in candidates:
+            added = step_ms(spec, shapes, swap | {j}, cost, prefetch) - now_ms
+            score = (added + 1e-3) / size[j]
+            if best is None or score < best[0]:
+                best = (score, j)
+        if best is None:
+            raise ValueError("budget of %.2f GiB cannot be met: %.2f GiB are needed with every idle tensor swapped"
+                             % (budget_bytes / GiB, peak / GiB))
+        swap.add(best[1])
+        now_ms = step_ms(spec, shapes, swap, cost, prefetch)
+    # the last pick may have freed more than was missing: put back what the budget can hold,
+    # dearest first
+    for _ in range(len(swap)):
+        gains = []
+        for j in swap:
+            rest = swap - {j}
+            if simulate(spec, shapes, rest, fixed_bytes, prefetch)[0] <= budget_bytes:
+                gains.append((now_ms - step_ms(spec, shapes, rest, cost, prefetch), j))
+        if not gains or max(gains)[0] <= 0:
+            break
+        swap.discard(max(gains)[1])
+        now_ms = step_ms(spec, shapes, swap, cost, prefetch)
+        peak = simulate(spec, shapes, swap, fixed_bytes, prefetch)[0]
+    split = {}
+    for li, layer in enumerate(spec):
+        if layer[0] == "conv" and li >= 1 and li in swap:
+            k = int(min(batch, max(1, -(-size[li] // piece_bytes))))
+            if k > 1:
+                split[li] = k
+    return MemoryPlan(swap, split, peak, now_ms, free_ms, fixed_bytes, budget_bytes, prefetch)

@@ -61,7 +61,7 @@ def param_shapes(spec):
         if layer[0] == "conv":
             _, name, cin, cout, k, _, _ = layer
             shapes[name + "_weight"] = (cout, cin, k, k)
-        elif layer[0] == "bn":
+        elif layer[0] in ("bn", "bnrelu"):
             _, name, c = layer
             shapes[name + "_scale"] = (1, c, 1, 1)
             shapes[name + "_bias"] = (1, c, 1, 1)
@@ -94,7 +94,7 @@ def _out_shape(layer, s):
     if kind == "conv":
         _, _, _, cout, k, pad, stride = layer
         return (s[0], cout, (s[2] + 2 * pad - k) // stride + 1, (s[3] + 2 * pad - k) // stride + 1)
-    if kind in ("bn", "relu"):
+    if kind in ("bn", "relu", "bnrelu"):
         return s
     if kind == "maxpool":
         _, k, pad, stride = layer
