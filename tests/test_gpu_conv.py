@@ -54,6 +54,13 @@ CASES = [
     (2, 16, 2, 2, 8, 3, 3, 1, 1, 1),       # 4 positions
     (2, 32, 10, 14, 24, 1, 7, 0, 3, 1),    # 140 positions, 1x7 filter
     (5, 48, 14, 14, 72, 3, 3, 1, 1, 1),    # 196 positions, odd image count
+    # ... and not a multiple of 4: the 16-byte gradient words start on 4-byte boundaries and the
+    # last word of an image straddles into the next row
+    (2, 16, 7, 7, 24, 3, 3, 1, 1, 1),      # 49 positions
+    (3, 32, 17, 17, 40, 1, 7, 0, 3, 1),    # 289 positions, 1x7
+    (2, 16, 5, 5, 8, 1, 1, 0, 0, 1),       # 25 positions, 1x1
+    (2, 16, 35, 35, 20, 3, 3, 1, 1, 1),    # 1225 positions
+    (3, 16, 3, 5, 136, 3, 3, 1, 1, 1),     # 15 positions: less than one k-step, two row tiles
 ]
 
 

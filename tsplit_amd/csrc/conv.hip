@@ -579,12 +579,13 @@ __global__ __launch_bounds__(kThreads) void conv_tap_zero_cut_tiles_kernel(TapCo
 }
 
 // ------------------------------------------------------------------ the tap-major filter-gradient kernel
-// Backward-filter for "same" stride-1 convolutions (oH = H, oW = W) with C % 16 == 0 and
-// H*W % 16 == 0, written like conv_tap_kernel so that the k-loop does almost no vector-ALU work.
+// Backward-filter for "same" stride-1 convolutions (oH = H, oW = W) with C % 16 == 0,
+// written like conv_tap_kernel so that the k-loop does almost no vector-ALU work.
 // The reduction runs over positions k = (img, p); because the convolution is "same", the
 // gathered element of tap (dr, dc) for output position p is x[img][c][p + dr*W + dc] - linear
 // in p - so the per-thread byte offset is a loop constant and the step's (img, p0) travels in
-// the scalar offset.  A 16-wide step never straddles two images (H*W % 16 == 0).  The padding
+// the scalar offset.  A 16-wide step never straddles two images (H*W % 16 == 0, or the TAIL
+// variant pads every image to that).  The padding
 // test needs the column of p, kept incrementally, and one range test on the linear index.
 struct TapWgradParams {
   const float *dy, *x;
@@ -596,8 +597,9 @@ struct TapWgradParams {
   int HWp;               // HW rounded up to a multiple of 16: the reduction runs over imgs*HWp positions
 };
 
-// TAIL: H*W is a multiple of 4 but not of 16.  Every image's positions are padded to HWp; the
-// padded ones read as zeros (one more compare per operand and step).
+// TAIL: H*W is not a multiple of 16.  Every image's positions are padded to HWp; the padded ones
+// read as zeros (a compare per operand and step, three selects per dy word).  When H*W is not a
+// multiple of 4 either, the 16-byte dy words start on 4-byte boundaries.
 template <int BM, int BN, int WM, int WN, bool TAIL>
 __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams P, float *__restrict__ part,
                                                                   TileGrid tg) {
@@ -661,13 +663,14 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
 
   u32x4 ra_regs[PA];
   unsigned rb_regs[KCOLS];
+  int a_cnt = 4;
 
   auto load_step = [&]() {
     const int soff_a = (img * P.O * P.HW + p0) * 4;
-    const bool word_ok = !TAIL || p0 + 4 * (tid & 3) < P.HW;     // H*W % 4 == 0: a word is all in or all out
+    if (TAIL) a_cnt = P.HW - (p0 + 4 * (tid & 3));               // positions of this thread's word inside the image
 #pragma unroll
     for (int s = 0; s < PA; ++s)
-      ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, word_ok ? a_voff[s] : kOobOffset, soff_a, 0);
+      ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_cnt > 0 ? a_voff[s] : kOobOffset, soff_a, 0);
     const int p = p0 + klocal;
     const bool ok = cols_ok && (!TAIL || p < P.HW) &&
                     static_cast<unsigned>(p + dr * P.W) < static_cast<unsigned>(P.HW) &&
@@ -688,8 +691,15 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
   };
   auto store_step = [&](float *sa, float *sb) {
 #pragma unroll
-    for (int s = 0; s < PA; ++s)
-      *reinterpret_cast<u32x4 *>(sa + ((tid >> 2) + 64 * s) * ALds::kStride + 4 * (tid & 3)) = ra_regs[s];
+    for (int s = 0; s < PA; ++s) {
+      u32x4 r = ra_regs[s];
+      if (TAIL) {        // a word that straddles the end of the image carries the next row's first values
+        r.y = a_cnt >= 2 ? r.y : 0u;
+        r.z = a_cnt >= 3 ? r.z : 0u;
+        r.w = a_cnt >= 4 ? r.w : 0u;
+      }
+      *reinterpret_cast<u32x4 *>(sa + ((tid >> 2) + 64 * s) * ALds::kStride + 4 * (tid & 3)) = r;
+    }
 #pragma unroll
     for (int i = 0; i < KCOLS; ++i)
       reinterpret_cast<unsigned *>(sb)[(jlocal0 + i) * BLds::kStride + klocal] = rb_regs[i];
@@ -1679,7 +1689,7 @@ int launch_wgrad_narrow(const ConvGeo &g, const float *x, const float *dy, float
 
 inline bool wgrad_tap_ok(const ConvGeo &g) {
   const int64_t bytes_x = static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4, bytes_dy = static_cast<int64_t>(g.imgs) * g.O * g.H * g.W * 4;
-  return g.s == 1 && g.oH == g.H && g.oW == g.W && (g.H * g.W) % 4 == 0 && g.C % BK == 0 &&
+  return g.s == 1 && g.oH == g.H && g.oW == g.W && g.C % BK == 0 &&
          bytes_x + 4 * (static_cast<int64_t>(g.ph) * g.W + g.pw) < (1ll << 31) && bytes_dy < (1ll << 31);
 }
 
