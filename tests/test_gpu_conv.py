@@ -43,6 +43,15 @@ CASES = [
     (2, 8, 20, 20, 12, 5, 5, 2, 2, 3),     # stride 3
     (1, 70, 12, 12, 130, 3, 3, 1, 1, 2),   # 128x128 tiles, ragged
     (1, 4, 9, 9, 6, 2, 2, 0, 0, 3),        # stride larger than the filter: some inputs get no gradient
+    # the same with output channels in multiples of 16: the phases run on the buffer-load kernel
+    (2, 24, 15, 15, 48, 3, 3, 1, 1, 2),
+    (2, 16, 17, 17, 32, 3, 3, 0, 0, 2),
+    (1, 8, 23, 19, 16, 7, 7, 3, 3, 2),
+    (2, 8, 20, 20, 16, 5, 5, 2, 2, 3),
+    (1, 70, 12, 12, 144, 3, 3, 1, 1, 2),
+    (1, 4, 9, 9, 16, 2, 2, 0, 0, 3),
+    (8, 64, 56, 56, 128, 3, 3, 1, 1, 2),   # ResNet stage transition: tiles cut between blocks
+    (4, 256, 28, 28, 512, 1, 1, 0, 0, 2),  # ResNet shortcut, 128x128 tiles in two rows
     # at most 32 filter columns (C*kH*kW): backward-filter takes the few-columns kernel
     (4, 3, 64, 64, 64, 3, 3, 1, 1, 1),     # several K slices, folded
     (3, 1, 19, 23, 100, 5, 5, 2, 2, 1),    # 25 columns, two row tiles, ragged K (oH*oW odd)

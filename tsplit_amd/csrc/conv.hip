@@ -276,7 +276,20 @@ struct TapConvParams {
   int M, N, K;
   int out_plane;        // elements per channel plane of the output
   int64_t out_img_stride;
+  // Column (i, j) of an image goes to element (out_a0 + out_s*i)*out_w + out_b0 + out_s*j of its
+  // output plane.  out_s == 1 with out_a0 = out_b0 = 0 and out_w = the column width: linear.
+  int out_s, out_a0, out_b0, out_w;
 };
+
+// offset of output column n (without the row term)
+__device__ __forceinline__ int64_t tap_out_col(const TapConvParams &P, int n) {
+  const uint32_t img = P.plane.div(n);
+  const uint32_t p = n - img * P.plane.d;
+  if (P.out_s == 1) return static_cast<int64_t>(img) * P.out_img_stride + p;
+  const uint32_t i = P.width.div(p), j = p - i * P.width.d;
+  return static_cast<int64_t>(img) * P.out_img_stride +
+         static_cast<int64_t>(P.out_a0 + P.out_s * static_cast<int>(i)) * P.out_w + (P.out_b0 + P.out_s * static_cast<int>(j));
+}
 
 constexpr int kBufFlags = 0x00020000;           // raw buffer, 32-bit untyped data (gfx9 family)
 constexpr unsigned kOobOffset = 0x80000000u;    // beyond any tensor this path accepts (< 2 GiB)
@@ -476,8 +489,7 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
       for (int ni = 0; ni < 2; ++ni) {
         const int n = n0 + wn0 + 32 * ni + (lane & 31);
         if (n >= P.N) continue;
-        const uint32_t img = P.plane.div(n);
-        const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
+        const int64_t coff = tap_out_col(P, n);
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi) {
           const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
@@ -495,8 +507,7 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
       for (int ni = 0; ni < 2; ++ni) {
         const int n = n0 + wn0 + 32 * ni + (lane & 31);
         if (n >= P.N) continue;
-        const uint32_t img = P.plane.div(n);
-        const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
+        const int64_t coff = tap_out_col(P, n);
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi) {
           const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
@@ -550,8 +561,7 @@ __global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvPara
   }
   const int n = n0 + wn0 + 32 * ni + (lane & 31);
   if (n >= P.N) return;
-  const uint32_t img = P.plane.div(n);
-  const int64_t coff = static_cast<int64_t>(img) * P.out_img_stride + (n - img * P.plane.d);
+  const int64_t coff = tap_out_col(P, n);
   const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
 #pragma unroll
   for (int e = 0; e < 16; ++e) {
@@ -571,10 +581,7 @@ __global__ __launch_bounds__(kThreads) void conv_tap_zero_cut_tiles_kernel(TapCo
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   for (int idx = threadIdx.x; idx < BM * BN; idx += kThreads) {
     const int m = m0 + idx / BN, n = n0 + idx % BN;
-    if (m < P.M && n < P.N) {
-      const uint32_t img = P.plane.div(n);
-      out[static_cast<int64_t>(img) * P.out_img_stride + static_cast<int64_t>(m) * P.out_plane + (n - img * P.plane.d)] = 0.f;
-    }
+    if (m < P.M && n < P.N) out[static_cast<int64_t>(m) * P.out_plane + tap_out_col(P, n)] = 0.f;
   }
 }
 
@@ -1324,10 +1331,38 @@ int launch_bwd_filter_tap_major(const ConvGeo &g, const float *x, const float *d
 }
 
 // launches conv_tap_kernel; `w_relaid` is [M][K] in the tap-major order
+// One stride phase of a strided backward-data pass, seen as a stride-1 backward-data problem:
+// dx[a0 + s*i][b0 + s*j] = sum over (o, u, v) of w[o][c][a + s*u][b + s*v] * dy[o][i + pad_r - u][j + pad_c - v].
+struct TapPhase {
+  int a, b;          // first filter row / column of the phase
+  int nu, nv;        // filter taps of the phase along each axis
+  int a0, b0;        // first input row / column of the phase
+  int hp, wp;        // positions of the phase along each axis
+  int pad_r, pad_c;  // (a0 + ph - a) / s, (b0 + pw - b) / s
+};
+
+// sub-filter of a phase in the tap-major order of conv_tap_kernel:
+// out[c][((o/16)*T + t)*16 + o%16] = w[o][c][a + s*u][b + s*v],  t = u*nv + v, T = nu*nv
+__global__ __launch_bounds__(256) void filter_phase_tap_major_kernel(const float *__restrict__ w, float *__restrict__ out,
+                                                                     int O, int C, int kH, int kW, int a, int b, int s,
+                                                                     int nu, int nv) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  const int T = nu * nv, K = O * T;
+  if (idx >= C * K) return;
+  const int c = idx / K, kp = idx - c * K;
+  const int lo = kp & 15, q = kp >> 4;
+  const int t = q % T, o = (q / T) * 16 + lo;
+  const int u = t / nv, v = t - u * nv;
+  out[idx] = w[((o * C + c) * kH + (a + s * u)) * kW + (b + s * v)];
+}
+
 template <int BM, int BN, int WM, int WN, bool BWD_DATA>
-int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, float *out, hipStream_t st) {
+int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, float *out, hipStream_t st,
+                    const TapPhase *phase = nullptr) {
   TapConvParams P;
-  const int taps = g.kH * g.kW;
+  int taps = g.kH * g.kW;
+  P.out_s = 1;
+  P.out_a0 = P.out_b0 = 0;
   if (BWD_DATA) {   // out = dx [imgs][C][H][W], src = dy [imgs][O][oH][oW]
     P.M = g.C;
     P.N = g.imgs * g.H * g.W;
@@ -1355,13 +1390,28 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
     P.out_img_stride = static_cast<int64_t>(g.O) * g.oH * g.oW;
     P.src_bytes = static_cast<unsigned>(static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4);
   }
-  P.wf = w_relaid;
-  P.src = src;
-  P.wf_bytes = static_cast<unsigned>(static_cast<int64_t>(P.M) * P.K * 4);
   P.ph = g.ph;
   P.pw = g.pw;
   P.s = g.s;
   P.kW = g.kW;
+  P.out_w = BWD_DATA ? g.W : g.oW;
+  if (phase) {      // one stride phase of a backward-data pass: a stride-1 problem on a sub-grid of dx
+    taps = phase->nu * phase->nv;
+    P.N = g.imgs * phase->hp * phase->wp;
+    P.K = g.O * taps;
+    P.plane = FastDiv(phase->hp * phase->wp);
+    P.width = FastDiv(phase->wp);
+    P.ph = phase->pad_r;
+    P.pw = phase->pad_c;
+    P.s = 1;
+    P.kW = phase->nv;
+    P.out_s = g.s;
+    P.out_a0 = phase->a0;
+    P.out_b0 = phase->b0;
+  }
+  P.wf = w_relaid;
+  P.src = src;
+  P.wf_bytes = static_cast<unsigned>(static_cast<int64_t>(P.M) * P.K * 4);
   P.taps = taps;
   const int tn = (P.N + BN - 1) / BN, tm = (P.M + BM - 1) / BM;
   const int tiles = tm * tn;
@@ -1408,6 +1458,53 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
   if (pieces)
     hipLaunchKernelGGL((conv_tap_assemble_kernel<BM, BN, WM, WN>), dim3(cut_tiles * 4), dim3(kThreads), 0, st, P, out,
                        pieces, sk);
+  return 0;
+}
+
+// Strided backward-data on conv_tap_kernel: one launch per stride phase (O % 16 == 0).
+template <int BM, int BN, int WM, int WN>
+int launch_bwd_data_phases_tap(const ConvGeo &g, const float *w, const float *dy, float *dx, float *wscratch,
+                               hipStream_t st) {
+  const int s = g.s;
+  TS_REQUIRE(s * s <= 64, "conv bwd-data: stride %d not supported", s);
+  TapPhase ph[64];
+  int count = 0;
+  bool any_empty = false;
+  for (int a = 0; a < s; ++a)
+    for (int b = 0; b < s; ++b) {
+      TapPhase t;
+      t.a = a;
+      t.b = b;
+      t.a0 = ((a - g.ph) % s + s) % s;
+      t.b0 = ((b - g.pw) % s + s) % s;
+      t.hp = t.a0 < g.H ? (g.H - t.a0 + s - 1) / s : 0;
+      t.wp = t.b0 < g.W ? (g.W - t.b0 + s - 1) / s : 0;
+      t.nu = a < g.kH ? (g.kH - a + s - 1) / s : 0;
+      t.nv = b < g.kW ? (g.kW - b + s - 1) / s : 0;
+      t.pad_r = (t.a0 + g.ph - a) / s;
+      t.pad_c = (t.b0 + g.pw - b) / s;
+      if (t.hp <= 0 || t.wp <= 0) continue;
+      if (t.nu == 0 || t.nv == 0) {
+        any_empty = true;        // positions no filter tap reaches: their gradient is zero
+        continue;
+      }
+      ph[count++] = t;
+    }
+  if (any_empty) {
+    const int64_t n = static_cast<int64_t>(g.imgs) * g.C * g.H * g.W;
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, dx, n);
+  }
+  int64_t woff = 0;
+  for (int i = 0; i < count; ++i) {
+    const TapPhase &t = ph[i];
+    const int K = g.O * t.nu * t.nv;
+    float *wp = wscratch + woff;          // every phase uses its own part of the re-laid filter
+    woff += static_cast<int64_t>(g.C) * K;
+    hipLaunchKernelGGL(filter_phase_tap_major_kernel, dim3((g.C * K + 255) / 256), dim3(256), 0, st, w, wp, g.O, g.C,
+                       g.kH, g.kW, t.a, t.b, s, t.nu, t.nv);
+    const int rc = launch_conv_tap<BM, BN, WM, WN, true>(g, dy, wp, dx, st, &t);
+    if (rc) return rc;
+  }
   return 0;
 }
 
@@ -1752,8 +1849,13 @@ int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray 
     } else {
       if (g.s > 1) {
         // the sub-filters of all phases together hold every filter element once
-        const int rc = g.C <= 64 ? launch_bwd_data_phases<64, 256, 1, 4>(g, cf(w), cf(dy), mf(dx), wt, st)
-                                 : launch_bwd_data_phases<128, 128, 2, 2>(g, cf(w), cf(dy), mf(dx), wt, st);
+        int rc;
+        if (g.O % BK == 0 && tap_kernel_ok(g, numel(dy), numel(w)))
+          rc = g.C <= 64 ? launch_bwd_data_phases_tap<64, 256, 1, 4>(g, cf(w), cf(dy), mf(dx), wt, st)
+                         : launch_bwd_data_phases_tap<128, 128, 2, 2>(g, cf(w), cf(dy), mf(dx), wt, st);
+        else
+          rc = g.C <= 64 ? launch_bwd_data_phases<64, 256, 1, 4>(g, cf(w), cf(dy), mf(dx), wt, st)
+                         : launch_bwd_data_phases<128, 128, 2, 2>(g, cf(w), cf(dy), mf(dx), wt, st);
         if (rc) return rc;
       } else {
         // taps index dy: off = o*oH*oW (the spatial part is recomputed because of the stride test)
