@@ -101,7 +101,9 @@ def test_optimizers(ts, n, rng):
     assert_close(v.asnumpy(), rv, TOL, "adam v")
 
 
-@pytest.mark.parametrize("rows,cols", [(128, 10), (64, 1000), (3, 1), (5, 4097), (300, 257)])
+# rows of at least 2048 columns in multiples of 4 take the block-per-row cross-entropy kernels
+@pytest.mark.parametrize("rows,cols", [(128, 10), (64, 1000), (3, 1), (5, 4097), (300, 257), (9, 4096), (7, 32000),
+                                       (5, 2050), (600, 2048)])
 def test_softmax_and_cross_entropy(ts, rows, cols, rng):
     y = (rng.normal(size=(rows, cols)) * 3).astype(np.float32)
     lab = np.eye(cols, dtype=np.float32)[rng.randint(0, cols, rows)]
@@ -121,12 +123,34 @@ def test_softmax_and_cross_entropy(ts, rows, cols, rng):
     assert_close(loss.asnumpy(), O.softmax_ce(y, sm), TOL, "ce smoothed")
 
 
-def test_cross_entropy_uniform_logits_is_log_c(ts):
-    y = np.full((8, 1000), -4.5, np.float32)
-    lab = np.eye(1000, dtype=np.float32)[np.arange(8)]
+@pytest.mark.parametrize("cols", [1000, 4096])
+def test_cross_entropy_uniform_logits_is_log_c(ts, cols):
+    y = np.full((8, cols), -4.5, np.float32)
+    lab = np.eye(cols, dtype=np.float32)[np.arange(8)]
     loss = ts.empty((1,))
     ts.links.softmax_cross_entropy(ts.arr(y), ts.arr(lab), loss, ts.stream)
-    assert abs(loss.asnumpy()[0] - np.log(1000)) < 1e-4 * np.log(1000)
+    assert abs(loss.asnumpy()[0] - np.log(cols)) < 1e-4 * np.log(cols)
+
+
+def test_cross_entropy_wide_rows_extreme_logits(ts, rng):
+    """One dominant logit per row (the others underflow), in a 3-D tensor as the Transformer loss
+    passes it: loss -> 0 where the label sits on it, gradient rows sum to zero."""
+    y = (rng.normal(size=(2, 3, 4096)) * 2).astype(np.float32)
+    hot = rng.randint(0, 4096, size=(2, 3))
+    for a in range(2):
+        for b in range(3):
+            y[a, b, hot[a, b]] = 200.0
+    lab = np.zeros_like(y)
+    for a in range(2):
+        for b in range(3):
+            lab[a, b, hot[a, b]] = 1.0
+    loss, out = ts.empty((1,)), ts.empty(y.shape)
+    ts.links.softmax_cross_entropy(ts.arr(y), ts.arr(lab), loss, ts.stream)
+    assert abs(float(loss.asnumpy()[0])) < 1e-3
+    g = ts.arr(np.array([1.0], np.float32))
+    ts.links.softmax_cross_entropy_gradient(ts.arr(y), ts.arr(lab), g, out, ts.stream)
+    got = out.asnumpy()
+    assert np.all(np.isfinite(got)) and np.abs(got.sum(axis=-1)).max() < 1e-5
 
 
 BN_SHAPES = [(4, 3, 5, 6), (2, 5, 7, 7), (16, 64, 56, 56), (8, 512, 14, 14), (3, 2, 1, 1), (64, 16, 32, 32)]

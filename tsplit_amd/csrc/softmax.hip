@@ -4,6 +4,9 @@
 // block barrier; a 256-thread block handles 4 rows.  The cross-entropy mean is a second,
 // single-block deterministic reduction over the per-row losses (the reference does that
 // mean serially in thread 0 of its only block: src/ops/SoftmaxCrossEntropy.cu:33-41).
+// Long rows (a 32 000-word vocabulary) get a whole block per row instead: 16-byte loads,
+// running (max, scaled sum) pairs so that the logits are read from memory once, and for the
+// loss the label sums of the same pass: loss_r = (log s + m) * sum(l) - sum(l * y).
 #include "common.h"
 #include "reduce.h"
 
@@ -76,6 +79,106 @@ __global__ __launch_bounds__(256) void ce_grad_kernel(const float *__restrict__ 
   for (int j = lane; j < ncol; j += kWave) o[j] = (expf(row[j] - m) * inv - l[j]) * scale;
 }
 
+// ---- one 256-thread block per row ---------------------------------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kWideMinCols = 2048;
+
+struct MaxSum {
+  float m, s;     // s = sum of exp(x - m) over the elements seen so far
+};
+
+__device__ __forceinline__ void ms_add(MaxSum &a, float x) {
+  if (x > a.m) {
+    a.s = a.s * expf(a.m - x) + 1.f;      // expf(-inf) = 0 covers the first element
+    a.m = x;
+  } else {
+    a.s += expf(x - a.m);
+  }
+}
+
+__device__ __forceinline__ MaxSum ms_merge(MaxSum a, MaxSum b) {
+  const float m = fmaxf(a.m, b.m);
+  if (m == -INFINITY) return MaxSum{m, 0.f};
+  return MaxSum{m, a.s * expf(a.m - m) + b.s * expf(b.m - m)};
+}
+
+__device__ __forceinline__ MaxSum ms_block(MaxSum v, float *smem /* 8 floats */) {
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) {
+    MaxSum o{__shfl_xor(v.m, d, kWave), __shfl_xor(v.s, d, kWave)};
+    v = ms_merge(v, o);
+  }
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  if (lane == 0) {
+    smem[2 * wave] = v.m;
+    smem[2 * wave + 1] = v.s;
+  }
+  __syncthreads();
+  MaxSum r{smem[0], smem[1]};
+#pragma unroll
+  for (int w = 1; w < 4; ++w) r = ms_merge(r, MaxSum{smem[2 * w], smem[2 * w + 1]});
+  __syncthreads();
+  return r;
+}
+
+__global__ __launch_bounds__(256) void ce_rows_wide_kernel(const float *__restrict__ y, const float *__restrict__ lab,
+                                                           float *__restrict__ row_loss, int ncol) {
+  __shared__ float sm[8];
+  __shared__ float sm2[8];
+  const int64_t r = blockIdx.x;
+  const f32x4 *row = reinterpret_cast<const f32x4 *>(y + r * ncol);
+  const f32x4 *l = reinterpret_cast<const f32x4 *>(lab + r * ncol);
+  MaxSum ms{-INFINITY, 0.f};
+  float sl = 0.f, sly = 0.f;
+  for (int j = threadIdx.x; j < ncol / 4; j += 256) {
+    const f32x4 v = row[j], w = __builtin_nontemporal_load(l + j);
+    ms_add(ms, v.x);
+    ms_add(ms, v.y);
+    ms_add(ms, v.z);
+    ms_add(ms, v.w);
+    sl += (w.x + w.y) + (w.z + w.w);
+    sly += (w.x * v.x + w.y * v.y) + (w.z * v.z + w.w * v.w);
+  }
+  ms = ms_block(ms, sm);
+  sl = block_sum<float, 4>(sl, sm2);
+  __syncthreads();
+  sly = block_sum<float, 4>(sly, sm2);
+  if (threadIdx.x == 0) row_loss[r] = (logf(ms.s) + ms.m) * sl - sly;
+}
+
+__global__ __launch_bounds__(256) void ce_grad_wide_kernel(const float *__restrict__ y, const float *__restrict__ lab,
+                                                           const float *__restrict__ g, float *__restrict__ out,
+                                                           int ncol, float inv_batch) {
+  __shared__ float sm[8];
+  const int64_t r = blockIdx.x;
+  const f32x4 *row = reinterpret_cast<const f32x4 *>(y + r * ncol);
+  const f32x4 *l = reinterpret_cast<const f32x4 *>(lab + r * ncol);
+  f32x4 *o = reinterpret_cast<f32x4 *>(out + r * ncol);
+  MaxSum ms{-INFINITY, 0.f};
+  for (int j = threadIdx.x; j < ncol / 4; j += 256) {
+    const f32x4 v = row[j];
+    ms_add(ms, v.x);
+    ms_add(ms, v.y);
+    ms_add(ms, v.z);
+    ms_add(ms, v.w);
+  }
+  ms = ms_block(ms, sm);
+  const float inv = 1.f / ms.s, scale = g[0] * inv_batch, m = ms.m;
+  for (int j = threadIdx.x; j < ncol / 4; j += 256) {     // second read of the row: from L2
+    const f32x4 v = row[j], w = __builtin_nontemporal_load(l + j);
+    f32x4 q;
+    q.x = (expf(v.x - m) * inv - w.x) * scale;
+    q.y = (expf(v.y - m) * inv - w.y) * scale;
+    q.z = (expf(v.z - m) * inv - w.z) * scale;
+    q.w = (expf(v.w - m) * inv - w.w) * scale;
+    __builtin_nontemporal_store(q, o + j);
+  }
+}
+
+inline bool wide_rows(int ncol, const void *a, const void *b, const void *c) {
+  return ncol >= kWideMinCols && ncol % 4 == 0 && aligned16(a) && aligned16(b) && (c == nullptr || aligned16(c));
+}
+
 inline bool rows_cols(const DLArray *a, int64_t &nrow, int &ncol) {
   if (a->ndim < 1) return false;
   nrow = 1;
@@ -119,8 +222,12 @@ int DLGpuSoftmaxCrossEntropy(const DLArrayHandle input_a, const DLArrayHandle in
   TS_REQUIRE(row_loss, "DLGpuSoftmaxCrossEntropy: no scratch memory");
   ProfileScope ps(p, s, 2 * numel(input_a), 1, nrow);
   const unsigned blocks = static_cast<unsigned>((nrow + kRowsPerBlock - 1) / kRowsPerBlock);
-  hipLaunchKernelGGL(ce_rows_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const float *>(input_a->data),
-                     static_cast<const float *>(input_b->data), row_loss, nrow, ncol);
+  if (wide_rows(ncol, input_a->data, input_b->data, nullptr) && nrow < (1ll << 31))
+    hipLaunchKernelGGL(ce_rows_wide_kernel, dim3(static_cast<unsigned>(nrow)), dim3(256), 0, s,
+                       static_cast<const float *>(input_a->data), static_cast<const float *>(input_b->data), row_loss, ncol);
+  else
+    hipLaunchKernelGGL(ce_rows_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const float *>(input_a->data),
+                       static_cast<const float *>(input_b->data), row_loss, nrow, ncol);
   hipLaunchKernelGGL(mean_kernel, dim3(1), dim3(256), 0, s, row_loss, static_cast<float *>(output->data), nrow);
   return ps.finish();
 }
@@ -139,9 +246,15 @@ int DLGpuSoftmaxCrossEntropy_Gradient(const DLArrayHandle input_a, const DLArray
   ProfileScope ps(p, s, 2 * numel(input_a) + 1, numel(output), 0);
   const unsigned blocks = static_cast<unsigned>((nrow + kRowsPerBlock - 1) / kRowsPerBlock);
   // scaled by 1/shape[0] (not 1/rows), as src/ops/SoftmaxCrossEntropy.cu:101,120 does
-  hipLaunchKernelGGL(ce_grad_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const float *>(input_a->data),
-                     static_cast<const float *>(input_b->data), static_cast<const float *>(input_c->data),
-                     static_cast<float *>(output->data), nrow, ncol, 1.f / static_cast<float>(input_a->shape[0]));
+  const float inv_batch = 1.f / static_cast<float>(input_a->shape[0]);
+  if (wide_rows(ncol, input_a->data, input_b->data, output->data) && nrow < (1ll << 31))
+    hipLaunchKernelGGL(ce_grad_wide_kernel, dim3(static_cast<unsigned>(nrow)), dim3(256), 0, s,
+                       static_cast<const float *>(input_a->data), static_cast<const float *>(input_b->data),
+                       static_cast<const float *>(input_c->data), static_cast<float *>(output->data), ncol, inv_batch);
+  else
+    hipLaunchKernelGGL(ce_grad_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const float *>(input_a->data),
+                       static_cast<const float *>(input_b->data), static_cast<const float *>(input_c->data),
+                       static_cast<float *>(output->data), nrow, ncol, inv_batch);
   return ps.finish();
 }
 
