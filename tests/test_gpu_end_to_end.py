@@ -14,7 +14,7 @@ def _onehot(idx, n):
 
 
 def test_mlp_20_steps_tracks_oracle():
-    """BASELINE config 1: 784-256-256-10 without bias, batch 128, 20 SGD steps, lr 0.1,
+    """The reference's CPU-runnable MLP: 784-256-256-10 without bias, batch 128, 20 SGD steps, lr 0.1,
     X ~ U[0,1), labels uniform, weights ~ N(0, 0.1)."""
     from tsplit_amd import ndarray, trainer
     rng = np.random.RandomState(123)

@@ -1,4 +1,4 @@
-"""Whole-graph parity for the branched example networks (BASELINE configs 3-5 at reduced
+"""Whole-graph parity for the branched example networks (ResNet-50, Inception-v4, Transformer at reduced
 size): the same builder code (tsplit_amd/workloads.py) runs on a tape over the C ABI and on a
 tape over the numpy oracle; loss, logits and every parameter gradient are compared, then a few
 SGD steps.  Tolerances: loss 1e-3 relative; logits and gradients 2e-3 of their largest entry
