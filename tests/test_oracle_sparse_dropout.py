@@ -13,12 +13,16 @@ import scipy.sparse
 from oracle import loops as LP
 from oracle import ops as O
 
-PHILOX_KAT = [
-    ((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
-    ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
-    ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
-     (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)),
-]
+def _load_kat():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "philox4x32_10_kat.json")) as f:
+        doc = json.load(f)
+    h = lambda words: tuple(int(w, 16) for w in words)
+    return [(h(v["counter"]), h(v["key"]), h(v["output"])) for v in doc["vectors"]]
+
+
+PHILOX_KAT = _load_kat()
 
 
 @pytest.mark.parametrize("ctr,key,expect", PHILOX_KAT)
