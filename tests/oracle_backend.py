@@ -69,6 +69,21 @@ class OracleBackend(object):
     def add_const(self, a, c, shape):
         return _s(O.add_const(a, c))
 
+    def mul(self, a, b, shape):
+        return _s(O.mul(a, b))
+
+    def sigmoid(self, x, shape):
+        return _s(O.sigmoid(x))
+
+    def tanh(self, x, shape):
+        return _s(O.tanh(x))
+
+    def slice(self, x, begin, out_shape):
+        return _s(O.slice_(x, begin, out_shape))
+
+    def slice_grad(self, dy, begin, in_shape):
+        return _s(O.slice_grad(dy, begin, in_shape))
+
     def broadcast_shape(self, x, out_shape):
         return _s(O.broadcast_shape(x, out_shape))
 

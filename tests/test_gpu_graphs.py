@@ -1,5 +1,5 @@
-"""Whole-graph parity for the branched example networks (ResNet-50, Inception-v4, Transformer at reduced
-size): the same builder code (tsplit_amd/workloads.py) runs on a tape over the C ABI and on a
+"""Whole-graph parity for the example networks (ResNet-50, Inception-v4, Transformer at reduced
+size, the LSTM at its own size): the same builder code (tsplit_amd/workloads.py) runs on a tape over the C ABI and on a
 tape over the numpy oracle; loss, logits and every parameter gradient are compared, then a few
 SGD steps.  Tolerances: loss 1e-3 relative; logits and gradients 2e-3 of their largest entry
 (the conv / matmul bar; these graphs chain tens of them)."""
@@ -87,3 +87,17 @@ def test_transformer_graph(rng):
     def build(t, b):
         return workloads.transformer(t, b, cfg, b.input(xs), b.input(ys_in), b.input(ys_out))
     _both(build, seed=7, steps=3, lr=0.01)
+
+
+def test_lstm_graph(rng):
+    """The LSTM classifier at the example's own size (28 frames of 28 values, 128 hidden units,
+    10 classes): slice, matmul, broadcast bias, sigmoid, tanh and elementwise products chained over
+    28 time steps, with the gradients the reference composes from elementwise operators."""
+    from tsplit_amd import workloads
+    x = rng.uniform(0, 1, size=(16, 28 * 28)).astype(np.float32)
+    y = _onehot(rng, 16, 10)
+
+    def build(t, b):
+        return workloads.lstm(t, b, b.input(x), b.input(y))
+    losses = _both(build, seed=9, steps=3, lr=0.5)
+    assert losses["gpu"][-1] < losses["gpu"][0]

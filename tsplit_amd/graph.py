@@ -141,6 +141,31 @@ class GpuBackend(object):
         L.matrix_elementwise_add_by_const(a, c, out, self.stream)
         return out
 
+    def mul(self, a, b, shape):
+        out = self.empty(shape)
+        L.matrix_elementwise_multiply(a, b, out, self.stream)
+        return out
+
+    def sigmoid(self, x, shape):
+        out = self.empty(shape)
+        L.sigmoid(x, out, self.stream)
+        return out
+
+    def tanh(self, x, shape):
+        out = self.empty(shape)
+        L.tanh(x, out, self.stream)
+        return out
+
+    def slice(self, x, begin, out_shape):
+        out = self.empty(out_shape)
+        L.matrix_slice(x, out, begin, self.stream)
+        return out
+
+    def slice_grad(self, dy, begin, in_shape):
+        out = self.empty(in_shape)
+        L.matrix_slice_gradient(dy, out, begin, self.stream)
+        return out
+
     def broadcast_shape(self, x, out_shape):
         out = self.empty(out_shape)
         L.broadcast_shape(x, out, None, self.stream)
@@ -307,6 +332,44 @@ class Tape(object):
     def shift(self, a, c):
         y = self.b.add_const(a.value, c, a.shape)
         return self._out(y, a.shape, [a], lambda g: self._acc(a, g))
+
+    def mul(self, a, b):
+        """gpu_ops/MultiplyElewise.py (compute; gradient: each input receives the other times the
+        output gradient)."""
+        assert a.shape == b.shape, (a.shape, b.shape)
+        y = self.b.mul(a.value, b.value, a.shape)
+
+        def back(g):
+            self._acc(a, self.b.mul(b.value, g, a.shape))
+            self._acc(b, self.b.mul(a.value, g, a.shape))
+        return self._out(y, a.shape, [a, b], back)
+
+    def sigmoid(self, x):
+        """gpu_ops/Sigmoid.py:58-61: gradient s * (1 + -1 * s) * g, built from the same elementwise
+        operators the reference's gradient graph uses."""
+        y = self.b.sigmoid(x.value, x.shape)
+
+        def back(g):
+            one_minus = self.b.add_const(self.b.mul_const(y, -1.0, x.shape), 1.0, x.shape)
+            self._acc(x, self.b.mul(self.b.mul(y, one_minus, x.shape), g, x.shape))
+        return self._out(y, x.shape, [x], back)
+
+    def tanh(self, x):
+        """gpu_ops/Tanh.py:59-61: gradient (1 + (-1 * t) * t) * g."""
+        y = self.b.tanh(x.value, x.shape)
+
+        def back(g):
+            d = self.b.add_const(self.b.mul(self.b.mul_const(y, -1.0, x.shape), y, x.shape), 1.0, x.shape)
+            self._acc(x, self.b.mul(d, g, x.shape))
+        return self._out(y, x.shape, [x], back)
+
+    def slice(self, x, begin, size):
+        """gpu_ops/Slice.py:47-81: tf.slice semantics, a size of -1 runs to the end; the gradient
+        writes the output gradient into zeros at `begin` (:126-141)."""
+        begin = tuple(int(v) for v in begin)
+        shape = tuple(int(x.shape[d] - begin[d] if n == -1 else n) for d, n in enumerate(size))
+        y = self.b.slice(x.value, begin, shape)
+        return self._out(y, shape, [x], lambda g: self._acc(x, self.b.slice_grad(g, begin, x.shape)))
 
     def reshape(self, a, shape):
         """gpu_ops/Reshape.py:42 (compute: a copy), :61 (gradient: reshaped back)."""

@@ -1,7 +1,7 @@
 """Times one training step (forward, backward, SGD) of the branched example networks at the
 sizes of the reference's benchmark configurations, on one MI355X through the C ABI.
 
-    python -m tsplit_amd.graphbench --net resnet50|inception_v4|transformer [--steps 5] [--warmup 2]
+    python -m tsplit_amd.graphbench --net resnet50|inception_v4|transformer|lstm [--steps 5] [--warmup 2]
 
 Prints one JSON object: samples/s, ms/step, final loss, operator calls per step.  Synthetic
 seeded inputs; parameters as in workloads.py.  (The headline benchmark of this repository is
@@ -16,7 +16,7 @@ import numpy as np
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--net", default="resnet50", choices=["resnet50", "inception_v4", "transformer"])
+    ap.add_argument("--net", default="resnet50", choices=["resnet50", "inception_v4", "transformer", "lstm"])
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--batch", type=int, default=0)
@@ -50,6 +50,16 @@ def main():
             return workloads.inception_v4(t, b, cache["x"], cache["y"])
         inputs = {"x": x, "y": y}
         desc = "Inception-v4, fp32 NCHW, batch %d, 3x299x299, 1000 classes" % n
+    elif a.net == "lstm":
+        n = a.batch or 512
+        x = rng.uniform(0, 1, size=(n, 28 * 28)).astype(np.float32)
+        y = np.zeros((n, 10), np.float32)
+        y[np.arange(n), rng.randint(0, 10, n)] = 1
+
+        def build(t, b, cache):
+            return workloads.lstm(t, b, cache["x"], cache["y"])
+        inputs = {"x": x, "y": y}
+        desc = "LSTM classifier, 28 frames x 28 values, 128 hidden units, 10 classes, batch %d" % n
     else:
         n = a.batch or 32
         # no softmax in this graph: masked scores are set to 0 and values are kept small so that twelve

@@ -314,3 +314,42 @@ def transformer(t, b, cfg, xs, ys_in, ys_out):
     onehot = t.one_hot(t.reshape(ys_out, (-1,)), cfg.vocab)
     labels = t.shift(t.scale(onehot, 1.0 - cfg.smoothing), cfg.smoothing / cfg.vocab)   # :184-186
     return t.softmax_ce(logits, labels), logits
+
+
+# ------------------------------------------------------------------ LSTM
+def lstm(t, b, x, labels, dim_input=28, dim_hidden=128, classes=10, steps=28, std=0.1):
+    """The reference's LSTM classifier (examples/LSTM.py:21-90): every row of x holds `steps`
+    frames of `dim_input` values, cut out with slice; one LSTM cell with separate forget / input
+    / output / candidate weights (W on the frame, U on the hidden state, bias broadcast); the
+    last hidden state feeds a linear layer and softmax cross-entropy.  All variables ~ N(0, std)
+    as the example draws them (LSTM.py:14-15).  Returns (loss, logits)."""
+    gates = {}
+    for g in ("forget_gate", "input_gate", "output_gate", "tanh"):
+        gates[g] = (b.get("lstm_%s_w" % g, (dim_input, dim_hidden), std), b.get("lstm_%s_u" % g, (dim_hidden, dim_hidden), std),
+                    b.get("lstm_%s_b" % g, (dim_hidden,), std))
+    out_w = b.get("lstm_out_weight", (dim_hidden, classes), std)
+    out_b = b.get("lstm_out_bias", (classes,), std)
+    initial = b.get("initial_state", (1,), std, trainable=False)
+    n = x.shape[0]
+
+    def gate(name, frame, h, act):
+        w, u, bias = gates[name]
+        z = t.add(t.matmul(h, u), t.matmul(frame, w))
+        z = t.add(z, t.broadcast_like(bias, z.shape))
+        return act(z)
+
+    c = h = None
+    for i in range(steps):
+        frame = t.slice(x, (0, i * dim_input), (-1, dim_input))
+        if i == 0:
+            c = t.broadcast_like(initial, (n, dim_hidden))
+            h = t.broadcast_like(initial, (n, dim_hidden))
+        f = gate("forget_gate", frame, h, t.sigmoid)
+        ig = gate("input_gate", frame, h, t.sigmoid)
+        o = gate("output_gate", frame, h, t.sigmoid)
+        cand = gate("tanh", frame, h, t.tanh)
+        c = t.add(t.mul(c, f), t.mul(ig, cand))
+        h = t.mul(t.tanh(c), o)
+    logits = t.matmul(h, out_w)
+    logits = t.add(logits, t.broadcast_like(out_b, logits.shape))
+    return t.softmax_ce(logits, labels), logits
