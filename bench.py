@@ -147,7 +147,7 @@ def main():
     spec, params, x, labels, split = vgg_workload(a.batch)
     if a.no_split:
         split = {}
-    timer = None if a.no_events else EventTimer(ctx)
+    timer = None if a.no_events else EventTimer(ctx, chained=True)
     t = trainer.Trainer(spec, params, x.shape, 1000, ctx, optimizer=("momentum", 1e-4, 0.9), split=split, timer=timer,
                         fuse_bn_relu=a.fused)
     gx, gy = ndarray.array(x, ctx), ndarray.array(labels, ctx)      # resident before timing
