@@ -153,7 +153,9 @@ def test_cross_entropy_wide_rows_extreme_logits(ts, rng):
     assert np.all(np.isfinite(got)) and np.abs(got.sum(axis=-1)).max() < 1e-5
 
 
-BN_SHAPES = [(4, 3, 5, 6), (2, 5, 7, 7), (16, 64, 56, 56), (8, 512, 14, 14), (3, 2, 1, 1), (64, 16, 32, 32)]
+# channels of at most 16384 values (N*H*W) take the one-pass kernels: 16, 32 or 64 values per thread
+BN_SHAPES = [(4, 3, 5, 6), (2, 5, 7, 7), (16, 64, 56, 56), (8, 512, 14, 14), (3, 2, 1, 1), (64, 16, 32, 32),
+             (64, 8, 14, 14), (32, 8, 17, 17), (20, 4, 20, 20), (64, 4, 16, 16), (64, 4, 16, 17), (17, 5, 16, 15)]
 
 
 @pytest.mark.parametrize("shape", BN_SHAPES)

@@ -15,6 +15,9 @@
 // E[x^2]-E[x]^2 and sum(dy*x)-mean*sum(dy) accurate.
 // Algorithmic traffic is 8 B/elem forward and 12 B/elem backward; these kernels move
 // 12 and 20 B/elem (x, and dy, are read by both passes).
+// Small channels (N*H*W <= 16384: 14x14 and smaller planes at batch 64, 17x17 at batch 32) take
+// one-pass kernels instead: one block per channel keeps the channel's values in registers, so
+// x (and dy) are read once - the algorithmic 8 and 12 B/elem - in one launch per direction.
 #include "common.h"
 #include "fastdiv.h"
 #include "reduce.h"
@@ -329,6 +332,147 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_dx_kernel(const float *__rest
   }
 }
 
+// ---- one block per channel, the channel in registers ------------------------------------
+constexpr int kOnePassMax = 64 * kThreads;      // elements per channel
+
+// element e of channel c: plane e / HW, offset e % HW
+__device__ __forceinline__ int64_t chan_addr(const FastDiv &hw, uint32_t e, int c, int C) {
+  const uint32_t n = hw.div(e);
+  return (static_cast<int64_t>(n) * C + c) * hw.d + (e - n * hw.d);
+}
+
+// R: values per thread (compile-time bound of the register arrays)
+template <int R, bool RELU>
+__global__ __launch_bounds__(kThreads) void bn_fwd_onepass_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                  const float *__restrict__ gamma,
+                                                                  const float *__restrict__ beta, FastDiv hw, int C,
+                                                                  uint32_t m, float eps, double inv_m,
+                                                                  float *__restrict__ save_mean,
+                                                                  float *__restrict__ save_istd) {
+  __shared__ double sm[kWaves];
+  __shared__ float coef[2];
+  const int c = blockIdx.x;
+  float v[R];
+  float s = 0.f;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t e = r * kThreads + threadIdx.x;
+    v[r] = e < m ? __builtin_nontemporal_load(x + chan_addr(hw, e, c, C)) : 0.f;
+    s += v[r];
+  }
+  const double mean = block_sum<double, kWaves>(static_cast<double>(s), sm) * inv_m;
+  // the values are at hand: the variance is the mean squared distance from the mean
+  const float mf32 = static_cast<float>(mean);
+  float q = 0.f;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t e = r * kThreads + threadIdx.x;
+    const float d = v[r] - mf32;
+    q += e < m ? d * d : 0.f;
+  }
+  double var = block_sum<double, kWaves>(static_cast<double>(q), sm) * inv_m;
+  // (x - float(mean)) leaves out mean - float(mean): var = E[(x - mf)^2] - (mean - mf)^2
+  const double dm = mean - static_cast<double>(mf32);
+  var -= dm * dm;
+  if (var < 0.0) var = 0.0;
+  if (threadIdx.x == 0) {
+    double istd = 1.0 / sqrt(var + static_cast<double>(eps));
+    double mean_used = mean;
+    if (RELU) {      // as in bn_apply_kernel: coefficients from the rounded statistics the backward pass will read
+      mean_used = static_cast<double>(static_cast<float>(mean));
+      istd = static_cast<double>(static_cast<float>(istd));
+    }
+    const double a = static_cast<double>(gamma[c]) * istd;
+    coef[0] = static_cast<float>(a);
+    coef[1] = static_cast<float>(static_cast<double>(beta[c]) - mean_used * a);
+    if (save_mean) save_mean[c] = static_cast<float>(mean);
+    if (save_istd) save_istd[c] = static_cast<float>(istd);
+  }
+  __syncthreads();
+  const float a = coef[0], b = coef[1];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t e = r * kThreads + threadIdx.x;
+    if (e < m) {
+      const float z = a * v[r] + b;
+      __builtin_nontemporal_store(RELU ? relu1(z) : z, y + chan_addr(hw, e, c, C));
+    }
+  }
+}
+
+template <int R, bool STATS, bool RELU>
+__global__ __launch_bounds__(kThreads) void bn_bwd_onepass_kernel(const float *__restrict__ dy, const float *__restrict__ x,
+                                                                  float *__restrict__ dx, const float *__restrict__ gamma,
+                                                                  const float *__restrict__ beta, FastDiv hw, int C,
+                                                                  uint32_t m, float eps, double inv_m,
+                                                                  const float *__restrict__ save_mean,
+                                                                  const float *__restrict__ save_istd,
+                                                                  float *__restrict__ dgamma, float *__restrict__ dbeta) {
+  __shared__ double sm[kWaves];
+  __shared__ float coef[3];
+  const int c = blockIdx.x;
+  float ga = 0.f, gb = 0.f;
+  if (RELU) {
+    const double a = static_cast<double>(gamma[c]) * static_cast<double>(save_istd[c]);
+    ga = static_cast<float>(a);
+    gb = static_cast<float>(static_cast<double>(beta[c]) - static_cast<double>(save_mean[c]) * a);
+  }
+  float xv[R], dv[R];
+  float sdy = 0.f, sdx = 0.f, sx = 0.f, sq = 0.f;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t e = r * kThreads + threadIdx.x;
+    const bool ok = e < m;
+    const int64_t at = ok ? chan_addr(hw, e, c, C) : 0;
+    xv[r] = ok ? __builtin_nontemporal_load(x + at) : 0.f;
+    dv[r] = ok ? __builtin_nontemporal_load(dy + at) : 0.f;
+    if (RELU) dv[r] = gated(dv[r], xv[r], ga, gb);
+    acc_dot(dv[r], xv[r], sdy, sdx);
+    if (STATS) acc2(xv[r], sx, sq);
+  }
+  const double r0 = block_sum<double, kWaves>(static_cast<double>(sdy), sm);
+  const double r1 = block_sum<double, kWaves>(static_cast<double>(sdx), sm);
+  double r2 = 0.0, r3 = 0.0;
+  if (STATS) {
+    r2 = block_sum<double, kWaves>(static_cast<double>(sx), sm);
+    r3 = block_sum<double, kWaves>(static_cast<double>(sq), sm);
+  }
+  if (threadIdx.x == 0) {
+    double mean, istd;
+    if (!STATS) {
+      mean = static_cast<double>(save_mean[c]);
+      istd = static_cast<double>(save_istd[c]);
+    } else {
+      mean = r2 * inv_m;
+      double var = r3 * inv_m - mean * mean;
+      if (var < 0.0) var = 0.0;
+      istd = 1.0 / sqrt(var + static_cast<double>(eps));
+    }
+    const double dbias = r0;
+    const double dscale = (r1 - mean * r0) * istd;
+    const double k1 = static_cast<double>(gamma[c]) * istd;
+    const double k2 = -k1 * istd * dscale * inv_m;
+    const double k3 = -k1 * dbias * inv_m - k2 * mean;
+    coef[0] = static_cast<float>(k1);
+    coef[1] = static_cast<float>(k2);
+    coef[2] = static_cast<float>(k3);
+    if (dgamma) dgamma[c] = static_cast<float>(dscale);
+    if (dbeta) dbeta[c] = static_cast<float>(dbias);
+  }
+  __syncthreads();
+  const float k1 = coef[0], k2 = coef[1], k3 = coef[2];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t e = r * kThreads + threadIdx.x;
+    if (e < m) __builtin_nontemporal_store(lin2(dv[r], xv[r], k1, k2, k3), dx + chan_addr(hw, e, c, C));
+  }
+}
+
+inline bool one_pass_ok(const DLArray *x) {
+  const int64_t m = x->shape[0] * x->shape[2] * x->shape[3];
+  return m > 0 && m <= kOnePassMax && numel(x) < (1ll << 31);
+}
+
 struct Plan {
   Geo g;
   int S;
@@ -383,6 +527,34 @@ static int bn_forward(const char *who, bool relu, const DLArrayHandle input_X, c
   TS_REQUIRE(!save_var_arr || numel(save_var_arr) == C, "%s: save_var must hold C elements", who);
   TS_REQUIRE(!relu || (save_mean_arr && save_var_arr), "%s: the fused form needs both save arrays", who);
   hipStream_t s = stream_of(stream_handle);
+  if (one_pass_ok(input_X)) {
+    const uint32_t hw = static_cast<uint32_t>(input_X->shape[2] * input_X->shape[3]);
+    const uint32_t m = static_cast<uint32_t>(input_X->shape[0]) * hw;
+    ProfileScope ps1(p, s, numel(input_X) + 2 * C, numel(output_Y), 0);
+    float *sm1 = save_mean_arr ? mf(save_mean_arr) : nullptr;
+    float *sv1 = save_var_arr ? mf(save_var_arr) : nullptr;
+    const int per = static_cast<int>((m + kThreads - 1) / kThreads);
+#define BN_FWD1(R, RL)                                                                                              \
+  hipLaunchKernelGGL((bn_fwd_onepass_kernel<R, RL>), dim3(static_cast<unsigned>(C)), dim3(kThreads), 0, s,         \
+                     cf(input_X), mf(output_Y), cf(bn_scale), cf(bn_bias), FastDiv(hw), static_cast<int>(C), m, eps, \
+                     1.0 / static_cast<double>(m), sm1, sv1)
+#define BN_FWD1_R(RL)   \
+  do {                  \
+    if (per <= 16)      \
+      BN_FWD1(16, RL);  \
+    else if (per <= 32) \
+      BN_FWD1(32, RL);  \
+    else                \
+      BN_FWD1(64, RL);  \
+  } while (0)
+    if (relu)
+      BN_FWD1_R(true);
+    else
+      BN_FWD1_R(false);
+#undef BN_FWD1_R
+#undef BN_FWD1
+    return ps1.finish();
+  }
   const bool al = aligned16(input_X->data) && aligned16(output_Y->data);
   Plan st, ap;
   TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 16384, st), "%s: unsupported shape", who);
@@ -448,6 +620,39 @@ static int bn_backward(const char *who, bool relu, const DLArrayHandle gradient_
   TS_REQUIRE(!relu || (saved && bn_bias && numel(bn_bias) == C),
              "%s: the fused form needs the bias and the statistics saved by the fused forward call", who);
   hipStream_t s = stream_of(stream_handle);
+  if (one_pass_ok(input_X)) {
+    const uint32_t hw = static_cast<uint32_t>(input_X->shape[2] * input_X->shape[3]);
+    const uint32_t m = static_cast<uint32_t>(input_X->shape[0]) * hw;
+    ProfileScope ps1(p, s, 2 * numel(input_X) + C, numel(gradient_X) + 2 * C, 0);
+    const float *sm1 = saved ? cf(save_mean_arr) : nullptr;
+    const float *sv1 = saved ? cf(save_var_arr) : nullptr;
+    const float *bias1 = bn_bias ? cf(bn_bias) : nullptr;
+    float *dg1 = gradient_bn_scale ? mf(gradient_bn_scale) : nullptr;
+    float *db1 = gradient_bn_bias ? mf(gradient_bn_bias) : nullptr;
+    const int per = static_cast<int>((m + kThreads - 1) / kThreads);
+#define BN_BWD1(R, ST, RL)                                                                                          \
+  hipLaunchKernelGGL((bn_bwd_onepass_kernel<R, ST, RL>), dim3(static_cast<unsigned>(C)), dim3(kThreads), 0, s,     \
+                     cf(gradient_Y), cf(input_X), mf(gradient_X), cf(bn_scale), bias1, FastDiv(hw),                 \
+                     static_cast<int>(C), m, eps, 1.0 / static_cast<double>(m), sm1, sv1, dg1, db1)
+#define BN_BWD1_R(ST, RL)   \
+  do {                      \
+    if (per <= 16)          \
+      BN_BWD1(16, ST, RL);  \
+    else if (per <= 32)     \
+      BN_BWD1(32, ST, RL);  \
+    else                    \
+      BN_BWD1(64, ST, RL);  \
+  } while (0)
+    if (relu)
+      BN_BWD1_R(false, true);
+    else if (saved)
+      BN_BWD1_R(false, false);
+    else
+      BN_BWD1_R(true, false);
+#undef BN_BWD1_R
+#undef BN_BWD1
+    return ps1.finish();
+  }
   const bool al = aligned16(input_X->data) && aligned16(gradient_Y->data) && aligned16(gradient_X->data);
   Plan rd, dxp;
   TS_REQUIRE(make_plan(input_X, al, 16 * kThreads, 16384, rd), "%s: unsupported shape", who);
