@@ -53,7 +53,7 @@ def vgg_workload(batch, seed=123):
     return spec, params, x, labels, split
 
 
-def cpu_baseline(sample_batch=8, seed=123):
+def cpu_baseline(sample_batch=16, seed=123):
     """The numpy oracle (float64, as the reference's numpy path computes) on `sample_batch`
     images of the same seeded workload: one forward+backward+momentum step."""
     from oracle import nets, ops
@@ -74,7 +74,7 @@ def cpu_baseline(sample_batch=8, seed=123):
                       "(%.1f s, loss %.4f)" % (sample_batch, dt, loss)}
 
 
-def cpu_baseline_onednn(sample_batch=8, seed=123):
+def cpu_baseline_onednn(sample_batch=16, seed=123):
     """The same step on the same seeded sample through oneDNN as bundled with PyTorch-CPU
     (conv / batch-norm / pooling / matmul primitives, fp32, all host cores): the closest
     available stand-in for the reference's dnnl CPU operator build (src/dnnl_ops), whose
@@ -91,7 +91,7 @@ def cpu_baseline_onednn(sample_batch=8, seed=123):
     vel = {k: torch.zeros_like(v) for k, v in P.items()}
     xt, yt = torch.tensor(x), torch.tensor(labels)
 
-    def step():
+    def step(update=True):
         h = xt
         for layer in spec:
             kind = layer[0]
@@ -112,11 +112,12 @@ def cpu_baseline_onednn(sample_batch=8, seed=123):
         loss.backward()
         with torch.no_grad():
             for k, p in P.items():
-                vel[k].mul_(0.9).sub_(p.grad, alpha=0.01)
-                p.add_(vel[k])
+                if update:
+                    vel[k].mul_(0.9).sub_(p.grad, alpha=0.01)
+                    p.add_(vel[k])
                 p.grad = None
         return float(loss.detach())
-    step()                       # warm-up: primitive creation, allocator
+    step(update=False)           # warm-up: primitive creation, allocator; parameters stay as seeded
     t0 = time.perf_counter()
     loss = step()
     dt = time.perf_counter() - t0
