@@ -19,7 +19,9 @@ divisibility and take one padding int, gpu_ops/Conv2d.py:36-37,
 gpu_ops/MaxPool.py:10-11): output sizes floor, and conv takes (pad_h, pad_w) as
 the GPU symbols do (src/ops/CudnnConv2d.cu:154-157).
 
-Parity status per function (what pins it, see tests/test_oracle_*.py):
+Parity status per function (what pins it, see tests/test_oracle*.py; conv, BN, the pools,
+softmax-CE and a whole backward sweep are also checked against PyTorch-CPU autograd in
+tests/test_oracle_vs_library.py):
   conv2d / conv2d_grad_data / conv2d_grad_filter  pinned: brute-force loops,
       scipy.signal.correlate2d, adjoint identities
   matmul                                           np.matmul is the reference
