@@ -241,9 +241,10 @@ class PlannedTrainer(object):
         for li in range(self.nl - 1, -1, -1):
             layer = self.spec[li]
             kind = layer[0]
-            # copy-in: this layer's input now if it is still away, the next `prefetch` ones ahead of time
-            for j in range(li, max(0, li - self.prefetch) - 1, -1):
-                if j >= 1:
+            # copy-ins the plan issues at this layer, the tensor needed first first; this layer's own
+            # input at the latest
+            for j in sorted(self.away, reverse=True):
+                if self.plan.issue_at.get(j, j) >= li or j >= li:
                     self._swap_in(j)
             a, y = self.acts[li], self.acts[li + 1]
             first = li == 0

@@ -18,7 +18,9 @@ schedule, which `simulate` replays byte for byte:
   forward  of layer i : allocate tensor i+1, run; then a swapped tensor i starts leaving
                         (it left the compute stream's hands) and is released once its copy is done
   backward of layer i : tensor i must be resident (a swapped one was re-allocated and its
-                        copy-in started while layer i+1 ran backward: one layer ahead);
+                        copy-in issued at the start of an earlier layer's backward: at least
+                        `prefetch` layers ahead, earlier where the budget has room, always in
+                        the order of need);
                         allocate the input gradient unless the layer writes it in place
                         (Relu, BatchNorm: elementwise in the gradient); run; release tensor
                         i+1 and the output gradient
@@ -76,10 +78,13 @@ IN_PLACE_BACKWARD = ("relu", "bn", "bnrelu")   # the input gradient may overwrit
 
 
 class MemoryPlan(object):
-    def __init__(self, swap, split, peak_bytes, est_step_ms, est_free_step_ms, fixed_bytes, budget_bytes, prefetch):
+    def __init__(self, swap, split, peak_bytes, est_step_ms, est_free_step_ms, fixed_bytes, budget_bytes, prefetch,
+                 issue_at=None):
         self.swap = frozenset(swap)          # tensor indices that leave the device after their forward use
         self.split = dict(split)             # layer index -> batch micro-tensors
-        self.prefetch = prefetch             # layers of lead a copy-in gets over the backward sweep
+        self.prefetch = prefetch             # least lead, in layers, of a copy-in over the backward sweep
+        # tensor -> backward layer at whose start its copy-in is issued
+        self.issue_at = dict(issue_at) if issue_at is not None else {j: j + prefetch for j in self.swap}
         self.peak_bytes = peak_bytes
         self.est_step_ms = est_step_ms             # cost-model step time with this plan ...
         self.est_free_step_ms = est_free_step_ms   # ... and with nothing swapped
@@ -88,7 +93,8 @@ class MemoryPlan(object):
 
     def describe(self):
         return {"swap": sorted(self.swap), "split": {int(k): int(v) for k, v in sorted(self.split.items())},
-                "prefetch": self.prefetch, "peak_GiB": self.peak_bytes / GiB, "est_step_ms": self.est_step_ms,
+                "prefetch": self.prefetch, "issue_at": {int(k): int(v) for k, v in sorted(self.issue_at.items())},
+                "peak_GiB": self.peak_bytes / GiB, "est_step_ms": self.est_step_ms,
                 "est_free_step_ms": self.est_free_step_ms,
                 "fixed_GiB": self.fixed_bytes / GiB,
                 "budget_GiB": None if self.budget_bytes is None else self.budget_bytes / GiB}
@@ -119,12 +125,18 @@ def tensor_bytes(shapes):
     return [4 * int(np.prod(s)) for s in shapes]
 
 
-def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3):
+def default_issue_at(swap, n_layers, prefetch):
+    """tensor -> backward layer at whose start its copy-in is issued: `prefetch` layers ahead."""
+    return {j: min(n_layers - 1, j + prefetch) for j in swap}
+
+
+def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3, issue_at=None):
     """Replays the executor's allocation schedule.  Returns (peak_bytes, events) where events is
     a list of (phase, layer, resident_bytes, resident_tensor_indices, busy_tensor_indices)."""
     L = len(spec)
     size = tensor_bytes(shapes)
     swap = set(swap)
+    issue_at = issue_at if issue_at is not None else default_issue_at(swap, L, prefetch)
     resident = set([0])
     grad_bytes = 0
     events = []
@@ -140,9 +152,9 @@ def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3):
             resident.discard(li)
     g_out = size[L]                    # the loss gradient has the logits' size
     for li in range(L - 1, -1, -1):
-        # the layer's own input must be there; copy-in of the next `prefetch` layers down starts now
-        for j in range(li, max(0, li - prefetch) - 1, -1):
-            if j >= 1 and j in swap:
+        # copy-ins issued at the start of this layer's backward (its own input at the latest)
+        for j in swap:
+            if 1 <= j <= li + 1 and (issue_at[j] >= li or j >= li):
                 resident.add(j)
         in_place = spec[li][0] in IN_PLACE_BACKWARD
         g_in = 0 if li == 0 else g_out if in_place else size[li]
@@ -155,7 +167,7 @@ def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3):
     return peak, events
 
 
-def step_ms(spec, shapes, swap, cost, prefetch=3):
+def step_ms(spec, shapes, swap, cost, prefetch=3, issue_at=None):
     """Estimated step time under the replayed schedule: one compute stream, one copy-out and one
     copy-in stream (each link direction carries one copy at a time, in issue order).  A swapped
     tensor starts leaving when its consumer starts and the sweep waits for it when that consumer
@@ -171,10 +183,11 @@ def step_ms(spec, shapes, swap, cost, prefetch=3):
         if li in swap:
             out_free = max(out_free, t0) + cost.copy_ms(size[li])
             t = max(t, out_free)
+    issue_at = issue_at if issue_at is not None else default_issue_at(swap, L, prefetch)
     in_free, arrival = 0.0, {}
     for li in range(L - 1, -1, -1):
-        for j in range(li, max(0, li - prefetch) - 1, -1):
-            if j >= 1 and j in swap and j not in arrival:
+        for j in sorted(swap, reverse=True):          # the tensor needed first is issued first
+            if j >= 1 and j not in arrival and (issue_at[j] >= li or j >= li):
                 in_free = max(in_free, t) + cost.copy_ms(size[j])
                 arrival[j] = in_free
         t = max(t, arrival.get(li, 0.0)) + cost.layer_ms(spec[li], shapes[li], shapes[li + 1], True, first=li == 0)
@@ -230,10 +243,27 @@ def plan_memory(spec, input_shape, budget_bytes=None, fixed_bytes=0, cost=None, 
         swap.discard(max(gains)[1])
         now_ms = step_ms(spec, shapes, swap, cost, prefetch)
         peak = simulate(spec, shapes, swap, fixed_bytes, prefetch)[0]
+    # copy-ins may start earlier than `prefetch` layers ahead where the budget has room for the
+    # tensor over the whole stretch; the order of issue stays the order of need
+    issue_at = default_issue_at(swap, L, prefetch)
+    if budget_bytes is not None and swap:
+        bound = L - 1
+        for j in sorted(swap, reverse=True):
+            best_at = issue_at[j]
+            for at in range(issue_at[j] + 1, bound + 1):
+                trial = dict(issue_at)
+                trial[j] = at
+                if simulate(spec, shapes, swap, fixed_bytes, prefetch, trial)[0] > budget_bytes:
+                    break
+                best_at = at
+            issue_at[j] = best_at
+            bound = best_at
+        now_ms = step_ms(spec, shapes, swap, cost, prefetch, issue_at)
+        peak = simulate(spec, shapes, swap, fixed_bytes, prefetch, issue_at)[0]
     split = {}
     for li, layer in enumerate(spec):
         if layer[0] == "conv" and li >= 1 and li in swap:
             k = int(min(batch, max(1, -(-size[li] // piece_bytes))))
             if k > 1:
                 split[li] = k
-    return MemoryPlan(swap, split, peak, now_ms, free_ms, fixed_bytes, budget_bytes, prefetch)
+    return MemoryPlan(swap, split, peak, now_ms, free_ms, fixed_bytes, budget_bytes, prefetch, issue_at)
