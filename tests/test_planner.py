@@ -86,3 +86,21 @@ def test_vgg16_batch64_numbers():
     assert p_plain.peak_bytes - p_fused.peak_bytes == conv_out    # the BatchNorm outputs never exist
     tight = planner.plan_memory(fused, (64, 3, 224, 224), 6 << 30, 1660 << 20)
     assert tight.peak_bytes <= 6 << 30 and tight.swap
+
+
+def test_copy_ins_start_early_where_the_budget_allows_and_keep_the_order_of_need():
+    spec = planner.fuse_spec(trainer.vgg16_spec(1000, 224))
+    shape = (64, 3, 224, 224)
+    p = planner.plan_memory(spec, shape, 7 << 30, 1660 << 20)
+    assert p.swap and set(p.issue_at) == set(p.swap)
+    order = sorted(p.swap, reverse=True)
+    for j in order:
+        assert p.issue_at[j] >= min(len(spec) - 1, j + p.prefetch)           # never later than the minimum lead
+    assert all(p.issue_at[a] >= p.issue_at[b] for a, b in zip(order, order[1:]))   # needed first, issued first
+    assert any(p.issue_at[j] > j + p.prefetch for j in order)                      # some did move
+    shapes = planner.layer_shapes(spec, shape)
+    peak, _ = planner.simulate(spec, shapes, p.swap, p.fixed_bytes, p.prefetch, p.issue_at)
+    assert peak == p.peak_bytes <= 7 << 30
+    cost = planner.CostModel()
+    assert planner.step_ms(spec, shapes, p.swap, cost, p.prefetch, p.issue_at) <= \
+        planner.step_ms(spec, shapes, p.swap, cost, p.prefetch)
