@@ -295,28 +295,21 @@ constexpr int kBufFlags = 0x00020000;           // raw buffer, 32-bit untyped da
 constexpr unsigned kOobOffset = 0x80000000u;    // beyond any tensor this path accepts (< 2 GiB)
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-// Work distribution ("stream-K"): the unit of work is one 16-wide k-step of one tile, numbered
-// tile-major.  Every block takes a contiguous range of `iters_per_block` units and the grid is
-// one full wave of resident blocks, so that 3.06 tiles per slot cost 3.06 tile-times, not 4,
-// and 392 tiles on 768 slots keep every slot busy.  A tile computed by one block is stored
-// directly.  Cut tiles are completed in one of two ways, both independent of scheduling:
-//   - ranges at least one tile long (more tiles than slots): a tile has at most two
-//     contributors, which add with float atomics into an output that a small kernel zeroed
-//     before; 0 + a + b does not depend on the order;
-//   - shorter ranges (fewer tiles than slots): every block parks the accumulators of its (at
-//     most two) partial pieces in scratch -- slot 0 for a piece that is the first segment of
-//     its range, slot 1 for a partial last segment -- and a second kernel adds the pieces of
-//     each tile in ascending block order and writes the tile.
-// Results do depend on where the cuts fall, i.e. on the problem shape.
-// The tiles of one M row (tile_m fixed) form a chain of tn * ksteps k-steps, cut into equal
-// ranges for the blocks of that row; block `logical` works on row logical % tm, range
-// logical / tm.  Blocks with consecutive ids therefore sit on the tm tiles that share one set
-// of gathered columns, at the same k-step at about the same time, in one XCD: the gathered
-// operand comes from HBM once and from that XCD's L2 for the other tm - 1 tiles.
-// A row's first whole_waves * ranges tiles are taken whole, one per block and wave of blocks:
-// all blocks of an XCD then walk k together and share each step's filter words in its L2 as
-// well.  Only the rest of the chain (between one and two tiles per block, or everything when
-// there are fewer tiles than blocks) is cut into equal ranges.
+// Work distribution.  The tiles of one M row (tile_m fixed) form a chain; block `logical`
+// works on row logical % tm, so the tm blocks with consecutive ids sit on the tiles that share
+// one set of gathered columns, at the same k-step at about the same time, in one XCD (ids are
+// transposed so that an XCD owns consecutive ids): the gathered operand comes from HBM once
+// and from that XCD's L2 for the other tm - 1 tiles.  The grid is one full wave of resident
+// blocks.  A row's tiles are first taken whole, one per block and wave of blocks - all blocks
+// of an XCD then walk k together and share each step's filter words in its L2 as well - and
+// the tiles left over (fewer than there are blocks; all of them in a layer with few tiles) are
+// cut "stream-K" fashion: the unit of work is one 16-wide k-step, every block takes an equal
+// contiguous range of the leftover chain, so 3.06 tiles per slot cost 3.06 tile-times, not 4,
+// and 392 tiles keep 512 slots busy.  A range is shorter than a tile; a block parks the
+// accumulators of its (at most two) partial pieces in scratch - slot 0 for a piece that is
+// the first segment of its range, slot 1 for a partial last segment - and a second kernel
+// adds the pieces of each cut tile in ascending block order and writes the tile.  Nothing
+// depends on scheduling; results do depend on where the cuts fall, i.e. on the problem shape.
 struct StreamK {
   int ksteps;            // k-steps per tile
   int total;             // k-steps of the cut part of one M row's chain
@@ -500,26 +493,8 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
           }
         }
       }
-    } else if (pieces == nullptr) {
-      // ranges are at least one tile long: a cut tile has exactly two contributors, which add into
-      // an output zeroed beforehand (0 + a + b does not depend on the order)
-#pragma unroll
-      for (int ni = 0; ni < 2; ++ni) {
-        const int n = n0 + wn0 + 32 * ni + (lane & 31);
-        if (n >= P.N) continue;
-        const int64_t coff = tap_out_col(P, n);
-#pragma unroll
-        for (int mi = 0; mi < 2; ++mi) {
-          const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int m = mb + 8 * (e >> 2) + (e & 3);
-            if (m < P.M) unsafeAtomicAdd(out + static_cast<int64_t>(m) * P.out_plane + coff, acc[mi][ni][e]);
-          }
-        }
-      }
     } else {
-      // a piece of a tile cut more than once: registers go to scratch as they are, [register][thread]
+      // a piece of a cut tile: registers go to scratch as they are, [register][thread]
       const int slot = (it - (ks1 - ks0)) == it_begin ? 0 : 1;
       float *pc = pieces + (static_cast<int64_t>(logical) * 2 + slot) * (BM * BN) + tid;
 #pragma unroll
@@ -567,21 +542,6 @@ __global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvPara
   for (int e = 0; e < 16; ++e) {
     const int m = mb + 8 * (e >> 2) + (e & 3);
     if (m < P.M) out[static_cast<int64_t>(m) * P.out_plane + coff] = acc[e];
-  }
-}
-
-// zeroes the output tiles that the stream-K ranges cut in two (block g looks at its range start)
-template <int BM, int BN>
-__global__ __launch_bounds__(kThreads) void conv_tap_zero_cut_tiles_kernel(TapConvParams P, float *__restrict__ out,
-                                                                           StreamK sk) {
-  const int range = blockIdx.x / sk.tm, tile_m = blockIdx.x - range * sk.tm;
-  const int start = (range + 1) * sk.iters_per_block;            // first k-step of the next range of this row
-  if (start >= sk.total || start % sk.ksteps == 0) return;       // falls on a tile boundary: nothing is cut
-  const int tile_n = sk.cut_first + start / sk.ksteps;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
-  for (int idx = threadIdx.x; idx < BM * BN; idx += kThreads) {
-    const int m = m0 + idx / BN, n = n0 + idx % BN;
-    if (m < P.M && n < P.N) out[static_cast<int64_t>(m) * P.out_plane + tap_out_col(P, n)] = 0.f;
   }
 }
 
@@ -1423,7 +1383,6 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
   const int slots = 256 * occ;
   unsigned grid;
   float *pieces = nullptr;
-  bool zero_cut = false;
   sk.whole_waves = 0;
   sk.cut_first = 0;
   int cut_tiles = tiles;         // tiles the assemble kernel looks at
@@ -1437,22 +1396,16 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
     sk.ranges = std::max(8, slots / tm / 8 * 8);
     grid = static_cast<unsigned>(sk.ranges) * tm;
     const int full = tn / sk.ranges;
-    sk.whole_waves = tn % sk.ranges == 0 ? full : std::max(0, full - 1);
+    sk.whole_waves = full;
     sk.cut_first = sk.whole_waves * sk.ranges;
     sk.total = (tn - sk.cut_first) * sk.ksteps;
     cut_tiles = (tn - sk.cut_first) * tm;
     sk.iters_per_block = std::max(1, (sk.total + sk.ranges - 1) / sk.ranges);
-    if (sk.total == 0) {
-      // whole waves cover every row exactly: nothing is cut
-    } else if (sk.iters_per_block >= sk.ksteps) {
-      zero_cut = true;           // at most two contributors per tile: atomics onto zeroed tiles
-    } else {
+    if (sk.total > 0) {          // (whole waves may cover every row exactly: then nothing is cut)
       pieces = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(grid) * 2 * BM * BN * sizeof(float)));
       TS_REQUIRE(pieces, "conv: no scratch memory for the pieces of cut tiles");
     }
   }
-  if (zero_cut)
-    hipLaunchKernelGGL((conv_tap_zero_cut_tiles_kernel<BM, BN>), dim3(grid), dim3(kThreads), 0, st, P, out, sk);
   hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>), dim3(grid), dim3(kThreads), 0, st, P, out, pieces,
                      sk);
   if (pieces)
