@@ -192,8 +192,19 @@ def main():
                            "frac": dd["rate"] / (PEAK_TFLOPS_FP32_MFMA if dd["unit"] == "flop" else PEAK_HBM_GBS),
                            "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom) if split and a.batch == 64 else None,
                            "per_launch": dd["work_per_call"], "ms_avg": dd["ms_avg"]}
+        # all conv FLOP over all conv time; the thin first layer (Cin*kH*kW = 27) is timed in bytes
+        # because HBM bounds it, so its FLOP (forward and filter gradient) are added here
         conv = [d for tag, d in k.items() if tag.startswith("conv_")]
-        conv_flop, conv_ms = sum(d["work"] for d in conv), sum(d["ms_total"] for d in conv)
+        conv_flop = sum(d["work"] for d in conv if d["unit"] == "flop")
+        shape = x.shape
+        for layer in spec:
+            if layer[0] == "conv":
+                if layer[2] * layer[4] * layer[4] <= 32:
+                    conv_flop += a.steps * 2 * 2.0 * shape[0] * layer[3] * shape[2] * shape[3] * layer[2] * layer[4] ** 2
+                shape = (shape[0], layer[3], shape[2], shape[3])
+            elif layer[0] == "maxpool":
+                shape = (shape[0], shape[1], shape[2] // 2, shape[3] // 2)
+        conv_ms = sum(d["ms_total"] for d in conv)
         out["conv_mfma_util_pct"] = 100.0 * conv_flop / (conv_ms * 1e-3) / 1e12 / PEAK_TFLOPS_FP32_MFMA
         out["kernels"] = kernels
     if not a.no_cpu_baseline:

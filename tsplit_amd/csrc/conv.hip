@@ -1743,6 +1743,117 @@ inline bool wgrad_tap_ok(const ConvGeo &g) {
          bytes_x + 4 * (static_cast<int64_t>(g.ph) * g.W + g.pw) < (1ll << 31) && bytes_dy < (1ll << 31);
 }
 
+// ------------------------------------------------------------------ thin forward (first layer)
+// Forward pass with at most 32 reduction indices (Cin*kH*kW: a first layer on 3 channels).  Two
+// 16-wide k-steps cannot amortise a tile's gather set-up and the layer is bound by writing its
+// output, so it runs on the vector ALU: a wave takes 64 consecutive output positions and 16
+// output channels; the filter, re-laid [k][Cout], is wave-uniform and feeds the multiply-adds
+// from scalar registers; every output plane gets 256-byte stores.  Algorithmic bytes =
+// 4 * (x + w + y), almost all of it y.
+constexpr int kThinMaxK = 32;
+constexpr int kThinChans = 16;       // output channels per thread
+
+struct ThinParams {
+  int C, H, W, O, Opad, kH, kW, ph, pw, s, oH, oW, K;
+  FastDiv plane, width;              // oH*oW, oW
+  int64_t n_total;                   // imgs * oH * oW
+};
+
+__global__ __launch_bounds__(256) void filter_thin_kernel(const float *__restrict__ w, float *__restrict__ out, int O,
+                                                          int Opad, int K) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= K * Opad) return;
+  const int k = idx / Opad, o = idx - k * Opad;
+  out[idx] = o < O ? w[o * K + k] : 0.f;
+}
+
+// wt: the filter as [K][Opad], Opad = O rounded up to 16
+__global__ __launch_bounds__(256) void conv_thin_fwd_kernel(ThinParams P, const float *__restrict__ x,
+                                                            const float *__restrict__ wt, float *__restrict__ y) {
+  __shared__ int tab[kThinMaxK][4];     // per reduction index: kh, kw, offset inside one image of x
+  if (threadIdx.x < P.K) {
+    const int taps = P.kH * P.kW;
+    const int c = threadIdx.x / taps, t = threadIdx.x - c * taps;
+    const int kh = t / P.kW, kw = t - kh * P.kW;
+    tab[threadIdx.x][0] = kh;
+    tab[threadIdx.x][1] = kw;
+    tab[threadIdx.x][2] = (c * P.H + kh) * P.W + kw;
+    tab[threadIdx.x][3] = 0;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63;
+  const int og = __builtin_amdgcn_readfirstlane(blockIdx.y * 4 + (threadIdx.x >> 6));   // channel group of this wave
+  if (og * kThinChans >= P.O) return;
+  const int64_t n = static_cast<int64_t>(blockIdx.x) * 64 + lane;
+  const bool ok = n < P.n_total;
+  const uint32_t nn = ok ? static_cast<uint32_t>(n) : 0u;
+  const uint32_t img = P.plane.div(nn);
+  const uint32_t p = nn - img * P.plane.d;
+  const uint32_t oh = P.width.div(p), ow = p - oh * P.width.d;
+  const int ih0 = static_cast<int>(oh) * P.s - P.ph, iw0 = static_cast<int>(ow) * P.s - P.pw;
+  const float *xi = x + static_cast<int64_t>(img) * P.C * P.H * P.W + ih0 * P.W + iw0;
+  const float *wg = wt + og * kThinChans;
+  // all gathered values first (independent loads, all in flight), then the multiply-adds
+  float xv[kThinMaxK];
+#pragma unroll
+  for (int k = 0; k < kThinMaxK; ++k) {
+    xv[k] = 0.f;
+    if (k < P.K) {
+      const int kh = tab[k][0], kw = tab[k][1], off = tab[k][2];
+      const bool in = ok && static_cast<unsigned>(ih0 + kh) < static_cast<unsigned>(P.H) &&
+                      static_cast<unsigned>(iw0 + kw) < static_cast<unsigned>(P.W);
+      if (in) xv[k] = xi[off];
+    }
+  }
+  float acc[kThinChans];
+#pragma unroll
+  for (int o = 0; o < kThinChans; ++o) acc[o] = 0.f;
+#pragma unroll
+  for (int k = 0; k < kThinMaxK; ++k) {
+    if (k < P.K) {
+      const float *wk = wg + k * P.Opad;         // wave-uniform: scalar loads
+#pragma unroll
+      for (int o = 0; o < kThinChans; ++o) acc[o] += xv[k] * wk[o];
+    }
+  }
+  if (!ok) return;
+  float *yo = y + (static_cast<int64_t>(img) * P.O + og * kThinChans) * P.plane.d + p;
+#pragma unroll
+  for (int o = 0; o < kThinChans; ++o)
+    if (og * kThinChans + o < P.O) __builtin_nontemporal_store(acc[o], yo + static_cast<int64_t>(o) * P.plane.d);
+}
+
+inline bool thin_fwd_ok(const ConvGeo &g) {
+  return g.C * g.kH * g.kW <= kThinMaxK && static_cast<int64_t>(g.imgs) * g.oH * g.oW < (1ll << 31);
+}
+
+int launch_conv_thin_fwd(const ConvGeo &g, const float *x, const float *w, float *y, hipStream_t st) {
+  ThinParams P;
+  P.K = g.C * g.kH * g.kW;
+  P.Opad = (g.O + kThinChans - 1) / kThinChans * kThinChans;
+  float *wt = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(P.K) * P.Opad * 4));
+  TS_REQUIRE(wt, "conv: no scratch memory for the re-laid filter");
+  hipLaunchKernelGGL(filter_thin_kernel, dim3((P.K * P.Opad + 255) / 256), dim3(256), 0, st, w, wt, g.O, P.Opad, P.K);
+  P.C = g.C;
+  P.H = g.H;
+  P.W = g.W;
+  P.O = g.O;
+  P.kH = g.kH;
+  P.kW = g.kW;
+  P.ph = g.ph;
+  P.pw = g.pw;
+  P.s = g.s;
+  P.oH = g.oH;
+  P.oW = g.oW;
+  P.plane = FastDiv(g.oH * g.oW);
+  P.width = FastDiv(g.oW);
+  P.n_total = static_cast<int64_t>(g.imgs) * g.oH * g.oW;
+  const unsigned groups = static_cast<unsigned>(P.Opad / kThinChans);
+  hipLaunchKernelGGL(conv_thin_fwd_kernel, dim3(static_cast<unsigned>((P.n_total + 63) / 64), (groups + 3) / 4), dim3(256), 0,
+                     st, P, x, wt, y);
+  return 0;
+}
+
 int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y, int ph, int pw, int s,
                  DLStreamHandle sh, ProfilerHandle p) {
   ConvGeo g;
@@ -1750,7 +1861,10 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
   hipStream_t st = stream_of(sh);
   ProfileScope ps(p, st, numel(x) + numel(w), numel(y), 0);
   if (numel(y) > 0) {
-    if (g.C % BK == 0) {
+    if (thin_fwd_ok(g)) {
+      const int rc = launch_conv_thin_fwd(g, cf(x), cf(w), mf(y), st);
+      if (rc) return rc;
+    } else if (g.C % BK == 0) {
       float *wf = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(numel(w)) * 4));
       TS_REQUIRE(wf, "%s: no scratch memory", who);
       const int total = static_cast<int>(numel(w));

@@ -188,10 +188,16 @@ class Trainer(object):
             if kind == "conv":
                 _, name, cin, cout, k, pad, stride = layer
                 w = self.params[name + "_weight"]
-                tag = "conv_fwd_" + self._tile(cout)
+                thin = cin * k * k <= 32      # a first layer (3 input channels): bound by HBM, timed in bytes
+                tag = "conv_fwd_thin" if thin else "conv_fwd_" + self._tile(cout)
                 pairs = list(zip(a.sTensor, out.sTensor)) if li in self.split else [(a, out)]
                 for xa, ya in pairs:
-                    self._run(tag, 2.0 * n(ya.shape) * cin * k * k, "flop", L.CuDNN_conv2d, xa, w, ya, pad, pad, stride)
+                    if thin:
+                        self._run(tag, 4.0 * (n(xa.shape) + n(w.shape) + n(ya.shape)), "byte", L.CuDNN_conv2d, xa, w, ya,
+                                  pad, pad, stride)
+                    else:
+                        self._run(tag, 2.0 * n(ya.shape) * cin * k * k, "flop", L.CuDNN_conv2d, xa, w, ya, pad, pad,
+                                  stride)
             elif kind == "bn" and li in self.fused:
                 name = layer[1]
                 sm, sv = self.saved[li]
@@ -239,9 +245,14 @@ class Trainer(object):
                 gs = g_out.sTensor if split else [g_out]
                 for i, (xa, ga) in enumerate(zip(xs, gs)):
                     # filter gradient first, as the reference reorders it (executor.py:327-332)
-                    self._run("conv_bwd_filter_" + self._tile(cout), 2.0 * n(ga.shape) * cin * k * k, "flop",
-                              L.CuDNN_conv2d_gradient_of_filter, xa, ga, dw if i == 0 else self.dw_piece[li],
-                              pad, pad, stride)
+                    if cin * k * k <= 32:
+                        self._run("conv_bwd_filter_thin", 4.0 * (n(xa.shape) + n(ga.shape) + n(dw.shape)), "byte",
+                                  L.CuDNN_conv2d_gradient_of_filter, xa, ga, dw if i == 0 else self.dw_piece[li],
+                                  pad, pad, stride)
+                    else:
+                        self._run("conv_bwd_filter_" + self._tile(cout), 2.0 * n(ga.shape) * cin * k * k, "flop",
+                                  L.CuDNN_conv2d_gradient_of_filter, xa, ga, dw if i == 0 else self.dw_piece[li],
+                                  pad, pad, stride)
                     if i > 0:
                         self._run("add", 12.0 * n(dw.shape), "byte", L.matrix_elementwise_add, dw, self.dw_piece[li], dw)
                 if not first:
