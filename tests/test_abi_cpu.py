@@ -155,3 +155,43 @@ def test_pool_split_rule_and_growth_and_limit(pool_lib):
     assert pool_lib.pool_test_free(h, b) == 1
     assert pool_lib.pool_test_try(h, 100 * MiB) == 1                                                 # from the freed slab
     pool_lib.pool_test_destroy(h)
+
+
+def test_header_compiles_as_c_and_cxx_and_links(tmp_path):
+    """A C translation unit and a C++ one that include the public header, take the address of a few
+    entry points with their declared types, and link against the built library: the header is
+    self-contained plain C, and the declarations agree with the definitions' C linkage."""
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib_dir = os.path.join(root, "tsplit_amd", "lib")
+    if not os.path.exists(os.path.join(lib_dir, "libc_runtime_api.so")):
+        pytest.skip("library not built")
+    body = '''
+#include "c_runtime_api.h"
+#include <stddef.h>
+typedef int (*relu_fn)(const DLArrayHandle, DLArrayHandle, DLStreamHandle, ProfilerHandle);
+typedef int (*conv_fn)(const DLArrayHandle, const DLArrayHandle, DLArrayHandle, const int, const int, const int,
+                       DLStreamHandle, ProfilerHandle);
+int main(void) {
+  relu_fn r = DLGpuRelu;
+  conv_fn c = CuDNN_DLGpuConv2d;
+  DLArray a;
+  a.data = NULL;
+  a.ndim = 0;
+  a.shape = NULL;
+  return (r != NULL && c != NULL && a.data == NULL && a.ndim == 0 && a.shape == NULL && sizeof(DLArray) == 32 && sizeof(DLContext) == 8 && sizeof(Profiler) == 16) ? 0 : 1;
+}
+'''
+    for compiler, name, std in (("gcc", "t.c", "-std=c99"), ("g++", "t.cpp", "-std=c++11")):
+        if shutil.which(compiler) is None:
+            pytest.skip(compiler + " not found")
+        src = tmp_path / name
+        src.write_text(body)
+        exe = tmp_path / (name + ".out")
+        cmd = [compiler, std, "-Wall", "-Werror", "-I", os.path.join(root, "include"), str(src), "-o", str(exe),
+               "-L", lib_dir, "-lc_runtime_api", "-Wl,-rpath," + lib_dir, "-Wl,--allow-shlib-undefined"]
+        done = subprocess.run(cmd, capture_output=True, text=True)
+        assert done.returncode == 0, done.stderr
+        ran = subprocess.run([str(exe)], capture_output=True, text=True)
+        assert ran.returncode == 0, ran.stderr
