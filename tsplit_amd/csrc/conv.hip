@@ -1746,15 +1746,16 @@ inline bool wgrad_tap_ok(const ConvGeo &g) {
 // ------------------------------------------------------------------ thin forward (first layer)
 // Forward pass with at most 32 reduction indices (Cin*kH*kW: a first layer on 3 channels).  Two
 // 16-wide k-steps cannot amortise a tile's gather set-up and the layer is bound by writing its
-// output, so it runs on the vector ALU: a wave takes 64 consecutive output positions and 16
-// output channels; the filter, re-laid [k][Cout], is wave-uniform and feeds the multiply-adds
-// from scalar registers; every output plane gets 256-byte stores.  Algorithmic bytes =
+// output, so it runs on the vector ALU: a wave takes 64 consecutive output positions and 32
+// output channels (measured best of 16 / 32 / 64: more channels per thread repeat the gather of
+// the <= 32 inputs less often but leave fewer waves to hide its latency); the filter, re-laid
+// [k][Cout], is wave-uniform and feeds the multiply-adds from scalar registers; every output
+// plane gets 256-byte stores.  Algorithmic bytes =
 // 4 * (x + w + y), almost all of it y.
 constexpr int kThinMaxK = 32;
-constexpr int kThinChans = 16;       // output channels per thread
 
 struct ThinParams {
-  int C, H, W, O, Opad, kH, kW, ph, pw, s, oH, oW, K;
+  int C, H, W, O, Opad, kH, kW, ph, pw, s, oH, oW, K;   // Opad: O rounded up to the channels per thread
   FastDiv plane, width;              // oH*oW, oW
   int64_t n_total;                   // imgs * oH * oW
 };
@@ -1767,7 +1768,8 @@ __global__ __launch_bounds__(256) void filter_thin_kernel(const float *__restric
   out[idx] = o < O ? w[o * K + k] : 0.f;
 }
 
-// wt: the filter as [K][Opad], Opad = O rounded up to 16
+// wt: the filter as [K][Opad]; kThinChans: output channels per thread
+template <int kThinChans>
 __global__ __launch_bounds__(256) void conv_thin_fwd_kernel(ThinParams P, const float *__restrict__ x,
                                                             const float *__restrict__ wt, float *__restrict__ y) {
   __shared__ int tab[kThinMaxK][4];     // per reduction index: kh, kw, offset inside one image of x
@@ -1830,7 +1832,8 @@ inline bool thin_fwd_ok(const ConvGeo &g) {
 int launch_conv_thin_fwd(const ConvGeo &g, const float *x, const float *w, float *y, hipStream_t st) {
   ThinParams P;
   P.K = g.C * g.kH * g.kW;
-  P.Opad = (g.O + kThinChans - 1) / kThinChans * kThinChans;
+  const int chans = g.O > 16 ? 32 : 16;
+  P.Opad = (g.O + chans - 1) / chans * chans;
   float *wt = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(P.K) * P.Opad * 4));
   TS_REQUIRE(wt, "conv: no scratch memory for the re-laid filter");
   hipLaunchKernelGGL(filter_thin_kernel, dim3((P.K * P.Opad + 255) / 256), dim3(256), 0, st, w, wt, g.O, P.Opad, P.K);
@@ -1848,9 +1851,12 @@ int launch_conv_thin_fwd(const ConvGeo &g, const float *x, const float *w, float
   P.plane = FastDiv(g.oH * g.oW);
   P.width = FastDiv(g.oW);
   P.n_total = static_cast<int64_t>(g.imgs) * g.oH * g.oW;
-  const unsigned groups = static_cast<unsigned>(P.Opad / kThinChans);
-  hipLaunchKernelGGL(conv_thin_fwd_kernel, dim3(static_cast<unsigned>((P.n_total + 63) / 64), (groups + 3) / 4), dim3(256), 0,
-                     st, P, x, wt, y);
+  const unsigned groups = static_cast<unsigned>(P.Opad / chans);
+  const dim3 grid(static_cast<unsigned>((P.n_total + 63) / 64), (groups + 3) / 4);
+  if (chans == 32)
+    hipLaunchKernelGGL(conv_thin_fwd_kernel<32>, grid, dim3(256), 0, st, P, x, wt, y);
+  else
+    hipLaunchKernelGGL(conv_thin_fwd_kernel<16>, grid, dim3(256), 0, st, P, x, wt, y);
   return 0;
 }
 
