@@ -408,6 +408,28 @@ int TSplit_BatchNormRelu_gradient(const DLArrayHandle gradient_Y, const DLArrayH
                                   DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
                                   DLStreamHandle stream_handle, ProfilerHandle p);
 
+/* ---- Recorded steps.  NO counterpart in the reference (every step there is issued call by
+ *      call from Python); for steps made of thousands of tiny kernels (recurrent nets, small
+ *      MLPs) whose time is the host's launch rate.  Between TSplit_StreamBeginRecord and
+ *      TSplit_StreamEndRecord every call of this library on `stream` is recorded into a HIP graph
+ *      instead of being run; TSplit_GraphLaunch replays the recorded calls on a stream, with the
+ *      arrays and scalar arguments they had when recorded (a step whose scalars change - Adam's
+ *      bias-correction powers - cannot be replayed).  `stream` must be a created stream, not NULL.
+ *      Run the step once before recording it: first-use set-up (tap tables, scratch growth) is
+ *      refused while recording and the call that needs it returns -1, as TSplit_StreamEndRecord
+ *      then does.  Host-visible calls (DLStreamSync, a copy with a NULL stream, an operator with
+ *      a non-NULL profiler) are not allowed while recording.  The arrays a recorded step touches
+ *      must stay allocated for as long as the graph is launched. ---- */
+typedef struct {
+  int device_id;
+  void *handle;     /* an instantiated hipGraphExec_t */
+} DLGraph;
+typedef DLGraph *DLGraphHandle;
+int TSplit_StreamBeginRecord(DLStreamHandle stream);
+int TSplit_StreamEndRecord(DLStreamHandle stream, DLGraphHandle *graph);
+int TSplit_GraphLaunch(DLGraphHandle graph, DLStreamHandle stream);
+int TSplit_GraphDestroy(DLGraphHandle graph);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

@@ -198,6 +198,13 @@ void *scratch_get(hipStream_t stream, int slot, size_t bytes) {
   ScratchBuf &b = g_scratch[ScratchKey{stream, slot}];
   if (b.bytes >= bytes && b.p) return b.p;
   if (b.p) {
+    // a recorded step keeps the address it was recorded with: growing is set-up, not part of a step
+    hipStreamCaptureStatus recording = hipStreamCaptureStatusNone;
+    if (stream && hipStreamIsCapturing(stream, &recording) == hipSuccess && recording != hipStreamCaptureStatusNone) {
+      std::fprintf(stderr, "[libc_runtime_api] scratch memory would have to grow while a step is being recorded; "
+                           "run the step once before recording it\n");
+      return nullptr;
+    }
     // the old buffer may still be read by a kernel in flight on this stream
     (void)hipStreamSynchronize(stream);
     (void)hipFree(b.p);
@@ -312,6 +319,52 @@ int DLEventQuery(DLEventHandle handle) {
   hipError_t e = hipEventQuery(*static_cast<hipEvent_t *>(handle->handle));
   if (e == hipSuccess) return 1;
   (void)hipGetLastError();   // hipErrorNotReady is sticky in the last-error slot otherwise
+  return 0;
+}
+
+// ------------------------------------------------------------ recorded steps (HIP graphs)
+int TSplit_StreamBeginRecord(DLStreamHandle stream) {
+  TS_REQUIRE(stream != nullptr && stream->handle != nullptr, "TSplit_StreamBeginRecord: a created stream is required");
+  // relaxed mode: device allocations made by this thread while recording (a new pool slab) are allowed
+  TS_HIP(hipStreamBeginCapture(stream_of(stream), hipStreamCaptureModeRelaxed));
+  return 0;
+}
+
+int TSplit_StreamEndRecord(DLStreamHandle stream, DLGraphHandle *out) {
+  TS_REQUIRE(stream != nullptr && stream->handle != nullptr && out != nullptr, "TSplit_StreamEndRecord: NULL argument");
+  *out = nullptr;
+  hipGraph_t graph = nullptr;
+  hipError_t e = hipStreamEndCapture(stream_of(stream), &graph);
+  if (e != hipSuccess || graph == nullptr) {
+    (void)hipGetLastError();
+    if (graph) (void)hipGraphDestroy(graph);
+    TS_FAIL("TSplit_StreamEndRecord: the recording was invalidated (%s)", hipGetErrorString(e));
+  }
+  hipGraphExec_t exec = nullptr;
+  e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    TS_FAIL("TSplit_StreamEndRecord: hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  }
+  DLGraph *g = new DLGraph();
+  g->device_id = stream->device_id;
+  g->handle = exec;
+  *out = g;
+  return 0;
+}
+
+int TSplit_GraphLaunch(DLGraphHandle graph, DLStreamHandle stream) {
+  TS_REQUIRE(graph != nullptr && graph->handle != nullptr, "TSplit_GraphLaunch: NULL graph");
+  TS_REQUIRE(stream != nullptr && stream->handle != nullptr, "TSplit_GraphLaunch: a created stream is required");
+  TS_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph->handle), stream_of(stream)));
+  return 0;
+}
+
+int TSplit_GraphDestroy(DLGraphHandle graph) {
+  if (!graph) return 0;
+  if (graph->handle) TS_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph->handle)));
+  delete graph;
   return 0;
 }
 

@@ -1,7 +1,10 @@
 """Times one training step (forward, backward, SGD) of the branched example networks at the
 sizes of the reference's benchmark configurations, on one MI355X through the C ABI.
 
-    python -m tsplit_amd.graphbench --net resnet50|inception_v4|transformer|lstm [--steps 5] [--warmup 2]
+    python -m tsplit_amd.graphbench --net resnet50|inception_v4|transformer|lstm|mlp [--steps 5] [--warmup 2] [--record]
+
+--record issues the step once into a HIP graph after the warm-up and times replays of that graph
+(one host call per step) instead of Python issuing every operator again.
 
 Prints one JSON object: samples/s, ms/step, final loss, operator calls per step.  Synthetic
 seeded inputs; parameters as in workloads.py.  (The headline benchmark of this repository is
@@ -16,14 +19,17 @@ import numpy as np
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--net", default="resnet50", choices=["resnet50", "inception_v4", "transformer", "lstm"])
+    ap.add_argument("--net", default="resnet50", choices=["resnet50", "inception_v4", "transformer", "lstm", "mlp"])
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--lr", type=float, default=1e-4)
+    ap.add_argument("--record", action="store_true", help="record the step into a graph and time its replays")
     a = ap.parse_args()
     from . import graph, ndarray, stream, workloads
     ctx = ndarray.gpu(0)
+    if a.net == "mlp":
+        return mlp(a, ctx)
     st = stream.create_stream_handle(ctx)
     backend = graph.GpuBackend(ctx, st)
     rng = np.random.RandomState(123)
@@ -96,15 +102,61 @@ def main():
     for _ in range(a.warmup):
         one_step()
     backend.sync()
-    t0 = time.perf_counter()
-    for _ in range(a.steps):
-        loss = one_step()
-    backend.sync()
-    dt = time.perf_counter() - t0
+    if a.record:
+        with stream.recording(st) as rec:
+            loss = one_step()
+        rec.graph.launch(st)            # first launch uploads the graph
+        backend.sync()
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            rec.graph.launch(st)
+        backend.sync()
+        dt = time.perf_counter() - t0
+    else:
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            loss = one_step()
+        backend.sync()
+        dt = time.perf_counter() - t0
     loss_val = float(loss.value.asnumpy()[0])
     print(json.dumps({"net": a.net, "workload": desc, "samples_per_s": n * a.steps / dt, "ms_per_step": dt / a.steps * 1e3,
-                      "steps": a.steps, "warmup": a.warmup, "final_loss": loss_val, "forward_ops_per_step": calls[0],
+                      "steps": a.steps, "warmup": a.warmup, "final_loss": loss_val, "forward_ops_per_step": calls[0], "recorded": bool(a.record),
                       "dtype": "f32", "data": "synthetic"}))
+
+
+def mlp(a, ctx):
+    """The 784-256-256-10 MLP of the smallest benchmark configuration (batch 128, SGD 0.1) on the
+    layer-list trainer: 13 launches per step, so the step is the host's launch rate unless recorded."""
+    from . import ndarray, trainer
+    n = a.batch or 128
+    rng = np.random.RandomState(123)
+    spec = trainer.mlp_spec()
+    params = trainer.init_params(spec, seed=123)
+    x = rng.uniform(0, 1, size=(n, 784)).astype(np.float32)
+    y = np.zeros((n, 10), np.float32)
+    y[np.arange(n), rng.randint(0, 10, n)] = 1
+    t = trainer.Trainer(spec, params, x.shape, 10, ctx, optimizer=("sgd", 0.1))
+    gx, gy = ndarray.array(x, ctx), ndarray.array(y, ctx)
+    for _ in range(max(1, a.warmup)):
+        t.step(gx, gy)
+    t.sync()
+    steps = a.steps
+    if a.record:
+        g = t.record_step(gx, gy)
+        g.launch(t.stream)
+        t.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            g.launch(t.stream)
+    else:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            t.step(gx, gy)
+    t.sync()
+    dt = time.perf_counter() - t0
+    print(json.dumps({"net": "mlp", "workload": "MLP 784-256-256-10, batch %d, SGD" % n, "samples_per_s": n * steps / dt,
+                      "ms_per_step": dt / steps * 1e3, "steps": steps, "warmup": a.warmup, "final_loss": t.loss_value(),
+                      "recorded": bool(a.record), "dtype": "f32", "data": "synthetic"}))
 
 
 if __name__ == "__main__":

@@ -13,7 +13,7 @@ import ctypes
 import numpy as np
 
 from ._base import _LIB, c_array, check_call
-from .stream import create_event_handle
+from .stream import create_event_handle, current_keeper
 
 # 0: raw device malloc/free per tensor; != 0: pooled allocator (ndarray.py:8)
 MEMORY_MANAGE_RULE = 1
@@ -57,7 +57,7 @@ def is_gpu_ctx(ctx):
 class NDArray(object):
     """A buffer object: no arithmetic, only allocation, copies and micro-tensor views."""
     __slots__ = ["handle", "auto_deleted", "swap", "in_gpu", "_events", "splitted", "sTensor",
-                 "split_number", "split_dimension", "_owner", "_is_view"]
+                 "split_number", "split_dimension", "_owner", "_is_view", "_keeper"]
 
     def __init__(self, handle, auto_deleted=True, owner=None, is_view=False):
         self.handle = handle
@@ -71,6 +71,7 @@ class NDArray(object):
         self._events = {}
         self._owner = owner          # keeps the parent allocation alive for views
         self._is_view = is_view
+        self._keeper = current_keeper()     # set while a step is being recorded into a graph
 
     def __del__(self):
         h = getattr(self, "handle", None)
@@ -81,7 +82,10 @@ class NDArray(object):
             h.contents.data = None
             _LIB.DLArrayFree(h, ctypes.c_int(MEMORY_MANAGE_RULE))
         elif self.auto_deleted:
-            _LIB.DLArrayFree(h, ctypes.c_int(MEMORY_MANAGE_RULE))
+            # an array born inside a recorded step outlives this object: the graph replays into it
+            keeper = getattr(self, "_keeper", None)
+            if keeper is None or h.contents.ctx.device_type != 2 or not keeper.take(h, MEMORY_MANAGE_RULE):
+                _LIB.DLArrayFree(h, ctypes.c_int(MEMORY_MANAGE_RULE))
         self.handle = None
 
     # ---- events used by swapping executors (created lazily) ----

@@ -312,6 +312,20 @@ class Trainer(object):
         self.update()
         return self.loss
 
+    def record_step(self, x, labels):
+        """Records one training step on (x, labels) into a graph and returns it: graph.launch(
+        self.stream) then runs the whole step with one host call, reading whatever x and labels
+        hold at that time.  For nets whose step is bound by the host's launch rate.  The step must
+        have run once before (first-use set-up cannot be recorded); per-call timers stay off."""
+        from .stream import recording
+        timer, self.timer = self.timer, None
+        try:
+            with recording(self.stream) as rec:
+                self.step(x, labels)
+        finally:
+            self.timer = timer
+        return rec.graph
+
     def sync(self):
         self.stream.sync()
 
