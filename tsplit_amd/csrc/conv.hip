@@ -17,6 +17,8 @@
 // cached on the device; the (img,oh,ow) decomposition uses multiply-shift division and is
 // done once per thread (forward, bwd-data: a thread's columns never change) or once per
 // k-step (bwd-filter).
+#include <algorithm>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -556,7 +558,7 @@ __global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvPara
 // test needs the column of p, kept incrementally, and one range test on the linear index.
 struct TapWgradParams {
   const float *dy, *x;
-  unsigned dy_bytes, x_bytes;
+  int64_t dy_bytes, x_bytes;   // whole tensors; a block addresses from the first image of its k range
   int O, C, HW, W, kW, taps;
   int ph, pw;
   int M, N, K;           // O, C*taps, imgs*HWp
@@ -590,11 +592,18 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
   const int kbegin = zsplit * P.kchunk;
   const int kend = min(P.K, kbegin + P.kchunk);
 
+  // 32-bit offsets count from the first image of this block's k range, so only the images of one
+  // split have to lie within 2 GiB of each other, not the whole tensors
   const int bias = P.ph * P.W + P.pw;
+  const int img_first = kbegin / P.HWp;
+  const int64_t a_base = static_cast<int64_t>(img_first) * P.O * P.HW, b_base = static_cast<int64_t>(img_first) * P.C * P.HW;
+  const int64_t a_left = P.dy_bytes - 4 * a_base, b_left = P.x_bytes - 4 * b_base + 4 * bias;
+  const int a_records = static_cast<int>(a_left < 0 ? 0 : (a_left < 0x7fffffffll ? a_left : 0x7fffffffll));
+  const int b_records = static_cast<int>(b_left < 0 ? 0 : (b_left < 0x7fffffffll ? b_left : 0x7fffffffll));
   const __amdgpu_buffer_rsrc_t ra =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.dy), 0, static_cast<int>(P.dy_bytes), kBufFlags);
-  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float *>(P.x) - bias, 0, static_cast<int>(P.x_bytes + 4u * bias), kBufFlags);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.dy) + a_base, 0, a_records, kBufFlags);
+  const __amdgpu_buffer_rsrc_t rb =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.x) + b_base - bias, 0, b_records, kBufFlags);
 
   // ---- dy operand: thread -> (row tid/4 + 64 s, 4 consecutive positions tid%4)
   unsigned a_voff[PA];
@@ -624,7 +633,7 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
       for (int e = 0; e < 16; ++e) acc[i][jx][e] = 0.f;
 
   // uniform position of the NEXT step to load, and this thread's column within the image row
-  int img = kbegin / P.HWp, p0 = kbegin - img * P.HWp;
+  int img = 0, p0 = kbegin - img_first * P.HWp;   // img counts from img_first
   int ow = (p0 + klocal) % P.W;
   const int ow_first = klocal % P.W;   // column of this thread's position in the first step of an image
 
@@ -1461,10 +1470,50 @@ int launch_bwd_data_phases_tap(const ConvGeo &g, const float *w, const float *dy
   return 0;
 }
 
-// the buffer-load path addresses with 32-bit byte offsets and a 32-tap bit mask
-inline bool tap_kernel_ok(const ConvGeo &g, int64_t src_elems, int64_t w_elems) {
-  return g.kH * g.kW <= 32 && src_elems * 4 + 4 * (static_cast<int64_t>(g.kH) * g.W + g.kW + g.ph * g.W + g.pw) < (1ll << 31) &&
-         w_elems * 4 < (1ll << 31);
+// Bytes a block may address from its base pointer: 2 GiB - 1 (offsets are signed 32-bit and the
+// out-of-range marker is 0x80000000).  TSPLIT_CONV_REACH_BYTES lowers it, which makes small tensors
+// take the paths of tensors beyond 2 GiB (for tests of those paths against a CPU result).
+inline int64_t conv_reach_bytes() {
+  const int64_t full = (1ll << 31) - 1;
+  if (const char *e = std::getenv("TSPLIT_CONV_REACH_BYTES")) {
+    const long long v = std::atoll(e);
+    if (v > 0 && v < full) return v;
+  }
+  return full;
+}
+
+// The buffer-load path addresses with 32-bit byte offsets and a 32-tap bit mask.  A gathered
+// tensor beyond 2 GiB is taken in runs of whole images, one launch each (images are independent
+// in the forward and backward-data passes): -> images per launch, 0 if the path cannot be used.
+inline int tap_kernel_images(const ConvGeo &g, int64_t src_elems_per_img, int64_t w_elems) {
+  if (g.kH * g.kW > 32 || w_elems * 4 >= (1ll << 31) || g.imgs <= 0) return 0;
+  const int64_t room = conv_reach_bytes() - 4 * (static_cast<int64_t>(g.kH) * g.W + g.kW + g.ph * g.W + g.pw);
+  const int64_t fit = room / (src_elems_per_img * 4);
+  if (fit < 1) return 0;
+  if (fit >= g.imgs) return g.imgs;
+  const int64_t launches = (g.imgs + fit - 1) / fit;          // equal runs rather than a short last one
+  return static_cast<int>((g.imgs + launches - 1) / launches);
+}
+
+// Runs f(geometry of the run, first image) over runs of `per` images.
+template <class F>
+inline int for_image_runs(const ConvGeo &g, int per, F f) {
+  for (int first = 0; first < g.imgs; first += per) {
+    ConvGeo run = g;
+    run.imgs = std::min(per, g.imgs - first);
+    const int rc = f(run, static_cast<int64_t>(first));
+    if (rc) return rc;
+  }
+  return 0;
+}
+
+// Images that fit into the 2 GiB a block of conv_wgrad_tap_kernel addresses from the first image of
+// its k range, in the larger of x and dy.  A split of kchunk positions touches at most
+// kchunk / HWp + 2 images.
+inline int wgrad_tap_span_images(const ConvGeo &g) {
+  const int64_t img_bytes = static_cast<int64_t>(std::max(g.C, g.O)) * g.H * g.W * 4;
+  const int64_t room = conv_reach_bytes() - 8 * (static_cast<int64_t>(g.ph) * g.W + g.pw) - 64;
+  return static_cast<int>(std::min<int64_t>(room / img_bytes, 1 << 20));
 }
 
 // bwd-filter on conv_wgrad_tap_kernel ("same" stride-1 convolutions)
@@ -1473,8 +1522,8 @@ int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *d
   TapWgradParams P;
   P.dy = dy;
   P.x = x;
-  P.dy_bytes = static_cast<unsigned>(static_cast<int64_t>(g.imgs) * g.O * g.H * g.W * 4);
-  P.x_bytes = static_cast<unsigned>(static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4);
+  P.dy_bytes = static_cast<int64_t>(g.imgs) * g.O * g.H * g.W * 4;
+  P.x_bytes = static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4;
   P.O = g.O;
   P.C = g.C;
   P.HW = g.H * g.W;
@@ -1492,6 +1541,12 @@ int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *d
   int S;
   static const int occ = blocks_per_cu(conv_wgrad_tap_kernel<BM, BN, WM, WN, false>);
   plan_splitk(tm * tn, P.K, 1024, occ, S, P.kchunk);
+  // the images one split touches must lie within 2 GiB in both tensors: shorten the splits until they do
+  const int span = wgrad_tap_span_images(g);
+  if (P.kchunk / P.HWp + 2 > span) {
+    P.kchunk = std::max(BK, (span - 2) * P.HWp / BK * BK);
+    S = (P.K + P.kchunk - 1) / P.kchunk;
+  }
   const int64_t mn = static_cast<int64_t>(P.M) * P.N;
   float *part = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(S) * mn * 4));
   TS_REQUIRE(part, "conv bwd-filter: no scratch memory for split-K");
@@ -1738,9 +1793,9 @@ int launch_wgrad_narrow(const ConvGeo &g, const float *x, const float *dy, float
 }
 
 inline bool wgrad_tap_ok(const ConvGeo &g) {
-  const int64_t bytes_x = static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4, bytes_dy = static_cast<int64_t>(g.imgs) * g.O * g.H * g.W * 4;
-  return g.s == 1 && g.oH == g.H && g.oW == g.W && g.C % BK == 0 &&
-         bytes_x + 4 * (static_cast<int64_t>(g.ph) * g.W + g.pw) < (1ll << 31) && bytes_dy < (1ll << 31);
+  // three images within a block's reach: a split of at least one image's positions stays addressable
+  return g.s == 1 && g.oH == g.H && g.oW == g.W && g.C % BK == 0 && wgrad_tap_span_images(g) >= 3 &&
+         static_cast<int64_t>(g.imgs) * ((g.H * g.W + BK - 1) / BK * BK) < (1ll << 31) - BK;
 }
 
 // ------------------------------------------------------------------ thin forward (first layer)
@@ -1876,9 +1931,12 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
       const int total = static_cast<int>(numel(w));
       hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wf, g.O, g.C,
                          g.kH * g.kW, false);
-      if (tap_kernel_ok(g, numel(x), numel(w))) {
-        const int rc = g.O <= 64 ? launch_conv_tap<64, 256, 1, 4, false>(g, cf(x), wf, mf(y), st)
-                                 : launch_conv_tap<128, 128, 2, 2, false>(g, cf(x), wf, mf(y), st);
+      const int64_t x_img = static_cast<int64_t>(g.C) * g.H * g.W, y_img = static_cast<int64_t>(g.O) * g.oH * g.oW;
+      if (const int per = tap_kernel_images(g, x_img, numel(w))) {
+        const int rc = for_image_runs(g, per, [&](const ConvGeo &run, int64_t first) {
+          return g.O <= 64 ? launch_conv_tap<64, 256, 1, 4, false>(run, cf(x) + first * x_img, wf, mf(y) + first * y_img, st)
+                           : launch_conv_tap<128, 128, 2, 2, false>(run, cf(x) + first * x_img, wf, mf(y) + first * y_img, st);
+        });
         if (rc) return rc;
       } else if (g.O <= 64) {
         launch_fwd_tap_major<64, 256, 1, 4>(g, cf(x), wf, mf(y), st);
@@ -1907,12 +1965,17 @@ int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray 
     float *wt = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(numel(w)) * 4));
     TS_REQUIRE(wt, "%s: no scratch memory", who);
     const int total = static_cast<int>(numel(w));
+    const int64_t dy_img = static_cast<int64_t>(g.O) * g.oH * g.oW, dx_img = static_cast<int64_t>(g.C) * g.H * g.W;
+    const int per = tap_kernel_images(g, dy_img, numel(w));
     if (g.s == 1 && g.O % BK == 0) {
       hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
                          g.kH * g.kW, true);
-      if (tap_kernel_ok(g, numel(dy), numel(w))) {
-        const int rc = g.C <= 64 ? launch_conv_tap<64, 256, 1, 4, true>(g, cf(dy), wt, mf(dx), st)
-                                 : launch_conv_tap<128, 128, 2, 2, true>(g, cf(dy), wt, mf(dx), st);
+      if (per) {
+        const int rc = for_image_runs(g, per, [&](const ConvGeo &run, int64_t first) {
+          return g.C <= 64
+                     ? launch_conv_tap<64, 256, 1, 4, true>(run, cf(dy) + first * dy_img, wt, mf(dx) + first * dx_img, st)
+                     : launch_conv_tap<128, 128, 2, 2, true>(run, cf(dy) + first * dy_img, wt, mf(dx) + first * dx_img, st);
+        });
         if (rc) return rc;
       } else if (g.C <= 64) {
         launch_bwd_data_tap_major<64, 256, 1, 4>(g, wt, cf(dy), mf(dx), st);
@@ -1923,9 +1986,13 @@ int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray 
       if (g.s > 1) {
         // the sub-filters of all phases together hold every filter element once
         int rc;
-        if (g.O % BK == 0 && tap_kernel_ok(g, numel(dy), numel(w)))
-          rc = g.C <= 64 ? launch_bwd_data_phases_tap<64, 256, 1, 4>(g, cf(w), cf(dy), mf(dx), wt, st)
-                         : launch_bwd_data_phases_tap<128, 128, 2, 2>(g, cf(w), cf(dy), mf(dx), wt, st);
+        if (g.O % BK == 0 && per)
+          rc = for_image_runs(g, per, [&](const ConvGeo &run, int64_t first) {
+            return g.C <= 64 ? launch_bwd_data_phases_tap<64, 256, 1, 4>(run, cf(w), cf(dy) + first * dy_img,
+                                                                        mf(dx) + first * dx_img, wt, st)
+                             : launch_bwd_data_phases_tap<128, 128, 2, 2>(run, cf(w), cf(dy) + first * dy_img,
+                                                                          mf(dx) + first * dx_img, wt, st);
+          });
         else
           rc = g.C <= 64 ? launch_bwd_data_phases<64, 256, 1, 4>(g, cf(w), cf(dy), mf(dx), wt, st)
                          : launch_bwd_data_phases<128, 128, 2, 2>(g, cf(w), cf(dy), mf(dx), wt, st);
