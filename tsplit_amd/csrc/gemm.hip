@@ -102,7 +102,10 @@ extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, co
     float *C = static_cast<float *>(matC->data);
     const int64_t lda = matA->shape[1], ldb = matB->shape[1];
     const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
-    if (!transposeA && !transposeB) rc = dispatch_tile<false, false>(A, lda, B, ldb, C, m, n, k, s, &ws);
+    // large untransposed products run on the forward convolution kernel (tiles cut between blocks
+    // instead of split-K slices); everything else on the tile engine of this file
+    if (!transposeA && !transposeB && !gemm_nn_on_conv_kernel(A, B, C, m, n, k, s, &rc))
+      rc = dispatch_tile<false, false>(A, lda, B, ldb, C, m, n, k, s, &ws);
     if (!transposeA && transposeB) rc = dispatch_tile<false, true>(A, lda, B, ldb, C, m, n, k, s, &ws);
     if (transposeA && !transposeB) rc = dispatch_tile<true, false>(A, lda, B, ldb, C, m, n, k, s, &ws);
     if (transposeA && transposeB) rc = dispatch_tile<true, true>(A, lda, B, ldb, C, m, n, k, s, &ws);
