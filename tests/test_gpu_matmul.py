@@ -15,7 +15,7 @@ CASES = [
     (784, 256, 128), (256, 10, 128), (128, 256, 10),           # MLP backward shapes
     (64, 1000, 4096), (64, 4096, 4096),                        # VGG classifier (skinny, split-K)
     (1, 1, 1), (3, 5, 7), (65, 129, 17), (130, 250, 33), (200, 64, 300), (64, 300, 5000),
-    # enough work for the untransposed form to run on the forward convolution kernel (K % 16 == 0)
+    # large and ragged: many tiles, split-free; a long reduction on skinny tiles
     (8192, 512, 512), (2000, 1030, 1040), (64, 4096, 8192),
 ]
 

@@ -27,8 +27,6 @@ inline float mib(int64_t elems) { return static_cast<float>(elems) * 4.0f / (102
 // that stream without waiting; ops on different streams never share one.
 void *scratch_get(hipStream_t stream, int slot, size_t bytes);
 
-// Row-major C = A B on the forward convolution kernel (conv.hip); false = shape not taken, nothing done.
-bool gemm_nn_on_conv_kernel(const float *A, const float *B, float *C, int M, int N, int K, hipStream_t st, int *rc);
 
 #define TS_FAIL(...)                                  \
   do {                                                \

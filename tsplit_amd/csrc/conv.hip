@@ -293,9 +293,6 @@ __device__ __forceinline__ int64_t tap_out_col(const TapConvParams &P, int n) {
          static_cast<int64_t>(P.out_a0 + P.out_s * static_cast<int>(i)) * P.out_w + (P.out_b0 + P.out_s * static_cast<int>(j));
 }
 
-constexpr int kBufFlags = 0x00020000;           // raw buffer, 32-bit untyped data (gfx9 family)
-constexpr unsigned kOobOffset = 0x80000000u;    // beyond any tensor this path accepts (< 2 GiB)
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // Work distribution.  The tiles of one M row (tile_m fixed) form a chain; block `logical`
 // works on row logical % tm, so the tm blocks with consecutive ids sit on the tiles that share
@@ -2049,24 +2046,6 @@ int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArra
 }
 
 }  // namespace
-
-// ------------------------------------------------------------------ a plain matrix product on the forward kernel
-// A 1x1 convolution of one image IS a row-major matrix product, C[M,N] = A[M,K] B[K,N] with
-// filter = A (K contiguous) and image = B (N positions), so DLGpuMatrixMultiply runs its
-// untransposed form here when there is enough work for the tiles to be cut between blocks
-// (5-15 % faster than the tile engine's split-K slices at 4 GFLOP and more); below that the
-// launcher would give each tile to one block, which is slow for a few tiles with a long K.
-// Returns false, having done nothing, when the shape is not taken.
-bool gemm_nn_on_conv_kernel(const float *A, const float *B, float *C, int M, int N, int K, hipStream_t st, int *rc) {
-  if (K % BK != 0 || M < 1 || N < 1 || (reinterpret_cast<uintptr_t>(A) & 15) != 0) return false;
-  const int bm = M <= 64 ? 64 : 128, bn = M <= 64 ? 256 : 128;
-  const int64_t tiles = static_cast<int64_t>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-  if (tiles * (K / BK) < 8192) return false;
-  ConvGeo g{1, K, 1, N, M, 1, 1, 0, 0, 1, 1, N};
-  if (tap_kernel_images(g, static_cast<int64_t>(K) * N, static_cast<int64_t>(M) * K) != 1) return false;
-  *rc = M <= 64 ? launch_conv_tap<64, 256, 1, 4, false>(g, B, A, C, st) : launch_conv_tap<128, 128, 2, 2, false>(g, B, A, C, st);
-  return true;
-}
 
 }  // namespace tsplit
 

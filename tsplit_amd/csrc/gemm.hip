@@ -17,13 +17,28 @@ namespace {
 
 using namespace mg;
 
-template <int BM, int BN, int WM, int WN, bool TA, bool TB>
+// stored rows of an operand: (M or N, K) by (transposed or not)
+inline int64_t stored_rows(bool k_rows, int mn, int K) { return k_rows ? K : mn; }
+
+// BUF: both operands lie within 2 GiB and are read with buffer loads (the usual case)
+template <int BM, int BN, int WM, int WN, bool TA, bool TB, bool BUF>
 int launch_gemm(const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int M, int N, int K,
                 hipStream_t s, int64_t *ws_elems) {
-  using AL = typename std::conditional<TA, MnContigLoader<BM>, KContigLoader<BM>>::type;
-  using BL = typename std::conditional<TB, KContigLoader<BN>, MnContigLoader<BN>>::type;
-  typename AL::Params ap{A, lda, M, lda % 4 == 0 && aligned16(A)};
-  typename BL::Params bp{B, ldb, N, ldb % 4 == 0 && aligned16(B)};
+  using AL = typename std::conditional<
+      BUF, typename std::conditional<TA, MnContigBufLoader<BM>, KContigBufLoader<BM>>::type,
+      typename std::conditional<TA, MnContigLoader<BM>, KContigLoader<BM>>::type>::type;
+  using BL = typename std::conditional<
+      BUF, typename std::conditional<TB, KContigBufLoader<BN>, MnContigBufLoader<BN>>::type,
+      typename std::conditional<TB, KContigLoader<BN>, MnContigLoader<BN>>::type>::type;
+  typename AL::Params ap;
+  typename BL::Params bp;
+  if constexpr (BUF) {
+    ap = {A, lda, M, K};
+    bp = {B, ldb, N, K};
+  } else {
+    ap = {A, lda, M, lda % 4 == 0 && aligned16(A)};
+    bp = {B, ldb, N, ldb % 4 == 0 && aligned16(B)};
+  }
   const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
   int S, kchunk;
   static const int occ = blocks_per_cu(mfma_gemm_kernel<BM, BN, WM, WN, AL, BL, RowMajorCols>);
@@ -44,20 +59,40 @@ int launch_gemm(const float *A, int64_t lda, const float *B, int64_t ldb, float 
   return 0;
 }
 
+template <int BM, int BN, int WM, int WN, bool TA, bool TB>
+int launch_gemm_any(const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int M, int N, int K,
+                    hipStream_t s, int64_t *ws) {
+  const bool buf = K < (1 << 29) && dense_fits_buffer(stored_rows(TA, M, K), lda, TA ? BK : BM) &&
+                   dense_fits_buffer(stored_rows(!TB, N, K), ldb, TB ? BN : BK);
+  if (buf) return launch_gemm<BM, BN, WM, WN, TA, TB, true>(A, lda, B, ldb, C, M, N, K, s, ws);
+  return launch_gemm<BM, BN, WM, WN, TA, TB, false>(A, lda, B, ldb, C, M, N, K, s, ws);
+}
+
 template <bool TA, bool TB>
 int dispatch_tile(const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int M, int N, int K,
                   hipStream_t s, int64_t *ws) {
-  if (M <= 64) return launch_gemm<64, 256, 1, 4, TA, TB>(A, lda, B, ldb, C, M, N, K, s, ws);
-  return launch_gemm<128, 128, 2, 2, TA, TB>(A, lda, B, ldb, C, M, N, K, s, ws);
+  if (M <= 64) return launch_gemm_any<64, 256, 1, 4, TA, TB>(A, lda, B, ldb, C, M, N, K, s, ws);
+  return launch_gemm_any<128, 128, 2, 2, TA, TB>(A, lda, B, ldb, C, M, N, K, s, ws);
 }
 
-template <int BM, int BN, int WM, int WN, bool TA, bool TB>
+template <int BM, int BN, int WM, int WN, bool TA, bool TB, bool BUF>
 int launch_batched(const float *A, int64_t lda, int64_t sa, const float *B, int64_t ldb, int64_t sb, float *C, int batch,
                    int M, int N, int K, hipStream_t s) {
-  using AL = typename std::conditional<TA, MnContigLoader<BM>, KContigLoader<BM>>::type;
-  using BL = typename std::conditional<TB, KContigLoader<BN>, MnContigLoader<BN>>::type;
-  typename AL::Params ap{A, lda, M, lda % 4 == 0 && sa % 4 == 0 && aligned16(A)};
-  typename BL::Params bp{B, ldb, N, ldb % 4 == 0 && sb % 4 == 0 && aligned16(B)};
+  using AL = typename std::conditional<
+      BUF, typename std::conditional<TA, MnContigBufLoader<BM>, KContigBufLoader<BM>>::type,
+      typename std::conditional<TA, MnContigLoader<BM>, KContigLoader<BM>>::type>::type;
+  using BL = typename std::conditional<
+      BUF, typename std::conditional<TB, KContigBufLoader<BN>, MnContigBufLoader<BN>>::type,
+      typename std::conditional<TB, KContigLoader<BN>, MnContigLoader<BN>>::type>::type;
+  typename AL::Params ap;
+  typename BL::Params bp;
+  if constexpr (BUF) {
+    ap = {A, lda, M, K};
+    bp = {B, ldb, N, K};
+  } else {
+    ap = {A, lda, M, lda % 4 == 0 && sa % 4 == 0 && aligned16(A)};
+    bp = {B, ldb, N, ldb % 4 == 0 && sb % 4 == 0 && aligned16(B)};
+  }
   const int tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
   const int64_t blocks = static_cast<int64_t>(tm) * tn * batch;
   TS_REQUIRE(blocks < (1ll << 31) - 8, "DLGpuBatchMatrixMultiply: too many tiles");
@@ -67,12 +102,21 @@ int launch_batched(const float *A, int64_t lda, int64_t sa, const float *B, int6
   return 0;
 }
 
+template <int BM, int BN, int WM, int WN, bool TA, bool TB>
+int launch_batched_any(const float *A, int64_t lda, int64_t sa, const float *B, int64_t ldb, int64_t sb, float *C,
+                       int batch, int M, int N, int K, hipStream_t s) {
+  const bool buf = K < (1 << 29) && dense_fits_buffer(stored_rows(TA, M, K), lda, TA ? BK : BM) &&
+                   dense_fits_buffer(stored_rows(!TB, N, K), ldb, TB ? BN : BK);
+  if (buf) return launch_batched<BM, BN, WM, WN, TA, TB, true>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
+  return launch_batched<BM, BN, WM, WN, TA, TB, false>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
+}
+
 template <bool TA, bool TB>
 int dispatch_batched(const float *A, int64_t lda, int64_t sa, const float *B, int64_t ldb, int64_t sb, float *C,
                      int batch, int M, int N, int K, hipStream_t s) {
-  if (M <= 64) return launch_batched<64, 256, 1, 4, TA, TB>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
-  if (N <= 64) return launch_batched<256, 64, 4, 1, TA, TB>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
-  return launch_batched<128, 128, 2, 2, TA, TB>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
+  if (M <= 64) return launch_batched_any<64, 256, 1, 4, TA, TB>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
+  if (N <= 64) return launch_batched_any<256, 64, 4, 1, TA, TB>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
+  return launch_batched_any<128, 128, 2, 2, TA, TB>(A, lda, sa, B, ldb, sb, C, batch, M, N, K, s);
 }
 
 }  // namespace
@@ -102,10 +146,7 @@ extern "C" int DLGpuMatrixMultiply(const DLArrayHandle matA, bool transposeA, co
     float *C = static_cast<float *>(matC->data);
     const int64_t lda = matA->shape[1], ldb = matB->shape[1];
     const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
-    // large untransposed products run on the forward convolution kernel (tiles cut between blocks
-    // instead of split-K slices); everything else on the tile engine of this file
-    if (!transposeA && !transposeB && !gemm_nn_on_conv_kernel(A, B, C, m, n, k, s, &rc))
-      rc = dispatch_tile<false, false>(A, lda, B, ldb, C, m, n, k, s, &ws);
+    if (!transposeA && !transposeB) rc = dispatch_tile<false, false>(A, lda, B, ldb, C, m, n, k, s, &ws);
     if (!transposeA && transposeB) rc = dispatch_tile<false, true>(A, lda, B, ldb, C, m, n, k, s, &ws);
     if (transposeA && !transposeB) rc = dispatch_tile<true, false>(A, lda, B, ldb, C, m, n, k, s, &ws);
     if (transposeA && transposeB) rc = dispatch_tile<true, true>(A, lda, B, ldb, C, m, n, k, s, &ws);

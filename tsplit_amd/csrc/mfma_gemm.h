@@ -166,6 +166,121 @@ struct MnContigLoader {
   }
 };
 
+// ------------------------------------------------------------------ dense-matrix loaders on buffer loads
+// The same two layouts read with raw buffer loads: a thread's byte offset is fixed when the tile
+// starts and the k position of a step travels in the scalar offset, so a step costs no vector-ALU
+// address arithmetic and no branch (vector-ALU instructions issued while the matrix pipe is
+// saturated cost MFMA issue time).  Rows or columns outside the matrix get an offset beyond the
+// buffer, for which the load returns 0; the buffer ends with the matrix, so the rows of a ragged
+// last k-step read as zeros by themselves.  For matrices below 2 GiB (32-bit offsets); 16-byte
+// loads need only 4-byte alignment here, so any leading dimension takes the wide path.
+constexpr int kBufFlags = 0x00020000;           // raw buffer, 32-bit untyped data (gfx9 family)
+constexpr unsigned kOobOffset = 0x80000000u;    // beyond any buffer these paths accept (< 2 GiB)
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+struct DenseParams {
+  const float *p;
+  int64_t ld;
+  int mn_total;
+  int k_total;
+};
+
+inline bool dense_fits_buffer(int64_t rows, int64_t ld, int tile_rows) {
+  return rows * ld * 4 < (1ll << 31) && tile_rows * ld * 4 < (1ll << 31);
+}
+
+template <int MN>
+struct KContigBufLoader {   // element (mn, k) at p[mn * ld + k]
+  using Lds = MnMajorLds<MN>;
+  using Params = DenseParams;
+  static constexpr int kPasses = MN / 64;   // 64 rows x 4 quads per pass
+  u32x4 r[kPasses];
+  unsigned voff[kPasses];
+  __amdgpu_buffer_rsrc_t rsrc;
+  int kq;
+
+  __device__ __forceinline__ void init(const Params &P, int mn0, int tid) {
+    kq = tid & 3;
+    const int rows_left = P.mn_total - mn0;
+    const int64_t bytes = static_cast<int64_t>(rows_left) * P.ld * 4;
+    // offsets count from the tile's first row
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.p) + static_cast<int64_t>(mn0) * P.ld, 0,
+                                             static_cast<int>(bytes < 0x7fffffffll ? bytes : 0x7fffffffll), kBufFlags);
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s) {
+      const int row = (tid >> 2) + 64 * s;
+      voff[s] = row < rows_left ? (static_cast<unsigned>(row) * static_cast<unsigned>(P.ld) + 4u * kq) * 4u : kOobOffset;
+    }
+  }
+  __device__ __forceinline__ void load(int k0, int kend) {
+    if (k0 + BK <= kend) {
+#pragma unroll
+      for (int s = 0; s < kPasses; ++s) r[s] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff[s], k0 * 4, 0);
+    } else {
+      // ragged last step: a word may run past the end of its row into the next one
+      const int cnt = kend - (k0 + 4 * kq);
+#pragma unroll
+      for (int s = 0; s < kPasses; ++s) {
+        u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, cnt > 0 ? voff[s] : kOobOffset, k0 * 4, 0);
+        v.y = cnt >= 2 ? v.y : 0u;
+        v.z = cnt >= 3 ? v.z : 0u;
+        v.w = cnt >= 4 ? v.w : 0u;
+        r[s] = v;
+      }
+    }
+  }
+  __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s)
+      *reinterpret_cast<u32x4 *>(lds + ((tid >> 2) + 64 * s) * Lds::kStride + 4 * kq) = r[s];
+  }
+};
+
+template <int MN>
+struct MnContigBufLoader {   // element (k, mn) at p[k * ld + mn]
+  using Lds = KMajorLds<MN>;
+  using Params = DenseParams;
+  static constexpr int kQuads = MN / 4;                 // 16-byte words per row
+  static constexpr int kRowsPerPass = kThreads / kQuads;
+  static constexpr int kPasses = BK / kRowsPerPass;
+  u32x4 r[kPasses];
+  __amdgpu_buffer_rsrc_t rsrc;
+  unsigned voff;
+  int ncols, krow, row_bytes;   // valid columns of this thread's word (>= 4: all), row within a pass
+
+  __device__ __forceinline__ void init(const Params &P, int mn0, int tid) {
+    const int col = mn0 + 4 * (tid % kQuads);
+    krow = tid / kQuads;
+    ncols = P.mn_total - col;
+    row_bytes = static_cast<int>(P.ld) * 4;
+    const int64_t bytes = static_cast<int64_t>(P.k_total) * P.ld * 4;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.p), 0, static_cast<int>(bytes), kBufFlags);
+    voff = ncols > 0 ? (static_cast<unsigned>(krow) * static_cast<unsigned>(P.ld) + static_cast<unsigned>(col)) * 4u
+                     : kOobOffset;
+  }
+  __device__ __forceinline__ void load(int k0, int /*kend*/) {
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s) {
+      const int soff = (k0 + s * kRowsPerPass) * row_bytes;     // rows past the matrix end are out of range
+      if (ncols >= 4 || ncols <= 0) {
+        r[s] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
+      } else {                                                   // the word holding the last 1-3 columns
+        u32x4 v;
+        v.x = __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, soff, 0);
+        v.y = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ncols > 1 ? voff + 4u : kOobOffset, soff, 0);
+        v.z = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ncols > 2 ? voff + 8u : kOobOffset, soff, 0);
+        v.w = 0u;
+        r[s] = v;
+      }
+    }
+  }
+  __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+    for (int s = 0; s < kPasses; ++s)
+      *reinterpret_cast<u32x4 *>(lds + (krow + s * kRowsPerPass) * Lds::kStride + 4 * (tid % kQuads)) = r[s];
+  }
+};
+
 // ------------------------------------------------------------------ column maps
 struct RowMajorCols {   // out[m * row_stride + n]
   __device__ __forceinline__ int64_t operator()(int n) const { return n; }
