@@ -70,6 +70,18 @@ CASES = [
     (2, 16, 5, 5, 8, 1, 1, 0, 0, 1),       # 25 positions, 1x1
     (2, 16, 35, 35, 20, 3, 3, 1, 1, 1),    # 1225 positions
     (3, 16, 3, 5, 136, 3, 3, 1, 1, 1),     # 15 positions: less than one k-step, two row tiles
+    # strided and "valid" filters with input channels in multiples of 16: the same backward-filter
+    # kernel with every thread tracking the (row, column) of its output position
+    (3, 32, 21, 21, 32, 3, 3, 0, 0, 1),    # 3x3 valid (Inception stem): 361 positions
+    (2, 16, 32, 32, 24, 3, 3, 0, 0, 1),    # 900 positions, a multiple of 4 only
+    (2, 16, 18, 18, 24, 3, 3, 0, 0, 1),    # 256 positions: whole k-steps
+    (5, 16, 9, 9, 40, 3, 3, 1, 1, 2),      # 25 output positions per image, stride 2
+    (2, 48, 16, 16, 136, 1, 1, 0, 0, 2),   # 1x1 stride 2: 64 positions, two row tiles
+    (2, 16, 23, 19, 24, 7, 7, 3, 3, 2),    # 7x7 stride 2, non-square
+    (2, 16, 20, 20, 12, 5, 5, 2, 2, 3),    # stride 3
+    (3, 16, 6, 40, 8, 1, 7, 0, 0, 1),      # 1x7 valid: output narrower than the input
+    (2, 32, 5, 5, 16, 5, 5, 0, 0, 1),      # one output position per image
+    (1, 16, 9, 9, 16, 2, 2, 0, 0, 3),      # stride larger than the filter
 ]
 
 

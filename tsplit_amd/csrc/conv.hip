@@ -545,14 +545,18 @@ __global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvPara
 }
 
 // ------------------------------------------------------------------ the tap-major filter-gradient kernel
-// Backward-filter for "same" stride-1 convolutions (oH = H, oW = W) with C % 16 == 0,
-// written like conv_tap_kernel so that the k-loop does almost no vector-ALU work.
+// Backward-filter for convolutions with C % 16 == 0, written like conv_tap_kernel so that the
+// k-loop does almost no vector-ALU work.  First the "same" stride-1 case (oH = H, oW = W):
 // The reduction runs over positions k = (img, p); because the convolution is "same", the
 // gathered element of tap (dr, dc) for output position p is x[img][c][p + dr*W + dc] - linear
 // in p - so the per-thread byte offset is a loop constant and the step's (img, p0) travels in
 // the scalar offset.  A 16-wide step never straddles two images (H*W % 16 == 0, or the TAIL
 // variant pads every image to that).  The padding
 // test needs the column of p, kept incrementally, and one range test on the linear index.
+// GEN (any stride, padding and output size): the gathered element of output position (oh, ow)
+// is x[c][oh*s - ph + kh][ow*s - pw + kw], no longer linear in p, so every thread keeps the
+// (oh, ow) of its position incrementally and rebuilds its byte offset each step: two
+// multiply-adds and two range tests more than the "same" case.
 struct TapWgradParams {
   const float *dy, *x;
   int64_t dy_bytes, x_bytes;   // whole tensors; a block addresses from the first image of its k range
@@ -561,12 +565,14 @@ struct TapWgradParams {
   int M, N, K;           // O, C*taps, imgs*HWp
   int kchunk;            // k range per split (multiple of 16)
   int HWp;               // HW rounded up to a multiple of 16: the reduction runs over imgs*HWp positions
+  // GEN only (HW and W above are then the OUTPUT plane oH*oW and width oW)
+  int s, xH, xW, xHW;    // stride, input height, width and plane
 };
 
 // TAIL: H*W is not a multiple of 16.  Every image's positions are padded to HWp; the padded ones
 // read as zeros (a compare per operand and step, three selects per dy word).  When H*W is not a
 // multiple of 4 either, the 16-byte dy words start on 4-byte boundaries.
-template <int BM, int BN, int WM, int WN, bool TAIL>
+template <int BM, int BN, int WM, int WN, bool TAIL, bool GEN>
 __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams P, float *__restrict__ part,
                                                                   TileGrid tg) {
   static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
@@ -591,9 +597,10 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
 
   // 32-bit offsets count from the first image of this block's k range, so only the images of one
   // split have to lie within 2 GiB of each other, not the whole tensors
-  const int bias = P.ph * P.W + P.pw;
+  const int bias = GEN ? 0 : P.ph * P.W + P.pw;
+  const int x_plane = GEN ? P.xHW : P.HW;
   const int img_first = kbegin / P.HWp;
-  const int64_t a_base = static_cast<int64_t>(img_first) * P.O * P.HW, b_base = static_cast<int64_t>(img_first) * P.C * P.HW;
+  const int64_t a_base = static_cast<int64_t>(img_first) * P.O * P.HW, b_base = static_cast<int64_t>(img_first) * P.C * x_plane;
   const int64_t a_left = P.dy_bytes - 4 * a_base, b_left = P.x_bytes - 4 * b_base + 4 * bias;
   const int a_records = static_cast<int>(a_left < 0 ? 0 : (a_left < 0x7fffffffll ? a_left : 0x7fffffffll));
   const int b_records = static_cast<int>(b_left < 0 ? 0 : (b_left < 0x7fffffffll ? b_left : 0x7fffffffll));
@@ -619,7 +626,8 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
   const int kh = tap / P.kW, kw = tap - kh * P.kW;
   const int dr = kh - P.ph, dc = kw - P.pw;
   const int shift = dr * P.W + dc;                // x index = p + shift
-  const unsigned b_voff = static_cast<unsigned>(c_first * P.HW + klocal + shift + bias) * 4u;
+  const unsigned b_voff = GEN ? static_cast<unsigned>(c_first * x_plane) * 4u
+                              : static_cast<unsigned>(c_first * P.HW + klocal + shift + bias) * 4u;
 
   acc16 acc[2][2];
 #pragma unroll
@@ -633,6 +641,8 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
   int img = 0, p0 = kbegin - img_first * P.HWp;   // img counts from img_first
   int ow = (p0 + klocal) % P.W;
   const int ow_first = klocal % P.W;   // column of this thread's position in the first step of an image
+  int oh = (p0 + klocal) / P.W;        // GEN: its row
+  const int oh_first = klocal / P.W;
 
   u32x4 ra_regs[PA];
   unsigned rb_regs[KCOLS];
@@ -645,21 +655,36 @@ __global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams
     for (int s = 0; s < PA; ++s)
       ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_cnt > 0 ? a_voff[s] : kOobOffset, soff_a, 0);
     const int p = p0 + klocal;
-    const bool ok = cols_ok && (!TAIL || p < P.HW) &&
-                    static_cast<unsigned>(p + dr * P.W) < static_cast<unsigned>(P.HW) &&
-                    static_cast<unsigned>(ow + dc) < static_cast<unsigned>(P.W);
-    const unsigned voff = ok ? b_voff : kOobOffset;
-    const int soff_b = (img * P.C * P.HW + p0) * 4;
+    if (GEN) {
+      const int ih = oh * P.s + dr, iw = ow * P.s + dc;
+      const bool ok = cols_ok && (!TAIL || p < P.HW) && static_cast<unsigned>(ih) < static_cast<unsigned>(P.xH) &&
+                      static_cast<unsigned>(iw) < static_cast<unsigned>(P.xW);
+      const unsigned voff = ok ? b_voff + static_cast<unsigned>(ih * P.xW + iw) * 4u : kOobOffset;
+      const int soff_b = img * P.C * x_plane * 4;
 #pragma unroll
-    for (int i = 0; i < KCOLS; ++i)
-      rb_regs[i] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, soff_b + i * P.HW * 4, 0);
+      for (int i = 0; i < KCOLS; ++i)
+        rb_regs[i] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, soff_b + i * x_plane * 4, 0);
+    } else {
+      const bool ok = cols_ok && (!TAIL || p < P.HW) &&
+                      static_cast<unsigned>(p + dr * P.W) < static_cast<unsigned>(P.HW) &&
+                      static_cast<unsigned>(ow + dc) < static_cast<unsigned>(P.W);
+      const unsigned voff = ok ? b_voff : kOobOffset;
+      const int soff_b = (img * P.C * P.HW + p0) * 4;
+#pragma unroll
+      for (int i = 0; i < KCOLS; ++i)
+        rb_regs[i] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, soff_b + i * P.HW * 4, 0);
+    }
     p0 += BK;
     ow += BK;                      // BK may exceed W for tiny images: reduce until in range
-    while (ow >= P.W) ow -= P.W;
+    while (ow >= P.W) {
+      ow -= P.W;
+      if (GEN) ++oh;
+    }
     if (p0 >= P.HWp) {
       p0 = 0;
       ++img;
       if (TAIL) ow = ow_first;     // positions do not continue across the padded tail
+      if (GEN) oh = oh_first;
     }
   };
   auto store_step = [&](float *sa, float *sb) {
@@ -1508,7 +1533,7 @@ inline int for_image_runs(const ConvGeo &g, int per, F f) {
 // its k range, in the larger of x and dy.  A split of kchunk positions touches at most
 // kchunk / HWp + 2 images.
 inline int wgrad_tap_span_images(const ConvGeo &g) {
-  const int64_t img_bytes = static_cast<int64_t>(std::max(g.C, g.O)) * g.H * g.W * 4;
+  const int64_t img_bytes = std::max(static_cast<int64_t>(g.C) * g.H * g.W, static_cast<int64_t>(g.O) * g.oH * g.oW) * 4;
   const int64_t room = conv_reach_bytes() - 8 * (static_cast<int64_t>(g.ph) * g.W + g.pw) - 64;
   return static_cast<int>(std::min<int64_t>(room / img_bytes, 1 << 20));
 }
@@ -1516,15 +1541,20 @@ inline int wgrad_tap_span_images(const ConvGeo &g) {
 // bwd-filter on conv_wgrad_tap_kernel ("same" stride-1 convolutions)
 template <int BM, int BN, int WM, int WN>
 int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *dw, hipStream_t st, int64_t *ws_elems) {
+  const bool gen = !(g.s == 1 && g.oH == g.H && g.oW == g.W);
   TapWgradParams P;
   P.dy = dy;
   P.x = x;
-  P.dy_bytes = static_cast<int64_t>(g.imgs) * g.O * g.H * g.W * 4;
+  P.dy_bytes = static_cast<int64_t>(g.imgs) * g.O * g.oH * g.oW * 4;
   P.x_bytes = static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4;
   P.O = g.O;
   P.C = g.C;
-  P.HW = g.H * g.W;
-  P.W = g.W;
+  P.HW = g.oH * g.oW;
+  P.W = g.oW;
+  P.s = g.s;
+  P.xH = g.H;
+  P.xW = g.W;
+  P.xHW = g.H * g.W;
   P.kW = g.kW;
   P.taps = g.kH * g.kW;
   P.ph = g.ph;
@@ -1536,7 +1566,7 @@ int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *d
   const bool tail = P.HWp != P.HW;
   const int tm = (P.M + BM - 1) / BM, tn = (P.N + BN - 1) / BN;
   int S;
-  static const int occ = blocks_per_cu(conv_wgrad_tap_kernel<BM, BN, WM, WN, false>);
+  static const int occ = blocks_per_cu(conv_wgrad_tap_kernel<BM, BN, WM, WN, false, false>);
   plan_splitk(tm * tn, P.K, 1024, occ, S, P.kchunk);
   // the images one split touches must lie within 2 GiB in both tensors: shorten the splits until they do
   const int span = wgrad_tap_span_images(g);
@@ -1548,12 +1578,16 @@ int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *d
   float *part = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(S) * mn * 4));
   TS_REQUIRE(part, "conv bwd-filter: no scratch memory for split-K");
   *ws_elems = S * mn;
-  if (tail)
-    hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN, true>), dim3(grid_blocks(tm, tn, S)), dim3(kThreads), 0,
-                       st, P, part, TileGrid{tm, tn, tm * tn * S});
+  const dim3 grid(grid_blocks(tm, tn, S));
+  const TileGrid tg{tm, tn, tm * tn * S};
+  if (gen && tail)
+    hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN, true, true>), grid, dim3(kThreads), 0, st, P, part, tg);
+  else if (gen)
+    hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN, false, true>), grid, dim3(kThreads), 0, st, P, part, tg);
+  else if (tail)
+    hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN, true, false>), grid, dim3(kThreads), 0, st, P, part, tg);
   else
-    hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN, false>), dim3(grid_blocks(tm, tn, S)), dim3(kThreads), 0,
-                       st, P, part, TileGrid{tm, tn, tm * tn * S});
+    hipLaunchKernelGGL((conv_wgrad_tap_kernel<BM, BN, WM, WN, false, false>), grid, dim3(kThreads), 0, st, P, part, tg);
   hipLaunchKernelGGL(fold_tap_major_kernel, dim3(static_cast<unsigned>((mn + 63) / 64)), dim3(256), 0, st, part, dw,
                      g.O, g.C, g.kH * g.kW, mn, S);
   return 0;
@@ -1791,8 +1825,8 @@ int launch_wgrad_narrow(const ConvGeo &g, const float *x, const float *dy, float
 
 inline bool wgrad_tap_ok(const ConvGeo &g) {
   // three images within a block's reach: a split of at least one image's positions stays addressable
-  return g.s == 1 && g.oH == g.H && g.oW == g.W && g.C % BK == 0 && wgrad_tap_span_images(g) >= 3 &&
-         static_cast<int64_t>(g.imgs) * ((g.H * g.W + BK - 1) / BK * BK) < (1ll << 31) - BK;
+  return g.C % BK == 0 && wgrad_tap_span_images(g) >= 3 &&
+         static_cast<int64_t>(g.imgs) * ((g.oH * g.oW + BK - 1) / BK * BK) < (1ll << 31) - BK;
 }
 
 // ------------------------------------------------------------------ thin forward (first layer)
