@@ -1957,11 +1957,16 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
       const int rc = launch_conv_thin_fwd(g, cf(x), cf(w), mf(y), st);
       if (rc) return rc;
     } else if (g.C % BK == 0) {
-      float *wf = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(numel(w)) * 4));
-      TS_REQUIRE(wf, "%s: no scratch memory", who);
-      const int total = static_cast<int>(numel(w));
-      hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wf, g.O, g.C,
-                         g.kH * g.kW, false);
+      // a 1x1 filter [O][C] already is tap-major: used where it lies
+      const float *wf = cf(w);
+      if (g.kH * g.kW != 1 || !aligned16(wf)) {
+        float *relaid = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(numel(w)) * 4));
+        TS_REQUIRE(relaid, "%s: no scratch memory", who);
+        const int total = static_cast<int>(numel(w));
+        hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), relaid, g.O,
+                           g.C, g.kH * g.kW, false);
+        wf = relaid;
+      }
       const int64_t x_img = static_cast<int64_t>(g.C) * g.H * g.W, y_img = static_cast<int64_t>(g.O) * g.oH * g.oW;
       if (const int per = tap_kernel_images(g, x_img, numel(w))) {
         const int rc = for_image_runs(g, per, [&](const ConvGeo &run, int64_t first) {
