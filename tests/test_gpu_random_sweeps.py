@@ -102,3 +102,87 @@ def test_random_pooling(shape, kH, kW, pad, stride):
     L.average_pooling2d_gradient(gdy, kH, kW, dx, pad, stride)
     assert_close(y.asnumpy(), O.avg_pool(x, kH, kW, pad, stride), 1e-4, "avg_pool")
     assert_close(dx.asnumpy(), O.avg_pool_grad(dy, shape, kH, kW, pad, stride), 1e-4, "avg_pool_grad")
+
+
+def _bn_cases(seed, count):
+    rng = np.random.RandomState(seed)
+    out = []
+    for _ in range(count):
+        N, C = int(rng.choice([1, 2, 3, 8, 32])), int(rng.choice([1, 3, 16, 33, 64, 130]))
+        H, W = int(rng.randint(1, 40)), int(rng.randint(1, 40))
+        if rng.rand() < 0.25:
+            H, W = int(rng.choice([56, 64, 75])), int(rng.choice([56, 64, 75]))     # beyond one pass per channel
+        if N * C * H * W > 3e6:
+            N = 1
+        out.append(((N, C, H, W), bool(rng.randint(2))))
+    return out
+
+
+@pytest.mark.parametrize("shape,saved", _bn_cases(5, 80))
+def test_random_batchnorm(shape, saved):
+    """Plain and fused BatchNorm(+Relu), forward and gradient, with and without saved statistics."""
+    from tsplit_amd import gpu_links as L, ndarray
+    ctx = ndarray.gpu(0)
+    C = shape[1]
+    rng = np.random.RandomState((shape[0] * 7 + C * 131 + shape[2] * 31 + shape[3]) % (2 ** 31))
+    x = (rng.normal(size=shape) * 2 + rng.normal(size=(1, C, 1, 1)) * 3).astype(np.float32)
+    gamma = rng.normal(size=(1, C, 1, 1)).astype(np.float32)
+    beta = rng.normal(size=(1, C, 1, 1)).astype(np.float32)
+    dy = rng.normal(size=shape).astype(np.float32)
+    eps = 0.01
+    arr = lambda a: ndarray.array(a, ctx)
+    gx, gg, gb, gdy = arr(x), arr(gamma), arr(beta), arr(dy)
+    y, dx = ndarray.empty(shape, ctx), ndarray.empty(shape, ctx)
+    dg, db = ndarray.empty((1, C, 1, 1), ctx), ndarray.empty((1, C, 1, 1), ctx)
+    sm, sv = ndarray.empty((1, C, 1, 1), ctx), ndarray.empty((1, C, 1, 1), ctx)
+    L.CuDNN_Batch_Normalization(gx, gg, gb, y, sm if saved else None, sv if saved else None, 0.99, eps)
+    ry, mean, var = O.batchnorm_forward(x, gamma, beta, eps)
+    assert_close(y.asnumpy(), ry, 1e-4, "bn fwd")
+    L.CuDNN_Batch_Normalization_gradient(gdy, gx, gg, dx, dg, db, sm if saved else None, sv if saved else None, eps)
+    rdx, rdg, rdb = O.batchnorm_backward(dy, x, gamma, eps)
+    assert_close(dx.asnumpy(), rdx, 1e-4, "bn dx")
+    assert_close(dg.asnumpy().ravel(), rdg, 1e-4, "bn dgamma")
+    assert_close(db.asnumpy().ravel(), rdb, 1e-4, "bn dbeta")
+    # fused with Relu: max(BN(x), 0) and the reference's Relu derivative (1/2 at zero) in front of the BN gradient
+    L.batch_norm_relu(gx, gg, gb, y, sm, sv, eps)
+    fused_y = y.asnumpy()
+    assert_close(fused_y, np.maximum(ry, 0), 1e-4, "bn+relu fwd")
+    L.batch_norm_relu_gradient(gdy, gx, gg, gb, dx, dg, db, sm, sv, eps)
+    # the gate follows the sign fp32 arithmetic gave z = BN(x) (a z within rounding of zero may have
+    # the other sign in float64; exact zeros, where the derivative is 1/2, do not occur in random data)
+    gated = O.relu_grad(np.where(fused_y > 0, 1.0, -1.0), dy)
+    fdx, fdg, fdb = O.batchnorm_backward(gated.astype(np.float32), x, gamma, eps)
+    assert_close(dx.asnumpy(), fdx, 1e-4, "bn+relu dx")
+    assert_close(dg.asnumpy().ravel(), fdg, 1e-4, "bn+relu dgamma")
+    assert_close(db.asnumpy().ravel(), fdb, 1e-4, "bn+relu dbeta")
+
+
+def _ce_cases(seed, count):
+    rng = np.random.RandomState(seed)
+    return [(int(rng.choice([1, 2, 7, 64, 300])), int(rng.choice([1, 2, 10, 33, 1000, 1001, 2048, 2050, 2052, 4096, 32000])))
+            for _ in range(count)]
+
+
+@pytest.mark.parametrize("rows,cols", sorted(set(_ce_cases(9, 60))))
+def test_random_softmax_cross_entropy(rows, cols):
+    from tsplit_amd import gpu_links as L, ndarray
+    ctx = ndarray.gpu(0)
+    rng = np.random.RandomState(rows * 1009 + cols)
+    logits = (rng.normal(size=(rows, cols)) * 3).astype(np.float32)
+    labels = np.zeros((rows, cols), np.float32)
+    labels[np.arange(rows), rng.randint(0, cols, rows)] = 1.0
+    if cols > 1 and rows % 2 == 0:                        # smoothed labels on half of the cases
+        labels = (labels * 0.9 + 0.1 / cols).astype(np.float32)
+    g = np.array([rng.uniform(0.5, 2.0)], np.float32)
+    arr = lambda a: ndarray.array(a, ctx)
+    gl, gy, gg = arr(logits), arr(labels), arr(g)
+    loss, grad, sm = ndarray.empty((1,), ctx), ndarray.empty((rows, cols), ctx), ndarray.empty((rows, cols), ctx)
+    L.softmax_cross_entropy(gl, gy, loss)
+    L.softmax_cross_entropy_gradient(gl, gy, gg, grad)
+    L.softmax(gl, sm)
+    # the loss is a difference of terms the size of the logits (log-sum-exp minus the label's logit): a
+    # confident row gives a loss far below them, so the error is measured against their scale as well
+    ref_loss = float(np.asarray(O.softmax_ce(logits, labels)).reshape(-1)[0])
+    assert abs(float(loss.asnumpy()[0]) - ref_loss) <= 1e-4 * max(abs(ref_loss), 1e-2 * float(np.abs(logits).max()))
+    assert_close(grad.asnumpy(), O.softmax_ce_grad(logits, labels, g), 1e-4, "ce grad")
+    assert_close(sm.asnumpy(), O.softmax(logits), 1e-4, "softmax")
