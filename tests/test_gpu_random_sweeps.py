@@ -186,3 +186,74 @@ def test_random_softmax_cross_entropy(rows, cols):
     assert abs(float(loss.asnumpy()[0]) - ref_loss) <= 1e-4 * max(abs(ref_loss), 1e-2 * float(np.abs(logits).max()))
     assert_close(grad.asnumpy(), O.softmax_ce_grad(logits, labels, g), 1e-4, "ce grad")
     assert_close(sm.asnumpy(), O.softmax(logits), 1e-4, "softmax")
+
+
+def _shape(rng, ndim, big):
+    ext = [1, 2, 3, 4, 5, 7, 8, 16, 17, 33, 64, 65] + ([130, 257] if big else [])
+    while True:
+        s = tuple(int(rng.choice(ext)) for _ in range(ndim))
+        if np.prod(s) <= 2_000_000:
+            return s
+
+
+def _layout_cases(seed, count):
+    rng = np.random.RandomState(seed)
+    return [(_shape(rng, int(rng.randint(1, 6)), rng.rand() < 0.3), int(rng.randint(1 << 30))) for _ in range(count)]
+
+
+@pytest.mark.parametrize("shape,seed", _layout_cases(21, 120))
+def test_random_layout_ops(shape, seed):
+    """Transpose with a random permutation, reduce-sum over a random axis subset, concat and slice along
+    a random axis with their gradients, constant padding: data movement is bit-exact, sums 1e-4."""
+    from tsplit_amd import gpu_links as L, ndarray
+    ctx = ndarray.gpu(0)
+    rng = np.random.RandomState(seed)
+    nd = len(shape)
+    x = rng.normal(size=shape).astype(np.float32)
+    gx = ndarray.array(x, ctx)
+    # transpose
+    perm = tuple(int(p) for p in rng.permutation(nd))
+    ref = O.transpose(x, perm)
+    out = ndarray.empty(ref.shape, ctx)
+    L.matrix_transpose(gx, out, perm)
+    np.testing.assert_array_equal(out.asnumpy(), ref)
+    # reduce-sum
+    axes = sorted(int(a) for a in rng.choice(nd, size=rng.randint(1, nd + 1), replace=False))
+    ref = O.reduce_sum(x, axes)
+    out = ndarray.empty(ref.shape or (1,), ctx)
+    L.reduce_sum(gx, out, axes)
+    assert_close(out.asnumpy().reshape(ref.shape), ref, 1e-4, f"reduce_sum {shape} {axes}")
+    # concat with a second array that differs along the axis, and the gradients back
+    axis = int(rng.randint(nd))
+    sb = list(shape)
+    sb[axis] = int(rng.choice([1, 2, 5, 16, 33]))
+    b = rng.normal(size=sb).astype(np.float32)
+    ref = O.concat(x, b, axis)
+    out = ndarray.empty(ref.shape, ctx)
+    L.concat(gx, ndarray.array(b, ctx), out, axis)
+    np.testing.assert_array_equal(out.asnumpy(), ref)
+    ga, gb = ndarray.empty(shape, ctx), ndarray.empty(tuple(sb), ctx)
+    L.concat_gradient(out, ga, axis, 0)
+    L.concat_gradient(out, gb, axis, 1)
+    np.testing.assert_array_equal(ga.asnumpy(), x)
+    np.testing.assert_array_equal(gb.asnumpy(), b)
+    # slice a random box out of the concatenated array, and scatter it back into zeros
+    begin = [int(rng.randint(0, e)) for e in ref.shape]
+    size = [int(rng.randint(1, e - b0 + 1)) for e, b0 in zip(ref.shape, begin)]
+    box = ndarray.empty(tuple(size), ctx)
+    L.matrix_slice(out, box, begin)
+    np.testing.assert_array_equal(box.asnumpy(), O.slice_(ref, begin, size))
+    back = ndarray.empty(ref.shape, ctx)
+    L.matrix_slice_gradient(box, back, begin)
+    np.testing.assert_array_equal(back.asnumpy(), O.slice_grad(box.asnumpy(), begin, ref.shape))
+    # constant padding of the trailing axes of a 4-D array
+    if nd == 4:
+        k = int(rng.randint(0, 5))
+        paddings = [(int(rng.randint(0, 4)), int(rng.randint(0, 4))) for _ in range(k)]
+        ref = O.pad(x, paddings, 0.25)
+        out = ndarray.empty(ref.shape, ctx)
+        L.pad(gx, out, paddings, "CONSTANT", 0.25)
+        np.testing.assert_array_equal(out.asnumpy(), ref.astype(np.float32))
+        dx = ndarray.empty(shape, ctx)
+        L.pad_gradient(out, dx, paddings, "CONSTANT")
+        np.testing.assert_array_equal(dx.asnumpy(), x)
