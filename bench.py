@@ -34,9 +34,9 @@ PEAK_HBM_GBS = 8000.0
 # be the step's largest, from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
 # profiles/vgg16_b64_train_step_hbm_traffic.txt (counter units calibrated on the Relu kernel).
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "conv_fwd_128x128": (324.6 + 137.7) * 1e6,
-    "conv_bwd_data_128x128": (440.9 + 129.3) * 1e6,
-    "conv_bwd_filter_128x128": (498.9 + 64.2) * 1e6,
+    "conv_fwd_128x128": (324.4 + 137.5) * 1e6,
+    "conv_bwd_data_128x128": (440.2 + 129.5) * 1e6,
+    "conv_bwd_filter_128x128": (555.1 + 64.2) * 1e6,
 }
 
 
