@@ -79,6 +79,20 @@ def _cases(L, A, E, S):
     dv = E((32, 8, 256, 64))
     add("batch_matmul/pv", 2.0 * nb * 256 * 64 * 256, "flop", lambda s: L.batch_matrix_multiply(pr, False, vh, False, ctxo, s))
     add("batch_matmul/p_t_dctx", 2.0 * nb * 256 * 64 * 256, "flop", lambda s: L.batch_matrix_multiply(pr, True, vh, False, dv, s))
+    # plain matrix products: Transformer projections / FFN / vocabulary (forward A B, input gradient A B^T,
+    # weight gradient A^T B) and the batch-64 fully-connected layers of VGG-16
+    for tag, m, k, nn in (("proj_8192x512x512", 8192, 512, 512), ("ffn_8192x512x2048", 8192, 512, 2048),
+                          ("vocab_8160x512x32000", 8160, 512, 32000), ("vgg_fc1_64x25088x4096", 64, 25088, 4096),
+                          ("vgg_fc2_64x4096x4096", 64, 4096, 4096)):
+        ma, mb, mc = A((m, k)), A((k, nn)), A((m, nn))
+        da, db = E((m, k)), E((k, nn))
+        fl = 2.0 * m * nn * k
+        add("matmul/" + tag + "/A_B", fl, "flop",
+            lambda s, ma=ma, mb=mb, mc=mc: L.matrix_multiply(ma, False, mb, False, mc, s))
+        add("matmul/" + tag + "/dY_Bt", fl, "flop",
+            lambda s, mc=mc, mb=mb, da=da: L.matrix_multiply(mc, False, mb, True, da, s))
+        add("matmul/" + tag + "/At_dY", fl, "flop",
+            lambda s, ma=ma, mc=mc, db=db: L.matrix_multiply(ma, True, mc, False, db, s))
     # pad (Inception-style spatial padding), one-hot labels, where, embedding
     xp, yp = A((32, 96, 35, 35)), E((32, 96, 37, 37))
     add("pad/35_to_37", 4 * (n(32, 96, 35, 35) + n(32, 96, 37, 37)), "byte",
