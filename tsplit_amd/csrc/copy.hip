@@ -1,8 +1,8 @@
 // Copying concat / slice kernels (the zero-copy batch split needs no kernel at all).
 //
-// Concat along `axis` of two tensors is, per input, a copy of `outer` rows of
-// len = axis_extent * inner contiguous elements into rows of the wider output; the gradient
-// is the same copy in the other direction.  Rows move as 16-byte words whenever lengths,
+// Concat along `axis` of two tensors writes `outer` output rows, each the row of the first input
+// (axis_extent * inner contiguous elements) followed by the row of the second, in one launch; the
+// gradient copies one input's part of every row back.  Rows move as 16-byte words whenever lengths,
 // strides, offsets and base pointers allow, else element-wise.  Slice is a general n-D
 // window copy; shapes travel as kernel arguments (the reference stages them through three
 // synchronous host-to-device copies per call: src/ops/Slice.cu:48-56).
@@ -47,6 +47,41 @@ void rows_copy(const float *src, float *dst, int64_t rows, int64_t len, int64_t 
     hipLaunchKernelGGL(rows_copy_kernel<float>, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
                        dim3(kThreads), 0, s, src, dst, FastDiv(static_cast<uint32_t>(len)),
                        static_cast<uint32_t>(src_stride), static_cast<uint32_t>(dst_stride), total);
+  }
+}
+
+// Concat of two tensors in one launch: output row r = x row r (lx words) followed by y row r (ly words).
+template <typename W>
+__global__ __launch_bounds__(kThreads) void concat_rows_kernel(const W *__restrict__ x, const W *__restrict__ y,
+                                                               W *__restrict__ dst, FastDiv row, uint32_t lx,
+                                                               uint32_t ly, int64_t total) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx >= total) return;
+  uint32_t r, j;
+  if (total < (1ll << 32)) {
+    r = row.div(static_cast<uint32_t>(idx));
+    j = static_cast<uint32_t>(idx) - r * row.d;
+  } else {
+    r = static_cast<uint32_t>(idx / row.d);
+    j = static_cast<uint32_t>(idx - static_cast<int64_t>(r) * row.d);
+  }
+  dst[idx] = j < lx ? x[static_cast<int64_t>(r) * lx + j] : y[static_cast<int64_t>(r) * ly + (j - lx)];
+}
+
+void concat_rows(const float *x, const float *y, float *dst, int64_t rows, int64_t lx, int64_t ly, hipStream_t s) {
+  if (rows <= 0 || lx + ly <= 0) return;
+  const bool vec = lx % 4 == 0 && ly % 4 == 0 && aligned16(x) && aligned16(y) && aligned16(dst);
+  if (vec) {
+    const int64_t total = rows * ((lx + ly) / 4);
+    hipLaunchKernelGGL(concat_rows_kernel<float4>, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
+                       dim3(kThreads), 0, s, reinterpret_cast<const float4 *>(x), reinterpret_cast<const float4 *>(y),
+                       reinterpret_cast<float4 *>(dst), FastDiv(static_cast<uint32_t>((lx + ly) / 4)),
+                       static_cast<uint32_t>(lx / 4), static_cast<uint32_t>(ly / 4), total);
+  } else {
+    const int64_t total = rows * (lx + ly);
+    hipLaunchKernelGGL(concat_rows_kernel<float>, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
+                       dim3(kThreads), 0, s, x, y, dst, FastDiv(static_cast<uint32_t>(lx + ly)),
+                       static_cast<uint32_t>(lx), static_cast<uint32_t>(ly), total);
   }
 }
 
@@ -134,9 +169,7 @@ int DLGpuConcat(const DLArrayHandle input_x, const DLArrayHandle input_y, DLArra
   TS_REQUIRE((ax + ay) * inner < (1ll << 32), "DLGpuConcat: row too long");
   hipStream_t s = stream_of(stream_handle);
   ProfileScope ps(p, s, numel(input_x) + numel(input_y), numel(output), 0);
-  const int64_t lo = (ax + ay) * inner;
-  rows_copy(cf(input_x), mf(output), outer, ax * inner, ax * inner, lo, s);
-  rows_copy(cf(input_y), mf(output) + ax * inner, outer, ay * inner, ay * inner, lo, s);
+  concat_rows(cf(input_x), cf(input_y), mf(output), outer, ax * inner, ay * inner, s);
   return ps.finish();
 }
 
