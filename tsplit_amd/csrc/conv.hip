@@ -1417,14 +1417,20 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
   sk.whole_waves = 0;
   sk.cut_first = 0;
   int cut_tiles = tiles;         // tiles the assemble kernel looks at
-  if (tiles % slots == 0 || static_cast<int64_t>(tiles) * sk.ksteps < slots * 8) {
+  // With little work, pieces stay at least kMinPiece k-steps long (shorter ones are all prologue and
+  // assembly), and nothing is cut unless that at least halves the longest block's work.
+  constexpr int kMinPiece = 8;
+  const bool little = static_cast<int64_t>(tiles) * sk.ksteps < slots * kMinPiece;
+  const bool cut_little = little && tiles * 2 <= slots && sk.ksteps >= 2 * kMinPiece && sk.total / kMinPiece >= 8;
+  if (tiles % slots == 0 || (little && !cut_little)) {
     // whole tiles fill whole waves of blocks, or there is too little work to cut: one tile per block
     sk.iters_per_block = sk.ksteps;
     sk.ranges = tn;
     grid = (tiles + 7) / 8 * 8;
-  } else {                       // one full wave of blocks
+  } else {                       // one full wave of blocks (fewer when the work is little)
     // ranges per row: a multiple of 8, so that the tm blocks of one range share an XCD
     sk.ranges = std::max(8, slots / tm / 8 * 8);
+    if (cut_little) sk.ranges = std::max(8, std::min(sk.ranges, sk.total / kMinPiece / 8 * 8));
     grid = static_cast<unsigned>(sk.ranges) * tm;
     const int full = tn / sk.ranges;
     sk.whole_waves = full;
