@@ -115,6 +115,16 @@ def test_conv_cudnn_family(case, rng):
     _run(case, "cudnn", rng)
 
 
+@pytest.mark.parametrize("raw", ["0", "1"])
+@pytest.mark.parametrize("case", [c for c in CASES if c[9] == 1 and c[4] % 16 == 0])
+def test_conv_backward_data_with_and_without_filter_relay(case, raw, rng, monkeypatch):
+    """Stride-1 backward-data with output channels in multiples of 16 has two kernels: one reads a
+    re-laid copy of the filter, one (chosen for small layers) the filter where it lies.  Both run on
+    every such shape."""
+    monkeypatch.setenv("TSPLIT_CONV_RAW", raw)
+    _run(case, "cudnn", rng)
+
+
 @pytest.mark.parametrize("case", [c for c in CASES if c[7] == c[8]][:8])
 def test_conv_plain_family(case, rng):
     _run(case, "plain", rng)

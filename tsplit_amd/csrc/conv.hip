@@ -268,7 +268,11 @@ struct TapMajorColsLoader {
 //     whose tap falls into the padding gets an out-of-range offset, for which a buffer load
 //     returns 0 - no zero-fill, no divergent branch.
 struct TapConvParams {
-  const float *wf;      // filter re-laid as [M][K], k' = ((ch/16)*taps + tap)*16 + ch%16
+  // filter re-laid as [M][K], k' = ((ch/16)*taps + tap)*16 + ch%16 - or, for the RAW kernels, the
+  // filter as it lies in memory, [O][C][taps]: element (row m, channel ch, tap) at
+  // m*raw_row + ch*raw_ch + tap (forward: rows are O, channels C; backward-data: the other way)
+  const float *wf;
+  int raw_row, raw_ch;
   const float *src;     // x (forward) or dy (backward-data)
   unsigned wf_bytes, src_bytes;
   FastDiv plane, width; // output columns per image / per row
@@ -319,7 +323,10 @@ struct StreamK {
   int cut_first;         // tile_n of the first tile of the cut part (= whole_waves * ranges)
 };
 
-template <int BM, int BN, int WM, int WN, bool BWD_DATA>
+// RAW: the filter operand is read from the [O][C][taps] filter itself with four 4-byte loads per
+// 16-byte word of the re-laid form; for small backward-data passes, where a re-lay kernel in
+// front of every call costs more than the extra loads.
+template <int BM, int BN, int WM, int WN, bool BWD_DATA, bool RAW>
 __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, float *__restrict__ out,
                                                             float *__restrict__ pieces, StreamK sk) {
   static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
@@ -370,8 +377,10 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
 #pragma unroll
     for (int s = 0; s < PA; ++s) {
       const int row = min(m0 + (tid >> 2) + 64 * s, P.M - 1);
-      a_voff[s] = (static_cast<unsigned>(row) * P.K + 4u * (tid & 3)) * 4u;
+      a_voff[s] = RAW ? (static_cast<unsigned>(row) * P.raw_row + 4u * (tid & 3) * P.raw_ch) * 4u
+                      : (static_cast<unsigned>(row) * P.K + 4u * (tid & 3)) * 4u;
     }
+    const unsigned a_next = static_cast<unsigned>(P.raw_ch) * 4u;    // RAW: bytes between two channels
     // ---- gathered operand: thread -> (column tid % BN, KPT consecutive k' starting at klocal0)
     unsigned b_voff, vmask = 0;
     {
@@ -415,9 +424,20 @@ __global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, flo
 
     auto load_step = [&](int step) {
       // filter words: scalar offset = k position of the step
-      const int soff_a = step * (BK * 4);
+      if (RAW) {
+        const int soff_a = (ch0 * P.raw_ch + tap) * 4;
 #pragma unroll
-      for (int s = 0; s < PA; ++s) ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[s], soff_a, 0);
+        for (int s = 0; s < PA; ++s) {
+          ra_regs[s].x = __builtin_amdgcn_raw_buffer_load_b32(ra, a_voff[s], soff_a, 0);
+          ra_regs[s].y = __builtin_amdgcn_raw_buffer_load_b32(ra, a_voff[s] + a_next, soff_a, 0);
+          ra_regs[s].z = __builtin_amdgcn_raw_buffer_load_b32(ra, a_voff[s] + 2u * a_next, soff_a, 0);
+          ra_regs[s].w = __builtin_amdgcn_raw_buffer_load_b32(ra, a_voff[s] + 3u * a_next, soff_a, 0);
+        }
+      } else {
+        const int soff_a = step * (BK * 4);
+#pragma unroll
+        for (int s = 0; s < PA; ++s) ra_regs[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[s], soff_a, 0);
+      }
       // gathered values: scalar offset = channel block + tap displacement
       const int kh = tap / P.kW, kw = tap - kh * P.kW;
       const int disp = BWD_DATA ? bias - (kh * P.src_w + kw) : kh * P.src_w + kw;
@@ -1347,7 +1367,7 @@ __global__ __launch_bounds__(256) void filter_phase_tap_major_kernel(const float
   out[idx] = w[((o * C + c) * kH + (a + s * u)) * kW + (b + s * v)];
 }
 
-template <int BM, int BN, int WM, int WN, bool BWD_DATA>
+template <int BM, int BN, int WM, int WN, bool BWD_DATA, bool RAW = false>
 int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, float *out, hipStream_t st,
                     const TapPhase *phase = nullptr) {
   TapConvParams P;
@@ -1401,6 +1421,8 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
     P.out_b0 = phase->b0;
   }
   P.wf = w_relaid;
+  P.raw_row = BWD_DATA ? taps : g.C * taps;      // (only read by the RAW kernels; never with stride phases)
+  P.raw_ch = BWD_DATA ? g.C * taps : taps;
   P.src = src;
   P.wf_bytes = static_cast<unsigned>(static_cast<int64_t>(P.M) * P.K * 4);
   P.taps = taps;
@@ -1410,7 +1432,7 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
   sk.ksteps = P.K / BK;
   sk.total = tn * sk.ksteps;
   sk.tm = tm;
-  static const int occ = blocks_per_cu(conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>);
+  static const int occ = blocks_per_cu(conv_tap_kernel<BM, BN, WM, WN, BWD_DATA, RAW>);
   const int slots = 256 * occ;
   unsigned grid;
   float *pieces = nullptr;
@@ -1443,8 +1465,8 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
       TS_REQUIRE(pieces, "conv: no scratch memory for the pieces of cut tiles");
     }
   }
-  hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA>), dim3(grid), dim3(kThreads), 0, st, P, out, pieces,
-                     sk);
+  hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA, RAW>), dim3(grid), dim3(kThreads), 0, st, P, out,
+                     pieces, sk);
   if (pieces)
     hipLaunchKernelGGL((conv_tap_assemble_kernel<BM, BN, WM, WN>), dim3(cut_tiles * 4), dim3(kThreads), 0, st, P, out,
                        pieces, sk);
@@ -1521,6 +1543,17 @@ inline int tap_kernel_images(const ConvGeo &g, int64_t src_elems_per_img, int64_
   if (fit >= g.imgs) return g.imgs;
   const int64_t launches = (g.imgs + fit - 1) / fit;          // equal runs rather than a short last one
   return static_cast<int>((g.imgs + launches - 1) / launches);
+}
+
+// Small backward-data passes read the filter where it lies instead of re-laying it first (RAW
+// kernels): in that pass neighbouring rows of the operand are neighbours in memory (4*taps bytes
+// apart), so the four 4-byte loads cost less than a re-lay kernel in front of every call.  The
+// forward pass reads rows C*taps apart with taps between the words of a row and loses more than
+// the re-lay costs (measured), so it keeps it.
+// TSPLIT_CONV_RAW=0 / 1 forces the choice (tests run both kernels on the same shapes).
+inline bool raw_filter_pays(const ConvGeo &g) {
+  if (const char *e = std::getenv("TSPLIT_CONV_RAW")) return e[0] == '1';
+  return 2.0 * g.imgs * g.O * g.oH * g.oW * g.C * g.kH * g.kW < 12e9;
 }
 
 // Runs f(geometry of the run, first image) over runs of `per` images.
@@ -1965,6 +1998,8 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
     } else if (g.C % BK == 0) {
       // a 1x1 filter [O][C] already is tap-major: used where it lies
       const float *wf = cf(w);
+      const int64_t x_img = static_cast<int64_t>(g.C) * g.H * g.W, y_img = static_cast<int64_t>(g.O) * g.oH * g.oW;
+      const int per = tap_kernel_images(g, x_img, numel(w));
       if (g.kH * g.kW != 1 || !aligned16(wf)) {
         float *relaid = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(numel(w)) * 4));
         TS_REQUIRE(relaid, "%s: no scratch memory", who);
@@ -1973,11 +2008,12 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
                            g.C, g.kH * g.kW, false);
         wf = relaid;
       }
-      const int64_t x_img = static_cast<int64_t>(g.C) * g.H * g.W, y_img = static_cast<int64_t>(g.O) * g.oH * g.oW;
-      if (const int per = tap_kernel_images(g, x_img, numel(w))) {
+      if (per) {
         const int rc = for_image_runs(g, per, [&](const ConvGeo &run, int64_t first) {
-          return g.O <= 64 ? launch_conv_tap<64, 256, 1, 4, false>(run, cf(x) + first * x_img, wf, mf(y) + first * y_img, st)
-                           : launch_conv_tap<128, 128, 2, 2, false>(run, cf(x) + first * x_img, wf, mf(y) + first * y_img, st);
+          const float *xr = cf(x) + first * x_img;
+          float *yr = mf(y) + first * y_img;
+          return g.O <= 64 ? launch_conv_tap<64, 256, 1, 4, false>(run, xr, wf, yr, st)
+                           : launch_conv_tap<128, 128, 2, 2, false>(run, xr, wf, yr, st);
         });
         if (rc) return rc;
       } else if (g.O <= 64) {
@@ -2010,13 +2046,19 @@ int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray 
     const int64_t dy_img = static_cast<int64_t>(g.O) * g.oH * g.oW, dx_img = static_cast<int64_t>(g.C) * g.H * g.W;
     const int per = tap_kernel_images(g, dy_img, numel(w));
     if (g.s == 1 && g.O % BK == 0) {
-      hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
-                         g.kH * g.kW, true);
+      const bool raw = per && raw_filter_pays(g);
+      if (!raw)
+        hipLaunchKernelGGL(filter_tap_major_kernel, dim3((total + 255) / 256), dim3(256), 0, st, cf(w), wt, g.O, g.C,
+                           g.kH * g.kW, true);
       if (per) {
         const int rc = for_image_runs(g, per, [&](const ConvGeo &run, int64_t first) {
-          return g.C <= 64
-                     ? launch_conv_tap<64, 256, 1, 4, true>(run, cf(dy) + first * dy_img, wt, mf(dx) + first * dx_img, st)
-                     : launch_conv_tap<128, 128, 2, 2, true>(run, cf(dy) + first * dy_img, wt, mf(dx) + first * dx_img, st);
+          const float *dyr = cf(dy) + first * dy_img;
+          float *dxr = mf(dx) + first * dx_img;
+          if (raw)
+            return g.C <= 64 ? launch_conv_tap<64, 256, 1, 4, true, true>(run, dyr, cf(w), dxr, st)
+                             : launch_conv_tap<128, 128, 2, 2, true, true>(run, dyr, cf(w), dxr, st);
+          return g.C <= 64 ? launch_conv_tap<64, 256, 1, 4, true>(run, dyr, wt, dxr, st)
+                           : launch_conv_tap<128, 128, 2, 2, true>(run, dyr, wt, dxr, st);
         });
         if (rc) return rc;
       } else if (g.C <= 64) {
