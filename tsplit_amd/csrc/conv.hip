@@ -1577,7 +1577,13 @@ inline int wgrad_tap_span_images(const ConvGeo &g) {
   return static_cast<int>(std::min<int64_t>(room / img_bytes, 1 << 20));
 }
 
-// bwd-filter on conv_wgrad_tap_kernel ("same" stride-1 convolutions)
+template <int BM, int BN, int WM, int WN, bool TAIL, bool GEN>
+int wgrad_tap_occupancy() {
+  static const int occ = blocks_per_cu(conv_wgrad_tap_kernel<BM, BN, WM, WN, TAIL, GEN>);
+  return occ;
+}
+
+// bwd-filter on conv_wgrad_tap_kernel
 template <int BM, int BN, int WM, int WN>
 int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *dw, hipStream_t st, int64_t *ws_elems) {
   const bool gen = !(g.s == 1 && g.oH == g.H && g.oW == g.W);
@@ -1605,7 +1611,11 @@ int launch_wgrad_tap(const ConvGeo &g, const float *x, const float *dy, float *d
   const bool tail = P.HWp != P.HW;
   const int tm = (P.M + BM - 1) / BM, tn = (P.N + BN - 1) / BN;
   int S;
-  static const int occ = blocks_per_cu(conv_wgrad_tap_kernel<BM, BN, WM, WN, false, false>);
+  // resident blocks per CU of the variant that will run (the padded-tail and general-geometry
+  // variants need a few more registers and may fit one block fewer): the K split aims at exactly
+  // one full wave of resident blocks
+  const int occ = gen ? (tail ? wgrad_tap_occupancy<BM, BN, WM, WN, true, true>() : wgrad_tap_occupancy<BM, BN, WM, WN, false, true>())
+                      : (tail ? wgrad_tap_occupancy<BM, BN, WM, WN, true, false>() : wgrad_tap_occupancy<BM, BN, WM, WN, false, false>());
   plan_splitk(tm * tn, P.K, 1024, occ, S, P.kchunk);
   // the images one split touches must lie within 2 GiB in both tensors: shorten the splits until they do
   const int span = wgrad_tap_span_images(g);
