@@ -593,7 +593,7 @@ struct TapWgradParams {
 // read as zeros (a compare per operand and step, three selects per dy word).  When H*W is not a
 // multiple of 4 either, the 16-byte dy words start on 4-byte boundaries.
 template <int BM, int BN, int WM, int WN, bool TAIL, bool GEN>
-__global__ __launch_bounds__(kThreads) void conv_wgrad_tap_kernel(TapWgradParams P, float *__restrict__ part,
+__global__ __launch_bounds__(kThreads, (BM == 128 ? 4 : 1)) void conv_wgrad_tap_kernel(TapWgradParams P, float *__restrict__ part,
                                                                   TileGrid tg) {
   static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
   using ALds = MnMajorLds<BM>;
