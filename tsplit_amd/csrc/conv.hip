@@ -326,9 +326,13 @@ struct StreamK {
 // RAW: the filter operand is read from the [O][C][taps] filter itself with four 4-byte loads per
 // 16-byte word of the re-laid form; for small backward-data passes, where a re-lay kernel in
 // front of every call costs more than the extra loads.
-template <int BM, int BN, int WM, int WN, bool BWD_DATA, bool RAW>
-__global__ __launch_bounds__(kThreads) void conv_tap_kernel(TapConvParams P, float *__restrict__ out,
-                                                            float *__restrict__ pieces, StreamK sk) {
+// MINB: resident blocks per CU the register budget is cut for.  2 leaves every value in registers;
+// 3 spills a dozen set-up values but keeps a third block resident, which pays on layers with
+// thousands of tiles (+1-4 % on the VGG layers) and costs on small ones (finer pieces, -1-3 % on
+// the ResNet-50 / Inception-v4 steps), so the launcher picks by tile count.
+template <int BM, int BN, int WM, int WN, bool BWD_DATA, bool RAW, int MINB>
+__global__ __launch_bounds__(kThreads, MINB) void conv_tap_kernel(TapConvParams P, float *__restrict__ out,
+                                                               float *__restrict__ pieces, StreamK sk) {
   static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
   using ALds = MnMajorLds<BM>;
   using BLds = MnMajorLds<BN>;
@@ -1367,6 +1371,8 @@ __global__ __launch_bounds__(256) void filter_phase_tap_major_kernel(const float
   out[idx] = w[((o * C + c) * kH + (a + s * u)) * kW + (b + s * v)];
 }
 
+constexpr int kManyTiles = 1024;
+
 template <int BM, int BN, int WM, int WN, bool BWD_DATA, bool RAW = false>
 int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, float *out, hipStream_t st,
                     const TapPhase *phase = nullptr) {
@@ -1432,8 +1438,11 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
   sk.ksteps = P.K / BK;
   sk.total = tn * sk.ksteps;
   sk.tm = tm;
-  static const int occ = blocks_per_cu(conv_tap_kernel<BM, BN, WM, WN, BWD_DATA, RAW>);
-  const int slots = 256 * occ;
+  // many tiles: the variant with three resident blocks per CU (never with RAW, which is for small layers)
+  const bool many = !RAW && tiles >= kManyTiles;
+  static const int occ2 = blocks_per_cu(conv_tap_kernel<BM, BN, WM, WN, BWD_DATA, RAW, 2>);
+  static const int occ3 = RAW ? occ2 : blocks_per_cu(conv_tap_kernel<BM, BN, WM, WN, BWD_DATA, false, 3>);
+  const int slots = 256 * (many ? occ3 : occ2);
   unsigned grid;
   float *pieces = nullptr;
   sk.whole_waves = 0;
@@ -1465,8 +1474,12 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
       TS_REQUIRE(pieces, "conv: no scratch memory for the pieces of cut tiles");
     }
   }
-  hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA, RAW>), dim3(grid), dim3(kThreads), 0, st, P, out,
-                     pieces, sk);
+  if (many)
+    hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA, false, 3>), dim3(grid), dim3(kThreads), 0, st, P, out,
+                       pieces, sk);
+  else
+    hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, BWD_DATA, RAW, 2>), dim3(grid), dim3(kThreads), 0, st, P, out,
+                       pieces, sk);
   if (pieces)
     hipLaunchKernelGGL((conv_tap_assemble_kernel<BM, BN, WM, WN>), dim3(cut_tiles * 4), dim3(kThreads), 0, st, P, out,
                        pieces, sk);
