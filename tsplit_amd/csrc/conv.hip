@@ -2141,7 +2141,7 @@ int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArra
     if (wgrad_narrow_ok(g)) {
       rc = launch_wgrad_narrow(g, cf(x), cf(dy), mf(dw), st, &ws);
     } else if (wgrad_tap_ok(g)) {
-      if (g.O <= 64)
+      if (short_tiles(g.O))
         rc = launch_wgrad_tap<64, 256, 1, 4>(g, cf(x), cf(dy), mf(dw), st, &ws);
       else
         rc = launch_wgrad_tap<128, 128, 2, 2>(g, cf(x), cf(dy), mf(dw), st, &ws);
