@@ -32,11 +32,12 @@ PEAK_TFLOPS_FP32_MFMA = 157.3
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch (read + write, mean over the launches of one step) of the kernels that can
 # be the step's largest, from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
-# profiles/vgg16_b64_train_step_hbm_traffic.txt (counter units calibrated on the Relu kernel).
+# profiles/vgg16_b64_train_step_hbm_traffic.txt (counter units calibrated on the Relu kernel; forward and
+# backward-data run as two register-budget variants of one kernel, averaged here over both by launch count).
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "conv_fwd_128x128": (324.4 + 137.5) * 1e6,
-    "conv_bwd_data_128x128": (440.2 + 129.5) * 1e6,
-    "conv_bwd_filter_128x128": (555.1 + 64.2) * 1e6,
+    "conv_fwd_128x128": (388.2 + 158.1) * 1e6,
+    "conv_bwd_data_128x128": (523.5 + 147.5) * 1e6,
+    "conv_bwd_filter_128x128": (523.2 + 64.2) * 1e6,
 }
 
 
