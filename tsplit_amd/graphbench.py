@@ -1,7 +1,7 @@
 """Times one training step (forward, backward, SGD) of the branched example networks at the
 sizes of the reference's benchmark configurations, on one MI355X through the C ABI.
 
-    python -m tsplit_amd.graphbench --net resnet50|inception_v4|transformer|lstm|mlp [--steps 5] [--warmup 2] [--record]
+    python -m tsplit_amd.graphbench --net resnet50|resnet101|inception_v4|transformer|lstm|mlp|vgg19 [--steps 5] [--warmup 2] [--record]
 
 --record issues the step once into a HIP graph after the warm-up and times replays of that graph
 (one host call per step) instead of Python issuing every operator again.
@@ -19,7 +19,7 @@ import numpy as np
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--net", default="resnet50", choices=["resnet50", "inception_v4", "transformer", "lstm", "mlp"])
+    ap.add_argument("--net", default="resnet50", choices=["resnet50", "resnet101", "inception_v4", "transformer", "lstm", "mlp", "vgg19"])
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--batch", type=int, default=0)
@@ -28,24 +28,25 @@ def main():
     a = ap.parse_args()
     from . import graph, ndarray, stream, workloads
     ctx = ndarray.gpu(0)
-    if a.net == "mlp":
-        return mlp(a, ctx)
+    if a.net in ("mlp", "vgg19"):
+        return layer_list(a, ctx)
     st = stream.create_stream_handle(ctx)
     backend = graph.GpuBackend(ctx, st)
     rng = np.random.RandomState(123)
     store = workloads.ParamStore(123)
     calls = [0]
 
-    if a.net == "resnet50":
+    if a.net in ("resnet50", "resnet101"):
         n = a.batch or 64
+        stages = (3, 4, 6, 3) if a.net == "resnet50" else (3, 4, 23, 3)
         x = rng.standard_normal((n, 3, 224, 224)).astype(np.float32)
         y = np.zeros((n, 1000), np.float32)
         y[np.arange(n), rng.randint(0, 1000, n)] = 1
 
         def build(t, b, cache):
-            return workloads.resnet(t, b, cache["x"], cache["y"])
+            return workloads.resnet(t, b, cache["x"], cache["y"], blocks=stages)
         inputs = {"x": x, "y": y}
-        desc = "ResNet-50, fp32 NCHW, batch %d, 3x224x224, 1000 classes" % n
+        desc = "ResNet-%s, fp32 NCHW, batch %d, 3x224x224, 1000 classes" % (a.net[6:], n)
     elif a.net == "inception_v4":
         n = a.batch or 32
         x = rng.standard_normal((n, 3, 299, 299)).astype(np.float32)
@@ -124,18 +125,26 @@ def main():
                       "dtype": "f32", "data": "synthetic"}))
 
 
-def mlp(a, ctx):
-    """The 784-256-256-10 MLP of the smallest benchmark configuration (batch 128, SGD 0.1) on the
-    layer-list trainer: 13 launches per step, so the step is the host's launch rate unless recorded."""
+def layer_list(a, ctx):
+    """Nets that are plain layer lists, on the layer-list trainer: the 784-256-256-10 MLP of the smallest
+    benchmark configuration (batch 128, SGD 0.1; 13 launches per step, so the step is the host's launch
+    rate unless recorded) and VGG-19 (batch 64, momentum SGD, as bench.py runs VGG-16)."""
     from . import ndarray, trainer
-    n = a.batch or 128
     rng = np.random.RandomState(123)
-    spec = trainer.mlp_spec()
+    if a.net == "mlp":
+        n, classes = a.batch or 128, 10
+        spec, opt = trainer.mlp_spec(), ("sgd", 0.1)
+        x = rng.uniform(0, 1, size=(n, 784)).astype(np.float32)
+        desc = "MLP 784-256-256-10, batch %d, SGD" % n
+    else:
+        n, classes = a.batch or 64, 1000
+        spec, opt = trainer.vgg19_spec(1000, 224), ("momentum", 1e-4, 0.9)
+        x = rng.standard_normal(size=(n, 3, 224, 224)).astype(np.float32)
+        desc = "VGG-19, fp32 NCHW, batch %d, 3x224x224, 1000 classes, momentum SGD" % n
     params = trainer.init_params(spec, seed=123)
-    x = rng.uniform(0, 1, size=(n, 784)).astype(np.float32)
-    y = np.zeros((n, 10), np.float32)
-    y[np.arange(n), rng.randint(0, 10, n)] = 1
-    t = trainer.Trainer(spec, params, x.shape, 10, ctx, optimizer=("sgd", 0.1))
+    y = np.zeros((n, classes), np.float32)
+    y[np.arange(n), rng.randint(0, classes, n)] = 1
+    t = trainer.Trainer(spec, params, x.shape, classes, ctx, optimizer=opt)
     gx, gy = ndarray.array(x, ctx), ndarray.array(y, ctx)
     for _ in range(max(1, a.warmup)):
         t.step(gx, gy)
@@ -154,7 +163,7 @@ def mlp(a, ctx):
             t.step(gx, gy)
     t.sync()
     dt = time.perf_counter() - t0
-    print(json.dumps({"net": "mlp", "workload": "MLP 784-256-256-10, batch %d, SGD" % n, "samples_per_s": n * steps / dt,
+    print(json.dumps({"net": a.net, "workload": desc, "samples_per_s": n * steps / dt,
                       "ms_per_step": dt / steps * 1e3, "steps": steps, "warmup": a.warmup, "final_loss": t.loss_value(),
                       "recorded": bool(a.record), "dtype": "f32", "data": "synthetic"}))
 

@@ -38,12 +38,21 @@ def mlp_spec(sizes=(784, 256, 256, 10)):
 
 
 def vgg16_spec(num_classes=1000, in_hw=224):
-    """VGG-16 as examples/imagenet_vgg.py:24-98 builds it: 13 x (conv3x3 pad 1, BN, Relu),
-    5 max-pools 2x2/2, flatten, three bias-free fully connected layers with no activation
+    return vgg_spec(16, num_classes, in_hw)
+
+
+def vgg19_spec(num_classes=1000, in_hw=224):
+    return vgg_spec(19, num_classes, in_hw)
+
+
+def vgg_spec(depth=16, num_classes=1000, in_hw=224):
+    """VGG-16 / VGG-19 as examples/imagenet_vgg.py:24-98 builds them: 13 or 16 x (conv3x3 pad 1, BN,
+    Relu), 5 max-pools 2x2/2, flatten, three bias-free fully connected layers with no activation
     in between."""
+    per_block = {16: (2, 2, 3, 3, 3), 19: (2, 2, 4, 4, 4)}[depth]
     spec = []
     cin = 3
-    for bi, (n, cout) in enumerate([(2, 64), (2, 128), (3, 256), (3, 512), (3, 512)], 1):
+    for bi, (n, cout) in enumerate(zip(per_block, (64, 128, 256, 512, 512)), 1):
         for li in range(1, n + 1):
             name = "vgg_block%d_layer%d" % (bi, li)
             spec += [("conv", name, cin, cout, 3, 1, 1), ("bn", name + "_bn", cout), ("relu",)]
