@@ -104,3 +104,28 @@ def test_copy_ins_start_early_where_the_budget_allows_and_keep_the_order_of_need
     cost = planner.CostModel()
     assert planner.step_ms(spec, shapes, p.swap, cost, p.prefetch, p.issue_at) <= \
         planner.step_ms(spec, shapes, p.swap, cost, p.prefetch)
+
+
+def test_max_batch_grows_with_the_budget_and_with_planning():
+    """The largest batch under a budget: never smaller with a bigger budget, larger with planning than
+    with everything resident, its plan replays within the budget, and one image more does not fit."""
+    from tsplit_amd import planner, trainer
+    from tsplit_amd.planned_trainer import fixed_bytes, make_plan, max_batch
+    spec = trainer.vgg16_spec(10, 32)
+    opt = ("momentum", 0.01, 0.9)
+    image = (3, 32, 32)
+    last = (0, 0)
+    for mib in (600, 800, 1200):
+        budget = mib << 20
+        resident, _ = max_batch(spec, image, 10, budget, opt, swap=False)
+        planned, plan = max_batch(spec, image, 10, budget, opt, swap=True)
+        assert planned > resident > 0
+        assert resident >= last[0] and planned >= last[1]
+        last = (resident, planned)
+        shapes = planner.layer_shapes(spec, (planned,) + image)
+        peak, _ = planner.simulate(spec, shapes, plan.swap, fixed_bytes(spec, (planned,) + image, 10, opt, tuple(plan.split)))
+        assert peak <= budget
+        with pytest.raises(ValueError):
+            make_plan(spec, (planned + 1,) + image, 10, budget, opt)
+        free = make_plan(spec, (resident + 1,) + image, 10, None, opt)
+        assert free.peak_bytes > budget

@@ -56,6 +56,46 @@ def make_plan(spec, input_shape, num_classes, budget_bytes, optimizer=("sgd", 0.
     return plan
 
 
+def max_batch(spec, image_shape, num_classes, budget_bytes, optimizer=("sgd", 0.1), swap=True, limit=1 << 14):
+    """Largest batch of `image_shape` (C, H, W) images that trains within `budget_bytes`: with `swap`
+    the planner may send activations to host memory and split layers, without it everything stays on
+    the device (the budget must then hold the unplanned peak).  The counterpart of the reference's
+    batch-size sweeps, which raise the batch until a policy runs out of memory
+    (examples/imagenet_vgg.py:168-178).  Tensors are limited to 2^31 elements, as in the library.
+    -> (batch, plan); (0, None) if not even one image fits."""
+    from .planner import layer_shapes
+
+    def plan_for(batch):
+        shape = (batch,) + tuple(image_shape)
+        if any(int(np.prod(s)) >= (1 << 31) for s in layer_shapes(spec, shape)):
+            return None
+        try:
+            if swap:
+                return make_plan(spec, shape, num_classes, budget_bytes, optimizer)
+            plan = make_plan(spec, shape, num_classes, None, optimizer)
+            return plan if plan.peak_bytes <= budget_bytes else None
+        except ValueError:
+            return None
+
+    best, best_plan = 0, None
+    hi = 1
+    while hi <= limit:                 # double until it no longer fits
+        plan = plan_for(hi)
+        if plan is None:
+            break
+        best, best_plan = hi, plan
+        hi *= 2
+    lo, hi = best, min(hi, limit + 1)  # fits at lo (or lo == 0), not at hi
+    while hi - lo > 1:
+        mid = (lo + hi) // 2
+        plan = plan_for(mid)
+        if plan is None:
+            hi = mid
+        else:
+            lo, best, best_plan = mid, mid, plan
+    return best, best_plan
+
+
 class PlannedTrainer(object):
     def __init__(self, spec, params, input_shape, num_classes, plan, ctx=None, optimizer=("sgd", 0.1), bn_eps=0.01):
         self.spec = list(spec)
