@@ -37,7 +37,7 @@ def _plain_losses(spec_fused, steps, rng_seed=5):
     return out, {k: v.asnumpy() for k, v in t.params.items()}
 
 
-def _planned(spec, budget_frac, steps, piece_bytes=64 << 10, rng_seed=5):
+def _planned(spec, budget_frac, steps, piece_bytes=64 << 10, rng_seed=5, allow_recompute=False):
     from tsplit_amd import ndarray
     from tsplit_amd.planned_trainer import PlannedTrainer, make_plan
     rng = np.random.RandomState(rng_seed)
@@ -48,7 +48,7 @@ def _planned(spec, budget_frac, steps, piece_bytes=64 << 10, rng_seed=5):
         shapes = planner.layer_shapes(spec, IN)
         floor, _ = planner.simulate(spec, shapes, range(1, len(spec)), free.fixed_bytes)
         budget = int(floor + budget_frac * (free.peak_bytes - floor))
-    plan = make_plan(spec, IN, 10, budget, OPT, piece_bytes=piece_bytes)
+    plan = make_plan(spec, IN, 10, budget, OPT, piece_bytes=piece_bytes, allow_recompute=allow_recompute)
     t = PlannedTrainer(spec, params, IN, 10, plan, optimizer=OPT)
     x, labels = _data(rng)
     gx, gl = ndarray.array(x, t.ctx), ndarray.array(labels, t.ctx)
@@ -98,3 +98,28 @@ def test_impossible_budget_is_refused():
     from tsplit_amd.planned_trainer import make_plan
     with pytest.raises(ValueError, match="cannot be met"):
         make_plan(SPEC, IN, 10, 64 << 10, OPT)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("frac", [0.6, 0.3, 0.1])
+def test_recomputation_meets_the_budget_with_the_same_bits(fused, frac):
+    """With recomputation allowed the plan drops BatchNorm / Relu outputs and computes them again in the
+    backward sweep; computing a tensor again gives the bits it had, so the results equal the plain
+    trainer's exactly wherever no convolution is split, and the executor's peak is the replayed one."""
+    spec = planner.fuse_spec(SPEC) if fused else SPEC
+    want, wp = _plain_losses(fused, 4)
+    got, gp, t, plan, free = _planned(spec, frac, 4, allow_recompute=True)
+    assert plan.recompute and plan.budget_bytes < free.peak_bytes
+    assert all(spec[j - 1][0] in planner.CHEAP_TO_REDO for j in plan.recompute)
+    assert t.peak <= plan.budget_bytes and not t.dropped
+    np.testing.assert_allclose(got, want, rtol=2e-5)
+    for k in wp:
+        np.testing.assert_allclose(gp[k], wp[k], rtol=1e-4, atol=2e-5, err_msg=k)
+    if not plan.split:
+        assert got == want
+        for k in wp:
+            assert np.array_equal(gp[k], wp[k]), k
+    # the plan is at least as fast, by the cost model, as the one that may only swap
+    from tsplit_amd.planned_trainer import make_plan
+    swap_only = make_plan(spec, IN, 10, plan.budget_bytes, OPT, piece_bytes=64 << 10)
+    assert plan.est_step_ms <= swap_only.est_step_ms + 1e-9

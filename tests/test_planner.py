@@ -129,3 +129,45 @@ def test_max_batch_grows_with_the_budget_and_with_planning():
             make_plan(spec, (planned + 1,) + image, 10, budget, opt)
         free = make_plan(spec, (resident + 1,) + image, 10, None, opt)
         assert free.peak_bytes > budget
+
+
+def test_recomputation_replay_and_choice():
+    """Dropped tensors leave after their forward use and are back, with the tensor they are computed
+    from, when their layer's backward runs; chains (Relu output from BatchNorm output from the kept
+    convolution output) replay in order; a tensor something is recomputed from is never swapped; the
+    estimated step never gets slower by allowing recomputation."""
+    from tsplit_amd import planner, trainer
+    from tsplit_amd.planned_trainer import fixed_bytes, make_plan
+    spec = trainer.vgg16_spec(10, 32)
+    shape = (64, 3, 32, 32)
+    opt = ("momentum", 0.01, 0.9)
+    shapes = planner.layer_shapes(spec, shape)
+    size = planner.tensor_bytes(shapes)
+    # hand-made: drop BN output (tensor 2) and Relu output (tensor 3) of the first block
+    peak0, _ = planner.simulate(spec, shapes)
+    peak, events = planner.simulate(spec, shapes, recompute=(2, 3))
+    assert peak <= peak0
+    fwd = {li: res for ph, li, _, res, _ in events if ph == "fwd"}
+    assert 2 in fwd[2] and 2 not in fwd[3] and 3 in fwd[3] and 3 not in fwd[4]
+    redone = [(li, res) for ph, li, _, res, _ in events if ph == "re"]
+    assert [li for li, _ in redone] == [2, 3]                  # the chain is rebuilt front to back
+    assert {1, 2} <= redone[0][1] and {2, 3} <= redone[1][1]
+    bwd = {li: res for ph, li, _, res, _ in events if ph == "bwd"}
+    assert {3, 4} <= bwd[3] and {2, 3} <= bwd[2] and 3 not in bwd[1]
+    free = make_plan(spec, shape, 10, None, opt)
+    floor = planner.simulate(spec, shapes, range(1, len(spec)), free.fixed_bytes)[0]
+    for frac in (0.7, 0.4, 0.15):
+        budget = int(floor + frac * (free.peak_bytes - floor))
+        both = make_plan(spec, shape, 10, budget, opt, allow_recompute=True)
+        swap_only = make_plan(spec, shape, 10, budget, opt)
+        assert both.recompute and both.peak_bytes <= budget
+        assert both.est_step_ms <= swap_only.est_step_ms + 1e-9
+        for j in both.recompute:
+            assert spec[j - 1][0] in planner.CHEAP_TO_REDO
+            k = j - 1
+            while k in both.recompute:
+                k -= 1
+            assert k not in both.swap
+        again = planner.simulate(spec, shapes, both.swap, fixed_bytes(spec, shape, 10, opt, tuple(both.split)),
+                                 issue_at=both.issue_at, recompute=both.recompute)[0]
+        assert again == both.peak_bytes

@@ -56,7 +56,8 @@ def make_plan(spec, input_shape, num_classes, budget_bytes, optimizer=("sgd", 0.
     return plan
 
 
-def max_batch(spec, image_shape, num_classes, budget_bytes, optimizer=("sgd", 0.1), swap=True, limit=1 << 14):
+def max_batch(spec, image_shape, num_classes, budget_bytes, optimizer=("sgd", 0.1), swap=True, limit=1 << 14,
+              allow_recompute=False):
     """Largest batch of `image_shape` (C, H, W) images that trains within `budget_bytes`: with `swap`
     the planner may send activations to host memory and split layers, without it everything stays on
     the device (the budget must then hold the unplanned peak).  The counterpart of the reference's
@@ -71,7 +72,7 @@ def max_batch(spec, image_shape, num_classes, budget_bytes, optimizer=("sgd", 0.
             return None
         try:
             if swap:
-                return make_plan(spec, shape, num_classes, budget_bytes, optimizer)
+                return make_plan(spec, shape, num_classes, budget_bytes, optimizer, allow_recompute=allow_recompute)
             plan = make_plan(spec, shape, num_classes, None, optimizer)
             return plan if plan.peak_bytes <= budget_bytes else None
         except ValueError:
@@ -138,6 +139,7 @@ class PlannedTrainer(object):
         self.acts = [None] * (self.nl + 1)
         self.in_events = {}                    # tensor -> list of per-piece copy-in events
         self.away = set()                      # tensors whose device copy is released
+        self.dropped = set()                   # tensors dropped after their forward use, to be computed again
 
     # ------------------------------------------------------------------ memory accounting
     @staticmethod
@@ -269,9 +271,36 @@ class PlannedTrainer(object):
                 copied = self._swap_out(li, produced)
                 self._release(a, [copied], keep_struct=True)
                 self.away.add(li)
+            elif li in self.plan.recompute:
+                self._release(a, [after])      # gone once this layer, its only reader, has run
+                self.acts[li] = None
+                self.dropped.add(li)
             produced = after
         L.softmax_cross_entropy(self.acts[-1], labels, self.loss, self.stream)
         return self.loss
+
+    def _redo(self, j):
+        """Computes dropped tensor j again from tensor j - 1 (itself computed again first if it was
+        dropped too): the forward call of layer j - 1, which gives the same bits as the first time."""
+        if j not in self.dropped:
+            return
+        self._redo(j - 1)
+        src, layer = self.acts[j - 1], self.spec[j - 1]
+        out = self.acts[j] = self._alloc(self.shapes[j])
+        kind = layer[0]
+        if kind == "bnrelu":
+            sm, sv = self.saved[j - 1]
+            L.batch_norm_relu(src, self.params[layer[1] + "_scale"], self.params[layer[1] + "_bias"], out, sm, sv,
+                              self.eps, self.stream)
+        elif kind == "bn":
+            sm, sv = self.saved[j - 1]
+            L.CuDNN_Batch_Normalization(src, self.params[layer[1] + "_scale"], self.params[layer[1] + "_bias"], out,
+                                        sm, sv, 0.99, self.eps, self.stream)
+        elif kind == "relu":
+            L.relu(src, out, self.stream)
+        else:
+            raise ValueError("layer %d (%s) is not one the plan may compute again" % (j - 1, kind))
+        self.dropped.discard(j)
 
     # ------------------------------------------------------------------ backward
     def backward(self, labels):
@@ -286,6 +315,7 @@ class PlannedTrainer(object):
             for j in sorted(self.away, reverse=True):
                 if self.plan.issue_at.get(j, j) >= li or j >= li:
                     self._swap_in(j)
+            self._redo(li)
             a, y = self.acts[li], self.acts[li + 1]
             first = li == 0
             in_place = kind in IN_PLACE_BACKWARD

@@ -75,12 +75,18 @@ class CostModel(object):
 
 
 IN_PLACE_BACKWARD = ("relu", "bn", "bnrelu")   # the input gradient may overwrite the output gradient
+# layers whose output is cheap to compute again from their input (two or three passes over HBM):
+# such an output may be dropped after its forward use and recomputed when the backward sweep needs it
+CHEAP_TO_REDO = ("relu", "bn", "bnrelu")
 
 
 class MemoryPlan(object):
     def __init__(self, swap, split, peak_bytes, est_step_ms, est_free_step_ms, fixed_bytes, budget_bytes, prefetch,
-                 issue_at=None):
+                 issue_at=None, recompute=()):
         self.swap = frozenset(swap)          # tensor indices that leave the device after their forward use
+        # tensor indices dropped after their forward use and computed again, from the tensor before,
+        # when the backward sweep reaches them
+        self.recompute = frozenset(recompute)
         self.split = dict(split)             # layer index -> batch micro-tensors
         self.prefetch = prefetch             # least lead, in layers, of a copy-in over the backward sweep
         # tensor -> backward layer at whose start its copy-in is issued
@@ -92,7 +98,7 @@ class MemoryPlan(object):
         self.budget_bytes = budget_bytes
 
     def describe(self):
-        return {"swap": sorted(self.swap), "split": {int(k): int(v) for k, v in sorted(self.split.items())},
+        return {"swap": sorted(self.swap), "recompute": sorted(self.recompute), "split": {int(k): int(v) for k, v in sorted(self.split.items())},
                 "prefetch": self.prefetch, "issue_at": {int(k): int(v) for k, v in sorted(self.issue_at.items())},
                 "peak_GiB": self.peak_bytes / GiB, "est_step_ms": self.est_step_ms,
                 "est_free_step_ms": self.est_free_step_ms,
@@ -130,12 +136,14 @@ def default_issue_at(swap, n_layers, prefetch):
     return {j: min(n_layers - 1, j + prefetch) for j in swap}
 
 
-def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3, issue_at=None):
+def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3, issue_at=None, recompute=()):
     """Replays the executor's allocation schedule.  Returns (peak_bytes, events) where events is
-    a list of (phase, layer, resident_bytes, resident_tensor_indices, busy_tensor_indices)."""
+    a list of (phase, layer, resident_bytes, resident_tensor_indices, busy_tensor_indices); phase
+    "re" is the moment tensor `layer` has just been computed again."""
     L = len(spec)
     size = tensor_bytes(shapes)
     swap = set(swap)
+    redo = set(recompute)
     issue_at = issue_at if issue_at is not None else default_issue_at(swap, L, prefetch)
     resident = set([0])
     grad_bytes = 0
@@ -148,14 +156,25 @@ def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3, issue_at=None):
     for li in range(L):
         resident.add(li + 1)
         note("fwd", li)
-        if li in swap:
+        if li in swap or li in redo:
             resident.discard(li)
     g_out = size[L]                    # the loss gradient has the logits' size
+    grad_bytes = g_out
     for li in range(L - 1, -1, -1):
         # copy-ins issued at the start of this layer's backward (its own input at the latest)
         for j in swap:
             if 1 <= j <= li + 1 and (issue_at[j] >= li or j >= li):
                 resident.add(j)
+        # this layer's input, if it was dropped, is computed again (and what it is computed from first)
+        chain = []
+        j = li
+        while j in redo and j not in resident:
+            chain.append(j)
+            j -= 1
+        for j in reversed(chain):
+            resident.add(j)
+            events.append(("re", j, fixed_bytes + sum(size[k] for k in resident) + grad_bytes, frozenset(resident),
+                           frozenset((j - 1, j))))
         in_place = spec[li][0] in IN_PLACE_BACKWARD
         g_in = 0 if li == 0 else g_out if in_place else size[li]
         grad_bytes = g_out if (li == 0 or in_place) else g_out + g_in
@@ -167,7 +186,7 @@ def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3, issue_at=None):
     return peak, events
 
 
-def step_ms(spec, shapes, swap, cost, prefetch=3, issue_at=None):
+def step_ms(spec, shapes, swap, cost, prefetch=3, issue_at=None, recompute=()):
     """Estimated step time under the replayed schedule: one compute stream, one copy-out and one
     copy-in stream (each link direction carries one copy at a time, in issue order).  A swapped
     tensor starts leaving when its consumer starts and the sweep waits for it when that consumer
@@ -185,64 +204,100 @@ def step_ms(spec, shapes, swap, cost, prefetch=3, issue_at=None):
             t = max(t, out_free)
     issue_at = issue_at if issue_at is not None else default_issue_at(swap, L, prefetch)
     in_free, arrival = 0.0, {}
+    redo, redone = set(recompute), set()
     for li in range(L - 1, -1, -1):
         for j in sorted(swap, reverse=True):          # the tensor needed first is issued first
             if j >= 1 and j not in arrival and (issue_at[j] >= li or j >= li):
                 in_free = max(in_free, t) + cost.copy_ms(size[j])
                 arrival[j] = in_free
+        j = li
+        while j in redo and j not in redone:          # every dropped tensor is computed again once
+            t += cost.layer_ms(spec[j - 1], shapes[j - 1], shapes[j], False)
+            redone.add(j)
+            j -= 1
         t = max(t, arrival.get(li, 0.0)) + cost.layer_ms(spec[li], shapes[li], shapes[li + 1], True, first=li == 0)
     return t
 
 
-def plan_memory(spec, input_shape, budget_bytes=None, fixed_bytes=0, cost=None, piece_bytes=128 << 20, prefetch=3):
+def plan_memory(spec, input_shape, budget_bytes=None, fixed_bytes=0, cost=None, piece_bytes=128 << 20, prefetch=3,
+                allow_recompute=False):
     """-> MemoryPlan for `spec` (already fused, if fusion is wanted).  Raises ValueError when
-    even swapping every idle tensor does not fit the budget."""
+    even removing every idle tensor does not fit the budget.  With `allow_recompute` an idle
+    tensor that a BatchNorm / Relu layer produced may also be dropped and computed again in the
+    backward sweep instead of travelling to the host and back; the planner takes whichever of the
+    two adds less estimated step time per byte freed."""
     cost = cost or CostModel()
     shapes = layer_shapes(spec, input_shape)
     batch = shapes[0][0]
     size = tensor_bytes(shapes)
     L = len(spec)
-    swap = set()
-    free_ms = now_ms = step_ms(spec, shapes, swap, cost, prefetch)
+    swap, redo = set(), set()
+
+    def replay(sw, rd, issue=None):
+        return simulate(spec, shapes, sw, fixed_bytes, prefetch, issue, rd)
+
+    def est(sw, rd, issue=None):
+        return step_ms(spec, shapes, sw, cost, prefetch, issue, rd)
+
+    def may_redo(j):
+        # produced by a cheap layer, and what it is computed from stays on the device
+        if not allow_recompute or j < 1 or j >= L or spec[j - 1][0] not in CHEAP_TO_REDO:
+            return False
+        k = j - 1
+        while k in redo:
+            k -= 1
+        return k not in swap
+
+    free_ms = now_ms = est(swap, redo)
     while True:
-        peak, events = simulate(spec, shapes, swap, fixed_bytes, prefetch)
+        peak, events = replay(swap, redo)
         if budget_bytes is None or peak <= budget_bytes:
             break
-        # moments at the peak; candidates = resident, idle, not yet swapped, neither batch nor logits
+        # moments at the peak; candidates = resident, idle, still kept, neither batch nor logits
         candidates = set()
         for phase, li, total, resident, busy in events:
             if total < peak:
                 continue
-            for j in resident - busy - swap:
+            for j in resident - busy - swap - redo:
                 if j == 0 or j >= L:
                     continue
-                if phase == "bwd" and li - prefetch <= j < li:
+                if phase != "fwd" and li - prefetch <= j < li:
                     continue            # on its way back in at that moment
                 candidates.add(j)
         best = None
         for j in candidates:
-            added = step_ms(spec, shapes, swap | {j}, cost, prefetch) - now_ms
-            score = (added + 1e-3) / size[j]
-            if best is None or score < best[0]:
-                best = (score, j)
+            options = []
+            if j + 1 not in redo:       # a tensor something is recomputed from stays on the device
+                options.append(("swap", est(swap | {j}, redo)))
+            if may_redo(j):
+                options.append(("redo", est(swap, redo | {j})))
+            for how, ms in options:
+                score = (ms - now_ms + 1e-3) / size[j]
+                if best is None or score < best[0]:
+                    best = (score, j, how)
         if best is None:
-            raise ValueError("budget of %.2f GiB cannot be met: %.2f GiB are needed with every idle tensor swapped"
+            raise ValueError("budget of %.2f GiB cannot be met: %.2f GiB are needed with every idle tensor removed"
                              % (budget_bytes / GiB, peak / GiB))
-        swap.add(best[1])
-        now_ms = step_ms(spec, shapes, swap, cost, prefetch)
+        (redo if best[2] == "redo" else swap).add(best[1])
+        now_ms = est(swap, redo)
     # the last pick may have freed more than was missing: put back what the budget can hold,
     # dearest first
-    for _ in range(len(swap)):
+    for _ in range(len(swap) + len(redo)):
         gains = []
         for j in swap:
             rest = swap - {j}
-            if simulate(spec, shapes, rest, fixed_bytes, prefetch)[0] <= budget_bytes:
-                gains.append((now_ms - step_ms(spec, shapes, rest, cost, prefetch), j))
+            if replay(rest, redo)[0] <= budget_bytes:
+                gains.append((now_ms - est(rest, redo), 0, j))
+        for j in redo:
+            rest = redo - {j}
+            if replay(swap, rest)[0] <= budget_bytes:
+                gains.append((now_ms - est(swap, rest), 1, j))
         if not gains or max(gains)[0] <= 0:
             break
-        swap.discard(max(gains)[1])
-        now_ms = step_ms(spec, shapes, swap, cost, prefetch)
-        peak = simulate(spec, shapes, swap, fixed_bytes, prefetch)[0]
+        _, which, j = max(gains)
+        (redo if which else swap).discard(j)
+        now_ms = est(swap, redo)
+        peak = replay(swap, redo)[0]
     # copy-ins may start earlier than `prefetch` layers ahead where the budget has room for the
     # tensor over the whole stretch; the order of issue stays the order of need
     issue_at = default_issue_at(swap, L, prefetch)
@@ -253,17 +308,17 @@ def plan_memory(spec, input_shape, budget_bytes=None, fixed_bytes=0, cost=None, 
             for at in range(issue_at[j] + 1, bound + 1):
                 trial = dict(issue_at)
                 trial[j] = at
-                if simulate(spec, shapes, swap, fixed_bytes, prefetch, trial)[0] > budget_bytes:
+                if replay(swap, redo, trial)[0] > budget_bytes:
                     break
                 best_at = at
             issue_at[j] = best_at
             bound = best_at
-        now_ms = step_ms(spec, shapes, swap, cost, prefetch, issue_at)
-        peak = simulate(spec, shapes, swap, fixed_bytes, prefetch, issue_at)[0]
+        now_ms = est(swap, redo, issue_at)
+        peak = replay(swap, redo, issue_at)[0]
     split = {}
     for li, layer in enumerate(spec):
         if layer[0] == "conv" and li >= 1 and li in swap:
             k = int(min(batch, max(1, -(-size[li] // piece_bytes))))
             if k > 1:
                 split[li] = k
-    return MemoryPlan(swap, split, peak, now_ms, free_ms, fixed_bytes, budget_bytes, prefetch, issue_at)
+    return MemoryPlan(swap, split, peak, now_ms, free_ms, fixed_bytes, budget_bytes, prefetch, issue_at, redo)
