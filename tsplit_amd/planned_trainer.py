@@ -24,7 +24,7 @@ import numpy as np
 
 from . import gpu_links as L
 from . import ndarray
-from .planner import IN_PLACE_BACKWARD, layer_shapes
+from .planner import IN_PLACE_BACKWARD, NEEDS_OUTPUT_BACKWARD, layer_shapes
 from .stream import create_event_handle, create_stream_handle
 from .trainer import param_shapes
 
@@ -310,6 +310,11 @@ class PlannedTrainer(object):
         for li in range(self.nl - 1, -1, -1):
             layer = self.spec[li]
             kind = layer[0]
+            if kind not in NEEDS_OUTPUT_BACKWARD and self.acts[li + 1] is not None:
+                # the output was the input of the layer behind, which is through: dead before anything
+                # is allocated for this layer
+                self._release(self.acts[li + 1])
+                self.acts[li + 1] = None
             # copy-ins the plan issues at this layer, the tensor needed first first; this layer's own
             # input at the latest
             for j in sorted(self.away, reverse=True):
@@ -362,9 +367,10 @@ class PlannedTrainer(object):
                     L.matrix_multiply(a, True, g_out, False, self.grads[layer[1] + "_weight"], self.stream)
                     if not first:
                         L.matrix_multiply(g_out, False, w, True, g_in, self.stream)
-            # the layer's output and output gradient are dead now
-            self._release(y)
-            self.acts[li + 1] = None
+            # the layer's output (if still held) and output gradient are dead now
+            if y is not None:
+                self._release(y)
+                self.acts[li + 1] = None
             if not in_place or first:
                 self._release(g_out)
             g_out = g_in

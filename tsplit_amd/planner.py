@@ -75,6 +75,7 @@ class CostModel(object):
 
 
 IN_PLACE_BACKWARD = ("relu", "bn", "bnrelu")   # the input gradient may overwrite the output gradient
+NEEDS_OUTPUT_BACKWARD = ("maxpool",)           # CuDNN_DLGpuMax_Pooling2d_gradient takes y as well as x
 # layers whose output is cheap to compute again from their input (two or three passes over HBM):
 # such an output may be dropped after its forward use and recomputed when the backward sweep needs it
 CHEAP_TO_REDO = ("relu", "bn", "bnrelu")
@@ -161,6 +162,10 @@ def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3, issue_at=None, re
     g_out = size[L]                    # the loss gradient has the logits' size
     grad_bytes = g_out
     for li in range(L - 1, -1, -1):
+        # only max pooling reads its own output in the backward pass; every other layer's output is dead
+        # as soon as the layer behind it has been through, before anything is allocated for this one
+        if spec[li][0] not in NEEDS_OUTPUT_BACKWARD:
+            resident.discard(li + 1)
         # copy-ins issued at the start of this layer's backward (its own input at the latest)
         for j in swap:
             if 1 <= j <= li + 1 and (issue_at[j] >= li or j >= li):
@@ -254,20 +259,20 @@ def plan_memory(spec, input_shape, budget_bytes=None, fixed_bytes=0, cost=None, 
         if budget_bytes is None or peak <= budget_bytes:
             break
         # moments at the peak; candidates = resident, idle, still kept, neither batch nor logits
-        candidates = set()
+        candidates, coming_back = set(), set()
         for phase, li, total, resident, busy in events:
             if total < peak:
                 continue
             for j in resident - busy - swap - redo:
                 if j == 0 or j >= L:
                     continue
-                if phase != "fwd" and li - prefetch <= j < li:
-                    continue            # on its way back in at that moment
                 candidates.add(j)
+                if phase != "fwd" and li - prefetch <= j < li:
+                    coming_back.add(j)  # swapped, it would be on its way back in at that moment: only dropping helps
         best = None
         for j in candidates:
             options = []
-            if j + 1 not in redo:       # a tensor something is recomputed from stays on the device
+            if j + 1 not in redo and j not in coming_back:   # a tensor something is recomputed from stays on the device
                 options.append(("swap", est(swap | {j}, redo)))
             if may_redo(j):
                 options.append(("redo", est(swap, redo | {j})))
