@@ -179,3 +179,41 @@ def test_recomputation_replay_and_choice():
         again = planner.simulate(spec, shapes, both.swap, fixed_bytes(spec, shape, 10, opt, tuple(both.split)),
                                  issue_at=both.issue_at, recompute=both.recompute)[0]
         assert again == both.peak_bytes
+
+
+def test_step_estimate_waits_only_where_the_executor_does():
+    """One swapped tensor, worked by hand: the copy-out starts with its consumer and holds nothing up
+    before the turn; the copy-in is issued `prefetch` layers ahead and the consumer's backward waits for
+    it; a budget that leaves no room makes an allocation wait for the copy-out instead."""
+    shapes = planner.layer_shapes(SMALL, IN)
+    size = planner.tensor_bytes(shapes)
+    cost = planner.CostModel(link_gbs=0.05, host_wait_ms=0.0)        # slow link: the copies outlast the layers
+    f, b = planner.layer_times(SMALL, shapes, cost)
+    L, c = len(SMALL), cost.copy_ms(size[1])
+    free = planner.step_ms(SMALL, shapes, (), cost)
+    assert free == pytest.approx(sum(f) + sum(b))
+    t = max(sum(f), f[0] + c)                                          # the turn waits for the copy-out
+    issue = min(L - 1, 1 + 3)
+    t += sum(b[issue + 1:])                                            # backward of the layers behind the issue point
+    arrival = t + c
+    t += sum(b[2:issue + 1])
+    t = max(t, arrival) + b[1] + b[0]
+    assert planner.step_ms(SMALL, shapes, (1,), cost) == pytest.approx(t)
+    # each host-side wait of a swap (one on the way out, one on the way in) is charged to the compute stream
+    quick = planner.CostModel(link_gbs=1e6, host_wait_ms=0.5)
+    assert planner.step_ms(SMALL, shapes, (1,), quick) == pytest.approx(planner.step_ms(SMALL, shapes, (), quick) + 1.0, abs=1e-3)
+    # with room for everything the budget changes nothing; at the replayed peak of this plan the first
+    # allocation that does not fit beside tensor 1 waits for it to have left, and the rest of the forward
+    # pass runs after the copy instead of under it
+    roomy, _ = planner.simulate(SMALL, shapes, ())
+    assert planner.step_ms(SMALL, shapes, (1,), cost, budget_bytes=roomy) == pytest.approx(t)
+    tight, _ = planner.simulate(SMALL, shapes, (1,))
+    assert tight < roomy and f[0] + c > sum(f)
+    held, first_wait = size[0], None
+    for li in range(L):
+        held += size[li + 1]
+        if held > tight:
+            first_wait = li
+            break
+    assert first_wait is not None and first_wait >= 2
+    assert planner.step_ms(SMALL, shapes, (1,), cost, budget_bytes=tight) == pytest.approx(t + sum(f[first_wait:]))

@@ -34,6 +34,9 @@ cheap, and a run of neighbouring small tensors that would queue on the link is n
 whose input is swapped run in micro-tensors of at most `piece_bytes`, so that a backward
 micro-op starts as soon as its own piece has arrived.
 """
+import collections
+import math
+
 import numpy as np
 
 GiB = float(1 << 30)
@@ -41,10 +44,13 @@ GiB = float(1 << 30)
 
 class CostModel(object):
     """Rates measured on one MI355X with this library (fp32): contractions, streaming
-    kernels on the bytes they move, and the pinned-host link each way."""
+    kernels on the bytes they move, the pinned-host link each way, and what one host-side
+    event wait costs the compute stream (the host has to catch up with its launches afterwards;
+    a swapped tensor brings one such wait on the way out and one on the way in)."""
 
     def __init__(self, conv_tflops=110.0, conv_tflops_narrow=90.0, matmul_tflops=65.0, stream_gbs=5500.0,
-                 link_gbs=55.0):
+                 link_gbs=55.0, host_wait_ms=0.2):
+        self.host_wait_ms = host_wait_ms
         self.conv_tflops = conv_tflops
         self.conv_tflops_narrow = conv_tflops_narrow
         self.matmul_tflops = matmul_tflops
@@ -129,7 +135,7 @@ def layer_shapes(spec, input_shape):
 
 
 def tensor_bytes(shapes):
-    return [4 * int(np.prod(s)) for s in shapes]
+    return [4 * int(math.prod(s)) for s in shapes]
 
 
 def default_issue_at(swap, n_layers, prefetch):
@@ -191,37 +197,100 @@ def simulate(spec, shapes, swap=(), fixed_bytes=0, prefetch=3, issue_at=None, re
     return peak, events
 
 
-def step_ms(spec, shapes, swap, cost, prefetch=3, issue_at=None, recompute=()):
+def layer_times(spec, shapes, cost):
+    """-> (forward ms, backward ms) per layer under `cost`; `step_ms` takes them ready-made when
+    it is called many times for one net."""
+    L = len(spec)
+    return ([cost.layer_ms(spec[li], shapes[li], shapes[li + 1], False) for li in range(L)],
+            [cost.layer_ms(spec[li], shapes[li], shapes[li + 1], True, first=li == 0) for li in range(L)])
+
+
+def step_ms(spec, shapes, swap, cost, prefetch=3, issue_at=None, recompute=(), budget_bytes=None, fixed_bytes=0,
+            times=None):
     """Estimated step time under the replayed schedule: one compute stream, one copy-out and one
     copy-in stream (each link direction carries one copy at a time, in issue order).  A swapped
-    tensor starts leaving when its consumer starts and the sweep waits for it when that consumer
-    ends (the release point of the replay); a copy-in is issued `prefetch` layers ahead and the
-    layer that needs the tensor waits for its arrival."""
+    tensor starts leaving when its consumer starts; its memory comes back when both the consumer
+    and the copy are done, and releases are handed back in the order they were made.  As in the
+    executor, nothing waits for a release until an allocation would not fit `budget_bytes` without
+    it (no budget: never), except at the turn, where the backward sweep starts only after every
+    copy-out has finished.  A copy-in is issued `prefetch` layers ahead (or where `issue_at` says)
+    and the layer that needs the tensor waits for its arrival."""
     L = len(spec)
     size = tensor_bytes(shapes)
-    swap = set(swap)
-    t = out_free = 0.0
-    for li in range(L):
-        t0 = t
-        t += cost.layer_ms(spec[li], shapes[li], shapes[li + 1], False)
-        if li in swap:
-            out_free = max(out_free, t0) + cost.copy_ms(size[li])
-            t = max(t, out_free)
+    fwd_ms, bwd_ms = times if times is not None else layer_times(spec, shapes, cost)
+    swap, redo = set(swap), set(recompute)
     issue_at = issue_at if issue_at is not None else default_issue_at(swap, L, prefetch)
+    clock = [0.0, fixed_bytes + size[0]]      # compute-stream time (ms), bytes held
+    pending = collections.deque()             # (bytes, time the release is through), in order of release
+
+    def alloc(nbytes):
+        while pending:
+            held, ready = pending[0]
+            if ready > clock[0]:
+                if budget_bytes is None or clock[1] + nbytes <= budget_bytes:
+                    break
+                clock[0] = ready              # the allocation waits for the oldest release
+            pending.popleft()
+            clock[1] -= held
+        clock[1] += nbytes
+
+    def release(nbytes, ready=0.0):
+        pending.append((nbytes, max(clock[0], ready)))
+
+    out_free = 0.0
+    for li in range(L):
+        alloc(size[li + 1])
+        started = clock[0]
+        clock[0] += fwd_ms[li]
+        if li in swap:
+            out_free = max(out_free, started) + cost.copy_ms(size[li])
+            release(size[li], out_free)
+            clock[0] += cost.host_wait_ms
+        elif li in redo:
+            release(size[li])
+    while pending:                            # the turn: every tensor that left has really left
+        held, ready = pending.popleft()
+        clock[0] = max(clock[0], ready)
+        clock[1] -= held
+    alloc(size[L])
+    g_out = size[L]
     in_free, arrival = 0.0, {}
-    redo, redone = set(recompute), set()
+    away, dropped = set(j for j in swap if j >= 1), set(redo)
+    here = set(range(L + 1)) - away - dropped
     for li in range(L - 1, -1, -1):
-        for j in sorted(swap, reverse=True):          # the tensor needed first is issued first
-            if j >= 1 and j not in arrival and (issue_at[j] >= li or j >= li):
-                in_free = max(in_free, t) + cost.copy_ms(size[j])
+        if spec[li][0] not in NEEDS_OUTPUT_BACKWARD and li + 1 in here:
+            here.discard(li + 1)
+            release(size[li + 1])
+        for j in sorted(away, reverse=True):          # the tensor needed first is issued first
+            if issue_at[j] >= li or j >= li:
+                away.discard(j)
+                here.add(j)
+                alloc(size[j])
+                in_free = max(in_free, clock[0]) + cost.copy_ms(size[j])
                 arrival[j] = in_free
+                clock[0] += cost.host_wait_ms
+        chain = []
         j = li
-        while j in redo and j not in redone:          # every dropped tensor is computed again once
-            t += cost.layer_ms(spec[j - 1], shapes[j - 1], shapes[j], False)
-            redone.add(j)
+        while j in dropped:
+            chain.append(j)
             j -= 1
-        t = max(t, arrival.get(li, 0.0)) + cost.layer_ms(spec[li], shapes[li], shapes[li + 1], True, first=li == 0)
-    return t
+        for j in reversed(chain):                     # every dropped tensor is computed again once
+            dropped.discard(j)
+            here.add(j)
+            alloc(size[j])
+            clock[0] += fwd_ms[j - 1]
+        in_place = spec[li][0] in IN_PLACE_BACKWARD
+        g_in = 0 if li == 0 else g_out if in_place else size[li]
+        if li and not in_place:
+            alloc(g_in)
+        clock[0] = max(clock[0], arrival.get(li, 0.0)) + bwd_ms[li]
+        if li + 1 in here:
+            here.discard(li + 1)
+            release(size[li + 1])
+        if not in_place or li == 0:
+            release(g_out)
+        g_out = g_in
+    return clock[0]
 
 
 def plan_memory(spec, input_shape, budget_bytes=None, fixed_bytes=0, cost=None, piece_bytes=128 << 20, prefetch=3,
@@ -241,8 +310,10 @@ def plan_memory(spec, input_shape, budget_bytes=None, fixed_bytes=0, cost=None, 
     def replay(sw, rd, issue=None):
         return simulate(spec, shapes, sw, fixed_bytes, prefetch, issue, rd)
 
+    times = layer_times(spec, shapes, cost)
+
     def est(sw, rd, issue=None):
-        return step_ms(spec, shapes, sw, cost, prefetch, issue, rd)
+        return step_ms(spec, shapes, sw, cost, prefetch, issue, rd, budget_bytes, fixed_bytes, times)
 
     def may_redo(j):
         # produced by a cheap layer, and what it is computed from stays on the device
@@ -253,73 +324,96 @@ def plan_memory(spec, input_shape, budget_bytes=None, fixed_bytes=0, cost=None, 
             k -= 1
         return k not in swap
 
-    free_ms = now_ms = est(swap, redo)
-    while True:
-        peak, events = replay(swap, redo)
-        if budget_bytes is None or peak <= budget_bytes:
-            break
-        # moments at the peak; candidates = resident, idle, still kept, neither batch nor logits
-        candidates, coming_back = set(), set()
-        for phase, li, total, resident, busy in events:
-            if total < peak:
-                continue
-            for j in resident - busy - swap - redo:
-                if j == 0 or j >= L:
+    def early_issue(swap, redo, now_ms, peak):
+        # copy-ins may start earlier than `prefetch` layers ahead where the budget has room for the
+        # tensor over the whole stretch; the order of issue stays the order of need
+        issue_at = default_issue_at(swap, L, prefetch)
+        if budget_bytes is not None and swap:
+            bound = L - 1
+            for j in sorted(swap, reverse=True):
+                best_at = issue_at[j]
+                for at in range(issue_at[j] + 1, bound + 1):
+                    trial = dict(issue_at)
+                    trial[j] = at
+                    if replay(swap, redo, trial)[0] > budget_bytes:
+                        break
+                    best_at = at
+                issue_at[j] = best_at
+                bound = best_at
+            now_ms = est(swap, redo, issue_at)
+            peak = replay(swap, redo, issue_at)[0]
+        return now_ms, peak, issue_at
+
+    free_ms = est(set(), set())
+
+    def choose(power):
+        """One greedy pass scoring a candidate by added time / size**power -> (ms, peak, issue_at, swap, redo)."""
+        swap.clear()
+        redo.clear()
+        now_ms = free_ms
+        while True:
+            peak, events = replay(swap, redo)
+            if budget_bytes is None or peak <= budget_bytes:
+                break
+            # moments at the peak; candidates = resident, idle, still kept, neither batch nor logits
+            candidates, coming_back = set(), set()
+            for phase, li, total, resident, busy in events:
+                if total < peak:
                     continue
-                candidates.add(j)
-                if phase != "fwd" and li - prefetch <= j < li:
-                    coming_back.add(j)  # swapped, it would be on its way back in at that moment: only dropping helps
-        best = None
-        for j in candidates:
-            options = []
-            if j + 1 not in redo and j not in coming_back:   # a tensor something is recomputed from stays on the device
-                options.append(("swap", est(swap | {j}, redo)))
-            if may_redo(j):
-                options.append(("redo", est(swap, redo | {j})))
-            for how, ms in options:
-                score = (ms - now_ms + 1e-3) / size[j]
-                if best is None or score < best[0]:
-                    best = (score, j, how)
-        if best is None:
-            raise ValueError("budget of %.2f GiB cannot be met: %.2f GiB are needed with every idle tensor removed"
-                             % (budget_bytes / GiB, peak / GiB))
-        (redo if best[2] == "redo" else swap).add(best[1])
-        now_ms = est(swap, redo)
-    # the last pick may have freed more than was missing: put back what the budget can hold,
-    # dearest first
-    for _ in range(len(swap) + len(redo)):
-        gains = []
-        for j in swap:
-            rest = swap - {j}
-            if replay(rest, redo)[0] <= budget_bytes:
-                gains.append((now_ms - est(rest, redo), 0, j))
-        for j in redo:
-            rest = redo - {j}
-            if replay(swap, rest)[0] <= budget_bytes:
-                gains.append((now_ms - est(swap, rest), 1, j))
-        if not gains or max(gains)[0] <= 0:
-            break
-        _, which, j = max(gains)
-        (redo if which else swap).discard(j)
-        now_ms = est(swap, redo)
-        peak = replay(swap, redo)[0]
-    # copy-ins may start earlier than `prefetch` layers ahead where the budget has room for the
-    # tensor over the whole stretch; the order of issue stays the order of need
-    issue_at = default_issue_at(swap, L, prefetch)
-    if budget_bytes is not None and swap:
-        bound = L - 1
-        for j in sorted(swap, reverse=True):
-            best_at = issue_at[j]
-            for at in range(issue_at[j] + 1, bound + 1):
-                trial = dict(issue_at)
-                trial[j] = at
-                if replay(swap, redo, trial)[0] > budget_bytes:
-                    break
-                best_at = at
-            issue_at[j] = best_at
-            bound = best_at
-        now_ms = est(swap, redo, issue_at)
-        peak = replay(swap, redo, issue_at)[0]
+                for j in resident - busy - swap - redo:
+                    if j == 0 or j >= L:
+                        continue
+                    candidates.add(j)
+                    if phase != "fwd" and li - prefetch <= j < li:
+                        coming_back.add(j)  # swapped, it would be on its way back in at that moment: only dropping helps
+            best = None
+            for j in candidates:
+                options = []
+                if j + 1 not in redo and j not in coming_back:   # a tensor something is recomputed from stays on the device
+                    options.append(("swap", est(swap | {j}, redo)))
+                if may_redo(j):
+                    options.append(("redo", est(swap, redo | {j})))
+                for how, ms in options:
+                    score = (ms - now_ms + 1e-3) / float(size[j]) ** power
+                    if best is None or score < best[0]:
+                        best = (score, j, how)
+            if best is None:
+                raise ValueError("budget of %.2f GiB cannot be met: %.2f GiB are needed with every idle tensor removed"
+                                 % (budget_bytes / GiB, peak / GiB))
+            (redo if best[2] == "redo" else swap).add(best[1])
+            now_ms = est(swap, redo)
+        # the last pick may have freed more than was missing: put back what the budget can hold,
+        # dearest first
+        for _ in range(len(swap) + len(redo)):
+            gains = []
+            for j in swap:
+                rest = swap - {j}
+                if replay(rest, redo)[0] <= budget_bytes:
+                    gains.append((now_ms - est(rest, redo), 0, j))
+            for j in redo:
+                rest = redo - {j}
+                if replay(swap, rest)[0] <= budget_bytes:
+                    gains.append((now_ms - est(swap, rest), 1, j))
+            if not gains or max(gains)[0] <= 0:
+                break
+            _, which, j = max(gains)
+            (redo if which else swap).discard(j)
+            now_ms = est(swap, redo)
+            peak = replay(swap, redo)[0]
+        return early_issue(set(swap), set(redo), now_ms, peak) + (set(swap), set(redo))
+
+    # time per byte freed is the natural score; weighting size less or more sometimes finds a cheaper set
+    # (fewer, larger tensors that hide behind long layers), so the estimate decides between a few passes
+    powers = (1.0,) if budget_bytes is None else (1.0, 0.5, 1.5)
+    passes, refusal = [], None
+    for pw in powers:
+        try:
+            passes.append(choose(pw))
+        except ValueError as e:
+            refusal = refusal or e
+    if not passes:
+        raise refusal
+    now_ms, peak, issue_at, swap, redo = min(passes, key=lambda r: (r[0], len(r[3]) + len(r[4])))
     split = {}
     for li, layer in enumerate(spec):
         if layer[0] == "conv" and li >= 1 and li in swap:
