@@ -26,11 +26,14 @@ schedule, which `simulate` replays byte for byte:
                         i+1 and the output gradient
 
 Choice.  Greedy: while the replayed peak exceeds the budget, take the moment of the peak and,
-among the tensors resident but idle then, swap the one that adds the least estimated step
-time per byte it frees.  The estimate (`step_ms`) walks the same schedule with a cost model:
-layer times from measured rates, one copy at a time per link direction, the sweep waiting
-where a copy has not finished - so a tensor whose transfer hides behind a long convolution is
-cheap, and a run of neighbouring small tensors that would queue on the link is not.  Layers
+among the tensors resident but idle then, remove the one that adds the least estimated step
+time per byte it frees - by swapping it, or (if allowed, and a cheap layer produced it) by
+dropping it and computing it again in the backward sweep.  The estimate (`step_ms`) walks the
+same schedule with a cost model: layer times from measured rates, one copy at a time per link
+direction, and waits where the executor waits (an allocation that does not fit the budget
+without an outstanding release, the turn, a layer whose copy-in has not arrived, the host-side
+event waits of a swap) - so a tensor whose transfer hides behind a long convolution is cheap,
+and a run of neighbouring small tensors that would queue on the link is not.  Layers
 whose input is swapped run in micro-tensors of at most `piece_bytes`, so that a backward
 micro-op starts as soon as its own piece has arrived.
 """
