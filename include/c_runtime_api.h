@@ -408,6 +408,18 @@ int TSplit_BatchNormRelu_gradient(const DLArrayHandle gradient_Y, const DLArrayH
                                   DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
                                   DLStreamHandle stream_handle, ProfilerHandle p);
 
+/* ---- Which routine a convolution takes.  NO counterpart in the reference (cuDNN's choice is
+ *      internal there, src/ops/CudnnConv2d.cu:66).  Returns 1 when CuDNN_DLGpuConv2d (data_gradient
+ *      = 0) or CuDNN_DLGpuConv2d_Gradient_of_Data (data_gradient = 1) would run a layer of this
+ *      shape through the Winograd F(4x4, 3x3) routine instead of the direct implicit GEMM, 0
+ *      otherwise; for benchmarks that label their timings.  in_channels / out_channels are the
+ *      filter's C and O whatever the direction.  Environment: TSPLIT_CONV_WINOGRAD=0 never,
+ *      =1 wherever the shape allows (3x3, stride 1, pad 1, the channel count that is summed over
+ *      a multiple of 16). ---- */
+int TSplit_ConvTakesWinograd(int images, int in_channels, int out_channels, int height, int width,
+                             int kernel_h, int kernel_w, int pad_h, int pad_w, int stride,
+                             int data_gradient);
+
 /* ---- Recorded steps.  NO counterpart in the reference (every step there is issued call by
  *      call from Python); for steps made of thousands of tiny kernels (recurrent nets, small
  *      MLPs) whose time is the host's launch rate.  Between TSplit_StreamBeginRecord and

@@ -1,5 +1,6 @@
-"""GPU parity of the three convolutions (implicit GEMM on fp32 MFMA) against the CPU oracle,
-through both symbol families.  Tolerance 2e-3 max relative error; measured errors are ~1e-6."""
+"""GPU parity of the three convolutions (implicit GEMM on fp32 MFMA; Winograd F(4x4, 3x3) for wide
+3x3 layers) against the CPU oracle, through both symbol families.  Tolerance 2e-3 max relative
+error; measured errors are ~1e-6 (direct) and below 2e-5 (Winograd)."""
 import numpy as np
 import pytest
 
@@ -123,6 +124,88 @@ def test_conv_backward_data_with_and_without_filter_relay(case, raw, rng, monkey
     every such shape."""
     monkeypatch.setenv("TSPLIT_CONV_RAW", raw)
     _run(case, "cudnn", rng)
+
+
+WINOGRAD_CASES = [c for c in CASES if c[5:] == (3, 3, 1, 1, 1) and c[1] % 16 == 0 and c[4] % 16 == 0] + [
+    (4, 128, 28, 28, 128, 3, 3, 1, 1, 1),   # whole 4x4 tiles, rows stored as quads
+    (2, 256, 14, 14, 144, 3, 3, 1, 1, 1),   # 14 = 3.5 tiles: the last tile row and column hang over the edge
+    (3, 32, 13, 17, 48, 3, 3, 1, 1, 1),     # odd, non-square planes
+    (2, 16, 5, 3, 16, 3, 3, 1, 1, 1),       # a plane narrower than one tile
+    (1, 16, 1, 1, 16, 3, 3, 1, 1, 1),       # one pixel: only the filter's centre counts
+    (3, 16, 40, 72, 32, 3, 3, 1, 1, 1),     # 18 tiles per row: tile rows do not line up with the 64 lanes of a wave
+    (2, 16, 300, 260, 16, 3, 3, 1, 1, 1),   # tile rows longer than a wave
+    (70, 32, 8, 8, 48, 3, 3, 1, 1, 1),      # 280 tiles: the tile count padded to a multiple of 4 and of 128
+]
+
+
+@pytest.mark.parametrize("winograd", ["0", "1"])
+@pytest.mark.parametrize("case", WINOGRAD_CASES)
+def test_conv_3x3_direct_and_winograd(case, winograd, rng, monkeypatch):
+    """3x3 / stride 1 / pad 1 layers have two routines for the forward pass and the data gradient:
+    the direct implicit GEMM and Winograd F(4x4, 3x3) (chosen for wide layers).  Both run on every
+    such shape; the Winograd transforms cost about a digit (errors of a few 1e-6 of the output's
+    magnitude against ~1e-7), far inside the 2e-3 bar, and `_run` holds both to 1e-4."""
+    from tsplit_amd import gpu_links as L
+    monkeypatch.setenv("TSPLIT_CONV_WINOGRAD", winograd)
+    N, C, H, W, Oc = case[:5]
+    assert L.conv_takes_winograd(N, C, Oc, H, W) == (winograd == "1")
+    assert L.conv_takes_winograd(N, C, Oc, H, W, data_gradient=True) == (winograd == "1")
+    _run(case, "cudnn", rng)
+
+
+def test_conv_winograd_choice(monkeypatch):
+    """Left to itself the library takes Winograd for wide 3x3 / stride 1 / pad 1 layers with enough
+    tiles, and never for another filter, stride or padding, whatever the environment says."""
+    from tsplit_amd import gpu_links as L
+    monkeypatch.delenv("TSPLIT_CONV_WINOGRAD", raising=False)
+    assert L.conv_takes_winograd(64, 256, 256, 56, 56) and L.conv_takes_winograd(64, 256, 256, 56, 56, data_gradient=True)
+    assert L.conv_takes_winograd(16, 64, 128, 112, 112) and L.conv_takes_winograd(64, 512, 512, 14, 14)
+    assert not L.conv_takes_winograd(64, 64, 64, 224, 224)           # too narrow: the transforms outweigh the GEMMs
+    assert not L.conv_takes_winograd(2, 256, 256, 14, 14)            # too few tiles
+    assert not L.conv_takes_winograd(64, 3, 64, 224, 224)
+    monkeypatch.setenv("TSPLIT_CONV_WINOGRAD", "1")
+    assert L.conv_takes_winograd(2, 16, 16, 5, 5)
+    assert not L.conv_takes_winograd(2, 24, 16, 5, 5)                # channels summed over must be a multiple of 16
+    assert L.conv_takes_winograd(2, 24, 16, 5, 5, data_gradient=True)
+    for kernel, pad, stride in ((3, 1, 2), (3, 0, 1), (1, 0, 1), (5, 2, 1)):
+        assert not L.conv_takes_winograd(64, 256, 256, 56, 56, kernel, pad, stride)
+    monkeypatch.setenv("TSPLIT_CONV_WINOGRAD", "0")
+    assert not L.conv_takes_winograd(64, 256, 256, 56, 56)
+
+
+def test_conv_winograd_is_per_image_and_repeatable(rng, monkeypatch):
+    """Tiles never span images and every GEMM sums the channels in one fixed order: a batch run as 4
+    micro-tensors, in runs of a few images (a small scratch allowance) or twice gives the same bits."""
+    from tsplit_amd import gpu_links as L, ndarray
+    monkeypatch.setenv("TSPLIT_CONV_WINOGRAD", "1")
+    ctx = ndarray.gpu(0)
+    x = rng.normal(size=(8, 32, 20, 24)).astype(np.float32)
+    w = rng.normal(size=(48, 32, 3, 3)).astype(np.float32)
+    dy = rng.normal(size=(8, 48, 20, 24)).astype(np.float32)
+    gx, gw, gdy = ndarray.array(x, ctx), ndarray.array(w, ctx), ndarray.array(dy, ctx)
+
+    def both(split):
+        y, dx = ndarray.empty(dy.shape, ctx), ndarray.empty(x.shape, ctx)
+        if split:
+            for a in (gx, gdy, y, dx):
+                a.split_tensor(4)
+            for i in range(4):
+                L.CuDNN_conv2d(gx.sTensor[i], gw, y.sTensor[i], 1, 1, 1)
+                L.CuDNN_conv2d_gradient_of_data(gw, gdy.sTensor[i], dx.sTensor[i], 1, 1, 1)
+        else:
+            L.CuDNN_conv2d(gx, gw, y, 1, 1, 1)
+            L.CuDNN_conv2d_gradient_of_data(gw, gdy, dx, 1, 1, 1)
+        return y.asnumpy(), dx.asnumpy()
+
+    whole = both(False)
+    again = both(False)
+    monkeypatch.setenv("TSPLIT_WINOGRAD_RUN_MIB", "1")     # 3 images per run
+    runs = both(False)
+    monkeypatch.delenv("TSPLIT_WINOGRAD_RUN_MIB")
+    parts = both(True)
+    for other in (again, runs, parts):
+        np.testing.assert_array_equal(whole[0], other[0])
+        np.testing.assert_array_equal(whole[1], other[1])
 
 
 @pytest.mark.parametrize("case", [c for c in CASES if c[7] == c[8]][:8])

@@ -30,6 +30,9 @@
 #include "mfma_gemm.h"
 
 namespace tsplit {
+// winograd.hip
+int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int gathered, int produced, int H, int W,
+                      bool rotated, hipStream_t st);
 namespace {
 
 using namespace mg;
@@ -2017,6 +2020,24 @@ int launch_conv_thin_fwd(const ConvGeo &g, const float *x, const float *w, float
   return 0;
 }
 
+// 3x3 / stride 1 / pad 1 layers wide enough to be bound by MFMA throughput go through the Winograd
+// F(4x4, 3x3) routine (winograd.hip): a quarter of the multiplications for 2.25x the activation
+// traffic.  TSPLIT_CONV_WINOGRAD=0 switches it off, =1 takes it wherever the shape allows.
+
+inline bool winograd_pays(const ConvGeo &g, int gathered, int produced) {
+  const char *e = std::getenv("TSPLIT_CONV_WINOGRAD");
+  const int forced = e ? (e[0] == '1' ? 1 : 0) : -1;
+  const bool fits = g.kH == 3 && g.kW == 3 && g.s == 1 && g.ph == 1 && g.pw == 1 && g.oH == g.H && g.oW == g.W &&
+                    gathered % BK == 0 && static_cast<int64_t>(std::max(gathered, produced)) * g.H * g.W < (1ll << 29);
+  if (!fits || forced == 0) return false;
+  if (forced == 1) return true;
+  // wide enough for the 36 GEMMs to outweigh the transforms, little of the 4x4 tiling hanging over
+  // the plane's edge, and enough tiles to fill the chip
+  const int64_t covered = static_cast<int64_t>((g.H + 3) / 4) * ((g.W + 3) / 4) * 16;
+  return std::min(gathered, produced) >= 64 && std::max(gathered, produced) >= 128 &&
+         covered * 3 <= static_cast<int64_t>(g.H) * g.W * 4 && static_cast<int64_t>(g.imgs) * covered >= 16 * 1024;
+}
+
 int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y, int ph, int pw, int s,
                  DLStreamHandle sh, ProfilerHandle p) {
   ConvGeo g;
@@ -2026,6 +2047,9 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
   if (numel(y) > 0) {
     if (thin_fwd_ok(g)) {
       const int rc = launch_conv_thin_fwd(g, cf(x), cf(w), mf(y), st);
+      if (rc) return rc;
+    } else if (winograd_pays(g, g.C, g.O)) {
+      const int rc = conv_winograd_3x3(cf(x), cf(w), mf(y), g.imgs, g.C, g.O, g.H, g.W, false, st);
       if (rc) return rc;
     } else if (g.C % BK == 0) {
       // a 1x1 filter [O][C] already is tap-major: used where it lies
@@ -2071,7 +2095,10 @@ int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray 
   if (geo_from(who, dx, w, dy, ph, pw, s, g)) return -1;
   hipStream_t st = stream_of(sh);
   ProfileScope ps(p, st, numel(dy) + numel(w), numel(dx), numel(w));
-  if (numel(dx) > 0) {
+  if (numel(dx) > 0 && winograd_pays(g, g.O, g.C)) {
+    const int rc = conv_winograd_3x3(cf(dy), cf(w), mf(dx), g.imgs, g.O, g.C, g.H, g.W, true, st);
+    if (rc) return rc;
+  } else if (numel(dx) > 0) {
     float *wt = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(numel(w)) * 4));
     TS_REQUIRE(wt, "%s: no scratch memory", who);
     const int total = static_cast<int>(numel(w));
@@ -2171,6 +2198,14 @@ int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArra
 using namespace tsplit;
 
 extern "C" {
+
+int TSplit_ConvTakesWinograd(int images, int in_channels, int out_channels, int height, int width, int kernel_h,
+                             int kernel_w, int pad_h, int pad_w, int stride, int data_gradient) {
+  if (images <= 0 || in_channels <= 0 || out_channels <= 0 || height <= 0 || width <= 0 || stride <= 0) return 0;
+  ConvGeo g{images, in_channels, height, width, out_channels, kernel_h, kernel_w, pad_h, pad_w, stride,
+            (height + 2 * pad_h - kernel_h) / stride + 1, (width + 2 * pad_w - kernel_w) / stride + 1};
+  return data_gradient ? winograd_pays(g, out_channels, in_channels) : winograd_pays(g, in_channels, out_channels);
+}
 
 int CuDNN_DLGpuConv2d(const DLArrayHandle input_x, const DLArrayHandle input_f, DLArrayHandle output,
                       const int padding, const int padding2, const int stride, DLStreamHandle stream_handle,

@@ -399,6 +399,15 @@ def sigmoid(in_arr, out_arr, stream=None, profiler=None):
     check_call(_LIB.DLGpuSigmoid(_h(in_arr), _h(out_arr), _s(stream), _p(profiler)))
 
 
+# ---- Which routine a convolution takes (no counterpart in the reference's gpu_links) ----
+def conv_takes_winograd(images, in_channels, out_channels, height, width, kernel=3, pad=1, stride=1, data_gradient=False):
+    """True when the library runs this layer's forward pass (or, with `data_gradient`, its data
+    gradient) through the Winograd F(4x4, 3x3) routine rather than the direct implicit GEMM."""
+    return bool(_LIB.TSplit_ConvTakesWinograd(int(images), int(in_channels), int(out_channels), int(height), int(width),
+                                              int(kernel), int(kernel), int(pad), int(pad), int(stride),
+                                              int(bool(data_gradient))))
+
+
 # ---- Fused BatchNorm + Relu (no counterpart in the reference's gpu_links) ----
 def batch_norm_relu(in_arr, bn_scale_arr, bn_bias_arr, out_arr, save_mean, save_var, eps=0.01, stream=None,
                     profiler=None):

@@ -198,8 +198,10 @@ class Trainer(object):
                 _, name, cin, cout, k, pad, stride = layer
                 w = self.params[name + "_weight"]
                 thin = cin * k * k <= 32      # a first layer (3 input channels): bound by HBM, timed in bytes
-                tag = "conv_fwd_thin" if thin else "conv_fwd_" + self._tile(cout)
                 pairs = list(zip(a.sTensor, out.sTensor)) if li in self.split else [(a, out)]
+                xs = pairs[0][0].shape
+                wino = L.conv_takes_winograd(xs[0], cin, cout, xs[2], xs[3], k, pad, stride)
+                tag = "conv_fwd_thin" if thin else "conv_fwd_winograd" if wino else "conv_fwd_" + self._tile(cout)
                 for xa, ya in pairs:
                     if thin:
                         self._run(tag, 4.0 * (n(xa.shape) + n(w.shape) + n(ya.shape)), "byte", L.CuDNN_conv2d, xa, w, ya,
@@ -266,8 +268,11 @@ class Trainer(object):
                         self._run("add", 12.0 * n(dw.shape), "byte", L.matrix_elementwise_add, dw, self.dw_piece[li], dw)
                 if not first:
                     gis = g_in.sTensor if split else [g_in]
+                    wino = L.conv_takes_winograd(gis[0].shape[0], cin, cout, gis[0].shape[2], gis[0].shape[3], k, pad, stride,
+                                                 data_gradient=True)
                     for ga, gi in zip(gs, gis):
-                        self._run("conv_bwd_data_" + self._tile(cin), 2.0 * n(ga.shape) * cin * k * k, "flop",
+                        self._run("conv_bwd_data_winograd" if wino else "conv_bwd_data_" + self._tile(cin),
+                                  2.0 * n(ga.shape) * cin * k * k, "flop",
                                   L.CuDNN_conv2d_gradient_of_data, w, ga, gi, pad, pad, stride)
             elif kind == "bn" and li in self.fused:
                 name = layer[1]
