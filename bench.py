@@ -147,7 +147,7 @@ def main():
         sys.exit("bench.py: this build is single-GPU by design (no collectives, no sharding); run with --gpus 1. "
                  "The one-GPU figure is the whole-job throughput.")
 
-    from tsplit_amd import ndarray, trainer
+    from tsplit_amd import gpu_links as L, ndarray, trainer
     from tsplit_amd.timing import EventTimer
     ctx = ndarray.gpu(0)
     spec, params, x, labels, split = vgg_workload(a.batch)
@@ -162,6 +162,7 @@ def main():
     t.sync()
     if timer:
         timer.enabled = True
+        L.winograd_gemm_timing(True)
     t0 = time.perf_counter()
     for _ in range(a.steps):
         t.step(gx, gy)
@@ -191,6 +192,18 @@ def main():
                             "unit": "TFLOP/s" if d["unit"] == "flop" else "GB/s", "frac": d["rate"] / peak}
             if tag.endswith("_winograd"):
                 kernels[tag]["note"] = "several kernels per call; rate of the direct algorithm's FLOP count"
+        # the GEMM kernels inside the Winograd calls, timed by the library with event pairs on the
+        # compute stream around each launch; their work is the FLOP they execute
+        for tag, grad in (("winograd_gemm", False), ("winograd_filter_grad_gemm", True)):
+            launches, ms, flop = L.winograd_gemm_times(filter_gradient=grad)
+            if launches:
+                k[tag] = {"calls": launches, "ms_total": ms, "ms_avg": ms / launches, "work": flop,
+                          "work_per_call": flop / launches, "rate": flop / (ms * 1e-3) / 1e12, "unit": "flop"}
+                kernels[tag] = {"calls_per_step": launches / a.steps, "ms_per_step": ms / a.steps, "ms_avg": ms / launches,
+                                "achieved": k[tag]["rate"], "unit": "TFLOP/s", "frac": k[tag]["rate"] / PEAK_TFLOPS_FP32_MFMA,
+                                "note": "one kernel inside the *_winograd calls above (its time is part of theirs)"}
+        L.winograd_gemm_timing(False)
+        kernels = dict(sorted(kernels.items(), key=lambda kv: -kv[1]["ms_per_step"]))
         dom = next(tag for tag in kernels if not tag.endswith("_winograd"))
         dd = k[dom]
         out["roofline"] = {"kernel": dom, "bound": "mfma" if dd["unit"] == "flop" else "hbm",
@@ -201,7 +214,7 @@ def main():
                            "per_launch": dd["work_per_call"], "ms_avg": dd["ms_avg"]}
         # all conv FLOP over all conv time; the thin first layer (Cin*kH*kW = 27) is timed in bytes
         # because HBM bounds it, so its FLOP (forward and filter gradient) are added here
-        conv = [d for tag, d in k.items() if tag.startswith("conv_")]
+        conv = [d for tag, d in k.items() if tag.startswith("conv_")]      # the Winograd GEMMs' time is inside these
         conv_flop = sum(d["work"] for d in conv if d["unit"] == "flop")
         shape = x.shape
         for layer in spec:

@@ -409,16 +409,25 @@ int TSplit_BatchNormRelu_gradient(const DLArrayHandle gradient_Y, const DLArrayH
                                   DLStreamHandle stream_handle, ProfilerHandle p);
 
 /* ---- Which routine a convolution takes.  NO counterpart in the reference (cuDNN's choice is
- *      internal there, src/ops/CudnnConv2d.cu:66).  Returns 1 when CuDNN_DLGpuConv2d (data_gradient
- *      = 0) or CuDNN_DLGpuConv2d_Gradient_of_Data (data_gradient = 1) would run a layer of this
- *      shape through the Winograd F(4x4, 3x3) routine instead of the direct implicit GEMM, 0
- *      otherwise; for benchmarks that label their timings.  in_channels / out_channels are the
- *      filter's C and O whatever the direction.  Environment: TSPLIT_CONV_WINOGRAD=0 never,
- *      =1 wherever the shape allows (3x3, stride 1, pad 1, the channel count that is summed over
- *      a multiple of 16). ---- */
+ *      internal there, src/ops/CudnnConv2d.cu:66).  Returns 1 when CuDNN_DLGpuConv2d (pass 0),
+ *      CuDNN_DLGpuConv2d_Gradient_of_Data (pass 1) or CuDNN_DLGpuConv2d_Gradient_of_Filter (pass 2)
+ *      would run a layer of this shape through the Winograd F(4x4, 3x3) routine instead of the
+ *      direct implicit GEMM, 0 otherwise; for benchmarks that label their timings.  in_channels /
+ *      out_channels are the filter's C and O whatever the pass.  Environment:
+ *      TSPLIT_CONV_WINOGRAD=0 never, =1 wherever the shape allows (3x3, stride 1, pad 1; for
+ *      passes 0 and 1 the channel count that is summed over a multiple of 16). ---- */
 int TSplit_ConvTakesWinograd(int images, int in_channels, int out_channels, int height, int width,
-                             int kernel_h, int kernel_w, int pad_h, int pad_w, int stride,
-                             int data_gradient);
+                             int kernel_h, int kernel_w, int pad_h, int pad_w, int stride, int pass);
+
+/* ---- Timing of the GEMM launches inside the Winograd routine.  NO counterpart in the reference;
+ *      for benchmarks that report a kernel's duration measured inside their own timed region.
+ *      TSplit_WinogradGemmTiming(1) makes every such launch record an event pair on its stream
+ *      (not while the stream is being recorded into a graph); (0) stops and forgets them.
+ *      TSplit_WinogradGemmTimes waits for the launches of kind `which` (0: forward and data
+ *      gradient, 1: filter gradient) and returns their count, summed milliseconds and summed
+ *      executed FLOP (2 * 36 * rows * columns * depth per launch). ---- */
+int TSplit_WinogradGemmTiming(int on);
+int TSplit_WinogradGemmTimes(int which, double *launches, double *ms, double *flop);
 
 /* ---- Recorded steps.  NO counterpart in the reference (every step there is issued call by
  *      call from Python); for steps made of thousands of tiny kernels (recurrent nets, small

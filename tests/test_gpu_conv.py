@@ -141,8 +141,8 @@ WINOGRAD_CASES = [c for c in CASES if c[5:] == (3, 3, 1, 1, 1) and c[1] % 16 == 
 @pytest.mark.parametrize("winograd", ["0", "1"])
 @pytest.mark.parametrize("case", WINOGRAD_CASES)
 def test_conv_3x3_direct_and_winograd(case, winograd, rng, monkeypatch):
-    """3x3 / stride 1 / pad 1 layers have two routines for the forward pass and the data gradient:
-    the direct implicit GEMM and Winograd F(4x4, 3x3) (chosen for wide layers).  Both run on every
+    """3x3 / stride 1 / pad 1 layers have two routines for each of the three passes: the direct
+    implicit GEMM and Winograd F(4x4, 3x3) (chosen for wide layers).  Both run on every
     such shape; the Winograd transforms cost about a digit (errors of a few 1e-6 of the output's
     magnitude against ~1e-7), far inside the 2e-3 bar, and `_run` holds both to 1e-4."""
     from tsplit_amd import gpu_links as L
@@ -150,6 +150,7 @@ def test_conv_3x3_direct_and_winograd(case, winograd, rng, monkeypatch):
     N, C, H, W, Oc = case[:5]
     assert L.conv_takes_winograd(N, C, Oc, H, W) == (winograd == "1")
     assert L.conv_takes_winograd(N, C, Oc, H, W, data_gradient=True) == (winograd == "1")
+    assert L.conv_takes_winograd(N, C, Oc, H, W, filter_gradient=True) == (winograd == "1")
     _run(case, "cudnn", rng)
 
 
@@ -160,6 +161,8 @@ def test_conv_winograd_choice(monkeypatch):
     monkeypatch.delenv("TSPLIT_CONV_WINOGRAD", raising=False)
     assert L.conv_takes_winograd(64, 256, 256, 56, 56) and L.conv_takes_winograd(64, 256, 256, 56, 56, data_gradient=True)
     assert L.conv_takes_winograd(16, 64, 128, 112, 112) and L.conv_takes_winograd(64, 512, 512, 14, 14)
+    assert L.conv_takes_winograd(64, 256, 256, 56, 56, filter_gradient=True)
+    assert not L.conv_takes_winograd(16, 64, 128, 112, 112, filter_gradient=True)   # two transforms: needs both wide
     assert not L.conv_takes_winograd(64, 64, 64, 224, 224)           # too narrow: the transforms outweigh the GEMMs
     assert not L.conv_takes_winograd(2, 256, 256, 14, 14)            # too few tiles
     assert not L.conv_takes_winograd(64, 3, 64, 224, 224)
@@ -167,6 +170,8 @@ def test_conv_winograd_choice(monkeypatch):
     assert L.conv_takes_winograd(2, 16, 16, 5, 5)
     assert not L.conv_takes_winograd(2, 24, 16, 5, 5)                # channels summed over must be a multiple of 16
     assert L.conv_takes_winograd(2, 24, 16, 5, 5, data_gradient=True)
+    assert L.conv_takes_winograd(2, 24, 20, 5, 5, filter_gradient=True)   # any channel counts
+    assert not L.conv_takes_winograd(2, 3, 20, 5, 5, filter_gradient=True)  # at most 32 filter columns: the narrow kernel
     for kernel, pad, stride in ((3, 1, 2), (3, 0, 1), (1, 0, 1), (5, 2, 1)):
         assert not L.conv_takes_winograd(64, 256, 256, 56, 56, kernel, pad, stride)
     monkeypatch.setenv("TSPLIT_CONV_WINOGRAD", "0")
@@ -183,6 +188,12 @@ def test_conv_winograd_is_per_image_and_repeatable(rng, monkeypatch):
     w = rng.normal(size=(48, 32, 3, 3)).astype(np.float32)
     dy = rng.normal(size=(8, 48, 20, 24)).astype(np.float32)
     gx, gw, gdy = ndarray.array(x, ctx), ndarray.array(w, ctx), ndarray.array(dy, ctx)
+    dws = []
+    for _ in range(2):                     # the filter gradient sums over images: repeatable, not splittable
+        dw = ndarray.empty(w.shape, ctx)
+        L.CuDNN_conv2d_gradient_of_filter(gx, gdy, dw, 1, 1, 1)
+        dws.append(dw.asnumpy())
+    np.testing.assert_array_equal(dws[0], dws[1])
 
     def both(split):
         y, dx = ndarray.empty(dy.shape, ctx), ndarray.empty(x.shape, ctx)

@@ -33,6 +33,8 @@ namespace tsplit {
 // winograd.hip
 int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int gathered, int produced, int H, int W,
                       bool rotated, hipStream_t st);
+int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, int imgs, int C, int O, int H, int W,
+                                  hipStream_t st);
 namespace {
 
 using namespace mg;
@@ -2024,18 +2026,36 @@ int launch_conv_thin_fwd(const ConvGeo &g, const float *x, const float *w, float
 // F(4x4, 3x3) routine (winograd.hip): a quarter of the multiplications for 2.25x the activation
 // traffic.  TSPLIT_CONV_WINOGRAD=0 switches it off, =1 takes it wherever the shape allows.
 
-inline bool winograd_pays(const ConvGeo &g, int gathered, int produced) {
+inline int winograd_forced() {
   const char *e = std::getenv("TSPLIT_CONV_WINOGRAD");
-  const int forced = e ? (e[0] == '1' ? 1 : 0) : -1;
-  const bool fits = g.kH == 3 && g.kW == 3 && g.s == 1 && g.ph == 1 && g.pw == 1 && g.oH == g.H && g.oW == g.W &&
-                    gathered % BK == 0 && static_cast<int64_t>(std::max(gathered, produced)) * g.H * g.W < (1ll << 29);
-  if (!fits || forced == 0) return false;
-  if (forced == 1) return true;
-  // wide enough for the 36 GEMMs to outweigh the transforms, little of the 4x4 tiling hanging over
-  // the plane's edge, and enough tiles to fill the chip
+  return e ? (e[0] == '1' ? 1 : 0) : -1;
+}
+
+inline bool winograd_shape(const ConvGeo &g) {
+  return g.kH == 3 && g.kW == 3 && g.s == 1 && g.ph == 1 && g.pw == 1 && g.oH == g.H && g.oW == g.W &&
+         static_cast<int64_t>(std::max(g.C, g.O)) * g.H * g.W < (1ll << 29);
+}
+
+// wide enough for the 36 GEMMs to outweigh the transforms (the filter gradient transforms two
+// activation tensors, so it needs both channel counts large), little of the 4x4 tiling hanging over
+// the plane's edge, and enough tiles to fill the chip
+inline bool winograd_wide(const ConvGeo &g, int narrowest) {
   const int64_t covered = static_cast<int64_t>((g.H + 3) / 4) * ((g.W + 3) / 4) * 16;
-  return std::min(gathered, produced) >= 64 && std::max(gathered, produced) >= 128 &&
+  return std::min(g.C, g.O) >= narrowest && std::max(g.C, g.O) >= 128 &&
          covered * 3 <= static_cast<int64_t>(g.H) * g.W * 4 && static_cast<int64_t>(g.imgs) * covered >= 16 * 1024;
+}
+
+// forward and data gradient: the channels summed over are the GEMMs' K
+inline bool winograd_pays(const ConvGeo &g, int gathered) {
+  const int forced = winograd_forced();
+  if (!winograd_shape(g) || gathered % BK != 0 || forced == 0) return false;
+  return forced == 1 || winograd_wide(g, 64);
+}
+
+inline bool winograd_filter_grad_pays(const ConvGeo &g) {
+  const int forced = winograd_forced();
+  if (!winograd_shape(g) || forced == 0) return false;
+  return forced == 1 || winograd_wide(g, 128);
 }
 
 int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y, int ph, int pw, int s,
@@ -2048,7 +2068,7 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
     if (thin_fwd_ok(g)) {
       const int rc = launch_conv_thin_fwd(g, cf(x), cf(w), mf(y), st);
       if (rc) return rc;
-    } else if (winograd_pays(g, g.C, g.O)) {
+    } else if (winograd_pays(g, g.C)) {
       const int rc = conv_winograd_3x3(cf(x), cf(w), mf(y), g.imgs, g.C, g.O, g.H, g.W, false, st);
       if (rc) return rc;
     } else if (g.C % BK == 0) {
@@ -2095,7 +2115,7 @@ int conv_bwd_data(const char *who, const DLArray *w, const DLArray *dy, DLArray 
   if (geo_from(who, dx, w, dy, ph, pw, s, g)) return -1;
   hipStream_t st = stream_of(sh);
   ProfileScope ps(p, st, numel(dy) + numel(w), numel(dx), numel(w));
-  if (numel(dx) > 0 && winograd_pays(g, g.O, g.C)) {
+  if (numel(dx) > 0 && winograd_pays(g, g.O)) {
     const int rc = conv_winograd_3x3(cf(dy), cf(w), mf(dx), g.imgs, g.O, g.C, g.H, g.W, true, st);
     if (rc) return rc;
   } else if (numel(dx) > 0) {
@@ -2167,6 +2187,8 @@ int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArra
   if (numel(dw) > 0) {
     if (wgrad_narrow_ok(g)) {
       rc = launch_wgrad_narrow(g, cf(x), cf(dy), mf(dw), st, &ws);
+    } else if (winograd_filter_grad_pays(g)) {
+      rc = conv_winograd_3x3_filter_grad(cf(x), cf(dy), mf(dw), g.imgs, g.C, g.O, g.H, g.W, st);
     } else if (wgrad_tap_ok(g)) {
       if (short_tiles(g.O))
         rc = launch_wgrad_tap<64, 256, 1, 4>(g, cf(x), cf(dy), mf(dw), st, &ws);
@@ -2200,11 +2222,12 @@ using namespace tsplit;
 extern "C" {
 
 int TSplit_ConvTakesWinograd(int images, int in_channels, int out_channels, int height, int width, int kernel_h,
-                             int kernel_w, int pad_h, int pad_w, int stride, int data_gradient) {
+                             int kernel_w, int pad_h, int pad_w, int stride, int pass) {
   if (images <= 0 || in_channels <= 0 || out_channels <= 0 || height <= 0 || width <= 0 || stride <= 0) return 0;
   ConvGeo g{images, in_channels, height, width, out_channels, kernel_h, kernel_w, pad_h, pad_w, stride,
             (height + 2 * pad_h - kernel_h) / stride + 1, (width + 2 * pad_w - kernel_w) / stride + 1};
-  return data_gradient ? winograd_pays(g, out_channels, in_channels) : winograd_pays(g, in_channels, out_channels);
+  if (pass == 2) return winograd_filter_grad_pays(g) && !wgrad_narrow_ok(g);
+  return winograd_pays(g, pass == 1 ? out_channels : in_channels);
 }
 
 int CuDNN_DLGpuConv2d(const DLArrayHandle input_x, const DLArrayHandle input_f, DLArrayHandle output,

@@ -21,6 +21,8 @@
 // differ from the directly summed one by a few 1e-6 of the output's magnitude.
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
+#include <vector>
 
 #include "common.h"
 #include "mfma_gemm.h"
@@ -202,6 +204,168 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const float *__restric
   }
 }
 
+// ---------------------------------------------------------------- filter gradient
+// The forward map is linear in the filter, y = A^T [(G g G^T) . (B^T d B)] A per tile, so the filter
+// gradient is its adjoint: dg = G^T [ sum over tiles (A dy A^T) . (B^T d B) ] G.
+//
+// rows of A applied to (d0 .. d3)
+__device__ __forceinline__ void a_rows(const float d[4], float o[6]) {
+  const float e = d[0] + d[2], f = d[1] + d[3], p = d[0] + 4.0f * d[2], q = 2.0f * d[1] + 8.0f * d[3];
+  o[0] = d[0];
+  o[1] = e + f;
+  o[2] = e - f;
+  o[3] = p + q;
+  o[4] = p - q;
+  o[5] = d[3];
+}
+
+// Y[xi][o][t] = (A dy A^T)[xi] of the 4x4 output tile t, channel o (zero beyond the plane's edge)
+template <bool QUADS>
+__global__ __launch_bounds__(256) void wino_grad_kernel(const float *__restrict__ dy, float *__restrict__ Y, WinoGeo g) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= g.ld) return;
+  const int o = blockIdx.y;
+  float *out = Y + static_cast<int64_t>(o) * g.ld + t;
+  const int64_t plane_stride = static_cast<int64_t>(g.chans) * g.ld;
+  if (t >= g.tiles) {   // padding of the reduction: contributes nothing
+#pragma unroll
+    for (int xi = 0; xi < kXi; ++xi) out[xi * plane_stride] = 0.0f;
+    return;
+  }
+  const int per_img = g.th * g.tw;
+  const int n = t / per_img, rem = t - n * per_img;
+  const int ty = rem / g.tw, tx = rem - ty * g.tw;
+  const float *plane = dy + (static_cast<int64_t>(n) * g.chans + o) * g.H * g.W;
+  float tmp[4][6];   // tmp[q][.] = A applied down column q
+  {
+    float d[4][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int h = 4 * ty + r;
+      const bool row_ok = h < g.H;
+      const float *row = plane + static_cast<int64_t>(row_ok ? h : 0) * g.W + 4 * tx;
+      if constexpr (QUADS) {
+        float4 v = *reinterpret_cast<const float4 *>(row);
+        if (!row_ok) v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        d[r][0] = v.x;
+        d[r][1] = v.y;
+        d[r][2] = v.z;
+        d[r][3] = v.w;
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) d[r][q] = row_ok && 4 * tx + q < g.W ? row[q] : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float col[4] = {d[0][q], d[1][q], d[2][q], d[3][q]};
+      a_rows(col, tmp[q]);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 6; ++r) {
+    const float row[4] = {tmp[0][r], tmp[1][r], tmp[2][r], tmp[3][r]};
+    float v[6];
+    a_rows(row, v);
+#pragma unroll
+    for (int q = 0; q < 6; ++q) out[(r * 6 + q) * plane_stride] = v[q];
+  }
+}
+
+// 36 GEMMs dU[xi] (O x C) = Y[xi] (O x tiles) V[xi]^T, each cut along the tiles into `splits`
+// ranges of `kchunk`: block group z = split * 36 + xi writes its partial sum to out + z * O * C
+template <class ALoader, class BLoader>
+__global__ __launch_bounds__(kThreads) void wino_grad_gemm_kernel(typename ALoader::Params ap, typename BLoader::Params bp,
+                                                                   float *__restrict__ out, int64_t a_xi, int64_t b_xi, int M,
+                                                                   int N, int K, int kchunk, TileGrid tg) {
+  int z, tile_m, tile_n;
+  if (!block_tile(tg, z, tile_m, tile_n)) return;
+  const int split = z / kXi, xi = z - split * kXi;
+  ap.p += xi * a_xi;
+  bp.p += xi * b_xi;
+  const int kbegin = split * kchunk;
+  mfma_gemm_tile<128, 128, 2, 2, ALoader, BLoader, RowMajorCols>(ap, bp, out + static_cast<int64_t>(z) * M * N,
+                                                                 static_cast<int64_t>(N), RowMajorCols{}, M, N, tile_m * 128,
+                                                                 tile_n * 128, kbegin, min(K, kbegin + kchunk));
+}
+
+// rows of G^T applied to (u0 .. u5)
+__device__ __forceinline__ void gt_rows(const float u[6], float w[3]) {
+  const float s12 = u[1] + u[2], s34 = u[3] + u[4];
+  w[0] = 0.25f * u[0] - s12 * (1.0f / 6.0f) + s34 * (1.0f / 24.0f);
+  w[1] = (u[2] - u[1]) * (1.0f / 6.0f) + (u[3] - u[4]) * (1.0f / 12.0f);
+  w[2] = (s34 - s12) * (1.0f / 6.0f) + u[5];
+}
+
+// dw[o][c][3][3] = G^T (sum of the partial dU, in ascending order) G; part[(p * 36 + xi) * O * C + o * C + c]
+__global__ __launch_bounds__(256) void wino_filter_grad_kernel(const float *__restrict__ part, float *__restrict__ dw,
+                                                               int oc, int parts) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= oc) return;
+  float t[6][3];   // t[q][.] = G^T applied down column q
+#pragma unroll
+  for (int q = 0; q < 6; ++q) {
+    float col[6];
+#pragma unroll
+    for (int r = 0; r < 6; ++r) {
+      const float *src = part + static_cast<int64_t>(r * 6 + q) * oc + i;
+      float sum = src[0];
+      for (int p = 1; p < parts; ++p) sum += src[static_cast<int64_t>(p) * kXi * oc];
+      col[r] = sum;
+    }
+    gt_rows(col, t[q]);
+  }
+#pragma unroll
+  for (int r = 0; r < 3; ++r) {
+    const float row[6] = {t[0][r], t[1][r], t[2][r], t[3][r], t[4][r], t[5][r]};
+    float w[3];
+    gt_rows(row, w);
+#pragma unroll
+    for (int q = 0; q < 3; ++q) dw[static_cast<int64_t>(i) * 9 + r * 3 + q] = w[q];
+  }
+}
+
+// ---------------------------------------------------------------- GEMM launch timing (opt-in)
+// With TSplit_WinogradGemmTiming(1) every GEMM launch below is bracketed by two events on its own
+// stream, so a benchmark can read the duration of these kernels inside its timed region.
+struct TimedLaunch {
+  hipEvent_t begin, end;
+  int which;       // 0: forward / data-gradient GEMMs, 1: filter-gradient GEMMs
+  double flop;
+};
+std::mutex g_timing_mu;
+bool g_timing_on = false;
+std::vector<TimedLaunch> g_timed;
+
+class GemmTiming {
+ public:
+  GemmTiming(hipStream_t st, int which, double flop) : st_(st) {
+    std::lock_guard<std::mutex> lk(g_timing_mu);
+    if (!g_timing_on) return;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return;
+    if (hipEventCreate(&t_.begin) != hipSuccess) return;
+    if (hipEventCreate(&t_.end) != hipSuccess) {
+      (void)hipEventDestroy(t_.begin);
+      return;
+    }
+    t_.which = which;
+    t_.flop = flop;
+    on_ = hipEventRecord(t_.begin, st) == hipSuccess;
+  }
+  ~GemmTiming() {
+    if (!on_) return;
+    (void)hipEventRecord(t_.end, st_);
+    std::lock_guard<std::mutex> lk(g_timing_mu);
+    g_timed.push_back(t_);
+  }
+
+ private:
+  hipStream_t st_;
+  TimedLaunch t_{};
+  bool on_ = false;
+};
+
 // bytes of V and M one run of images may take together
 inline int64_t run_bytes() {
   const char *e = std::getenv("TSPLIT_WINOGRAD_RUN_MIB");
@@ -247,13 +411,109 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
     const int tm = (produced + 127) / 128, tn = (gi.ld + 127) / 128;
     typename AL::Params ap{U, gathered, produced, gathered};
     typename BL::Params bp{V, gi.ld, gi.ld, gathered};
-    hipLaunchKernelGGL((mfma_batched_gemm_kernel<128, 128, 2, 2, AL, BL>), dim3(grid_blocks(tm, tn, kXi)), dim3(kThreads),
-                       0, st, ap, bp, M, static_cast<int64_t>(produced) * gathered, static_cast<int64_t>(gathered) * gi.ld,
-                       static_cast<int64_t>(produced) * gi.ld, produced, gi.ld, gathered, TileGrid{tm, tn, tm * tn * kXi});
+    {
+      GemmTiming timed(st, 0, 2.0 * kXi * produced * static_cast<double>(gi.ld) * gathered);
+      hipLaunchKernelGGL((mfma_batched_gemm_kernel<128, 128, 2, 2, AL, BL>), dim3(grid_blocks(tm, tn, kXi)),
+                         dim3(kThreads), 0, st, ap, bp, M, static_cast<int64_t>(produced) * gathered,
+                         static_cast<int64_t>(gathered) * gi.ld, static_cast<int64_t>(produced) * gi.ld, produced, gi.ld,
+                         gathered, TileGrid{tm, tn, tm * tn * kXi});
+    }
     hipLaunchKernelGGL(wino_output_kernel, dim3((go.tiles + 255) / 256, produced), dim3(256), 0, st, M,
                        y + static_cast<int64_t>(first) * produced * H * W, go);
   }
   return 0;
 }
 
+// dw[O][C][3][3] = filter gradient of the 3x3 / stride 1 / pad 1 convolution of x[n][C][H][W] whose output
+// gradient is dy[n][O][H][W]
+int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, int imgs, int C, int O, int H, int W,
+                                  hipStream_t st) {
+  const int th = (H + 3) / 4, tw = (W + 3) / 4;
+  const int per_img = th * tw;
+  const int64_t img_bytes = static_cast<int64_t>(C + O) * kXi * 4 * per_img;
+  int run = static_cast<int>(std::max<int64_t>(1, run_bytes() / img_bytes));
+  run = std::min(run, imgs);
+  const int runs = (imgs + run - 1) / run;
+  run = (imgs + runs - 1) / runs;
+  const int ld_max = (run * per_img + 3) / 4 * 4;
+  TS_REQUIRE(static_cast<int64_t>(std::max(C, O)) * ld_max * 4 < (1ll << 31),
+             "conv (Winograd): a run of %d images does not fit 32-bit offsets", run);
+  // enough blocks for three per CU, each with at least 16 k-steps
+  const int tm = (O + 127) / 128, tn = (C + 127) / 128;
+  int splits = std::max(1, (768 + kXi * tm * tn / 2) / (kXi * tm * tn));
+  splits = std::min(splits, std::max(1, ld_max / (16 * BK)));
+  const int kchunk = ((ld_max + splits - 1) / splits + BK - 1) / BK * BK;
+  const int parts_max = runs * ((ld_max + kchunk - 1) / kchunk);
+  const int64_t oc = static_cast<int64_t>(O) * C;
+  float *VY = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(kXi) * (C + O) * ld_max * 4));
+  float *part = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(parts_max) * kXi * oc * 4));
+  TS_REQUIRE(VY && part, "conv (Winograd): no scratch memory");
+  float *V = VY, *Y = VY + static_cast<int64_t>(kXi) * C * ld_max;
+  using KL = KContigBufLoader<128>;
+  int parts = 0;
+  for (int first = 0; first < imgs; first += run) {
+    const int n = std::min(run, imgs - first);
+    const float *xr = x + static_cast<int64_t>(first) * C * H * W, *dyr = dy + static_cast<int64_t>(first) * O * H * W;
+    WinoGeo gx{C, H, W, th, tw, n * per_img, (n * per_img + 3) / 4 * 4, false};
+    WinoGeo gy = gx;
+    gy.chans = O;
+    const dim3 grid_x((gx.ld + 255) / 256, C), grid_y((gx.ld + 255) / 256, O);
+    if ((W & 3) == 0 && (reinterpret_cast<uintptr_t>(xr) & 15) == 0)
+      hipLaunchKernelGGL(wino_input_kernel<true>, grid_x, dim3(256), 0, st, xr, V, gx);
+    else
+      hipLaunchKernelGGL(wino_input_kernel<false>, grid_x, dim3(256), 0, st, xr, V, gx);
+    if ((W & 3) == 0 && (reinterpret_cast<uintptr_t>(dyr) & 15) == 0)
+      hipLaunchKernelGGL(wino_grad_kernel<true>, grid_y, dim3(256), 0, st, dyr, Y, gy);
+    else
+      hipLaunchKernelGGL(wino_grad_kernel<false>, grid_y, dim3(256), 0, st, dyr, Y, gy);
+    const int here = (gx.ld + kchunk - 1) / kchunk;
+    typename KL::Params ap{Y, gx.ld, O, gx.ld};
+    typename KL::Params bp{V, gx.ld, C, gx.ld};
+    {
+      GemmTiming timed(st, 1, 2.0 * kXi * O * static_cast<double>(gx.ld) * C);
+      hipLaunchKernelGGL((wino_grad_gemm_kernel<KL, KL>), dim3(grid_blocks(tm, tn, kXi * here)), dim3(kThreads), 0, st, ap,
+                         bp, part + static_cast<int64_t>(parts) * kXi * oc, static_cast<int64_t>(O) * gx.ld,
+                         static_cast<int64_t>(C) * gx.ld, O, C, gx.ld, kchunk, TileGrid{tm, tn, tm * tn * kXi * here});
+    }
+    parts += here;
+  }
+  hipLaunchKernelGGL(wino_filter_grad_kernel, dim3(static_cast<unsigned>((oc + 255) / 256)), dim3(256), 0, st, part, dw,
+                     static_cast<int>(oc), parts);
+  return 0;
+}
+
 }  // namespace tsplit
+
+// Switches the timing of the Winograd routine's GEMM launches on or off (and forgets what was recorded).
+extern "C" int TSplit_WinogradGemmTiming(int on) {
+  using namespace tsplit;
+  std::lock_guard<std::mutex> lk(g_timing_mu);
+  for (TimedLaunch &t : g_timed) {
+    (void)hipEventDestroy(t.begin);
+    (void)hipEventDestroy(t.end);
+  }
+  g_timed.clear();
+  g_timing_on = on != 0;
+  return 0;
+}
+
+// Waits for the recorded launches of kind `which` and reports their number, summed duration in
+// milliseconds and summed GEMM FLOP (2 * 36 * rows * columns * depth per launch); -1 on a HIP error.
+extern "C" int TSplit_WinogradGemmTimes(int which, double *launches, double *ms, double *flop) {
+  using namespace tsplit;
+  std::lock_guard<std::mutex> lk(g_timing_mu);
+  double n = 0, total = 0, work = 0;
+  for (const TimedLaunch &t : g_timed) {
+    if (t.which != which) continue;
+    float one = 0.0f;
+    TS_HIP(hipEventSynchronize(t.end));
+    TS_HIP(hipEventElapsedTime(&one, t.begin, t.end));
+    n += 1;
+    total += one;
+    work += t.flop;
+  }
+  if (launches) *launches = n;
+  if (ms) *ms = total;
+  if (flop) *flop = work;
+  return 0;
+}

@@ -400,12 +400,28 @@ def sigmoid(in_arr, out_arr, stream=None, profiler=None):
 
 
 # ---- Which routine a convolution takes (no counterpart in the reference's gpu_links) ----
-def conv_takes_winograd(images, in_channels, out_channels, height, width, kernel=3, pad=1, stride=1, data_gradient=False):
-    """True when the library runs this layer's forward pass (or, with `data_gradient`, its data
-    gradient) through the Winograd F(4x4, 3x3) routine rather than the direct implicit GEMM."""
+def conv_takes_winograd(images, in_channels, out_channels, height, width, kernel=3, pad=1, stride=1, data_gradient=False,
+                        filter_gradient=False):
+    """True when the library runs this layer's forward pass (or, with `data_gradient` /
+    `filter_gradient`, that gradient) through the Winograd F(4x4, 3x3) routine rather than the
+    direct implicit GEMM."""
+    which = 2 if filter_gradient else 1 if data_gradient else 0
     return bool(_LIB.TSplit_ConvTakesWinograd(int(images), int(in_channels), int(out_channels), int(height), int(width),
-                                              int(kernel), int(kernel), int(pad), int(pad), int(stride),
-                                              int(bool(data_gradient))))
+                                              int(kernel), int(kernel), int(pad), int(pad), int(stride), which))
+
+
+def winograd_gemm_timing(on):
+    """Switch the event timing of the GEMM launches inside the Winograd routine on or off."""
+    check_call(_LIB.TSplit_WinogradGemmTiming(int(bool(on))))
+
+
+def winograd_gemm_times(filter_gradient=False):
+    """-> (launches, total ms, total executed FLOP) of the timed GEMM launches of the forward /
+    data-gradient routine, or of the filter-gradient routine."""
+    n, ms, flop = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+    check_call(_LIB.TSplit_WinogradGemmTimes(int(bool(filter_gradient)), ctypes.byref(n), ctypes.byref(ms),
+                                             ctypes.byref(flop)))
+    return int(n.value), ms.value, flop.value
 
 
 # ---- Fused BatchNorm + Relu (no counterpart in the reference's gpu_links) ----

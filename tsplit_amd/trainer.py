@@ -261,7 +261,10 @@ class Trainer(object):
                                   L.CuDNN_conv2d_gradient_of_filter, xa, ga, dw if i == 0 else self.dw_piece[li],
                                   pad, pad, stride)
                     else:
-                        self._run("conv_bwd_filter_" + self._tile(cout), 2.0 * n(ga.shape) * cin * k * k, "flop",
+                        wino = L.conv_takes_winograd(xa.shape[0], cin, cout, xa.shape[2], xa.shape[3], k, pad, stride,
+                                                     filter_gradient=True)
+                        self._run("conv_bwd_filter_winograd" if wino else "conv_bwd_filter_" + self._tile(cout),
+                                  2.0 * n(ga.shape) * cin * k * k, "flop",
                                   L.CuDNN_conv2d_gradient_of_filter, xa, ga, dw if i == 0 else self.dw_piece[li],
                                   pad, pad, stride)
                     if i > 0:
