@@ -46,14 +46,16 @@ GiB = float(1 << 30)
 
 
 class CostModel(object):
-    """Rates measured on one MI355X with this library (fp32): contractions, streaming
+    """Rates measured on one MI355X with this library (fp32): contractions (for wide 3x3 layers the
+    rate of the direct algorithm's FLOP count under the Winograd routine), streaming
     kernels on the bytes they move, the pinned-host link each way, and what one host-side
     event wait costs the compute stream (the host has to catch up with its launches afterwards;
     a swapped tensor brings one such wait on the way out and one on the way in)."""
 
     def __init__(self, conv_tflops=110.0, conv_tflops_narrow=90.0, matmul_tflops=65.0, stream_gbs=5500.0,
-                 link_gbs=55.0, host_wait_ms=0.2):
+                 link_gbs=55.0, host_wait_ms=0.2, conv_tflops_winograd=240.0):
         self.host_wait_ms = host_wait_ms
+        self.conv_tflops_winograd = conv_tflops_winograd
         self.conv_tflops = conv_tflops
         self.conv_tflops_narrow = conv_tflops_narrow
         self.matmul_tflops = matmul_tflops
@@ -68,9 +70,11 @@ class CostModel(object):
         n_in, n_out = float(np.prod(in_shape)), float(np.prod(out_shape))
         kind = layer[0]
         if kind == "conv":
-            _, _, cin, cout, k, _, _ = layer
+            _, _, cin, cout, k, pad, stride = layer
             flop = 2.0 * n_out * cin * k * k
             rate = self.conv_tflops if min(cin, cout) > 64 else self.conv_tflops_narrow
+            if (k, pad, stride) == (3, 1, 1) and min(cin, cout) >= 64 and max(cin, cout) >= 128:
+                rate = self.conv_tflops_winograd     # wide 3x3 layers run through the Winograd routine
             passes = (1 if first else 2) if backward else 1
             return passes * flop / (rate * 1e12) * 1e3
         if kind == "fc":
