@@ -297,6 +297,15 @@ __device__ __forceinline__ void gt_rows(const float u[6], float w[3]) {
   w[2] = (s34 - s12) * (1.0f / 6.0f) + u[5];
 }
 
+// part[i] = sum over p of part[p * n + i], p ascending (in place: every thread owns its elements)
+__global__ __launch_bounds__(256) void wino_fold_kernel(float *__restrict__ part, int64_t n, int parts) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n) return;
+  float sum = part[i];
+  for (int p = 1; p < parts; ++p) sum += part[p * n + i];
+  part[i] = sum;
+}
+
 // dw[o][c][3][3] = G^T (sum of the partial dU, in ascending order) G; part[(p * 36 + xi) * O * C + o * C + c]
 __global__ __launch_bounds__(256) void wino_filter_grad_kernel(const float *__restrict__ part, float *__restrict__ dw,
                                                                int oc, int parts) {
@@ -373,6 +382,18 @@ inline int64_t run_bytes() {
   return static_cast<int64_t>(mibs > 0 ? mibs : 1024) << 20;
 }
 
+// images per run: what the scratch allowance holds of both transformed tensors, within reach of the GEMM
+// loaders' 32-bit byte offsets (one transformed plane set is channels x tiles floats), in equal runs
+inline int run_images(int imgs, int per_img, int chans_a, int chans_b) {
+  const int64_t img_bytes = static_cast<int64_t>(chans_a + chans_b) * kXi * 4 * per_img;
+  const int64_t reach = ((1ll << 31) - 64) / (4ll * std::max(chans_a, chans_b)) / per_img;
+  int64_t run = std::min<int64_t>(std::max<int64_t>(1, run_bytes() / img_bytes), reach);
+  if (run < 1) return 0;
+  run = std::min<int64_t>(run, imgs);
+  const int64_t runs = (imgs + run - 1) / run;
+  return static_cast<int>((imgs + runs - 1) / runs);
+}
+
 }  // namespace
 
 // y[n][produced][H][W] = conv3x3(x[n][gathered][H][W], filter), stride 1, pad 1.  `rotated` selects
@@ -381,14 +402,9 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
                       bool rotated, hipStream_t st) {
   const int th = (H + 3) / 4, tw = (W + 3) / 4;
   const int per_img = th * tw;
-  const int64_t img_bytes = static_cast<int64_t>(gathered + produced) * kXi * 4 * per_img;
-  int run = static_cast<int>(std::max<int64_t>(1, run_bytes() / img_bytes));
-  run = std::min(run, imgs);
-  const int runs = (imgs + run - 1) / run;
-  run = (imgs + runs - 1) / runs;   // equal runs
+  const int run = run_images(imgs, per_img, gathered, produced);
+  TS_REQUIRE(run > 0, "conv (Winograd): one image's tiles do not fit 32-bit offsets");
   const int ld_max = (run * per_img + 3) / 4 * 4;
-  TS_REQUIRE(static_cast<int64_t>(std::max(gathered, produced)) * ld_max * 4 < (1ll << 31),
-             "conv (Winograd): a run of %d images does not fit 32-bit offsets", run);
   float *U = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(kXi) * produced * gathered * 4));
   float *VM = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(kXi) * (gathered + produced) * ld_max * 4));
   TS_REQUIRE(U && VM, "conv (Winograd): no scratch memory");
@@ -430,14 +446,10 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
                                   hipStream_t st) {
   const int th = (H + 3) / 4, tw = (W + 3) / 4;
   const int per_img = th * tw;
-  const int64_t img_bytes = static_cast<int64_t>(C + O) * kXi * 4 * per_img;
-  int run = static_cast<int>(std::max<int64_t>(1, run_bytes() / img_bytes));
-  run = std::min(run, imgs);
+  const int run = run_images(imgs, per_img, C, O);
+  TS_REQUIRE(run > 0, "conv (Winograd): one image's tiles do not fit 32-bit offsets");
   const int runs = (imgs + run - 1) / run;
-  run = (imgs + runs - 1) / runs;
   const int ld_max = (run * per_img + 3) / 4 * 4;
-  TS_REQUIRE(static_cast<int64_t>(std::max(C, O)) * ld_max * 4 < (1ll << 31),
-             "conv (Winograd): a run of %d images does not fit 32-bit offsets", run);
   // enough blocks for three per CU, each with at least 16 k-steps
   const int tm = (O + 127) / 128, tn = (C + 127) / 128;
   int splits = std::max(1, (768 + kXi * tm * tn / 2) / (kXi * tm * tn));
@@ -477,8 +489,13 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
     }
     parts += here;
   }
+  // many partial sums for few filter elements (narrow layers cut into many ranges): fold them with one
+  // thread per element first, so that the final transform's threads do not each walk all of them
+  if (parts > 1)
+    hipLaunchKernelGGL(wino_fold_kernel, dim3(static_cast<unsigned>((kXi * oc + 255) / 256)), dim3(256), 0, st, part,
+                       kXi * oc, parts);
   hipLaunchKernelGGL(wino_filter_grad_kernel, dim3(static_cast<unsigned>((oc + 255) / 256)), dim3(256), 0, st, part, dw,
-                     static_cast<int>(oc), parts);
+                     static_cast<int>(oc), 1);
   return 0;
 }
 
