@@ -67,10 +67,15 @@ def test_convnet_momentum_tracks_oracle_with_and_without_split(split, fuse):
         assert_close(t.params[k].asnumpy(), ref_params[k], 2e-3, k)
 
 
-def test_vgg16_topology_small_resolution_tracks_oracle():
+@pytest.mark.parametrize("winograd", [None, "1"])
+def test_vgg16_topology_small_resolution_tracks_oracle(winograd, monkeypatch):
     """The full VGG-16 layer list (13 conv+BN+Relu, 5 pools, 3 FC) at 32x32, batch 4, with the
-    two largest-resolution blocks run as 2 micro-tensors: 3 momentum steps against the oracle."""
+    two largest-resolution blocks run as 2 micro-tensors: 3 momentum steps against the oracle.
+    Once as the library routes these small layers itself (direct kernels), once with every layer but
+    the first forced through the Winograd routine in all three passes."""
     from tsplit_amd import ndarray, trainer
+    if winograd:
+        monkeypatch.setenv("TSPLIT_CONV_WINOGRAD", winograd)
     rng = np.random.RandomState(11)
     spec = trainer.vgg16_spec(num_classes=10, in_hw=32)
     X = rng.normal(size=(4, 3, 32, 32)).astype(np.float32)
