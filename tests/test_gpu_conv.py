@@ -162,7 +162,9 @@ def test_conv_winograd_choice(monkeypatch):
     assert L.conv_takes_winograd(64, 256, 256, 56, 56) and L.conv_takes_winograd(64, 256, 256, 56, 56, data_gradient=True)
     assert L.conv_takes_winograd(16, 64, 128, 112, 112) and L.conv_takes_winograd(64, 512, 512, 14, 14)
     assert L.conv_takes_winograd(64, 256, 256, 56, 56, filter_gradient=True)
-    assert not L.conv_takes_winograd(16, 64, 128, 112, 112, filter_gradient=True)   # two transforms: needs both wide
+    assert L.conv_takes_winograd(16, 64, 128, 112, 112, filter_gradient=True)
+    assert L.conv_takes_winograd(16, 64, 64, 224, 224, filter_gradient=True)        # no transformed output to write: pays earlier
+    assert not L.conv_takes_winograd(16, 32, 64, 224, 224, filter_gradient=True)
     assert not L.conv_takes_winograd(64, 64, 64, 224, 224)           # too narrow: the transforms outweigh the GEMMs
     assert not L.conv_takes_winograd(2, 256, 256, 14, 14)            # too few tiles
     assert not L.conv_takes_winograd(64, 3, 64, 224, 224)
