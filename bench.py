@@ -43,7 +43,7 @@ TRAFFIC_BYTES_PER_LAUNCH = {
     "conv_bwd_data_128x128": (523.5 + 147.5) * 1e6,
     "conv_bwd_filter_128x128": (523.2 + 64.2) * 1e6,
     "winograd_gemm": (243.6 + 220.6) * 1e6,
-    "winograd_filter_grad_gemm": (553.8 + 45.3) * 1e6,
+    "winograd_filter_grad_gemm": (586.8 + 35.1) * 1e6,
 }
 
 
