@@ -34,17 +34,41 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS_FP32_MFMA = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch (read + write, mean over the launches of one step) of the kernels that can
-# be the step's largest, from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
-# profiles/vgg16_b64_train_step_hbm_traffic.txt (counter units calibrated on the Relu kernel; forward and
-# backward-data run as two register-budget variants of one kernel, averaged here over both by launch count).
-TRAFFIC_BYTES_PER_LAUNCH = {
-    "conv_fwd_128x128": (388.2 + 158.1) * 1e6,
-    "conv_bwd_data_128x128": (523.5 + 147.5) * 1e6,
-    "conv_bwd_filter_128x128": (523.2 + 64.2) * 1e6,
-    "winograd_gemm": (243.6 + 220.6) * 1e6,
-    "winograd_filter_grad_gemm": (586.8 + 35.1) * 1e6,
+# Kernel names (as rocprofv3 prints them) behind the operator classes that can be the step's largest
+# single kernel; their HBM bytes per launch are read from the counter summary under profiles/.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "vgg16_b64_train_step_hbm_traffic.txt")
+TRAFFIC_KERNELS = {
+    "conv_fwd_128x128": ("conv_tap_kernel<128, 128, 2, 2, false",),
+    "conv_bwd_data_128x128": ("conv_tap_kernel<128, 128, 2, 2, true",),
+    "conv_fwd_64x256": ("conv_tap_kernel<64, 256, 1, 4, false",),
+    "conv_bwd_data_64x256": ("conv_tap_kernel<64, 256, 1, 4, true",),
+    "conv_bwd_filter_128x128": ("conv_wgrad_tap_kernel<128, 128",),
+    "winograd_gemm": ("wino_gemm_kernel", "mfma_batched_gemm_kernel<128, 128, 2, 2, KContigBufLoader<128>, MnContigBufLoader<128>"),
+    "winograd_filter_grad_gemm": ("wino_grad_gemm_kernel",),
 }
+
+
+def traffic_bytes_per_launch(tag):
+    """HBM bytes one launch of the class's kernel moves (read + write, mean over the launches of a step),
+    from the FETCH_SIZE / WRITE_SIZE summary committed under profiles/ (columns: kernel, launches, read MB,
+    write MB; several variants of one kernel are averaged by launch count).  None when the summary does
+    not list the kernel: the figure is never a constant typed in here."""
+    names = TRAFFIC_KERNELS.get(tag)
+    if not names or not os.path.exists(TRAFFIC_PROFILE):
+        return None
+    launches = total = 0.0
+    with open(TRAFFIC_PROFILE) as f:
+        for line in f:
+            if not any(line.startswith(n) for n in names):
+                continue
+            cols = line.split()
+            try:
+                n, rd, wr = float(cols[-3]), float(cols[-2]), float(cols[-1])
+            except (ValueError, IndexError):
+                continue
+            launches += n
+            total += n * (rd + wr) * 1e6
+    return total / launches if launches else None
 
 
 def vgg_workload(batch, seed=123):
@@ -76,9 +100,18 @@ def cpu_baseline(sample_batch=16, seed=123):
         cores = max([p.get("num_threads", 1) for p in threadpoolctl.threadpool_info()] or [1])
     except Exception:
         cores = os.cpu_count() or 1
-    return {"value": sample_batch / dt, "unit": "samples/s", "cores": int(cores), "kind": "port",
+    return {"value": sample_batch / dt, "unit": "samples/s", "cores": int(cores), "kind": "port", "loss": loss,
             "sample": "one VGG-16 fwd+bwd+momentum step on %d of the 64 seeded images, numpy oracle in float64 "
                       "(%.1f s, loss %.4f)" % (sample_batch, dt, loss)}
+
+
+def gpu_loss_on_sample(ctx, sample_batch=16, seed=123):
+    """First-step loss of the GPU path on the sample the CPU baselines run (untimed)."""
+    from tsplit_amd import ndarray, trainer
+    spec, params, x, labels, split = vgg_workload(sample_batch, seed)
+    t = trainer.Trainer(spec, params, x.shape, 1000, ctx, optimizer=("momentum", 0.01, 0.9), split=split)
+    t.forward(ndarray.array(x, ctx), ndarray.array(labels, ctx))
+    return t.loss_value()
 
 
 def cpu_baseline_onednn(sample_batch=16, seed=123):
@@ -129,7 +162,7 @@ def cpu_baseline_onednn(sample_batch=16, seed=123):
     loss = step()
     dt = time.perf_counter() - t0
     return {"value": sample_batch / dt, "unit": "samples/s", "cores": int(torch.get_num_threads()), "kind": "library",
-            "sample": "one VGG-16 fwd+bwd+momentum step on %d of the 64 seeded images, PyTorch-CPU %s with its "
+            "loss": loss, "sample": "one VGG-16 fwd+bwd+momentum step on %d of the 64 seeded images, PyTorch-CPU %s with its "
                       "bundled oneDNN, fp32 (%.2f s, loss %.4f)" % (sample_batch, torch.__version__, dt, loss)}
 
 
@@ -193,17 +226,27 @@ def main():
                             "ms_avg": d["ms_avg"], "achieved": d["rate"],
                             "unit": "TFLOP/s" if d["unit"] == "flop" else "GB/s", "frac": d["rate"] / peak}
             if tag.endswith("_winograd"):
-                kernels[tag]["note"] = "several kernels per call; rate of the direct algorithm's FLOP count"
+                # several kernels per call, and a quarter of the direct algorithm's multiplications are
+                # executed: the rate below is on the direct FLOP count and is no fraction of any peak
+                del kernels[tag]["frac"]
+                kernels[tag]["note"] = ("several kernels per call; rate of the direct algorithm's FLOP count, of which the "
+                                        "Winograd GEMMs execute a quarter (see winograd_gemm / winograd_filter_grad_gemm)")
+            if "bytes" in d:      # near the ridge: both fractions
+                kernels[tag]["hbm_achieved_gbs"] = d["bytes"] / (d["ms_total"] * 1e-3) / 1e9
+                kernels[tag]["hbm_frac"] = kernels[tag]["hbm_achieved_gbs"] / PEAK_HBM_GBS
         # the GEMM kernels inside the Winograd calls, timed by the library with event pairs on the
         # compute stream around each launch; their work is the FLOP they execute
+        wino_exec_flop = 0.0
         for tag, grad in (("winograd_gemm", False), ("winograd_filter_grad_gemm", True)):
             launches, ms, flop = L.winograd_gemm_times(filter_gradient=grad)
             if launches:
+                wino_exec_flop += flop
                 k[tag] = {"calls": launches, "ms_total": ms, "ms_avg": ms / launches, "work": flop,
                           "work_per_call": flop / launches, "rate": flop / (ms * 1e-3) / 1e12, "unit": "flop"}
                 kernels[tag] = {"calls_per_step": launches / a.steps, "ms_per_step": ms / a.steps, "ms_avg": ms / launches,
                                 "achieved": k[tag]["rate"], "unit": "TFLOP/s", "frac": k[tag]["rate"] / PEAK_TFLOPS_FP32_MFMA,
-                                "note": "one kernel inside the *_winograd calls above (its time is part of theirs)"}
+                                "note": "one kernel inside the *_winograd calls above (its time is part of theirs); "
+                                        "executed FLOP"}
         L.winograd_gemm_timing(False)
         kernels = dict(sorted(kernels.items(), key=lambda kv: -kv[1]["ms_per_step"]))
         dom = next(tag for tag in kernels if not tag.endswith("_winograd"))
@@ -212,31 +255,45 @@ def main():
                            "achieved": dd["rate"], "peak": PEAK_TFLOPS_FP32_MFMA if dd["unit"] == "flop" else PEAK_HBM_GBS,
                            "unit": "TFLOP/s" if dd["unit"] == "flop" else "GB/s",
                            "frac": dd["rate"] / (PEAK_TFLOPS_FP32_MFMA if dd["unit"] == "flop" else PEAK_HBM_GBS),
-                           "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dom) if split and a.batch == 64 else None,
+                           "traffic": traffic_bytes_per_launch(dom) if split and a.batch == 64 and not a.fused else None,
                            "per_launch": dd["work_per_call"], "ms_avg": dd["ms_avg"]}
-        # all conv FLOP over all conv time; the thin first layer (Cin*kH*kW = 27) is timed in bytes
-        # because HBM bounds it, so its FLOP (forward and filter gradient) are added here
-        conv = [d for tag, d in k.items() if tag.startswith("conv_")]      # the Winograd GEMMs' time is inside these
-        conv_flop = sum(d["work"] for d in conv if d["unit"] == "flop")
+        # Conv utilisation, two ways.  The thin first layer (Cin*kH*kW = 27) is timed in bytes because
+        # HBM bounds it, so its FLOP (forward and filter gradient) are added to both counts.
+        conv = {tag: d for tag, d in k.items() if tag.startswith("conv_")}      # the Winograd GEMMs' time is inside these
+        thin_flop = 0.0
         shape = x.shape
         for layer in spec:
             if layer[0] == "conv":
                 if layer[2] * layer[4] * layer[4] <= 32:
-                    conv_flop += a.steps * 2 * 2.0 * shape[0] * layer[3] * shape[2] * shape[3] * layer[2] * layer[4] ** 2
+                    thin_flop += a.steps * 2 * 2.0 * shape[0] * layer[3] * shape[2] * shape[3] * layer[2] * layer[4] ** 2
                 shape = (shape[0], layer[3], shape[2], shape[3])
             elif layer[0] == "maxpool":
                 shape = (shape[0], shape[1], shape[2] // 2, shape[3] // 2)
-        conv_ms = sum(d["ms_total"] for d in conv)
-        out["conv_mfma_util_pct"] = 100.0 * conv_flop / (conv_ms * 1e-3) / 1e12 / PEAK_TFLOPS_FP32_MFMA
-        # the same over the direct kernels alone, whose executed FLOP are the algorithmic ones
-        direct = [d for tag, d in k.items() if tag.startswith("conv_") and not tag.endswith("_winograd")
-                  and d["unit"] == "flop"]
-        if direct:
-            out["conv_mfma_util_direct_kernels_pct"] = 100.0 * sum(d["work"] for d in direct) / (
-                sum(d["ms_total"] for d in direct) * 1e-3) / 1e12 / PEAK_TFLOPS_FP32_MFMA
+        conv_ms = sum(d["ms_total"] for d in conv.values())
+        direct_flop = sum(d["work"] for tag, d in conv.items() if d["unit"] == "flop" and not tag.endswith("_winograd"))
+        equivalent_flop = sum(d["work"] for d in conv.values() if d["unit"] == "flop") + thin_flop
+
+        def pct(flop, ms):
+            return 100.0 * flop / (ms * 1e-3) / 1e12 / PEAK_TFLOPS_FP32_MFMA if ms > 0 else None
+        # executed: what the matrix pipe really multiplies (the Winograd calls count with their 36 GEMMs'
+        # FLOP, the direct kernels with the algorithm's) over ALL conv time, transforms included
+        out["conv_mfma_util_executed_pct"] = pct(direct_flop + thin_flop + wino_exec_flop, conv_ms)
+        # direct-equivalent: the direct algorithm's FLOP count of every layer over the same time; above 100
+        # because the Winograd layers execute a quarter of it.  A throughput figure, not a utilisation
+        out["conv_direct_equivalent_pct"] = pct(equivalent_flop, conv_ms)
+        out["conv_effective_tflops"] = equivalent_flop / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else None
+        # the direct kernels alone, whose executed FLOP are the algorithmic ones
+        direct_ms = sum(d["ms_total"] for tag, d in conv.items() if d["unit"] == "flop" and not tag.endswith("_winograd"))
+        if direct_ms > 0:
+            out["conv_mfma_util_direct_kernels_pct"] = pct(direct_flop, direct_ms)
         out["kernels"] = kernels
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+        # the same 16-image sample, same seeded parameters, once through the GPU path (forward of the first
+        # step, 4 micro-tensors on the first four convolutions): the loss the CPU figures report beside it
+        out["gpu_loss_on_cpu_sample"] = gpu_loss_on_sample(ctx)
+        out["gpu_vs_cpu_loss_rel_diff"] = abs(out["gpu_loss_on_cpu_sample"] - out["cpu_baseline"]["loss"]) / abs(
+            out["cpu_baseline"]["loss"])
         onednn = cpu_baseline_onednn()
         if onednn:
             out["cpu_baseline_onednn"] = onednn

@@ -37,6 +37,9 @@ def test_mlp_20_steps_tracks_oracle():
         assert_close(t.params[k].asnumpy(), ref_params[k], 1e-3, k)
 
 
+VGG_20_STEP_LR = 5e-7
+
+
 def _small_convnet():
     return [("conv", "c1", 3, 8, 3, 1, 1), ("bn", "c1_bn", 8), ("relu",),
             ("conv", "c2", 8, 16, 3, 1, 1), ("bn", "c2_bn", 16), ("relu",), ("maxpool", 2, 0, 2),
@@ -67,31 +70,98 @@ def test_convnet_momentum_tracks_oracle_with_and_without_split(split, fuse):
         assert_close(t.params[k].asnumpy(), ref_params[k], 2e-3, k)
 
 
-@pytest.mark.parametrize("winograd", [None, "1"])
-def test_vgg16_topology_small_resolution_tracks_oracle(winograd, monkeypatch):
-    """The full VGG-16 layer list (13 conv+BN+Relu, 5 pools, 3 FC) at 32x32, batch 4, with the
-    two largest-resolution blocks run as 2 micro-tensors: 3 momentum steps against the oracle.
-    Once as the library routes these small layers itself (direct kernels), once with every layer but
-    the first forced through the Winograd routine in all three passes."""
+def _train_gpu(spec, params, X, Y, steps, opt, split=None, fuse=False):
     from tsplit_amd import ndarray, trainer
-    if winograd:
-        monkeypatch.setenv("TSPLIT_CONV_WINOGRAD", winograd)
-    rng = np.random.RandomState(11)
-    spec = trainer.vgg16_spec(num_classes=10, in_hw=32)
-    X = rng.normal(size=(4, 3, 32, 32)).astype(np.float32)
-    Y = _onehot(rng.randint(0, 10, 4), 10)
-    params = trainer.init_params(spec, seed=3)
-    # a small step keeps the run in the regime where the loss falls smoothly; with larger steps this
-    # 4-image batch is memorised (or diverges) within two updates and rounding differences are amplified
-    ref_losses, _ = nets.train(spec, params, X, Y, steps=3, lr=1e-5, momentum=0.9)
     ctx = ndarray.gpu(0)
-    conv_idx = [i for i, l in enumerate(spec) if l[0] == "conv"]
-    t = trainer.Trainer(spec, params, X.shape, 10, ctx, optimizer=("momentum", 1e-5, 0.9),
-                        split={i: 2 for i in conv_idx[:4]})
+    t = trainer.Trainer(spec, params, X.shape, Y.shape[1], ctx, optimizer=opt, split=split, fuse_bn_relu=fuse)
     gx, gy = ndarray.array(X, ctx), ndarray.array(Y, ctx)
     losses = []
-    for _ in range(3):
+    for _ in range(steps):
         t.step(gx, gy)
         losses.append(t.loss_value())
+    return t, losses
+
+
+_VGG_20 = {}
+
+
+def _vgg_20_step_oracle():
+    """Spec, data, seeded parameters and the oracle's 20-step run, computed once for both routings."""
+    if not _VGG_20:
+        from tsplit_amd import trainer
+        rng = np.random.RandomState(11)
+        spec = trainer.vgg16_spec(num_classes=10, in_hw=32, fc_width=512)
+        X = rng.normal(size=(8, 3, 32, 32)).astype(np.float32)
+        Y = _onehot(rng.randint(0, 10, 8), 10)
+        params = trainer.init_params(spec, seed=3)
+        ref_losses, ref_params = nets.train(spec, params, X, Y, steps=20, lr=VGG_20_STEP_LR, momentum=0.9)
+        _VGG_20.update(spec=spec, X=X, Y=Y, params=params, ref_losses=ref_losses, ref_params=ref_params)
+    return _VGG_20
+
+
+@pytest.mark.parametrize("winograd", [None, "1"])
+def test_vgg16_topology_20_steps_tracks_oracle(winograd, monkeypatch):
+    """The full VGG-16 layer list (13 conv+BN+Relu at 64 ... 512 channels, 5 pools, 3 FC) at 32x32,
+    batch 8, with the two largest-resolution blocks run as 2 micro-tensors: 20 momentum steps against
+    the oracle.  The step size is the one under which this 8-image batch is learnt smoothly (the loss
+    falls from 4.8 to 0.7 over the 20 steps; ten times larger and the batch is memorised within three
+    updates, after which rounding differences decide the curve), so a wrong gradient or update shows in
+    the curve; what the 20 updates changed in every parameter is compared as well.  Once as the library
+    routes these small layers itself (direct kernels), once with every layer but the first forced
+    through the Winograd routine in all three passes."""
+    if winograd:
+        monkeypatch.setenv("TSPLIT_CONV_WINOGRAD", winograd)
+    o = _vgg_20_step_oracle()
+    spec, params, ref_losses, ref_params = o["spec"], o["params"], o["ref_losses"], o["ref_params"]
+    assert ref_losses[-1] < 0.5 * ref_losses[0], ref_losses       # the run does train
+    conv_idx = [i for i, l in enumerate(spec) if l[0] == "conv"]
+    t, losses = _train_gpu(spec, params, o["X"], o["Y"], 20, ("momentum", VGG_20_STEP_LR, 0.9),
+                           split={i: 2 for i in conv_idx[:4]})
     rel = np.max(np.abs(np.array(losses) - np.array(ref_losses)) / np.abs(ref_losses))
     assert rel <= 1e-3, (rel, losses, ref_losses)
+    for k in params:
+        got = t.params[k].asnumpy()
+        assert_close(got, ref_params[k], 2e-3, k)
+        # the updates themselves: parameters are stored in fp32 on both sides, so a change is known to
+        # about 1e-3 of itself
+        assert_close(got.astype(np.float64) - params[k], ref_params[k].astype(np.float64) - params[k], 2e-2, "change of " + k)
+
+
+def test_vgg16_224_natural_routing_gradients_match_oracle():
+    """VGG-16 at the benchmark's resolution (224x224, 1000 classes, He init), batch 8 with the first
+    four convolutions on 2 micro-tensors, routed by the library itself: at these sizes it sends the
+    112x112 and 56x56 layers through the Winograd routine in all three passes (asserted through the
+    routing query, so the test cannot silently run on the direct kernels) and cuts the direct layers'
+    tiles between blocks as it does at batch 64.  One step's loss and EVERY parameter gradient, then
+    the parameters after two momentum steps, against the float64 oracle."""
+    from tsplit_amd import gpu_links as L, ndarray, trainer
+    rng = np.random.RandomState(21)
+    spec = trainer.vgg16_spec(num_classes=1000, in_hw=224)
+    X = rng.standard_normal(size=(8, 3, 224, 224)).astype(np.float32)
+    Y = _onehot(rng.randint(0, 1000, 8), 1000)
+    params = trainer.init_params(spec, seed=9, scheme="he")
+    # the routing the library chooses for this run
+    for imgs, c, o, hw in ((4, 64, 128, 112), (4, 128, 128, 112), (8, 128, 256, 56), (8, 256, 256, 56)):
+        assert L.conv_takes_winograd(imgs, c, o, hw, hw, 3, 1, 1)
+        assert L.conv_takes_winograd(imgs, c, o, hw, hw, 3, 1, 1, filter_gradient=True)
+        assert L.conv_takes_winograd(imgs, c, o, hw, hw, 3, 1, 1, data_gradient=True) or (c, o) == (64, 128)
+    assert not L.conv_takes_winograd(4, 64, 64, 224, 224, 3, 1, 1)
+    lr = 0.01
+    loss0, _, ref_grads = nets.forward_backward(spec, params, X, Y)
+    ref_losses, ref_params = nets.train(spec, params, X, Y, steps=2, lr=lr, momentum=0.9)
+    assert abs(ref_losses[0] - loss0) < 1e-12
+    conv_idx = [i for i, l in enumerate(spec) if l[0] == "conv"]
+    ctx = ndarray.gpu(0)
+    t = trainer.Trainer(spec, params, X.shape, 1000, ctx, optimizer=("momentum", lr, 0.9),
+                        split={i: 2 for i in conv_idx[:4]})
+    gx, gy = ndarray.array(X, ctx), ndarray.array(Y, ctx)
+    t.forward(gx, gy)
+    t.backward(gy)
+    assert abs(t.loss_value() - loss0) <= 1e-3 * abs(loss0), (t.loss_value(), loss0)
+    for k, g in ref_grads.items():
+        assert_close(t.grads[k].asnumpy().reshape(g.shape), g, 2e-3, "gradient of " + k)
+    t.update()
+    t.step(gx, gy)
+    assert abs(t.loss_value() - ref_losses[1]) <= 1e-3 * abs(ref_losses[1]), (t.loss_value(), ref_losses)
+    for k in params:
+        assert_close(t.params[k].asnumpy(), ref_params[k], 2e-3, k)

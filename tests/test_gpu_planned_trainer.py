@@ -1,5 +1,8 @@
-"""The budgeted executor against the plain one on the GPU: same losses step by step, measured
-peak within the budget, tensors really leaving and coming back."""
+"""The budgeted executor on the GPU against the CPU oracle (loss curve and final parameters of the
+swap-only, recomputing and split plans) and against the plain executor (the same bits wherever no
+convolution is split): measured peak within the budget, the device pool holding exactly what the
+executor accounts for, tensors really leaving and coming back, and one run in a process whose
+device pool is capped at the budget."""
 import numpy as np
 import pytest
 
@@ -37,9 +40,37 @@ def _plain_losses(spec_fused, steps, rng_seed=5):
     return out, {k: v.asnumpy() for k, v in t.params.items()}
 
 
+_ORACLE = {}
+
+
+def _oracle(steps):
+    """The float64 oracle on the same seeded data and parameters: (losses, final parameters)."""
+    if steps not in _ORACLE:
+        from oracle import nets
+        rng = np.random.RandomState(5)
+        params = trainer.init_params(SPEC, seed=3)
+        x, labels = _data(rng)
+        _ORACLE[steps] = nets.train(SPEC, params, x, labels, steps=steps, lr=OPT[1], momentum=OPT[2])
+    return _ORACLE[steps]
+
+
+def _tracks_oracle(losses, params):
+    """North-star bars: loss curve within 1e-3 relative, parameters within 2e-3 of their largest entry."""
+    from util import assert_close
+    ref_losses, ref_params = _oracle(len(losses))
+    rel = np.max(np.abs(np.array(losses) - np.array(ref_losses)) / np.abs(ref_losses))
+    assert rel <= 1e-3, (rel, losses, ref_losses)
+    for k, v in ref_params.items():
+        assert_close(params[k], v, 2e-3, k)
+
+
 def _planned(spec, budget_frac, steps, piece_bytes=64 << 10, rng_seed=5, allow_recompute=False):
-    from tsplit_amd import ndarray
+    import gc
+
+    from tsplit_amd import gpu_memory_manager, ndarray
     from tsplit_amd.planned_trainer import PlannedTrainer, make_plan
+    gc.collect()
+    pool_before = gpu_memory_manager.pool_state().used
     rng = np.random.RandomState(rng_seed)
     params = trainer.init_params(SPEC, seed=3)
     free = make_plan(spec, IN, 10, None, OPT)
@@ -56,6 +87,10 @@ def _planned(spec, budget_frac, steps, piece_bytes=64 << 10, rng_seed=5, allow_r
     for _ in range(steps):
         t.step(gx, gl)
         out.append(t.loss_value())
+        # what the device pool holds for this run is what the executor accounts for (plus the caller's
+        # batch and labels): nothing released lingers in the pool
+        held = gpu_memory_manager.pool_state().used - pool_before
+        assert held == t.live + 4 * (x.size + labels.size), (held, t.live)
     return out, {k: v.asnumpy() for k, v in t.params.items()}, t, plan, free
 
 
@@ -66,6 +101,7 @@ def test_unlimited_budget_equals_plain_trainer(fused):
     got, gp, t, plan, _ = _planned(spec, None, 4)
     assert not plan.swap
     assert got == want                                  # same kernels on the same data: bit for bit
+    _tracks_oracle(got, gp)
     for k in wp:
         assert np.array_equal(gp[k], wp[k]), k
     # without a budget releases are not waited for, so the executor may hold a little more
@@ -86,6 +122,7 @@ def test_budget_is_met_and_results_do_not_change(fused, frac):
     got, gp, t, plan, free = _planned(spec, frac, 4)
     assert plan.swap and plan.budget_bytes < free.peak_bytes
     assert t.peak <= plan.budget_bytes
+    _tracks_oracle(got, gp)                             # swapped (and split) runs against the oracle itself
     # swapping moves bytes, it does not change them; split convolutions may round differently
     np.testing.assert_allclose(got, want, rtol=2e-5)
     for k in wp:
@@ -112,6 +149,7 @@ def test_recomputation_meets_the_budget_with_the_same_bits(fused, frac):
     assert plan.recompute and plan.budget_bytes < free.peak_bytes
     assert all(spec[j - 1][0] in planner.CHEAP_TO_REDO for j in plan.recompute)
     assert t.peak <= plan.budget_bytes and not t.dropped
+    _tracks_oracle(got, gp)                             # recomputed (and split) runs against the oracle itself
     np.testing.assert_allclose(got, want, rtol=2e-5)
     for k in wp:
         np.testing.assert_allclose(gp[k], wp[k], rtol=1e-4, atol=2e-5, err_msg=k)
@@ -123,3 +161,43 @@ def test_recomputation_meets_the_budget_with_the_same_bits(fused, frac):
     from tsplit_amd.planned_trainer import make_plan
     swap_only = make_plan(spec, IN, 10, plan.budget_bytes, OPT, piece_bytes=64 << 10)
     assert plan.est_step_ms <= swap_only.est_step_ms + 1e-9
+
+
+def _capped_child():
+    """Runs in a process whose device pool is capped (TSPLIT_POOL_LIMIT_BYTES): three steps of the
+    recomputing plan at 30 % of the way from the floor to the unplanned peak; prints the losses."""
+    import json
+    spec = SPEC
+    got, gp, t, plan, free = _planned(spec, 0.3, 3, allow_recompute=True)
+    from tsplit_amd import gpu_memory_manager
+    st = gpu_memory_manager.pool_state()
+    print(json.dumps({"losses": got, "peak": t.peak, "budget": plan.budget_bytes, "unplanned_peak": free.peak_bytes,
+                      "pool_total": st.used + st.unused_unavailable + st.unused_available}))
+
+
+def test_budgeted_run_inside_a_capped_device_pool():
+    """The budget is host-side bookkeeping; here the device pool itself is capped, so an allocation
+    beyond the cap fails in the library.  The cap is the plan's budget plus an eighth for the pool's
+    256-byte granules and unsplit slack, and lies below what the unplanned run needs, so only a run
+    that really releases what the plan says can finish."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from tsplit_amd.planned_trainer import make_plan
+    free = make_plan(SPEC, IN, 10, None, OPT)
+    shapes = planner.layer_shapes(SPEC, IN)
+    floor, _ = planner.simulate(SPEC, shapes, range(1, len(SPEC)), free.fixed_bytes)
+    budget = int(floor + 0.3 * (free.peak_bytes - floor))
+    cap = budget + budget // 8
+    assert cap < free.peak_bytes                     # the unplanned run would not fit
+    env = dict(os.environ, TSPLIT_POOL_LIMIT_BYTES=str(cap))
+    here = os.path.dirname(os.path.abspath(__file__))
+    r = subprocess.run([sys.executable, "-c", "import test_gpu_planned_trainer as m; m._capped_child()"], cwd=here, env=env,
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert out["budget"] == budget and out["peak"] <= budget and out["pool_total"] <= cap
+    ref_losses, _ = _oracle(3)
+    rel = np.max(np.abs(np.array(out["losses"]) - np.array(ref_losses)) / np.abs(ref_losses))
+    assert rel <= 1e-3, (out["losses"], ref_losses)

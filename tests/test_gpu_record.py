@@ -204,3 +204,43 @@ def test_first_use_set_up_is_refused_while_recording():
     lse = np.log(np.exp(z - z.max(1, keepdims=True)).sum(1)) + z.max(1)
     ref = float(np.mean(lse - (z * large[1].asnumpy()).sum(1)))
     assert abs(float(large[2].asnumpy()[0]) - ref) <= 1e-4 * abs(ref)
+
+
+def test_scratch_growing_after_a_recording_leaves_the_graph_its_buffer():
+    """A recorded step holds the address of the scratch buffer it was recorded with.  When a later
+    eager call on the same stream needs more scratch than that, the library takes a new buffer for
+    the stream and keeps the recorded one allocated until the graph is destroyed, so replays after
+    the growth still compute the same values (softmax cross-entropy keeps one partial loss per row
+    in per-stream scratch, in granules of 1 MiB)."""
+    from tsplit_amd import gpu_links as L, ndarray, stream
+    ctx = ndarray.gpu(0)
+    st = stream.create_stream_handle(ctx)
+    rng = np.random.RandomState(4)
+
+    def ce_arrays(rows):
+        logits = ndarray.array(rng.standard_normal((rows, 4)).astype(np.float32), ctx)
+        labels = ndarray.array(np.eye(4, dtype=np.float32)[rng.randint(0, 4, rows)], ctx)
+        return logits, labels, ndarray.empty((1,), ctx)
+
+    small, large = ce_arrays(1000), ce_arrays(600000)
+    L.softmax_cross_entropy(small[0], small[1], small[2], st)          # first use: scratch of 1 MiB
+    st.sync()
+    want = small[2].asnumpy().copy()
+    with stream.recording(st) as rec:
+        L.softmax_cross_entropy(small[0], small[1], small[2], st)
+    for _ in range(3):
+        L.array_set(small[2], -1.0, st)
+        rec.graph.launch(st)
+        st.sync()
+        np.testing.assert_array_equal(small[2].asnumpy(), want)
+        # eager work on the same stream that needs more than the recorded buffer holds (2.4 MB of
+        # row losses), then other allocations that could land where a freed buffer was
+        L.softmax_cross_entropy(large[0], large[1], large[2], st)
+        st.sync()
+        filler = [ndarray.array(np.full((1 << 18,), 7.0, np.float32), ctx) for _ in range(4)]
+        del filler
+    z = large[0].asnumpy().astype(np.float64)
+    lse = np.log(np.exp(z - z.max(1, keepdims=True)).sum(1)) + z.max(1)
+    ref = float(np.mean(lse - (z * large[1].asnumpy()).sum(1)))
+    assert abs(float(large[2].asnumpy()[0]) - ref) <= 1e-4 * abs(ref)
+    del rec

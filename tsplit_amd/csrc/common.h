@@ -73,11 +73,15 @@ class ProfileScope {
     float ms = -1.f;
     bool good = hipEventRecord(b_, s_) == hipSuccess && hipEventSynchronize(b_) == hipSuccess &&
                 hipEventElapsedTime(&ms, a_, b_) == hipSuccess;
-    (void)hipEventDestroy(a_);
-    (void)hipEventDestroy(b_);
     p_->time = ms;
     return good ? 0 : -1;
   }
+  ~ProfileScope() {   // also on the early-return paths of an operator call
+    if (a_) (void)hipEventDestroy(a_);
+    if (b_) (void)hipEventDestroy(b_);
+  }
+  ProfileScope(const ProfileScope &) = delete;
+  ProfileScope &operator=(const ProfileScope &) = delete;
 
  private:
   ProfilerHandle p_;

@@ -77,7 +77,10 @@ const Tap *tap_table(int chans, int kH, int kW, int plane_w, int plane_hw, int s
       }
   Tap *d = nullptr;
   if (hipMalloc(&d, h.size() * sizeof(Tap)) != hipSuccess) return nullptr;
-  if (hipMemcpy(d, h.data(), h.size() * sizeof(Tap), hipMemcpyHostToDevice) != hipSuccess) return nullptr;
+  if (hipMemcpy(d, h.data(), h.size() * sizeof(Tap), hipMemcpyHostToDevice) != hipSuccess) {
+    (void)hipFree(d);
+    return nullptr;
+  }
   g_taps[key] = d;
   return d;
 }

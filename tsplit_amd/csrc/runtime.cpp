@@ -7,6 +7,7 @@
 #include <new>
 #include <set>
 #include <stdexcept>
+#include <vector>
 
 #include "common.h"
 #include "pool.h"
@@ -178,8 +179,34 @@ struct ScratchKey {
 struct ScratchBuf {
   void *p;
   size_t bytes;
+  bool recorded;   // handed out while a step was being recorded: a graph holds this address
 };
 std::map<ScratchKey, ScratchBuf> g_scratch;
+// Buffers a recorded step still refers to after their (stream, slot) moved on to a larger one or
+// the stream was destroyed; owned here until the last graph is gone.
+std::vector<void *> g_scratch_parked;
+int g_live_graphs = 0;
+int g_open_recordings = 0;
+
+// g_mu held.  A buffer no recording refers to is freed, one a recording got is parked.
+void scratch_retire(ScratchBuf &b) {
+  if (!b.p) return;
+  if (b.recorded)
+    g_scratch_parked.push_back(b.p);
+  else
+    (void)hipFree(b.p);
+  b.p = nullptr;
+  b.bytes = 0;
+  b.recorded = false;
+}
+
+// g_mu held.  With no graph alive and none being recorded nothing refers to a parked buffer.
+void scratch_release_parked() {
+  if (g_live_graphs > 0 || g_open_recordings > 0) return;
+  for (void *p : g_scratch_parked) (void)hipFree(p);
+  g_scratch_parked.clear();
+  for (auto &kv : g_scratch) kv.second.recorded = false;
+}
 
 }  // namespace
 
@@ -196,20 +223,24 @@ void *device_pool_alloc(int device_id, size_t bytes) {
 void *scratch_get(hipStream_t stream, int slot, size_t bytes) {
   std::lock_guard<std::mutex> lk(g_mu);
   ScratchBuf &b = g_scratch[ScratchKey{stream, slot}];
-  if (b.bytes >= bytes && b.p) return b.p;
+  hipStreamCaptureStatus recording = hipStreamCaptureStatusNone;
+  const bool in_recording =
+      stream && hipStreamIsCapturing(stream, &recording) == hipSuccess && recording != hipStreamCaptureStatusNone;
+  if (b.bytes >= bytes && b.p) {
+    b.recorded |= in_recording;
+    return b.p;
+  }
   if (b.p) {
-    // a recorded step keeps the address it was recorded with: growing is set-up, not part of a step
-    hipStreamCaptureStatus recording = hipStreamCaptureStatusNone;
-    if (stream && hipStreamIsCapturing(stream, &recording) == hipSuccess && recording != hipStreamCaptureStatusNone) {
+    // growing is set-up, not part of a step: a recording cannot allocate on the way
+    if (in_recording) {
       std::fprintf(stderr, "[libc_runtime_api] scratch memory would have to grow while a step is being recorded; "
                            "run the step once before recording it\n");
       return nullptr;
     }
-    // the old buffer may still be read by a kernel in flight on this stream
+    // the old buffer may still be read by a kernel in flight on this stream; a recorded step that
+    // got it keeps its address, so such a buffer is parked instead of freed
     (void)hipStreamSynchronize(stream);
-    (void)hipFree(b.p);
-    b.p = nullptr;
-    b.bytes = 0;
+    scratch_retire(b);
   }
   size_t want = (bytes + (1 << 20) - 1) >> 20 << 20;
   if (hipMalloc(&b.p, want) != hipSuccess) {
@@ -218,7 +249,38 @@ void *scratch_get(hipStream_t stream, int slot, size_t bytes) {
     return nullptr;
   }
   b.bytes = want;
+  b.recorded = in_recording;
   return b.p;
+}
+
+// Bytes of scratch a destroyed stream leaves behind would stay allocated for good, keyed by a
+// handle value a later stream may get again: called by DLStreamDestroy after the stream has drained.
+void scratch_drop_stream(hipStream_t stream) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  for (auto it = g_scratch.begin(); it != g_scratch.end();) {
+    if (it->first.s == stream) {
+      scratch_retire(it->second);
+      it = g_scratch.erase(it);
+    } else {
+      ++it;
+    }
+  }
+}
+
+void scratch_recording_opened() {
+  std::lock_guard<std::mutex> lk(g_mu);
+  ++g_open_recordings;
+}
+void scratch_recording_closed(bool graph_made) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (g_open_recordings > 0) --g_open_recordings;
+  if (graph_made) ++g_live_graphs;
+  scratch_release_parked();
+}
+void scratch_graph_destroyed() {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (g_live_graphs > 0) --g_live_graphs;
+  scratch_release_parked();
 }
 
 }  // namespace tsplit
@@ -264,6 +326,7 @@ int DLStreamDestroy(DLStreamHandle handle) {
   hipStream_t *s = static_cast<hipStream_t *>(handle->handle);
   if (s) {
     (void)hipStreamSynchronize(*s);
+    scratch_drop_stream(*s);
     TS_HIP(hipStreamDestroy(*s));
     delete s;
   }
@@ -327,6 +390,7 @@ int TSplit_StreamBeginRecord(DLStreamHandle stream) {
   TS_REQUIRE(stream != nullptr && stream->handle != nullptr, "TSplit_StreamBeginRecord: a created stream is required");
   // relaxed mode: device allocations made by this thread while recording (a new pool slab) are allowed
   TS_HIP(hipStreamBeginCapture(stream_of(stream), hipStreamCaptureModeRelaxed));
+  scratch_recording_opened();
   return 0;
 }
 
@@ -338,6 +402,7 @@ int TSplit_StreamEndRecord(DLStreamHandle stream, DLGraphHandle *out) {
   if (e != hipSuccess || graph == nullptr) {
     (void)hipGetLastError();
     if (graph) (void)hipGraphDestroy(graph);
+    scratch_recording_closed(false);
     TS_FAIL("TSplit_StreamEndRecord: the recording was invalidated (%s)", hipGetErrorString(e));
   }
   hipGraphExec_t exec = nullptr;
@@ -345,8 +410,10 @@ int TSplit_StreamEndRecord(DLStreamHandle stream, DLGraphHandle *out) {
   (void)hipGraphDestroy(graph);
   if (e != hipSuccess) {
     (void)hipGetLastError();
+    scratch_recording_closed(false);
     TS_FAIL("TSplit_StreamEndRecord: hipGraphInstantiate failed: %s", hipGetErrorString(e));
   }
+  scratch_recording_closed(true);
   DLGraph *g = new DLGraph();
   g->device_id = stream->device_id;
   g->handle = exec;
@@ -365,6 +432,7 @@ int TSplit_GraphDestroy(DLGraphHandle graph) {
   if (!graph) return 0;
   if (graph->handle) TS_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph->handle)));
   delete graph;
+  scratch_graph_destroyed();
   return 0;
 }
 

@@ -167,6 +167,12 @@ class PlannedTrainer(object):
             if isinstance(arr, tuple):         # a swapped tensor keeps its struct: drop the data only
                 arr[0].delete_itself()
                 arr[0].sTensor = []
+            else:
+                # micro-tensor views refer to their parent and the parent lists them: without this the
+                # pair is a cycle that only the collector frees, and the pool would hold the bytes
+                # beyond this point
+                arr.sTensor = []
+            del arr
             self.live -= nbytes
 
     def _alloc(self, shape, reuse=None):

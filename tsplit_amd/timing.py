@@ -39,11 +39,13 @@ class EventTimer(object):
                 self._a = self._ev()
                 self._a.record(stream)
 
-    def end(self, stream, tag, work, unit):
+    def end(self, stream, tag, work, unit, moved=None):
+        """`work` in `unit` ("flop" or "byte"); `moved`: for a call counted in FLOP, also its
+        algorithmic bytes (operands read once, result written once)."""
         if self.enabled:
             b = self._ev()
             b.record(stream)
-            self.spans.append((tag, work, unit, self._a, b))
+            self.spans.append((tag, work, unit, self._a, b, moved))
             self._last = (b, stream)
 
     def elapsed_ms(self, a, b):
@@ -57,14 +59,16 @@ class EventTimer(object):
         self._used, self.spans, self._last = 0, [], None
 
     def collect(self):
-        """-> {tag: dict(calls, ms_total, ms_avg, work_per_call, unit, rate)}; rate in TFLOP/s
+        """-> {tag: dict(calls, ms_total, ms_avg, work_per_call, unit, rate[, bytes])}; rate in TFLOP/s
         (unit "flop") or GB/s (unit "byte")"""
         out = {}
-        for tag, work, unit, a, b in self.spans:
+        for tag, work, unit, a, b, moved in self.spans:
             d = out.setdefault(tag, {"calls": 0, "ms_total": 0.0, "work": 0.0, "unit": unit})
             d["calls"] += 1
             d["ms_total"] += self.elapsed_ms(a, b)
             d["work"] += work
+            if moved is not None:
+                d["bytes"] = d.get("bytes", 0.0) + moved
         for d in out.values():
             d["ms_avg"] = d["ms_total"] / d["calls"]
             d["work_per_call"] = d["work"] / d["calls"]

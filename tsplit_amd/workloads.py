@@ -353,3 +353,49 @@ def lstm(t, b, x, labels, dim_input=28, dim_hidden=128, classes=10, steps=28, st
     logits = t.matmul(h, out_w)
     logits = t.add(logits, t.broadcast_like(out_b, logits.shape))
     return t.softmax_ce(logits, labels), logits
+
+
+# ------------------------------------------------------------------ shapes only
+class _ShapeBackend(object):
+    """Runs a builder without arithmetic: every primitive returns None; convolutions are listed."""
+
+    def __init__(self):
+        self.convs = []
+
+    def conv2d(self, x, w, xs, ws, ph, pw, s):
+        self.convs.append((int(xs[0]), int(xs[1]), int(xs[2]), int(xs[3]), int(ws[0]), int(ws[2]), int(ws[3]), int(ph),
+                           int(pw), int(s)))
+
+    def __getattr__(self, name):
+        return lambda *a, **k: None
+
+
+class _ShapeStore(object):
+    trainable = {}
+
+    def get(self, name, shape, init, trainable=True):
+        return np.broadcast_to(np.float32(0), tuple(int(s) for s in shape))
+
+
+def conv_geometries(net, batch=None):
+    """The distinct convolution geometries of a full-size example network, in order of first use:
+    tuples (images, Cin, H, W, Cout, kH, kW, pad_h, pad_w, stride).  net: "resnet50" (batch 64,
+    224x224) or "inception_v4" (batch 32, 299x299), the sizes of the benchmark configurations."""
+    from . import graph
+    backend = _ShapeBackend()
+    t = graph.Tape(backend)
+    b = Binder(t, _ShapeStore())
+    if net == "resnet50":
+        n = batch or 64
+        resnet(t, b, t.const(None, (n, 3, 224, 224)), t.const(None, (n, 1000)))
+    elif net == "inception_v4":
+        n = batch or 32
+        inception_v4(t, b, t.const(None, (n, 3, 299, 299)), t.const(None, (n, 1000)))
+    else:
+        raise ValueError(net)
+    seen, out = set(), []
+    for g in backend.convs:
+        if g not in seen:
+            seen.add(g)
+            out.append(g)
+    return out
