@@ -116,7 +116,7 @@ def test_resnet50_full_size_step():
     first, second, store = _step_twice(lambda t, b, d: workloads.resnet(t, b, d["x"], d["y"]),
                                        _images(np.random.default_rng(1), 64, 224), seed=123)
     _check_step(first, second, store)
-    assert abs(first[0] - np.log(1000.0)) < 3.0          # He init, random labels: about log(classes)
+    assert abs(first[0] - np.log(1000.0)) < 6.0          # He init, random labels: log(classes) and a few units
 
 
 def test_inception_v4_full_size_step():
@@ -124,7 +124,7 @@ def test_inception_v4_full_size_step():
     first, second, store = _step_twice(lambda t, b, d: workloads.inception_v4(t, b, d["x"], d["y"]),
                                        _images(np.random.default_rng(2), 32, 299), seed=123)
     _check_step(first, second, store)
-    assert abs(first[0] - np.log(1000.0)) < 3.0
+    assert abs(first[0] - np.log(1000.0)) < 6.0
 
 
 def test_transformer_full_size_step():
@@ -141,4 +141,4 @@ def test_transformer_full_size_step():
     first, second, store = _step_twice(lambda t, b, d: workloads.transformer(t, b, cfg, d["xs"], d["yi"], d["yo"]),
                                        inputs, seed=123)
     _check_step(first, second, store, order_dependent=("embedding_table",))
-    assert abs(first[0] - np.log(32000.0)) < 3.0
+    assert abs(first[0] - np.log(32000.0)) < 6.0

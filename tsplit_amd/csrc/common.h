@@ -27,6 +27,10 @@ inline float mib(int64_t elems) { return static_cast<float>(elems) * 4.0f / (102
 // that stream without waiting; ops on different streams never share one.
 void *scratch_get(hipStream_t stream, int slot, size_t bytes);
 
+// Looks up, once per device, the address of the fixed scratch array behind
+// TSplit_SoftmaxCrossEntropyNoAlloc (called from the per-device init call).
+void softmax_noalloc_setup(int device_id);
+
 
 #define TS_FAIL(...)                                  \
   do {                                                \

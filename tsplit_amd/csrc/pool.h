@@ -34,8 +34,11 @@ class BinnedPool {
   static constexpr size_t kAlign = 256;                 // ref: chunk granularity 256 B
   static constexpr size_t kSplitSlack = 128ull << 20;   // ref: gpu_memory_manager.cc:222-223
 
-  BinnedPool(PoolBacking backing, size_t slab_bytes, size_t limit_bytes)
-      : backing_(backing), slab_bytes_(slab_bytes), limit_(limit_bytes) {}
+  // split_slack: a free block at most twice the request is handed out whole unless the part left over
+  // would reach this many bytes (the reference's 128 MiB by default; 0 splits always, which wastes
+  // nothing and is what a capacity limit close to the tensors' own total needs)
+  BinnedPool(PoolBacking backing, size_t slab_bytes, size_t limit_bytes, size_t split_slack = kSplitSlack)
+      : backing_(backing), slab_bytes_(slab_bytes), limit_(limit_bytes), split_slack_(split_slack) {}
 
   ~BinnedPool() {
     for (Chunk *c : all_) delete c;
@@ -55,7 +58,7 @@ class BinnedPool {
     c->used = bytes;
     // split rule of the reference: only when the block is more than twice the request or
     // the slack reaches 128 MiB; smaller slack stays attached ("unused unavailable").
-    if (c->size > 2 * need || c->size - need >= kSplitSlack) Split(c, need);
+    if (c->size > need && (c->size > 2 * need || c->size - need >= split_slack_)) Split(c, need);
     live_[c->ptr] = c;
     return c->ptr;
   }
@@ -189,6 +192,7 @@ class BinnedPool {
   PoolBacking backing_;
   size_t slab_bytes_;
   size_t limit_;
+  size_t split_slack_;
   size_t reserved_ = 0;
   std::vector<void *> slabs_;
   std::set<Chunk *, ByAddr> all_;

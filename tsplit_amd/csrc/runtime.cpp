@@ -50,7 +50,7 @@ BinnedPool *pool_for(int dev) {
   PoolBacking b{dev_alloc, dev_release, dev_available, nullptr};
   size_t slab = env_bytes("TSPLIT_POOL_SLAB_BYTES", 1ull << 30);
   size_t limit = env_bytes("TSPLIT_POOL_LIMIT_BYTES", ~size_t(0));
-  BinnedPool *p = new BinnedPool(b, slab, limit);
+  BinnedPool *p = new BinnedPool(b, slab, limit, env_bytes("TSPLIT_POOL_SPLIT_SLACK_BYTES", BinnedPool::kSplitSlack));
   g_pools[dev] = p;
   return p;
 }
@@ -440,7 +440,10 @@ void cuda_init(void) {
   int d = 0;
   if (hipGetDevice(&d) == hipSuccess) (void)hipSetDevice(d);
 }
-void cudnn_init(size_t dev_id, DLStreamHandle) { (void)hipSetDevice(static_cast<int>(dev_id)); }
+void cudnn_init(size_t dev_id, DLStreamHandle) {
+  (void)hipSetDevice(static_cast<int>(dev_id));
+  softmax_noalloc_setup(static_cast<int>(dev_id));
+}
 void cublas_init(size_t dev_id, DLStreamHandle) { (void)hipSetDevice(static_cast<int>(dev_id)); }
 void cusp_init(size_t dev_id, DLStreamHandle) { (void)hipSetDevice(static_cast<int>(dev_id)); }
 

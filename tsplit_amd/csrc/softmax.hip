@@ -7,8 +7,15 @@
 // Long rows (a 32 000-word vocabulary) get a whole block per row instead: 16-byte loads,
 // running (max, scaled sum) pairs so that the logits are read from memory once, and for the
 // loss the label sums of the same pass: loss_r = (log s + m) * sum(l) - sum(l * y).
+#include <mutex>
+
 #include "common.h"
 #include "reduce.h"
+
+// Per-row losses of TSplit_SoftmaxCrossEntropyNoAlloc (below): a fixed array in the code object, so
+// that call needs no device allocation.  No kernel names it: kernels get its address as an argument.
+constexpr int kNoAllocMaxRows = 1 << 18;
+static __device__ __align__(256) __attribute__((used)) float scratch[kNoAllocMaxRows];
 
 namespace tsplit {
 namespace {
@@ -187,12 +194,74 @@ inline bool rows_cols(const DLArray *a, int64_t &nrow, int &ncol) {
   return nrow > 0 && ncol > 0;
 }
 
+// ---------------------------------------------------------------- entry point that allocates nothing
+// Each GPU holds its own copy of `scratch` (1 MiB) at its own address, from the time the library is
+// loaded on it until the process ends.
+constexpr int kNoAllocMaxDevices = 64;
+std::mutex g_noalloc_mu;
+float *g_noalloc_ptr[kNoAllocMaxDevices] = {};
+
+// Device address of `scratch` on device `dev`, looked up once per device with that device current.
+// (In host code the array's name is only a handle for this lookup, never a device address.)
+float *noalloc_scratch(int dev) {
+  if (dev < 0 || dev >= kNoAllocMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lk(g_noalloc_mu);
+  if (g_noalloc_ptr[dev]) return g_noalloc_ptr[dev];
+  if (hipSetDevice(dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  void *ptr = nullptr;
+  const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || ptr == nullptr) {
+    (void)hipGetLastError();
+    std::fprintf(stderr, "[libc_runtime_api] hipGetSymbolAddress(scratch) failed on device %d: %s\n", dev,
+                 hipGetErrorString(e));
+    return nullptr;
+  }
+  g_noalloc_ptr[dev] = static_cast<float *>(ptr);
+  return g_noalloc_ptr[dev];
+}
+
 }  // namespace
+
+// Called from the library's per-device init call so that the first operator call finds the address.
+void softmax_noalloc_setup(int dev) { (void)noalloc_scratch(dev); }
+
 }  // namespace tsplit
 
 using namespace tsplit;
 
 extern "C" {
+
+int TSplit_SoftmaxCrossEntropyNoAlloc(const DLArrayHandle input_a, const DLArrayHandle input_b, DLArrayHandle output,
+                                      DLStreamHandle stream_handle) {
+  const char *who = "TSplit_SoftmaxCrossEntropyNoAlloc";
+  TS_REQUIRE(input_a && input_b && output, "%s: NULL array", who);
+  TS_REQUIRE(numel(input_a) == numel(input_b), "%s: logits and labels differ in size", who);
+  TS_REQUIRE(numel(output) >= 1, "%s: output must hold one element", who);
+  int64_t nrow;
+  int ncol;
+  TS_REQUIRE(rows_cols(input_a, nrow, ncol), "%s: empty input", who);
+  TS_REQUIRE(nrow <= kNoAllocMaxRows, "%s: %lld rows, the fixed scratch array holds %d; use DLGpuSoftmaxCrossEntropy", who,
+             static_cast<long long>(nrow), kNoAllocMaxRows);
+  float *row_loss = noalloc_scratch(input_a->ctx.device_id);
+  TS_REQUIRE(row_loss, "%s: the scratch array of device %d could not be located", who, input_a->ctx.device_id);
+  hipStream_t s = stream_of(stream_handle);
+  // every row's entry is written by the first kernel before the second reads rows [0, nrow): nothing of
+  // an earlier call's contents is read, so nothing has to be cleared
+  const unsigned blocks = static_cast<unsigned>((nrow + kRowsPerBlock - 1) / kRowsPerBlock);
+  if (wide_rows(ncol, input_a->data, input_b->data, nullptr))
+    hipLaunchKernelGGL(ce_rows_wide_kernel, dim3(static_cast<unsigned>(nrow)), dim3(256), 0, s,
+                       static_cast<const float *>(input_a->data), static_cast<const float *>(input_b->data), row_loss, ncol);
+  else
+    hipLaunchKernelGGL(ce_rows_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const float *>(input_a->data),
+                       static_cast<const float *>(input_b->data), row_loss, nrow, ncol);
+  hipLaunchKernelGGL(mean_kernel, dim3(1), dim3(256), 0, s, row_loss, static_cast<float *>(output->data), nrow);
+  const hipError_t le = hipGetLastError();
+  TS_REQUIRE(le == hipSuccess, "%s: kernel launch failed: %s", who, hipGetErrorString(le));
+  return 0;
+}
 
 int DLGpuSoftmax(const DLArrayHandle input, DLArrayHandle output, DLStreamHandle stream_handle, ProfilerHandle p) {
   TS_REQUIRE(input && output, "DLGpuSoftmax: NULL array");
