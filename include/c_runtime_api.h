@@ -153,6 +153,18 @@ int DLGpuSoftmaxCrossEntropy_Gradient(const DLArrayHandle input_a, const DLArray
                                       const DLArrayHandle input_c, DLArrayHandle output,
                                       DLStreamHandle stream_handle, ProfilerHandle p);
 
+/* ---- Softmax cross-entropy that allocates nothing.  NO counterpart in the reference.  For callers
+ *      that cannot allocate device memory inside the call: code being captured into a HIP graph,
+ *      tight serving loops, harnesses that forbid hipMalloc.  Same arguments, kernels and result
+ *      (bit for bit) as DLGpuSoftmaxCrossEntropy without the profiler; the per-row losses live in
+ *      a fixed 1 MiB array inside the library instead of its grow-on-demand scratch memory, so at
+ *      most 262144 rows (product of all but the last dimension): more returns -1 with a message.
+ *      Every GPU the library runs on holds its own copy of that array until the process ends; calls
+ *      that overlap on one GPU (different streams) share it and race.  The array's address is
+ *      looked up once per device, by cudnn_init(dev_id, ...) or else by the first call. ---- */
+int TSplit_SoftmaxCrossEntropyNoAlloc(const DLArrayHandle input_a, const DLArrayHandle input_b,
+                                      DLArrayHandle output, DLStreamHandle stream_handle);
+
 /* ---- Conv2d, cross-correlation, no bias, square stride, dilation 1.
  *      `CuDNN_` symbols (ref: c_runtime_api.h:323-327; impl src/ops/CudnnConv2d.cu:6,207,410)
  *      take (pad_h, pad_w, stride); they are the ones the graph ops call

@@ -14,8 +14,11 @@
 
 // Per-row losses of TSplit_SoftmaxCrossEntropyNoAlloc (below): a fixed array in the code object, so
 // that call needs no device allocation.  No kernel names it: kernels get its address as an argument.
+// The host code's reference to it (hipGetSymbolAddress below) is what makes the compiler give this
+// static variable a symbol the runtime can find; it must NOT carry __attribute__((used)), which keeps
+// the symbol local to the code object, and looking up a local symbol ends the process.
 constexpr int kNoAllocMaxRows = 1 << 18;
-static __device__ __align__(256) __attribute__((used)) float scratch[kNoAllocMaxRows];
+static __device__ __align__(256) float scratch[kNoAllocMaxRows];
 
 namespace tsplit {
 namespace {
@@ -201,9 +204,11 @@ constexpr int kNoAllocMaxDevices = 64;
 std::mutex g_noalloc_mu;
 float *g_noalloc_ptr[kNoAllocMaxDevices] = {};
 
+}  // namespace
+
 // Device address of `scratch` on device `dev`, looked up once per device with that device current.
 // (In host code the array's name is only a handle for this lookup, never a device address.)
-float *noalloc_scratch(int dev) {
+float *softmax_noalloc_scratch(int dev) {
   if (dev < 0 || dev >= kNoAllocMaxDevices) return nullptr;
   std::lock_guard<std::mutex> lk(g_noalloc_mu);
   if (g_noalloc_ptr[dev]) return g_noalloc_ptr[dev];
@@ -223,10 +228,8 @@ float *noalloc_scratch(int dev) {
   return g_noalloc_ptr[dev];
 }
 
-}  // namespace
-
 // Called from the library's per-device init call so that the first operator call finds the address.
-void softmax_noalloc_setup(int dev) { (void)noalloc_scratch(dev); }
+void softmax_noalloc_setup(int dev) { (void)softmax_noalloc_scratch(dev); }
 
 }  // namespace tsplit
 
@@ -245,7 +248,7 @@ int TSplit_SoftmaxCrossEntropyNoAlloc(const DLArrayHandle input_a, const DLArray
   TS_REQUIRE(rows_cols(input_a, nrow, ncol), "%s: empty input", who);
   TS_REQUIRE(nrow <= kNoAllocMaxRows, "%s: %lld rows, the fixed scratch array holds %d; use DLGpuSoftmaxCrossEntropy", who,
              static_cast<long long>(nrow), kNoAllocMaxRows);
-  float *row_loss = noalloc_scratch(input_a->ctx.device_id);
+  float *row_loss = softmax_noalloc_scratch(input_a->ctx.device_id);
   TS_REQUIRE(row_loss, "%s: the scratch array of device %d could not be located", who, input_a->ctx.device_id);
   hipStream_t s = stream_of(stream_handle);
   // every row's entry is written by the first kernel before the second reads rows [0, nrow): nothing of

@@ -96,6 +96,12 @@ def softmax_cross_entropy(in_arr_a, in_arr_b, out_arr, stream=None, profiler=Non
     check_call(_LIB.DLGpuSoftmaxCrossEntropy(_h(in_arr_a), _h(in_arr_b), _h(out_arr), _s(stream), _p(profiler)))
 
 
+def softmax_cross_entropy_no_alloc(in_arr_a, in_arr_b, out_arr, stream=None):
+    """The same loss from the entry point that allocates no device memory (no counterpart in the
+    reference's gpu_links): at most 262144 rows, per-row losses in a fixed array of the library."""
+    check_call(_LIB.TSplit_SoftmaxCrossEntropyNoAlloc(_h(in_arr_a), _h(in_arr_b), _h(out_arr), _s(stream)))
+
+
 def softmax_cross_entropy_gradient(in_arr_a, in_arr_b, in_arr_c, out_arr, stream=None, profiler=None):
     check_call(_LIB.DLGpuSoftmaxCrossEntropy_Gradient(_h(in_arr_a), _h(in_arr_b), _h(in_arr_c), _h(out_arr),
                                                       _s(stream), _p(profiler)))
