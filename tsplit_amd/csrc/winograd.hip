@@ -26,6 +26,7 @@
 
 #include "common.h"
 #include "mfma_gemm.h"
+#include "wino_gemm.h"
 
 namespace tsplit {
 using namespace mg;
@@ -375,6 +376,24 @@ class GemmTiming {
   bool on_ = false;
 };
 
+// compute units of the current device and resident blocks of the GEMM kernel on each, asked once
+inline int compute_units() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus < 1) {
+      (void)hipGetLastError();
+      cus = 256;
+    }
+    return cus;
+  }();
+  return n;
+}
+inline int gemm_blocks_per_cu() {
+  static const int n = blocks_per_cu(wg::wino_gemm_kernel);
+  return n;
+}
+
 // bytes of V and M one run of images may take together
 inline int64_t run_bytes() {
   const char *e = std::getenv("TSPLIT_WINOGRAD_RUN_MIB");
@@ -411,8 +430,6 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
   float *V = VM, *M = VM + static_cast<int64_t>(kXi) * gathered * ld_max;
   hipLaunchKernelGGL(wino_filter_kernel, dim3((produced * gathered + 255) / 256), dim3(256), 0, st, w, U, produced,
                      gathered, rotated);
-  using AL = KContigBufLoader<128>;
-  using BL = MnContigBufLoader<128>;
   for (int first = 0; first < imgs; first += run) {
     const int n = std::min(run, imgs - first);
     WinoGeo gi{gathered, H, W, th, tw, n * per_img, (n * per_img + 3) / 4 * 4,
@@ -424,15 +441,10 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
       hipLaunchKernelGGL(wino_input_kernel<true>, dim3((gi.ld + 255) / 256, gathered), dim3(256), 0, st, xr, V, gi);
     else
       hipLaunchKernelGGL(wino_input_kernel<false>, dim3((gi.ld + 255) / 256, gathered), dim3(256), 0, st, xr, V, gi);
-    const int tm = (produced + 127) / 128, tn = (gi.ld + 127) / 128;
-    typename AL::Params ap{U, gathered, produced, gathered};
-    typename BL::Params bp{V, gi.ld, gi.ld, gathered};
     {
       GemmTiming timed(st, 0, 2.0 * kXi * produced * static_cast<double>(gi.ld) * gathered);
-      hipLaunchKernelGGL((mfma_batched_gemm_kernel<128, 128, 2, 2, AL, BL>), dim3(grid_blocks(tm, tn, kXi)),
-                         dim3(kThreads), 0, st, ap, bp, M, static_cast<int64_t>(produced) * gathered,
-                         static_cast<int64_t>(gathered) * gi.ld, static_cast<int64_t>(produced) * gi.ld, produced, gi.ld,
-                         gathered, TileGrid{tm, tn, tm * tn * kXi});
+      wg::launch(wg::Problem{U, V, M, produced, gathered, gi.ld, (produced + 127) / 128, (gi.ld + 127) / 128}, st,
+                 gemm_blocks_per_cu(), compute_units());
     }
     hipLaunchKernelGGL(wino_output_kernel, dim3((go.tiles + 255) / 256, produced), dim3(256), 0, st, M,
                        y + static_cast<int64_t>(first) * produced * H * W, go);
