@@ -166,6 +166,299 @@ static __global__ __launch_bounds__(kThreads, 4) void wino_gemm_kernel(Problem p
   }
 }
 
+// ---------------------------------------------------------------- filter-gradient GEMMs of narrow layers
+// dU[xi] (rows x cols) = Y[xi] (rows x depth) V[xi]^T (cols x depth), both operands depth-contiguous, cut along
+// the depth (the tiles of the layer) into ranges; block group z = range * 36 + xi writes its partial sum
+// to out + z * rows * cols.  With 64 output or input channels a 128 x 128 block tile leaves two or three
+// of the four waves without a sub-tile.  Here the block tile is TM x TN (64 or 128 each, not both 128)
+// and the waves that have no sub-tile of their own share the depth instead: the 4 / (TM/64 * TN/64) = KG
+// waves on one 64 x 64 sub-tile each take every KG-th 16-wide k-step of a 16*KG-wide chunk, and their
+// accumulators are added through LDS at the end, in a fixed order.  A chunk row is 64*KG bytes, so a
+// row's loads cover whole 128-byte lines, and the LDS rows (16*KG + 4 floats) are free of bank conflicts
+// for both the 16-byte stores and the 16-byte fragment reads.  One LDS stage; the next chunk waits in
+// registers while the current one is multiplied.
+struct GradProblem {
+  const float *Y;   // [36][rows][ld]
+  const float *V;   // [36][cols][ld]
+  float *out;       // [ranges * 36][rows][cols]
+  int rows, cols, ld;
+  int kchunk;       // depth per range, a multiple of 64
+  int tm, tn;
+};
+
+template <int TM, int TN>
+static __global__ __launch_bounds__(kThreads, 3) void wino_grad_gemm_narrow_kernel(GradProblem p, TileGrid tg) {
+  constexpr int SUB = (TM / 64) * (TN / 64);   // 64 x 64 sub-tiles of the block tile
+  constexpr int KG = 4 / SUB;                  // waves per sub-tile
+  static_assert(SUB == 1 || SUB == 2, "narrow tiles only: 64x64, 128x64, 64x128");
+  constexpr int CH = BK * KG;                  // chunk depth
+  constexpr int STRIDE = CH + 4;               // LDS row pitch in floats
+  constexpr int LPR = CH / 4;                  // lanes (16-byte words) per row
+  constexpr int RPP = kThreads / LPR;          // rows per pass
+  constexpr int PA = TM / RPP, PB = TN / RPP;  // passes per operand
+  constexpr int kOperands = (TM + TN) * STRIDE;
+  constexpr int kReduce = (KG / 2) * SUB * 64 * 64;   // accumulators parked in one round of the final sum
+  constexpr int kLds = kOperands > kReduce ? kOperands : kReduce;
+  __shared__ __attribute__((aligned(16))) float lds[kLds];
+
+  int z, tile_m, tile_n;
+  if (!block_tile(tg, z, tile_m, tile_n)) return;
+  const int range = z / kXi, xi = z - range * kXi;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int sub = wave % SUB, g = wave / SUB;            // sub-tile and k-group of this wave
+  const int wm0 = TM == 128 ? 64 * sub : 0, wn0 = TN == 128 ? 64 * sub : 0;
+  const int m0 = tile_m * TM, n0 = tile_n * TN;
+  const int kbegin = range * p.kchunk, kend = min(p.ld, kbegin + p.kchunk);
+
+  // loaders: thread -> (row tid / LPR + RPP * pass, word tid % LPR); rows beyond the matrix and words
+  // beyond the range read as zeros through an out-of-range offset
+  const int quad = tid % LPR, prow = tid / LPR;
+  const float *abase = p.Y + static_cast<int64_t>(xi) * p.rows * p.ld + static_cast<int64_t>(m0) * p.ld;
+  const float *bbase = p.V + static_cast<int64_t>(xi) * p.cols * p.ld + static_cast<int64_t>(n0) * p.ld;
+  const int arows = min(TM, p.rows - m0), brows = min(TN, p.cols - n0);
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(abase), 0, static_cast<int>(static_cast<int64_t>(arows) * p.ld * 4), kBufFlags);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(bbase), 0, static_cast<int>(static_cast<int64_t>(brows) * p.ld * 4), kBufFlags);
+  unsigned a_voff[PA], b_voff[PB];
+#pragma unroll
+  for (int s = 0; s < PA; ++s) {
+    const int row = prow + RPP * s;
+    a_voff[s] = row < arows ? (static_cast<unsigned>(row) * static_cast<unsigned>(p.ld) + 4u * quad) * 4u : kOobOffset;
+  }
+#pragma unroll
+  for (int s = 0; s < PB; ++s) {
+    const int row = prow + RPP * s;
+    b_voff[s] = row < brows ? (static_cast<unsigned>(row) * static_cast<unsigned>(p.ld) + 4u * quad) * 4u : kOobOffset;
+  }
+  u32x4 areg[PA], breg[PB];
+  auto load = [&](int k0) {
+    // ld is a multiple of 4 and so is every word's position: a word lies wholly inside the range or outside
+    const bool in = k0 + 4 * quad < kend;
+#pragma unroll
+    for (int s = 0; s < PA; ++s) areg[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, in ? a_voff[s] : kOobOffset, k0 * 4, 0);
+#pragma unroll
+    for (int s = 0; s < PB; ++s) breg[s] = __builtin_amdgcn_raw_buffer_load_b128(rb, in ? b_voff[s] : kOobOffset, k0 * 4, 0);
+  };
+  float *lds_a = lds, *lds_b = lds + TM * STRIDE;
+  auto store = [&]() {
+#pragma unroll
+    for (int s = 0; s < PA; ++s) *reinterpret_cast<u32x4 *>(lds_a + (prow + RPP * s) * STRIDE + 4 * quad) = areg[s];
+#pragma unroll
+    for (int s = 0; s < PB; ++s) *reinterpret_cast<u32x4 *>(lds_b + (prow + RPP * s) * STRIDE + 4 * quad) = breg[s];
+  };
+
+  acc16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  if (kbegin < kend) {
+    load(kbegin);
+    store();
+  }
+  __syncthreads();
+  const bool live = m0 + wm0 < p.rows && n0 + wn0 < p.cols;
+  for (int k0 = kbegin; k0 < kend; k0 += CH) {
+    const bool more = k0 + CH < kend;
+    if (more) load(k0 + CH);
+    if (live) {
+      // this wave's 16 of the chunk's k values: lanes 0-31 supply k = 8j + i, lanes 32-63 k = 8j + 4 + i
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        float fa[2][4], fb[2][4];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const float4 qa = *reinterpret_cast<const float4 *>(lds_a + (wm0 + 32 * i + (lane & 31)) * STRIDE + BK * g + 8 * j +
+                                                              4 * (lane >> 5));
+          const float4 qb = *reinterpret_cast<const float4 *>(lds_b + (wn0 + 32 * i + (lane & 31)) * STRIDE + BK * g + 8 * j +
+                                                              4 * (lane >> 5));
+          fa[i][0] = qa.x, fa[i][1] = qa.y, fa[i][2] = qa.z, fa[i][3] = qa.w;
+          fb[i][0] = qb.x, fb[i][1] = qb.y, fb[i][2] = qb.z, fb[i][3] = qb.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+          for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+              acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
+      }
+    }
+    __syncthreads();   // every wave has read the chunk
+    if (more) {
+      store();
+      __syncthreads();
+    }
+  }
+
+  // sum over the k-groups: the upper half parks its accumulators ([register][lane] per wave), the lower
+  // half adds them; then once more until group 0 holds the sum.  The loop above ended with a barrier.
+#pragma unroll
+  for (int half = KG / 2; half >= 1; half /= 2) {
+    float *park = lds + ((g - half) * SUB + sub) * (64 * 64) + lane;
+    if (g >= half && g < 2 * half) {
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) park[((mi * 2 + ni) * 16 + e) * 64] = acc[mi][ni][e];
+    }
+    __syncthreads();
+    if (g < half) {
+      const float *from = lds + (g * SUB + sub) * (64 * 64) + lane;
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[mi][ni][e] += from[((mi * 2 + ni) * 16 + e) * 64];
+    }
+    __syncthreads();
+  }
+  if (g != 0 || !live) return;
+  float *__restrict__ o = p.out + static_cast<int64_t>(z) * p.rows * p.cols;
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const int n = n0 + wn0 + 32 * ni + (lane & 31);
+    if (n >= p.cols) continue;
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+      const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = mb + 8 * (e >> 2) + (e & 3);
+        if (m < p.rows) o[static_cast<int64_t>(m) * p.cols + n] = acc[mi][ni][e];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- filter-gradient GEMMs, 128 x 128 tiles
+// Same product and output layout as above.  The unit of work is one tile of one (range, xi) pair; the
+// grid is NB resident blocks on every compute unit and block L (in the XCD-aware order) takes units
+// L, L + G, L + 2G, ...: every block gets the same number of equal units when the host chooses the number
+// of ranges so that the units fill a whole number of rounds, and the blocks of one XCD work at any time
+// on the tiles of the same few (range, xi) pairs, which read the same rows of Y and V through that XCD's
+// L2.  (With one tile per block, a launch of 576 or 864 blocks left a quarter of the matrix pipes idle
+// in its last round, and a launch cut finer paid a prologue and a drained pipeline per block.)  As in the
+// forward kernel, the next unit's first loads are issued before the finished unit's stores.  The LDS
+// request is padded so that exactly NB blocks fit a compute unit: the dispatcher then cannot stack the
+// grid unevenly.
+template <int NB>
+static __global__ __launch_bounds__(kThreads, NB) void wino_grad_gemm_kernel(GradProblem p, int units) {
+  using Loader = KContigBufLoader<128>;
+  using Lds = typename Loader::Lds;
+  constexpr int kStage = 2 * Lds::kFloats;
+  constexpr int kFit = (160 * 1024 / (NB + 1)) / 4 + 64;   // more than an (NB+1)-th of the LDS
+  constexpr int kLds = 2 * kStage > kFit ? 2 * kStage : kFit;
+  __shared__ __attribute__((aligned(16))) float lds[kLds];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
+  const int per_group = p.tm * p.tn;
+  const int G = gridDim.x;
+  int u = (blockIdx.x & 7) * (G >> 3) + (blockIdx.x >> 3);
+  if (u >= units) return;
+
+  int z, m0, n0, kbegin, kend;
+  Loader la, lb;
+  auto start = [&](int unit) {
+    z = unit / per_group;
+    const int tile = unit - z * per_group;
+    const int tile_n = tile / p.tm;
+    m0 = (tile - tile_n * p.tm) * 128;
+    n0 = tile_n * 128;
+    const int range = z / kXi, xi = z - range * kXi;
+    kbegin = range * p.kchunk;
+    kend = min(p.ld, kbegin + p.kchunk);
+    typename Loader::Params ap{p.Y + static_cast<int64_t>(xi) * p.rows * p.ld, p.ld, p.rows, p.ld};
+    typename Loader::Params bp{p.V + static_cast<int64_t>(xi) * p.cols * p.ld, p.ld, p.cols, p.ld};
+    la.init(ap, m0, tid);
+    lb.init(bp, n0, tid);
+    la.load(kbegin, kend);
+    lb.load(kbegin, kend);
+  };
+  start(u);
+
+  for (;;) {
+    acc16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    // the last k-step of the previous unit ended with a barrier: stage 0 is free
+    la.store(lds, tid);
+    lb.store(lds + Lds::kFloats, tid);
+    __syncthreads();
+
+    const bool live = m0 + wm0 < p.rows && n0 + wn0 < p.cols;
+    int stage = 0;
+    for (int k0 = kbegin; k0 < kend; k0 += BK) {
+      const bool more = k0 + BK < kend;
+      if (more) {
+        la.load(k0 + BK, kend);
+        lb.load(k0 + BK, kend);
+      }
+      if (live) {
+        const float *sa = lds + stage * kStage, *sb = sa + Lds::kFloats;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          float fa[2][4], fb[2][4];
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            Lds::frag(sa, wm0 + 32 * i, j, lane, fa[i]);
+            Lds::frag(sb, wn0 + 32 * i, j, lane, fb[i]);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+              for (int ni = 0; ni < 2; ++ni)
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi][e], fb[ni][e], acc[mi][ni], 0, 0, 0);
+        }
+      }
+      if (more) {
+        float *sa = lds + (stage ^ 1) * kStage;
+        la.store(sa, tid);
+        lb.store(sa + Lds::kFloats, tid);
+      }
+      __syncthreads();
+      stage ^= 1;
+    }
+
+    float *__restrict__ o = p.out + static_cast<int64_t>(z) * p.rows * p.cols;
+    const int om0 = m0 + wm0, on0 = n0 + wn0;
+    u += G;
+    const bool again = u < units;
+    if (again) start(u);
+    if (live) {
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) {
+        const int n = on0 + 32 * ni + (lane & 31);
+        if (n >= p.cols) continue;
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) {
+          const int mb = om0 + 32 * mi + 4 * (lane >> 5);
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int m = mb + 8 * (e >> 2) + (e & 3);
+            if (m < p.rows) o[static_cast<int64_t>(m) * p.cols + n] = acc[mi][ni][e];
+          }
+        }
+      }
+    }
+    if (!again) break;
+  }
+}
+
 // One resident round of blocks: `blocks_per_cu` (what hipOccupancyMaxActiveBlocksPerMultiprocessor reports for
 // the kernel) on each of `cus` compute units, never more blocks than tiles.
 inline void launch(const Problem &p, hipStream_t st, int blocks_per_cu, int cus) {

@@ -273,23 +273,6 @@ __global__ __launch_bounds__(256) void wino_grad_kernel(const float *__restrict_
   }
 }
 
-// 36 GEMMs dU[xi] (O x C) = Y[xi] (O x tiles) V[xi]^T, each cut along the tiles into `splits`
-// ranges of `kchunk`: block group z = split * 36 + xi writes its partial sum to out + z * O * C
-template <class ALoader, class BLoader>
-__global__ __launch_bounds__(kThreads) void wino_grad_gemm_kernel(typename ALoader::Params ap, typename BLoader::Params bp,
-                                                                   float *__restrict__ out, int64_t a_xi, int64_t b_xi, int M,
-                                                                   int N, int K, int kchunk, TileGrid tg) {
-  int z, tile_m, tile_n;
-  if (!block_tile(tg, z, tile_m, tile_n)) return;
-  const int split = z / kXi, xi = z - split * kXi;
-  ap.p += xi * a_xi;
-  bp.p += xi * b_xi;
-  const int kbegin = split * kchunk;
-  mfma_gemm_tile<128, 128, 2, 2, ALoader, BLoader, RowMajorCols>(ap, bp, out + static_cast<int64_t>(z) * M * N,
-                                                                 static_cast<int64_t>(N), RowMajorCols{}, M, N, tile_m * 128,
-                                                                 tile_n * 128, kbegin, min(K, kbegin + kchunk));
-}
-
 // rows of G^T applied to (u0 .. u5)
 __device__ __forceinline__ void gt_rows(const float u[6], float w[3]) {
   const float s12 = u[1] + u[2], s34 = u[3] + u[4];
@@ -394,6 +377,76 @@ inline int gemm_blocks_per_cu() {
   return n;
 }
 
+// How the filter-gradient GEMMs of one run are cut: tile shape, depth per range, and (128 x 128 tiles) the
+// persistent grid.  Narrow layers (64 produced or gathered channels) take 64-wide tiles whose idle waves
+// share the depth, one tile per block, with as many ranges as give three blocks per compute unit.  The
+// others run on the persistent kernel: the number of ranges is chosen so that the units (tiles x ranges x
+// 36) fill one, two or three rounds of the grid as fully as possible, fewer rounds winning unless more
+// rounds fill at least 7 % better; a range keeps at least 12 k-steps.
+struct GradPlan {
+  int tile_m, tile_n;   // block tile
+  int tm, tn;           // tiles
+  int kchunk;           // depth per range
+  int grid;             // persistent grid (128 x 128 tiles), else 0
+};
+constexpr int kGradBlocksPerCu = 3;
+
+inline GradPlan plan_grad_gemm(int O, int C, int ld, int cus) {
+  GradPlan g{};
+  const int slots = cus * kGradBlocksPerCu / 8 * 8;
+  if (O <= 64 || C <= 64) {
+    g.tile_m = O <= 64 ? 64 : 128;
+    g.tile_n = (g.tile_m == 128 || C <= 64) ? 64 : 128;
+    g.tm = (O + g.tile_m - 1) / g.tile_m;
+    g.tn = (C + g.tile_n - 1) / g.tile_n;
+    const int per = kXi * g.tm * g.tn;
+    int ranges = std::max(1, (slots + per / 2) / per);
+    ranges = std::min(ranges, std::max(1, ld / 1024));
+    g.kchunk = ((ld + ranges - 1) / ranges + 63) / 64 * 64;
+    g.grid = 0;
+    return g;
+  }
+  g.tile_m = g.tile_n = 128;
+  g.tm = (O + 127) / 128;
+  g.tn = (C + 127) / 128;
+  const int per = kXi * g.tm * g.tn;
+  const int max_ranges = std::max(1, ld / (12 * BK));
+  int best_ranges = 1;
+  double best_fill = 0.0;
+  for (int rounds = 1; rounds <= 3; ++rounds) {
+    const int ranges = std::min(max_ranges, std::max(1, rounds * slots / per));
+    const int units = per * ranges;
+    const double fill = static_cast<double>(units) / (static_cast<double>((units + slots - 1) / slots) * slots);
+    if (fill > best_fill + 0.07 || (rounds == 1)) {
+      best_fill = fill;
+      best_ranges = ranges;
+    }
+  }
+  g.kchunk = ((ld + best_ranges - 1) / best_ranges + BK - 1) / BK * BK;
+  g.grid = slots;
+  return g;
+}
+
+// `here` ranges of p.kchunk cover p.ld; partial sum z = range * 36 + xi goes to p.out + z * rows * cols
+inline void launch_grad_gemm(const GradPlan &g, wg::GradProblem p, int here, hipStream_t st) {
+  p.tm = g.tm;
+  p.tn = g.tn;
+  const int units = g.tm * g.tn * kXi * here;
+  if (g.grid > 0) {
+    const int grid = std::min(g.grid, (units + 7) / 8 * 8);
+    hipLaunchKernelGGL((wg::wino_grad_gemm_kernel<kGradBlocksPerCu>), dim3(grid), dim3(kThreads), 0, st, p, units);
+    return;
+  }
+  const TileGrid tg{g.tm, g.tn, units};
+  const dim3 grid(grid_blocks(g.tm, g.tn, kXi * here));
+  if (g.tile_m == 64 && g.tile_n == 64)
+    hipLaunchKernelGGL((wg::wino_grad_gemm_narrow_kernel<64, 64>), grid, dim3(kThreads), 0, st, p, tg);
+  else if (g.tile_m == 128)
+    hipLaunchKernelGGL((wg::wino_grad_gemm_narrow_kernel<128, 64>), grid, dim3(kThreads), 0, st, p, tg);
+  else
+    hipLaunchKernelGGL((wg::wino_grad_gemm_narrow_kernel<64, 128>), grid, dim3(kThreads), 0, st, p, tg);
+}
+
 // bytes of V and M one run of images may take together
 inline int64_t run_bytes() {
   const char *e = std::getenv("TSPLIT_WINOGRAD_RUN_MIB");
@@ -462,18 +515,14 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
   TS_REQUIRE(run > 0, "conv (Winograd): one image's tiles do not fit 32-bit offsets");
   const int runs = (imgs + run - 1) / run;
   const int ld_max = (run * per_img + 3) / 4 * 4;
-  // enough blocks for three per CU, each with at least 16 k-steps
-  const int tm = (O + 127) / 128, tn = (C + 127) / 128;
-  int splits = std::max(1, (768 + kXi * tm * tn / 2) / (kXi * tm * tn));
-  splits = std::min(splits, std::max(1, ld_max / (16 * BK)));
-  const int kchunk = ((ld_max + splits - 1) / splits + BK - 1) / BK * BK;
+  const GradPlan plan = plan_grad_gemm(O, C, ld_max, compute_units());
+  const int kchunk = plan.kchunk;
   const int parts_max = runs * ((ld_max + kchunk - 1) / kchunk);
   const int64_t oc = static_cast<int64_t>(O) * C;
   float *VY = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(kXi) * (C + O) * ld_max * 4));
   float *part = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(parts_max) * kXi * oc * 4));
   TS_REQUIRE(VY && part, "conv (Winograd): no scratch memory");
   float *V = VY, *Y = VY + static_cast<int64_t>(kXi) * C * ld_max;
-  using KL = KContigBufLoader<128>;
   int parts = 0;
   for (int first = 0; first < imgs; first += run) {
     const int n = std::min(run, imgs - first);
@@ -491,13 +540,10 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
     else
       hipLaunchKernelGGL(wino_grad_kernel<false>, grid_y, dim3(256), 0, st, dyr, Y, gy);
     const int here = (gx.ld + kchunk - 1) / kchunk;
-    typename KL::Params ap{Y, gx.ld, O, gx.ld};
-    typename KL::Params bp{V, gx.ld, C, gx.ld};
     {
       GemmTiming timed(st, 1, 2.0 * kXi * O * static_cast<double>(gx.ld) * C);
-      hipLaunchKernelGGL((wino_grad_gemm_kernel<KL, KL>), dim3(grid_blocks(tm, tn, kXi * here)), dim3(kThreads), 0, st, ap,
-                         bp, part + static_cast<int64_t>(parts) * kXi * oc, static_cast<int64_t>(O) * gx.ld,
-                         static_cast<int64_t>(C) * gx.ld, O, C, gx.ld, kchunk, TileGrid{tm, tn, tm * tn * kXi * here});
+      launch_grad_gemm(plan, wg::GradProblem{Y, V, part + static_cast<int64_t>(parts) * kXi * oc, O, C, gx.ld, kchunk, 0, 0},
+                       here, st);
     }
     parts += here;
   }
