@@ -420,6 +420,28 @@ int TSplit_BatchNormRelu_gradient(const DLArrayHandle gradient_Y, const DLArrayH
                                   DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
                                   DLStreamHandle stream_handle, ProfilerHandle p);
 
+/* ---- Convolution that hands its output's batch statistics to the BatchNorm behind it.  NO counterpart
+ *      in the reference, where the BatchNorm call (src/ops/CudnnBn.cu:12-210) reads the convolution's
+ *      output (src/ops/CudnnConv2d.cu:6-206) once more to get them; for hosts that know a BatchNorm
+ *      follows.  `stats` is float32 storage, 8-byte aligned, viewed as [slots][out_channels][2] doubles.
+ *      TSplit_Conv2dBatchNormStats computes exactly what CuDNN_DLGpuConv2d computes (same kernels, same
+ *      bits) and writes the per-channel (sum, sum of squares) of `output` into row `slot`; a host that
+ *      runs the convolution on batch micro-tensors gives every piece its own row.
+ *      TSplit_BatchNormFromStats adds rows 0 .. slots-1 in that order, derives the batch mean and
+ *      variance over all of input_X, and applies the BatchNorm (relu == 0) or BatchNorm + Relu
+ *      (relu != 0: both save arrays required, as for TSplit_BatchNormRelu) in one pass over input_X.
+ *      The gradients are those of CuDNN_DLGpuBatch_Normalization_gradient /
+ *      TSplit_BatchNormRelu_gradient with the saved statistics. ---- */
+int TSplit_Conv2dBatchNormStats(const DLArrayHandle input_x, const DLArrayHandle input_f,
+                                DLArrayHandle output, const int padding, const int padding2,
+                                const int stride, DLArrayHandle stats, int slot,
+                                DLStreamHandle stream_handle, ProfilerHandle p);
+int TSplit_BatchNormFromStats(const DLArrayHandle input_X, const DLArrayHandle stats, int slots,
+                              const DLArrayHandle bn_scale, const DLArrayHandle bn_bias,
+                              DLArrayHandle output_Y, float eps, DLArrayHandle save_mean_arr,
+                              DLArrayHandle save_var_arr, int relu, DLStreamHandle stream_handle,
+                              ProfilerHandle p);
+
 /* ---- Which routine a convolution takes.  NO counterpart in the reference (cuDNN's choice is
  *      internal there, src/ops/CudnnConv2d.cu:66).  Returns 1 when CuDNN_DLGpuConv2d (pass 0),
  *      CuDNN_DLGpuConv2d_Gradient_of_Data (pass 1) or CuDNN_DLGpuConv2d_Gradient_of_Filter (pass 2)

@@ -134,17 +134,19 @@ template <int VEC, bool RELU>
 __global__ __launch_bounds__(kThreads) void bn_apply_kernel(const float *__restrict__ x, float *__restrict__ y,
                                                             const float *__restrict__ gamma,
                                                             const float *__restrict__ beta,
-                                                            const double *__restrict__ part, int S, Geo g, float eps,
-                                                            double inv_m, float *__restrict__ save_mean,
+                                                            const double *__restrict__ part, int S, int64_t part_c,
+                                                            int64_t part_k, Geo g, float eps, double inv_m,
+                                                            float *__restrict__ save_mean,
                                                             float *__restrict__ save_istd) {
   using W = typename Word<VEC>::T;
   __shared__ float coef[2];
   __shared__ double sm[kWaves];
   const int c = blockIdx.y;
   double s = 0.0, q = 0.0;
+  // partial k of channel c is the pair at part[(c * part_c + k * part_k) * 2]
   for (int k = threadIdx.x; k < S; k += kThreads) {   // fixed order per thread, fixed tree: deterministic
-    s += part[(static_cast<int64_t>(c) * S + k) * 2];
-    q += part[(static_cast<int64_t>(c) * S + k) * 2 + 1];
+    s += part[(c * part_c + k * part_k) * 2];
+    q += part[(c * part_c + k * part_k) * 2 + 1];
   }
   if (S > 1) {
     s = block_sum<double, kWaves>(s, sm);
@@ -505,10 +507,44 @@ bool make_plan(const DLArray *x, bool all_aligned, uint32_t words_per_block, int
   return true;
 }
 
+// dst[c * 2], dst[c * 2 + 1] = the sums of channel c's S partial pairs (one block per channel)
+__global__ __launch_bounds__(kThreads) void bn_sums_fold_kernel(const double *__restrict__ part, int S,
+                                                                double *__restrict__ dst) {
+  __shared__ double sm[kWaves];
+  const int c = blockIdx.x;
+  double s = 0.0, q = 0.0;
+  for (int k = threadIdx.x; k < S; k += kThreads) {
+    s += part[(static_cast<int64_t>(c) * S + k) * 2];
+    q += part[(static_cast<int64_t>(c) * S + k) * 2 + 1];
+  }
+  s = block_sum<double, kWaves>(s, sm);
+  q = block_sum<double, kWaves>(q, sm);
+  if (threadIdx.x == 0) {
+    dst[c * 2] = s;
+    dst[c * 2 + 1] = q;
+  }
+}
+
 inline const float *cf(const DLArray *a) { return static_cast<const float *>(a->data); }
 inline float *mf(DLArray *a) { return static_cast<float *>(a->data); }
 
 }  // namespace
+
+int bn_channel_sums(const DLArray *y, double *dst, hipStream_t st) {
+  Plan pl;
+  TS_REQUIRE(make_plan(y, aligned16(y->data), 16 * kThreads, 16384, pl), "channel sums: unsupported shape");
+  const int64_t C = y->shape[1];
+  double *part = static_cast<double *>(scratch_get(st, 1, static_cast<size_t>(C) * pl.S * 2 * sizeof(double)));
+  TS_REQUIRE(part, "channel sums: no scratch memory");
+  const dim3 gs(pl.S, static_cast<unsigned>(C));
+  if (pl.vec == 4)
+    hipLaunchKernelGGL(bn_stats_kernel<4>, gs, dim3(kThreads), 0, st, cf(y), part, pl.g, pl.S);
+  else
+    hipLaunchKernelGGL(bn_stats_kernel<1>, gs, dim3(kThreads), 0, st, cf(y), part, pl.g, pl.S);
+  hipLaunchKernelGGL(bn_sums_fold_kernel, dim3(static_cast<unsigned>(C)), dim3(kThreads), 0, st, part, pl.S, dst);
+  return 0;
+}
+
 }  // namespace tsplit
 
 using namespace tsplit;
@@ -568,7 +604,7 @@ static int bn_forward(const char *who, bool relu, const DLArrayHandle input_X, c
   dim3 gs(st.S, static_cast<unsigned>(C)), ga(ap.S, static_cast<unsigned>(C));
 #define BN_APPLY(V, R)                                                                                              \
   hipLaunchKernelGGL((bn_apply_kernel<V, R>), ga, dim3(kThreads), 0, s, cf(input_X), mf(output_Y), cf(bn_scale),    \
-                     cf(bn_bias), part, st.S, ap.g, eps, inv_m, sm, sv)
+                     cf(bn_bias), part, st.S, static_cast<int64_t>(st.S), int64_t(1), ap.g, eps, inv_m, sm, sv)
   if (st.vec == 4) {
     hipLaunchKernelGGL(bn_stats_kernel<4>, gs, dim3(kThreads), 0, s, cf(input_X), part, st.g, st.S);
     if (relu)
@@ -600,6 +636,54 @@ int TSplit_BatchNormRelu(const DLArrayHandle input_X, const DLArrayHandle bn_sca
                          DLStreamHandle stream_handle, ProfilerHandle p) {
   return bn_forward("TSplit_BatchNormRelu", true, input_X, bn_scale, bn_bias, output_Y, eps, save_mean_arr,
                     save_var_arr, stream_handle, p);
+}
+
+// BatchNorm (relu == 0) or BatchNorm + Relu (relu != 0) forward whose batch statistics come from sums a
+// producer left: `stats` is float32 storage viewed as [slots][C][2] doubles, row k holding the per-channel
+// (sum, sum of squares) over one part of the batch (TSplit_Conv2dBatchNormStats writes such rows); the rows
+// are added in ascending order.  One pass over x: 8 B per element.
+int TSplit_BatchNormFromStats(const DLArrayHandle input_X, const DLArrayHandle stats, int slots,
+                              const DLArrayHandle bn_scale, const DLArrayHandle bn_bias, DLArrayHandle output_Y,
+                              float eps, DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr, int relu,
+                              DLStreamHandle stream_handle, ProfilerHandle p) {
+  const char *who = "TSplit_BatchNormFromStats";
+  TS_REQUIRE(input_X && stats && bn_scale && bn_bias && output_Y, "%s: NULL array", who);
+  TS_REQUIRE(input_X->ndim == 4 && output_Y->ndim == 4, "%s: input and output must be 4-D NCHW", who);
+  TS_REQUIRE(numel(input_X) == numel(output_Y), "%s: input/output sizes differ", who);
+  const int64_t C = input_X->shape[1];
+  TS_REQUIRE(numel(bn_scale) == C && numel(bn_bias) == C, "%s: scale/bias must hold C=%lld elements", who, (long long)C);
+  TS_REQUIRE(!save_mean_arr || numel(save_mean_arr) == C, "%s: save_mean must hold C elements", who);
+  TS_REQUIRE(!save_var_arr || numel(save_var_arr) == C, "%s: save_var must hold C elements", who);
+  TS_REQUIRE(!relu || (save_mean_arr && save_var_arr), "%s: the fused form needs both save arrays", who);
+  TS_REQUIRE(slots >= 1 && numel(stats) >= static_cast<int64_t>(slots) * C * 4, "%s: stats must hold slots * C * 4 floats", who);
+  TS_REQUIRE((reinterpret_cast<uintptr_t>(stats->data) & 7) == 0, "%s: stats must be 8-byte aligned", who);
+  hipStream_t s = stream_of(stream_handle);
+  ProfileScope ps(p, s, numel(input_X) + 2 * C, numel(output_Y), 0);
+  if (numel(input_X) == 0) return ps.finish();
+  const bool al = aligned16(input_X->data) && aligned16(output_Y->data);
+  Plan ap;
+  TS_REQUIRE(make_plan(input_X, al, 4 * kThreads, 1 << 22, ap), "%s: unsupported shape", who);
+  const double inv_m = 1.0 / static_cast<double>(ap.m);
+  float *sm = save_mean_arr ? mf(save_mean_arr) : nullptr;
+  float *sv = save_var_arr ? mf(save_var_arr) : nullptr;
+  const double *part = static_cast<const double *>(stats->data);
+  const dim3 ga(ap.S, static_cast<unsigned>(C));
+#define BN_APPLY_FROM(V, R)                                                                                        \
+  hipLaunchKernelGGL((bn_apply_kernel<V, R>), ga, dim3(kThreads), 0, s, cf(input_X), mf(output_Y), cf(bn_scale),   \
+                     cf(bn_bias), part, slots, int64_t(1), static_cast<int64_t>(C), ap.g, eps, inv_m, sm, sv)
+  if (ap.vec == 4) {
+    if (relu)
+      BN_APPLY_FROM(4, true);
+    else
+      BN_APPLY_FROM(4, false);
+  } else {
+    if (relu)
+      BN_APPLY_FROM(1, true);
+    else
+      BN_APPLY_FROM(1, false);
+  }
+#undef BN_APPLY_FROM
+  return ps.finish();
 }
 
 static int bn_backward(const char *who, bool relu, const DLArrayHandle gradient_Y, const DLArrayHandle input_X,

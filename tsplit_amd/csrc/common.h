@@ -27,6 +27,20 @@ inline float mib(int64_t elems) { return static_cast<float>(elems) * 4.0f / (102
 // that stream without waiting; ops on different streams never share one.
 void *scratch_get(hipStream_t stream, int slot, size_t bytes);
 
+// Where a convolution leaves per-channel partial sums of its output for a BatchNorm that follows:
+// partial k of channel c is the pair (sum, sum of squares) at part[(k * channels + c) * 2]; `used`
+// counts the partials written so far (a call may run as several launches).
+struct StatsSink {
+  float *part;
+  int channels;
+  int capacity;   // partials the buffer holds per channel
+  int used;
+};
+
+// Per-channel (sum, sum of squares) of a 4-D NCHW array by a pass of its own, as doubles: dst[c * 2],
+// dst[c * 2 + 1] (batchnorm.hip).
+int bn_channel_sums(const DLArray *y, double *dst, hipStream_t st);
+
 // Looks up, once per device, the address of the fixed scratch array behind
 // TSplit_SoftmaxCrossEntropyNoAlloc (called from the per-device init call).
 void softmax_noalloc_setup(int device_id);

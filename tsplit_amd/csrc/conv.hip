@@ -32,7 +32,7 @@
 namespace tsplit {
 // winograd.hip
 int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int gathered, int produced, int H, int W,
-                      bool rotated, hipStream_t st);
+                      bool rotated, hipStream_t st, StatsSink *sink = nullptr);
 int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, int imgs, int C, int O, int H, int W,
                                   hipStream_t st);
 namespace {
@@ -293,7 +293,33 @@ struct TapConvParams {
   // Column (i, j) of an image goes to element (out_a0 + out_s*i)*out_w + out_b0 + out_s*j of its
   // output plane.  out_s == 1 with out_a0 = out_b0 = 0 and out_w = the column width: linear.
   int out_s, out_a0, out_b0, out_w;
+  // STATS kernels: partial (sum, sum of squares) of output row m over the 32 columns [32 g, 32 g + 32)
+  // goes to stats[(g * M + m) * 2]
+  float *stats;
 };
+
+// Sums over the 32 lanes of each half of a wave for NR registers at once, NR = 32 or 16: in step b the
+// lanes whose bit b is clear keep the lower half of the registers and the others the upper half, each
+// adding what its partner held of that half, so that NR + NR/2 + ... shuffles do the work of 5 NR.
+// Afterwards r[0] of lane l is the sum of register (l % 32) for NR = 32, of register (l % 32) / 2 for
+// NR = 16 (both lanes of a pair hold it).
+template <int NR>
+__device__ __forceinline__ void half_wave_sums(float (&r)[NR], int lane) {
+  static_assert(NR == 32 || NR == 16, "one or two registers per lane and row");
+  constexpr int kTop = NR == 32 ? 4 : 3;   // register halving runs over lane bits 4..0 or 4..1
+#pragma unroll
+  for (int step = 0; step <= kTop; ++step) {
+    const int h = NR >> (step + 1);
+    const int bit = 4 - step;
+    const bool up = (lane >> bit) & 1;
+#pragma unroll
+    for (int i = 0; i < h; ++i) {
+      const float send = up ? r[i] : r[i + h], keep = up ? r[i + h] : r[i];
+      r[i] = keep + __shfl_xor(send, 1 << bit, 64);
+    }
+  }
+  if (NR == 16) r[0] += __shfl_xor(r[0], 1, 64);
+}
 
 // offset of output column n (without the row term)
 __device__ __forceinline__ int64_t tap_out_col(const TapConvParams &P, int n) {
@@ -338,7 +364,9 @@ struct StreamK {
 // 3 spills a dozen set-up values but keeps a third block resident, which pays on layers with
 // thousands of tiles (+1-4 % on the VGG layers) and costs on small ones (finer pieces, -1-3 % on
 // the ResNet-50 / Inception-v4 steps), so the launcher picks by tile count.
-template <int BM, int BN, int WM, int WN, bool BWD_DATA, bool RAW, int MINB>
+// STATS: a block that stores a whole tile also leaves the per-row sums and sums of squares of each
+// 32-column group of it (partial sums for a BatchNorm that follows; columns beyond N are zeros).
+template <int BM, int BN, int WM, int WN, bool BWD_DATA, bool RAW, int MINB, bool STATS = false>
 __global__ __launch_bounds__(kThreads, MINB) void conv_tap_kernel(TapConvParams P, float *__restrict__ out,
                                                                float *__restrict__ pieces, StreamK sk) {
   static_assert(WM * WN == 4 && BM / WM == 64 && BN / WN == 64, "each of the 4 waves owns a 64x64 sub-tile");
@@ -346,8 +374,11 @@ __global__ __launch_bounds__(kThreads, MINB) void conv_tap_kernel(TapConvParams 
   using BLds = MnMajorLds<BN>;
   constexpr int PA = BM / 64;        // 16-byte filter words per thread and step
   constexpr int KPT = BN / 16;       // gathered values per thread and step (consecutive k')
-  __shared__ __attribute__((aligned(16))) float lds_a[2][ALds::kFloats];
-  __shared__ __attribute__((aligned(16))) float lds_b[2][BLds::kFloats];
+  // one array: the STATS epilogue borrows the stages (4 waves x 32 x 68 floats) for its transposition
+  __shared__ __attribute__((aligned(16))) float lds_all[2 * (ALds::kFloats + BLds::kFloats)];
+  static_assert(!STATS || 4 * 32 * 68 <= 2 * (ALds::kFloats + BLds::kFloats), "the operand stages hold the staging areas");
+  float(*lds_a)[ALds::kFloats] = reinterpret_cast<float(*)[ALds::kFloats]>(lds_all);
+  float(*lds_b)[BLds::kFloats] = reinterpret_cast<float(*)[BLds::kFloats]>(lds_all + 2 * ALds::kFloats);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
@@ -524,6 +555,43 @@ __global__ __launch_bounds__(kThreads, MINB) void conv_tap_kernel(TapConvParams 
           }
         }
       }
+      if (STATS) {
+        // Row sums through LDS (the k-loop ended with a barrier: the stages are free).  A wave lays a
+        // 64 x 32 half of its sub-tile down as [column][row] - a lane's four consecutive rows are one
+        // 16-byte word - and then every lane sums one row over the 32 columns: pitch 68 keeps both the
+        // words and the column walks free of bank conflicts, and the 64 lanes store 64 neighbouring
+        // channels' pairs.
+        constexpr int kPitch = 68;
+        float *mine = lds_all + wave * (32 * kPitch);
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) {
+#pragma unroll
+          for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+              typedef float f32x4 __attribute__((ext_vector_type(4)));
+              const f32x4 v = {acc[mi][ni][4 * g4], acc[mi][ni][4 * g4 + 1], acc[mi][ni][4 * g4 + 2], acc[mi][ni][4 * g4 + 3]};
+              *reinterpret_cast<f32x4 *>(mine + (lane & 31) * kPitch + 32 * mi + 8 * g4 + 4 * (lane >> 5)) = v;
+            }
+          __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): a wave's own staging area needs no block barrier
+          __builtin_amdgcn_wave_barrier();
+          float sum = 0.f, sq = 0.f;
+#pragma unroll
+          for (int col = 0; col < 32; ++col) {
+            const float v = mine[col * kPitch + lane];
+            sum += v;
+            sq += v * v;
+          }
+          const int m = m0 + wm0 + lane, col0 = n0 + wn0 + 32 * ni;
+          if (m < P.M && col0 < P.N) {
+            float2 *dst = reinterpret_cast<float2 *>(P.stats + (static_cast<int64_t>(col0 >> 5) * P.M + m) * 2);
+            *dst = make_float2(sum, sq);
+          }
+          __builtin_amdgcn_s_waitcnt(0xc07f);
+          __builtin_amdgcn_wave_barrier();
+        }
+        __syncthreads();   // the next tile's first step is staged into this memory
+      }
     } else {
       // a piece of a cut tile: registers go to scratch as they are, [register][thread]
       const int slot = (it - (ks1 - ks0)) == it_begin ? 0 : 1;
@@ -542,7 +610,7 @@ __global__ __launch_bounds__(kThreads, MINB) void conv_tap_kernel(TapConvParams 
 // accumulator block of every wave (registers 16q .. 16q+15): each adds the pieces in ascending
 // block order and stores its share of the tile.  Thread and register layout are those of
 // conv_tap_kernel's epilogue.
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, bool STATS = false>
 __global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvParams P, float *__restrict__ out,
                                                                      const float *__restrict__ pieces, StreamK sk) {
   const int tile = blockIdx.x >> 2, q = blockIdx.x & 3;
@@ -566,6 +634,25 @@ __global__ __launch_bounds__(kThreads) void conv_tap_assemble_kernel(TapConvPara
     for (int e = 0; e < 16; ++e) acc[e] += __builtin_nontemporal_load(pc + e * kThreads);
   }
   const int n = n0 + wn0 + 32 * ni + (lane & 31);
+  if (STATS) {
+    // the pieces of columns beyond N are zeros: every lane takes part in the sums
+    float r[16], q[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      r[e] = acc[e];
+      q[e] = acc[e] * acc[e];
+    }
+    half_wave_sums<16>(r, lane);
+    half_wave_sums<16>(q, lane);
+    const int e = (lane & 31) >> 1;
+    const int m = m0 + wm0 + 32 * mi + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+    const int col0 = n0 + wn0 + 32 * ni;
+    if ((lane & 1) == 0 && m < P.M && col0 < P.N) {
+      float *dst = P.stats + (static_cast<int64_t>(col0 >> 5) * P.M + m) * 2;
+      dst[0] = r[0];
+      dst[1] = q[0];
+    }
+  }
   if (n >= P.N) return;
   const int64_t coff = tap_out_col(P, n);
   const int mb = m0 + wm0 + 32 * mi + 4 * (lane >> 5);
@@ -1383,7 +1470,7 @@ constexpr int kManyTiles = 1024;
 
 template <int BM, int BN, int WM, int WN, bool BWD_DATA, bool RAW = false>
 int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, float *out, hipStream_t st,
-                    const TapPhase *phase = nullptr) {
+                    const TapPhase *phase = nullptr, StatsSink *sink = nullptr) {
   TapConvParams P;
   int taps = g.kH * g.kW;
   P.out_s = 1;
@@ -1434,6 +1521,13 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
     P.out_a0 = phase->a0;
     P.out_b0 = phase->b0;
   }
+  P.stats = nullptr;
+  if (sink) {     // forward passes only: one partial per channel and 32 output columns
+    const int groups = (P.N + 31) / 32;
+    TS_REQUIRE(!BWD_DATA && !RAW && !phase && sink->used + groups <= sink->capacity, "conv: statistics buffer too small");
+    P.stats = sink->part + static_cast<int64_t>(sink->used) * P.M * 2;
+    sink->used += groups;
+  }
   P.wf = w_relaid;
   P.raw_row = BWD_DATA ? taps : g.C * taps;      // (only read by the RAW kernels; never with stride phases)
   P.raw_ch = BWD_DATA ? g.C * taps : taps;
@@ -1480,6 +1574,20 @@ int launch_conv_tap(const ConvGeo &g, const float *src, const float *w_relaid, f
     if (sk.total > 0) {          // (whole waves may cover every row exactly: then nothing is cut)
       pieces = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(grid) * 2 * BM * BN * sizeof(float)));
       TS_REQUIRE(pieces, "conv: no scratch memory for the pieces of cut tiles");
+    }
+  }
+  if constexpr (!BWD_DATA && !RAW) {
+    if (sink) {
+      if (many)
+        hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, false, false, 3, true>), dim3(grid), dim3(kThreads), 0, st, P,
+                           out, pieces, sk);
+      else
+        hipLaunchKernelGGL((conv_tap_kernel<BM, BN, WM, WN, false, false, 2, true>), dim3(grid), dim3(kThreads), 0, st, P,
+                           out, pieces, sk);
+      if (pieces)
+        hipLaunchKernelGGL((conv_tap_assemble_kernel<BM, BN, WM, WN, true>), dim3(cut_tiles * 4), dim3(kThreads), 0, st, P,
+                           out, pieces, sk);
+      return 0;
     }
   }
   if (many)
@@ -2062,18 +2170,80 @@ inline bool winograd_filter_grad_pays(const ConvGeo &g) {
   return forced == 1 || winograd_wide(g, 64);
 }
 
+// ------------------------------------------------------------------ statistics of the output
+// Folds the partial (sum, sum of squares) pairs the forward kernels leave, part[(k * C + c) * 2], k < used,
+// in two steps with a fixed order: `slices` blocks per group of 32 channels each sum a contiguous range
+// of k in double (lanes of a wave read neighbouring channels), then one thread per channel adds the
+// slices in ascending order and writes dst[c * 2], dst[c * 2 + 1] as doubles.
+__global__ __launch_bounds__(256) void conv_stats_fold_kernel(const float *__restrict__ part, int used, int C,
+                                                              double *__restrict__ tmp, int chunk) {
+  __shared__ double sm[8][32][2];
+  const int cc = threadIdx.x & 31, kk = threadIdx.x >> 5;
+  const int c = blockIdx.x * 32 + cc, slice = blockIdx.y;
+  const int kend = min(used, (slice + 1) * chunk);
+  double s = 0.0, q = 0.0;
+  if (c < C)
+    for (int k = slice * chunk + kk; k < kend; k += 8) {
+      const float2 v = *reinterpret_cast<const float2 *>(part + (static_cast<int64_t>(k) * C + c) * 2);
+      s += static_cast<double>(v.x);
+      q += static_cast<double>(v.y);
+    }
+  sm[kk][cc][0] = s;
+  sm[kk][cc][1] = q;
+  __syncthreads();
+  if (kk == 0 && c < C) {
+#pragma unroll
+    for (int j = 1; j < 8; ++j) {
+      s += sm[j][cc][0];
+      q += sm[j][cc][1];
+    }
+    tmp[(static_cast<int64_t>(slice) * C + c) * 2] = s;
+    tmp[(static_cast<int64_t>(slice) * C + c) * 2 + 1] = q;
+  }
+}
+__global__ __launch_bounds__(256) void conv_stats_final_kernel(const double *__restrict__ tmp, int slices, int C,
+                                                               double *__restrict__ dst) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  double s = 0.0, q = 0.0;
+  for (int j = 0; j < slices; ++j) {
+    s += tmp[(static_cast<int64_t>(j) * C + c) * 2];
+    q += tmp[(static_cast<int64_t>(j) * C + c) * 2 + 1];
+  }
+  dst[c * 2] = s;
+  dst[c * 2 + 1] = q;
+}
+
+constexpr int kStatsSlices = 64;
+
+// `stats_dst` (optional): per-channel (sum, sum of squares) of y as doubles, [O][2], for a BatchNorm that
+// follows.  The Winograd routine and the tap-major kernels produce them in their epilogues; the other
+// routes by a pass over y.
 int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y, int ph, int pw, int s,
-                 DLStreamHandle sh, ProfilerHandle p) {
+                 DLStreamHandle sh, ProfilerHandle p, double *stats_dst = nullptr) {
   ConvGeo g;
   if (geo_from(who, x, w, y, ph, pw, s, g)) return -1;
   hipStream_t st = stream_of(sh);
   ProfileScope ps(p, st, numel(x) + numel(w), numel(y), 0);
+  StatsSink sink{nullptr, g.O, 0, 0};
+  StatsSink *sk = nullptr;
+  if (stats_dst && numel(y) > 0 && !thin_fwd_ok(g) &&
+      (winograd_pays(g, g.C) ||
+       (g.C % BK == 0 && tap_kernel_images(g, static_cast<int64_t>(g.C) * g.H * g.W, numel(w)) > 0))) {
+    // one partial per 32 output positions at most, and a ragged group per run of images
+    sink.capacity = static_cast<int>((static_cast<int64_t>(g.imgs) * g.oH * g.oW + 31) / 32) + g.imgs;
+    const size_t bytes = static_cast<size_t>(sink.capacity) * g.O * 2 * sizeof(float) +
+                         static_cast<size_t>(kStatsSlices) * g.O * 2 * sizeof(double);
+    sink.part = static_cast<float *>(scratch_get(st, 7, bytes));
+    TS_REQUIRE(sink.part, "%s: no scratch memory", who);
+    sk = &sink;
+  }
   if (numel(y) > 0) {
     if (thin_fwd_ok(g)) {
       const int rc = launch_conv_thin_fwd(g, cf(x), cf(w), mf(y), st);
       if (rc) return rc;
     } else if (winograd_pays(g, g.C)) {
-      const int rc = conv_winograd_3x3(cf(x), cf(w), mf(y), g.imgs, g.C, g.O, g.H, g.W, false, st);
+      const int rc = conv_winograd_3x3(cf(x), cf(w), mf(y), g.imgs, g.C, g.O, g.H, g.W, false, st, sk);
       if (rc) return rc;
     } else if (g.C % BK == 0) {
       // a 1x1 filter [O][C] already is tap-major: used where it lies
@@ -2092,8 +2262,8 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
         const int rc = for_image_runs(g, per, [&](const ConvGeo &run, int64_t first) {
           const float *xr = cf(x) + first * x_img;
           float *yr = mf(y) + first * y_img;
-          return short_tiles(g.O) ? launch_conv_tap<64, 256, 1, 4, false>(run, xr, wf, yr, st)
-                           : launch_conv_tap<128, 128, 2, 2, false>(run, xr, wf, yr, st);
+          return short_tiles(g.O) ? launch_conv_tap<64, 256, 1, 4, false>(run, xr, wf, yr, st, nullptr, sk)
+                           : launch_conv_tap<128, 128, 2, 2, false>(run, xr, wf, yr, st, nullptr, sk);
         });
         if (rc) return rc;
       } else if (g.O <= 64) {
@@ -2108,6 +2278,23 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
         launch_fwd<64, 256, 1, 4>(g, cf(x), cf(w), mf(y), taps, st);
       else
         launch_fwd<128, 128, 2, 2>(g, cf(x), cf(w), mf(y), taps, st);
+    }
+  }
+  if (stats_dst) {
+    if (sk) {
+      // the slices' sums live behind the partials in the same scratch buffer (8-byte aligned: the
+      // partials are pairs of floats)
+      double *tmp = reinterpret_cast<double *>(sink.part + static_cast<int64_t>(sink.capacity) * g.O * 2);
+      const int slices = std::max(1, std::min(kStatsSlices, (sink.used + 63) / 64));
+      const int chunk = (sink.used + slices - 1) / slices;
+      hipLaunchKernelGGL(conv_stats_fold_kernel, dim3((g.O + 31) / 32, slices), dim3(256), 0, st, sink.part, sink.used, g.O,
+                         tmp, chunk);
+      hipLaunchKernelGGL(conv_stats_final_kernel, dim3((g.O + 255) / 256), dim3(256), 0, st, tmp, slices, g.O, stats_dst);
+    } else if (numel(y) > 0) {
+      if (bn_channel_sums(y, stats_dst, st)) return -1;
+    } else {
+      hipLaunchKernelGGL(conv_stats_final_kernel, dim3((g.O + 255) / 256), dim3(256), 0, st,
+                         static_cast<const double *>(nullptr), 0, g.O, stats_dst);
     }
   }
   return ps.finish();
@@ -2238,6 +2425,22 @@ int CuDNN_DLGpuConv2d(const DLArrayHandle input_x, const DLArrayHandle input_f, 
                       const int padding, const int padding2, const int stride, DLStreamHandle stream_handle,
                       ProfilerHandle p) {
   return conv_forward("CuDNN_DLGpuConv2d", input_x, input_f, output, padding, padding2, stride, stream_handle, p);
+}
+
+// Convolution that also leaves the per-channel sum and sum of squares of its output, as doubles, in row
+// `slot` of `stats` (float32 storage viewed as [slots][C][2] doubles): the statistics pass of a BatchNorm
+// that follows (TSplit_BatchNormFromStats) then need not read the output again.
+int TSplit_Conv2dBatchNormStats(const DLArrayHandle input_x, const DLArrayHandle input_f, DLArrayHandle output,
+                                const int padding, const int padding2, const int stride, DLArrayHandle stats,
+                                int slot, DLStreamHandle stream_handle, ProfilerHandle p) {
+  TS_REQUIRE(input_x && input_f && output && stats, "Conv2dBatchNormStats: NULL array");
+  TS_REQUIRE(input_f->ndim == 4, "Conv2dBatchNormStats: filter must be 4-D");
+  const int64_t C = input_f->shape[0];
+  TS_REQUIRE(slot >= 0 && numel(stats) >= (static_cast<int64_t>(slot) + 1) * C * 4,
+             "Conv2dBatchNormStats: stats must hold (slot + 1) * out_channels * 4 floats");
+  TS_REQUIRE((reinterpret_cast<uintptr_t>(stats->data) & 7) == 0, "Conv2dBatchNormStats: stats must be 8-byte aligned");
+  double *dst = static_cast<double *>(stats->data) + static_cast<int64_t>(slot) * C * 2;
+  return conv_forward("Conv2dBatchNormStats", input_x, input_f, output, padding, padding2, stride, stream_handle, p, dst);
 }
 
 int CuDNN_DLGpuConv2d_Gradient_of_Filter(const DLArrayHandle input_x, const DLArrayHandle gradient_y,

@@ -26,6 +26,7 @@
 
 #include "common.h"
 #include "mfma_gemm.h"
+#include "reduce.h"
 #include "wino_gemm.h"
 
 namespace tsplit {
@@ -168,39 +169,71 @@ __device__ __forceinline__ void at_rows(const float m[6], float o[4]) {
   o[3] = d12 + 8.0f * d34 + m[5];
 }
 
-// one thread per (channel, tile): grid (ceil(tiles / 256), chans)
-__global__ __launch_bounds__(256) void wino_output_kernel(const float *__restrict__ M, float *__restrict__ y, WinoGeo g) {
+// one thread per (channel, tile): grid (ceil(tiles / 256), chans).  With STATS the block also leaves the
+// sum and the sum of squares of the outputs it stored (the values are at hand; the kernel is bound by
+// memory) at stats[(blockIdx.x * chans + channel) * 2]: partial sums for a BatchNorm that follows.
+template <bool STATS>
+__global__ __launch_bounds__(256) void wino_output_kernel(const float *__restrict__ M, float *__restrict__ y, WinoGeo g,
+                                                          float *__restrict__ stats) {
+  __shared__ float sm[8];
   const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t >= g.tiles) return;
   const int o = blockIdx.y;
-  const float *in = M + static_cast<int64_t>(o) * g.ld + t;
-  const int64_t plane_stride = static_cast<int64_t>(g.chans) * g.ld;
-  float tmp[6][4];   // tmp[q][.] = A^T applied down column q
+  float sum = 0.0f, sq = 0.0f;
+  if (t < g.tiles) {
+    const float *in = M + static_cast<int64_t>(o) * g.ld + t;
+    const int64_t plane_stride = static_cast<int64_t>(g.chans) * g.ld;
+    float tmp[6][4];   // tmp[q][.] = A^T applied down column q
 #pragma unroll
-  for (int q = 0; q < 6; ++q) {
-    float col[6];
+    for (int q = 0; q < 6; ++q) {
+      float col[6];
 #pragma unroll
-    for (int r = 0; r < 6; ++r) col[r] = in[(r * 6 + q) * plane_stride];
-    at_rows(col, tmp[q]);
+      for (int r = 0; r < 6; ++r) col[r] = in[(r * 6 + q) * plane_stride];
+      at_rows(col, tmp[q]);
+    }
+    const int per_img = g.th * g.tw;
+    const int n = t / per_img, rem = t - n * per_img;
+    const int ty = rem / g.tw, tx = rem - ty * g.tw;
+    float *plane = y + (static_cast<int64_t>(n) * g.chans + o) * g.H * g.W;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int h = 4 * ty + r;
+      if (h >= g.H) break;
+      const float row[6] = {tmp[0][r], tmp[1][r], tmp[2][r], tmp[3][r], tmp[4][r], tmp[5][r]};
+      float v[4];
+      at_rows(row, v);
+      float *dst = plane + static_cast<int64_t>(h) * g.W + 4 * tx;
+      if (g.quads) {
+        *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        if (STATS) {
+          sum += (v[0] + v[1]) + (v[2] + v[3]);
+          sq += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (4 * tx + q < g.W) {
+            dst[q] = v[q];
+            if (STATS) {
+              sum += v[q];
+              sq += v[q] * v[q];
+            }
+          }
+      }
+    }
   }
-  const int per_img = g.th * g.tw;
-  const int n = t / per_img, rem = t - n * per_img;
-  const int ty = rem / g.tw, tx = rem - ty * g.tw;
-  float *plane = y + (static_cast<int64_t>(n) * g.chans + o) * g.H * g.W;
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int h = 4 * ty + r;
-    if (h >= g.H) break;
-    const float row[6] = {tmp[0][r], tmp[1][r], tmp[2][r], tmp[3][r], tmp[4][r], tmp[5][r]};
-    float v[4];
-    at_rows(row, v);
-    float *dst = plane + static_cast<int64_t>(h) * g.W + 4 * tx;
-    if (g.quads) {
-      *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
-    } else {
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (4 * tx + q < g.W) dst[q] = v[q];
+  if (STATS) {
+    sum = wave_sum(sum);
+    sq = wave_sum(sq);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+      sm[wave] = sum;
+      sm[4 + wave] = sq;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float *dst = stats + (static_cast<int64_t>(blockIdx.x) * g.chans + o) * 2;
+      dst[0] = (sm[0] + sm[1]) + (sm[2] + sm[3]);
+      dst[1] = (sm[4] + sm[5]) + (sm[6] + sm[7]);
     }
   }
 }
@@ -372,10 +405,6 @@ inline int compute_units() {
   }();
   return n;
 }
-inline int gemm_blocks_per_cu() {
-  static const int n = blocks_per_cu(wg::wino_gemm_kernel);
-  return n;
-}
 
 // How the filter-gradient GEMMs of one run are cut: tile shape, depth per range, and (128 x 128 tiles) the
 // persistent grid.  Narrow layers (64 produced or gathered channels) take 64-wide tiles whose idle waves
@@ -470,8 +499,9 @@ inline int run_images(int imgs, int per_img, int chans_a, int chans_b) {
 
 // y[n][produced][H][W] = conv3x3(x[n][gathered][H][W], filter), stride 1, pad 1.  `rotated` selects
 // the data-gradient reading of the filter (stored [gathered][produced][3][3], rotated 180 degrees).
+// With a sink, every block of the output transform adds one partial (sum, sum of squares) per channel.
 int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int gathered, int produced, int H, int W,
-                      bool rotated, hipStream_t st) {
+                      bool rotated, hipStream_t st, StatsSink *sink) {
   const int th = (H + 3) / 4, tw = (W + 3) / 4;
   const int per_img = th * tw;
   const int run = run_images(imgs, per_img, gathered, produced);
@@ -497,10 +527,18 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
     {
       GemmTiming timed(st, 0, 2.0 * kXi * produced * static_cast<double>(gi.ld) * gathered);
       wg::launch(wg::Problem{U, V, M, produced, gathered, gi.ld, (produced + 127) / 128, (gi.ld + 127) / 128}, st,
-                 gemm_blocks_per_cu(), compute_units());
+                 compute_units());
     }
-    hipLaunchKernelGGL(wino_output_kernel, dim3((go.tiles + 255) / 256, produced), dim3(256), 0, st, M,
-                       y + static_cast<int64_t>(first) * produced * H * W, go);
+    const dim3 grid_out((go.tiles + 255) / 256, produced);
+    float *yr = y + static_cast<int64_t>(first) * produced * H * W;
+    if (sink) {
+      TS_REQUIRE(sink->used + static_cast<int>(grid_out.x) <= sink->capacity, "conv (Winograd): statistics buffer too small");
+      hipLaunchKernelGGL(wino_output_kernel<true>, grid_out, dim3(256), 0, st, M, yr, go,
+                         sink->part + static_cast<int64_t>(sink->used) * produced * 2);
+      sink->used += static_cast<int>(grid_out.x);
+    } else {
+      hipLaunchKernelGGL(wino_output_kernel<false>, grid_out, dim3(256), 0, st, M, yr, go, static_cast<float *>(nullptr));
+    }
   }
   return 0;
 }

@@ -26,7 +26,7 @@ __all__ = [
     "matrix_transpose", "batch_matrix_multiply", "one_hot", "where", "embedding_lookup",
     "embedding_lookup_gradient", "matrix_elementwise_divide", "matrix_elementwise_divide_const",
     "matrix_opposite", "matrix_sqrt", "matrix_rsqrt", "tanh", "sigmoid",
-    "batch_norm_relu", "batch_norm_relu_gradient",
+    "batch_norm_relu", "batch_norm_relu_gradient", "conv2d_batch_norm_stats", "batch_norm_from_stats",
     "CuDNN_Dropout", "CuDNN_Dropout_gradient", "CuSparse_Csrmv", "CuSparse_Csrmm",
 ]
 
@@ -435,6 +435,24 @@ def batch_norm_relu(in_arr, bn_scale_arr, bn_bias_arr, out_arr, save_mean, save_
                     profiler=None):
     check_call(_LIB.TSplit_BatchNormRelu(_h(in_arr), _h(bn_scale_arr), _h(bn_bias_arr), _h(out_arr),
                                          ctypes.c_float(eps), _h(save_mean), _h(save_var), _s(stream), _p(profiler)))
+
+
+def conv2d_batch_norm_stats(in_arr_x, in_arr_f, out_arr, stats, slot, padding=0, padding2=None, stride=1, stream=None,
+                            profiler=None):
+    """CuDNN_conv2d that also writes the per-channel (sum, sum of squares) of out_arr into row `slot` of
+    `stats` (float32 array of at least (slot + 1) * out_channels * 4 elements, read as doubles)."""
+    pad2 = padding if padding2 is None else padding2
+    check_call(_LIB.TSplit_Conv2dBatchNormStats(_h(in_arr_x), _h(in_arr_f), _h(out_arr), int(padding), int(pad2),
+                                                int(stride), _h(stats), int(slot), _s(stream), _p(profiler)))
+
+
+def batch_norm_from_stats(in_arr, stats, slots, bn_scale_arr, bn_bias_arr, out_arr, save_mean, save_var, eps=0.01,
+                          relu=False, stream=None, profiler=None):
+    """BatchNorm (+ Relu) forward with the batch statistics taken from rows 0 .. slots-1 of `stats`."""
+    check_call(_LIB.TSplit_BatchNormFromStats(_h(in_arr), _h(stats), int(slots), _h(bn_scale_arr), _h(bn_bias_arr),
+                                              _h(out_arr), ctypes.c_float(eps), _h(save_mean) if save_mean else None,
+                                              _h(save_var) if save_var else None, int(bool(relu)), _s(stream),
+                                              _p(profiler)))
 
 
 def batch_norm_relu_gradient(in_gradient_y, in_arr_x, in_bn_scale, in_bn_bias, out_gradient_x, out_gradient_bn_scale,

@@ -117,7 +117,7 @@ def _out_shape(layer, s):
 
 class Trainer(object):
     def __init__(self, spec, params, input_shape, num_classes, ctx=None, optimizer=("sgd", 0.1),
-                 split=None, bn_eps=0.01, timer=None, fuse_bn_relu=False):
+                 split=None, bn_eps=0.01, timer=None, fuse_bn_relu=False, conv_bn_stats=False):
         self.spec = list(spec)
         # with fuse_bn_relu a ("bn", ...) layer directly followed by ("relu",) runs as ONE fused call
         # in each direction (symbols outside the reference's ABI); the Relu layer's own arrays are
@@ -125,6 +125,13 @@ class Trainer(object):
         self.fused = set()
         if fuse_bn_relu:
             self.fused = {li for li, l in enumerate(self.spec[:-1]) if l[0] == "bn" and self.spec[li + 1][0] == "relu"}
+        # with conv_bn_stats a ("conv", ...) layer directly followed by ("bn", ...) hands the BatchNorm its
+        # batch statistics (one row of sums per micro-tensor; symbols outside the reference's ABI), so
+        # the BatchNorm reads the convolution's output once instead of twice
+        self.stats_of = {}
+        if conv_bn_stats:
+            self.stats_of = {li: None for li, l in enumerate(self.spec[:-1])
+                             if l[0] == "conv" and self.spec[li + 1][0] == "bn"}
         # optional per-call timing hook: timer.begin(stream) / timer.end(stream, tag, work, unit)
         self.timer = timer
         self.ctx = ctx if ctx is not None else ndarray.gpu(0)
@@ -158,6 +165,9 @@ class Trainer(object):
                 self.dacts[-1].split_tensor(self.split[li])
                 # per-piece filter gradient, summed into the layer's gradient
                 self.dw_piece[li] = ndarray.empty(param_shapes([layer])[layer[1] + "_weight"], self.ctx)
+            if li in self.stats_of:
+                # [pieces][Cout][2] doubles in float32 storage
+                self.stats_of[li] = ndarray.empty((self.split.get(li, 1) * layer[3] * 4,), self.ctx)
         assert self.shapes[-1] == (input_shape[0], num_classes), (self.shapes[-1], num_classes)
         self.loss = ndarray.empty((1,), self.ctx)
         self.ones = ndarray.empty((1,), self.ctx)
@@ -203,13 +213,23 @@ class Trainer(object):
                 xs = pairs[0][0].shape
                 wino = L.conv_takes_winograd(xs[0], cin, cout, xs[2], xs[3], k, pad, stride)
                 tag = "conv_fwd_thin" if thin else "conv_fwd_winograd" if wino else "conv_fwd_" + self._tile(cout)
-                for xa, ya in pairs:
-                    if thin:
-                        self._run(tag, 4.0 * (n(xa.shape) + n(w.shape) + n(ya.shape)), "byte", L.CuDNN_conv2d, xa, w, ya,
-                                  pad, pad, stride)
+                for i, (xa, ya) in enumerate(pairs):
+                    if li in self.stats_of:
+                        call, args = L.conv2d_batch_norm_stats, (xa, w, ya, self.stats_of[li], i, pad, pad, stride)
                     else:
-                        self._run(tag, 2.0 * n(ya.shape) * cin * k * k, "flop", L.CuDNN_conv2d, xa, w, ya, pad, pad,
-                                  stride)
+                        call, args = L.CuDNN_conv2d, (xa, w, ya, pad, pad, stride)
+                    if thin:
+                        self._run(tag, 4.0 * (n(xa.shape) + n(w.shape) + n(ya.shape)), "byte", call, *args)
+                    else:
+                        self._run(tag, 2.0 * n(ya.shape) * cin * k * k, "flop", call, *args)
+            elif kind == "bn" and li - 1 in self.stats_of:
+                name = layer[1]
+                sm, sv = self.saved[li]
+                fused = li in self.fused
+                self._run("bn_relu_fwd_from_stats" if fused else "bn_fwd_from_stats", 8.0 * n(a.shape), "byte",
+                          L.batch_norm_from_stats, a, self.stats_of[li - 1], self.split.get(li - 1, 1),
+                          self.params[name + "_scale"], self.params[name + "_bias"],
+                          self.acts[li + 2] if fused else out, sm, sv, self.eps, fused)
             elif kind == "bn" and li in self.fused:
                 name = layer[1]
                 sm, sv = self.saved[li]
