@@ -1,0 +1,130 @@
+"""The budgeted tape executor on the GPU: residual, multi-branch and attention graphs trained with
+part of their activations in pinned host memory.
+
+Bars: losses of the budgeted run equal those of the plain tape on the same library bit for bit (the same
+operators run on the same values; only where the values wait differs); against the numpy oracle the
+loss is within 1e-3 relative at every step (and the ResNet's weights after the steps within 2e-3 of their largest entry); the
+device pool's `used` figure stays within the replayed peak (plus the pool's rounding)."""
+import numpy as np
+import pytest
+
+from oracle_backend import OracleBackend
+from util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _onehot(rng, n, classes):
+    y = np.zeros((n, classes), np.float32)
+    y[np.arange(n), rng.randint(0, classes, n)] = 1
+    return y
+
+
+def _plain(build, inputs, seed, steps, lr, backend):
+    from tsplit_amd import graph, workloads
+    store = workloads.ParamStore(seed)
+    losses, binder, dev = [], None, None
+    for _ in range(steps):
+        t = graph.Tape(backend)
+        if binder is None:
+            binder = workloads.Binder(t, store)
+            dev = {k: binder.input(v) for k, v in inputs.items()}
+        else:
+            binder.t, binder._n = t, 0
+        loss, _ = build(t, binder, dev)
+        t.backward(loss)
+        losses.append(float(backend.to_numpy(loss.value).reshape(-1)[0]))
+        binder.sgd_step(lr)
+    binder.pull()
+    return losses, store.values
+
+
+def _cases(rng):
+    from tsplit_amd import workloads
+    cfg = workloads.TransformerConfig(batch=3, len1=10, len2=8, d_model=32, heads=4, d_ff=64, blocks=1, vocab=50,
+                                      mask_value=-1.0, embed_std=0.05, pos_amplitude=0.2)
+    xs = rng.randint(0, cfg.vocab, size=(cfg.batch, cfg.len1)).astype(np.float32)
+    ys_in = rng.randint(0, cfg.vocab, size=(cfg.batch, cfg.len2)).astype(np.float32)
+    ys_out = rng.randint(0, cfg.vocab, size=(cfg.batch, cfg.len2)).astype(np.float32)
+    xs[:, -2:] = 0
+    return {
+        "resnet": (lambda t, b, c: workloads.resnet(t, b, c["x"], c["y"], blocks=(2, 2), base=8, classes=10),
+                   {"x": rng.normal(size=(4, 3, 32, 32)).astype(np.float32), "y": _onehot(rng, 4, 10)}, 0.05),
+        "inception": (lambda t, b, c: workloads.inception_v4(t, b, c["x"], c["y"], n_a=1, n_b=1, n_c=1, div=8, classes=10),
+                      {"x": rng.normal(size=(3, 3, 107, 107)).astype(np.float32), "y": _onehot(rng, 3, 10)}, 0.01),
+        "transformer": (lambda t, b, c: workloads.transformer(t, b, cfg, c["xs"], c["yi"], c["yo"]),
+                        {"xs": xs, "yi": ys_in, "yo": ys_out}, 0.01),
+    }
+
+
+@pytest.mark.parametrize("net", ["resnet", "inception", "transformer"])
+def test_budgeted_graph_tracks_the_plain_tape_and_the_oracle(net, rng):
+    from tsplit_amd import graph, tape_budget as tb, workloads
+    build, inputs, lr = _cases(rng)[net]
+    steps = 3
+    ops, leaves = tb.record(build, {k: v.shape for k, v in inputs.items()})
+    free_peak = tb.replay(ops, leaves)[0]
+    # the tightest of these budgets the planner can meet (half of what the operators' values take, for
+    # the ResNet); these graphs are small, so values of any size may leave
+    plan = None
+    for frac in (0.5, 0.6, 0.7, 0.8, 0.9):
+        budget = leaves + int((free_peak - leaves) * frac)
+        try:
+            plan = tb.plan(ops, leaves, budget, min_bytes=0)
+            break
+        except ValueError:
+            continue
+    assert plan is not None and plan.away and plan.peak_bytes <= budget
+    assert net != "resnet" or frac == 0.5
+    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(5), budget, min_bytes=0)
+    assert run.plan.away == plan.away
+    got = []
+    for _ in range(steps):
+        loss = run.step(lr)
+        got.append(float(loss.value.asnumpy()[0]))
+    run.binder.pull()
+    plain_losses, plain_params = _plain(build, inputs, 5, steps, lr, graph.GpuBackend())
+    assert got == plain_losses or (net == "transformer" and np.allclose(got, plain_losses, rtol=1e-6)), (got, plain_losses)
+    for k, v in plain_params.items():
+        if net == "transformer":      # the embedding gradient adds with float atomics: sums differ in the last bits
+            np.testing.assert_allclose(run.store.values[k], v, rtol=1e-4, atol=1e-7)
+        else:
+            np.testing.assert_array_equal(run.store.values[k], v)
+    ref_losses, ref_params = _plain(build, inputs, 5, steps, lr, OracleBackend())
+    rel = max(abs(a - b) / abs(b) for a, b in zip(got, ref_losses))
+    assert rel <= 1e-3, (got, ref_losses)
+    for k, v in ref_params.items():
+        # (the BatchNorm scale and bias vectors move by sums that nearly cancel; three steps of a batch of
+        # four amplify their fp32 noise beyond any useful bar: they are held to the plain tape above, whose
+        # gradients tests/test_gpu_graphs.py holds to the oracle)
+        # (and the Inception graph at a batch of three drifts the same way in its weights: 6e-3 after three steps)
+        if net == "resnet" and k.endswith("weight"):
+            assert_close(run.store.values[k].reshape(v.shape), v, 2e-3, k)
+    assert run.state.host_waits > 0
+
+
+def test_pool_usage_stays_within_the_replayed_peak(rng):
+    """A ResNet of two stages at 96x96, batch 16 (activations of tens of MB): the pool's `used` figure,
+    read after every operator, against the planner's replay, unplanned and under half the budget."""
+    from tsplit_amd import tape_budget as tb, workloads
+    from tsplit_amd.gpu_memory_manager import pool_state
+
+    def build(t, b, c):
+        return workloads.resnet(t, b, c["x"], c["y"], blocks=(2, 2), base=32, classes=10)
+    inputs = {"x": rng.normal(size=(16, 3, 96, 96)).astype(np.float32), "y": _onehot(rng, 16, 10)}
+    ops, leaves = tb.record(build, {k: v.shape for k, v in inputs.items()})
+    free_peak = tb.replay(ops, leaves)[0]
+    peaks = {}
+    for tag, budget in (("free", None), ("half", leaves + (free_peak - leaves) // 2)):
+        base = pool_state().used
+        run = tb.BudgetedRun(build, inputs, workloads.ParamStore(3), budget, track_pool=True, min_bytes=0)
+        for _ in range(2):
+            run.step(0.01)
+        run.sync()
+        peaks[tag] = run.state.peak_used - base
+        # the pool rounds every block up and the executor's events, the loss seed and the library's
+        # bookkeeping are small allocations of their own: 3 % and 2 MiB of slack
+        assert peaks[tag] <= run.plan.peak_bytes * 1.03 + (2 << 20), (tag, peaks[tag], run.plan.peak_bytes)
+        assert peaks[tag] >= run.plan.peak_bytes * 0.9, (tag, peaks[tag], run.plan.peak_bytes)
+        del run
+    assert peaks["half"] < 0.65 * peaks["free"]

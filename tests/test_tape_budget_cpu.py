@@ -1,0 +1,77 @@
+"""Planner of the budgeted tape executor on recorded graphs (no GPU): the replay of the executor's
+schedule and the greedy choice of what leaves the device."""
+import numpy as np
+import pytest
+
+from tsplit_amd import tape_budget as tb, workloads
+
+
+def _resnet(t, b, c):
+    return workloads.resnet(t, b, c["x"], c["y"], blocks=(2, 2), base=8, classes=10)
+
+
+def _inception(t, b, c):
+    return workloads.inception_v4(t, b, c["x"], c["y"], n_a=1, n_b=1, n_c=1, div=8, classes=10)
+
+
+SHAPES = {"resnet": (_resnet, {"x": (4, 3, 32, 32), "y": (4, 10)}),
+          "inception": (_inception, {"x": (3, 3, 107, 107), "y": (3, 10)})}
+
+
+@pytest.mark.parametrize("net", sorted(SHAPES))
+def test_record_lists_every_operator_with_its_readers(net):
+    build, shapes = SHAPES[net]
+    ops, leaves = tb.record(build, shapes)
+    assert leaves > sum(4 * int(np.prod(s)) for s in shapes.values())      # parameters are leaves too
+    assert ops[-1].bytes == 4 and ops[-1].has_backward                      # the loss
+    for t, op in enumerate(ops):
+        assert all(i < t for i in op.inputs) and all(i <= t for i in op.saved)
+        assert set(op.grad_inputs) <= set(op.inputs)
+    # a convolution's backward reads its input, an addition's reads nothing
+    last_fwd, bwd = tb._uses(ops)
+    assert any(bwd[i] for i in range(len(ops))) and any(not bwd[i] for i in range(len(ops)))
+
+
+@pytest.mark.parametrize("net", sorted(SHAPES))
+def test_plan_meets_the_budget_by_sending_idle_values_away(net):
+    build, shapes = SHAPES[net]
+    ops, leaves = tb.record(build, shapes)
+    free_peak, at, idle = tb.replay(ops, leaves)
+    assert free_peak > leaves and 0 <= at < 2 * len(ops)
+    last_fwd, bwd = tb._uses(ops)
+    previous = free_peak
+    for frac in (0.9, 0.7, 0.55):
+        budget = leaves + int((free_peak - leaves) * frac)
+        p = tb.plan(ops, leaves, budget, min_bytes=0)
+        assert p.peak_bytes <= budget and p.free_peak_bytes == free_peak
+        assert p.peak_bytes == tb.replay(ops, leaves, p.away, p.lead)[0]
+        assert all(bwd[i] for i in p.away)            # only values the backward sweep reads again are worth moving
+        assert p.peak_bytes <= previous
+        previous = p.peak_bytes
+    assert tb.plan(ops, leaves, None).away == frozenset()
+    with pytest.raises(ValueError):
+        tb.plan(ops, leaves, leaves + 1, min_bytes=0)
+
+
+def test_sending_a_value_away_frees_it_between_its_uses():
+    build, shapes = SHAPES["resnet"]
+    ops, leaves = tb.record(build, shapes)
+    last_fwd, bwd = tb._uses(ops)
+    # the largest value that the backward sweep reads again
+    i = max((op.bytes, k) for k, op in enumerate(ops) if bwd[k])[1]
+    base = tb.replay(ops, leaves)[0]
+    assert tb.replay(ops, leaves, {i})[0] <= base
+
+
+def test_max_batch_grows_with_the_budget_and_with_planning():
+    def build_for(batch):
+        return _resnet
+
+    def shapes_for(batch):
+        return {"x": (batch, 3, 32, 32), "y": (batch, 10)}
+    budget = 8 << 20
+    plain, _ = tb.max_batch(build_for, shapes_for, budget, planned=False, limit=512)
+    planned, p = tb.max_batch(build_for, shapes_for, budget, planned=True, limit=512, min_bytes=0)
+    assert 0 < plain < planned and p.peak_bytes <= budget
+    more, _ = tb.max_batch(build_for, shapes_for, 2 * budget, planned=False, limit=512)
+    assert more > plain

@@ -18,11 +18,25 @@ from . import ndarray
 
 
 class Var(object):
-    """A value on the tape: backend array, shape, accumulated gradient."""
-    __slots__ = ["value", "shape", "grad", "needs_grad", "name"]
+    """A value on the tape: backend array, shape, accumulated gradient; `node` is the index of the
+    operator call that produced it on its tape (-1 for parameters, inputs and constants)."""
+    __slots__ = ["value", "shape", "grad", "needs_grad", "name", "node"]
 
     def __init__(self, value, shape, needs_grad, name=None):
         self.value, self.shape, self.grad, self.needs_grad, self.name = value, tuple(shape), None, needs_grad, name
+        self.node = -1
+
+
+class Node(object):
+    """One operator call: its output, the closure of its backward operators (None when no input
+    needs a gradient), the Vars it read and the Vars its backward closure reads again."""
+    __slots__ = ["out", "back", "inputs", "saved", "index"]
+
+    def __init__(self, out, back, inputs, saved, index):
+        self.out, self.back, self.inputs, self.saved, self.index = out, back, tuple(inputs), tuple(saved), index
+
+
+SELF = object()      # in a `saved` list: the operator's own output
 
 
 def _prod(shape):
@@ -252,7 +266,7 @@ class GpuBackend(object):
 class Tape(object):
     def __init__(self, backend):
         self.b = backend
-        self._nodes = []     # (output Var, backward closure)
+        self._nodes = []     # every operator call, in order (Node)
 
     # ---- leaves
     def param(self, value, shape, name=None):
@@ -261,11 +275,27 @@ class Tape(object):
     def const(self, value, shape, name=None):
         return Var(value, shape, False, name)
 
-    def _out(self, value, shape, inputs, backward):
+    def _out(self, value, shape, inputs, backward, saved=None):
+        """Registers an operator call.  `saved`: the Vars the backward closure reads (SELF for the
+        output itself); by default the inputs.  A closure must read them as `var.value` when it
+        runs, so that an executor may move a value off the device in between."""
         v = Var(value, shape, any(i.needs_grad for i in inputs))
-        if v.needs_grad:
-            self._nodes.append((v, backward))
+        saved = inputs if saved is None else [v if s is SELF else s for s in saved]
+        node = Node(v, backward if v.needs_grad else None, inputs, saved if v.needs_grad else (), len(self._nodes))
+        v.node = node.index
+        self._nodes.append(node)
+        self._after_forward(node)
         return v
+
+    # hooks of executors that manage memory (tsplit_amd.tape_budget)
+    def _after_forward(self, node):
+        pass
+
+    def _before_backward(self, node):
+        pass
+
+    def _after_backward(self, node):
+        pass
 
     def _acc(self, var, g):
         if not var.needs_grad:
@@ -283,7 +313,7 @@ class Tape(object):
                 self._acc(w, self.b.conv2d_grad_filter(x.value, g, w.shape, ph, pw, stride))
             if x.needs_grad:
                 self._acc(x, self.b.conv2d_grad_data(w.value, g, x.shape, ph, pw, stride))
-        return self._out(y, ys, [x, w], back)
+        return self._out(y, ys, [x, w], back, saved=[x, w])
 
     def batch_norm(self, x, gamma, beta, eps=0.01):
         """gpu_ops/BatchNorm.py:54-83 (compute), :166-227 (gradient node; statistics recomputed, no
@@ -295,7 +325,7 @@ class Tape(object):
             self._acc(x, dx)
             self._acc(gamma, dg)
             self._acc(beta, db)
-        return self._out(y, x.shape, [x, gamma, beta], back)
+        return self._out(y, x.shape, [x, gamma, beta], back, saved=[x, gamma])
 
     def relu(self, x):
         """gpu_ops/Relu.py:51,117."""
@@ -306,13 +336,19 @@ class Tape(object):
         """gpu_ops/MaxPool.py:119 (compute), :146 (gradient)."""
         y = self.b.max_pool(x.value, x.shape, k, pad, stride)
         ys = (x.shape[0], x.shape[1], conv_out(x.shape[2], k, pad, stride), conv_out(x.shape[3], k, pad, stride))
-        return self._out(y, ys, [x], lambda g: self._acc(x, self.b.max_pool_grad(x.value, y, g, x.shape, k, pad, stride)))
+        out = None
+        out = self._out(y, ys, [x], lambda g: self._acc(x, self.b.max_pool_grad(x.value, out.value, g, x.shape, k, pad, stride)),
+                        saved=[x, SELF])
+        return out
 
     def avg_pool(self, x, k, pad, stride):
         """gpu_ops/AvgPool.py:78 (compute), :103-104 (gradient)."""
         y = self.b.avg_pool(x.value, x.shape, k, pad, stride)
         ys = (x.shape[0], x.shape[1], conv_out(x.shape[2], k, pad, stride), conv_out(x.shape[3], k, pad, stride))
-        return self._out(y, ys, [x], lambda g: self._acc(x, self.b.avg_pool_grad(x.value, y, g, x.shape, k, pad, stride)))
+        out = None
+        out = self._out(y, ys, [x], lambda g: self._acc(x, self.b.avg_pool_grad(x.value, out.value, g, x.shape, k, pad, stride)),
+                        saved=[x, SELF])
+        return out
 
     def add(self, a, b):
         """gpu_ops/AddElewise.py:54 (compute), :95 (gradient: both inputs receive the output gradient)."""
@@ -322,16 +358,16 @@ class Tape(object):
         def back(g):
             self._acc(a, g)
             self._acc(b, g)
-        return self._out(y, a.shape, [a, b], back)
+        return self._out(y, a.shape, [a, b], back, saved=[])
 
     def scale(self, a, c):
         """gpu_ops/MultiplyConst.py:45 (compute), :63 (gradient: the output gradient times the constant)."""
         y = self.b.mul_const(a.value, c, a.shape)
-        return self._out(y, a.shape, [a], lambda g: self._acc(a, self.b.mul_const(g, c, a.shape)))
+        return self._out(y, a.shape, [a], lambda g: self._acc(a, self.b.mul_const(g, c, a.shape)), saved=[])
 
     def shift(self, a, c):
         y = self.b.add_const(a.value, c, a.shape)
-        return self._out(y, a.shape, [a], lambda g: self._acc(a, g))
+        return self._out(y, a.shape, [a], lambda g: self._acc(a, g), saved=[])
 
     def mul(self, a, b):
         """gpu_ops/MultiplyElewise.py (compute; gradient: each input receives the other times the
@@ -348,20 +384,24 @@ class Tape(object):
         """gpu_ops/Sigmoid.py:58-61: gradient s * (1 + -1 * s) * g, built from the same elementwise
         operators the reference's gradient graph uses."""
         y = self.b.sigmoid(x.value, x.shape)
+        out = None
 
         def back(g):
-            one_minus = self.b.add_const(self.b.mul_const(y, -1.0, x.shape), 1.0, x.shape)
-            self._acc(x, self.b.mul(self.b.mul(y, one_minus, x.shape), g, x.shape))
-        return self._out(y, x.shape, [x], back)
+            one_minus = self.b.add_const(self.b.mul_const(out.value, -1.0, x.shape), 1.0, x.shape)
+            self._acc(x, self.b.mul(self.b.mul(out.value, one_minus, x.shape), g, x.shape))
+        out = self._out(y, x.shape, [x], back, saved=[SELF])
+        return out
 
     def tanh(self, x):
         """gpu_ops/Tanh.py:59-61: gradient (1 + (-1 * t) * t) * g."""
         y = self.b.tanh(x.value, x.shape)
+        out = None
 
         def back(g):
-            d = self.b.add_const(self.b.mul(self.b.mul_const(y, -1.0, x.shape), y, x.shape), 1.0, x.shape)
+            d = self.b.add_const(self.b.mul(self.b.mul_const(out.value, -1.0, x.shape), out.value, x.shape), 1.0, x.shape)
             self._acc(x, self.b.mul(d, g, x.shape))
-        return self._out(y, x.shape, [x], back)
+        out = self._out(y, x.shape, [x], back, saved=[SELF])
+        return out
 
     def slice(self, x, begin, size):
         """gpu_ops/Slice.py:47-81: tf.slice semantics, a size of -1 runs to the end; the gradient
@@ -369,7 +409,7 @@ class Tape(object):
         begin = tuple(int(v) for v in begin)
         shape = tuple(int(x.shape[d] - begin[d] if n == -1 else n) for d, n in enumerate(size))
         y = self.b.slice(x.value, begin, shape)
-        return self._out(y, shape, [x], lambda g: self._acc(x, self.b.slice_grad(g, begin, x.shape)))
+        return self._out(y, shape, [x], lambda g: self._acc(x, self.b.slice_grad(g, begin, x.shape)), saved=[])
 
     def reshape(self, a, shape):
         """gpu_ops/Reshape.py:42 (compute: a copy), :61 (gradient: reshaped back)."""
@@ -379,7 +419,7 @@ class Tape(object):
             shape[shape.index(-1)] = _prod(a.shape) // known
         shape = tuple(shape)
         y = self.b.reshape(a.value, shape)
-        return self._out(y, shape, [a], lambda g: self._acc(a, self.b.reshape(g, a.shape)))
+        return self._out(y, shape, [a], lambda g: self._acc(a, self.b.reshape(g, a.shape)), saved=[])
 
     def concat(self, a, b, axis):
         """gpu_ops/Concat.py:47-60 (compute), :65 (gradient: two concat_gradient nodes, idx 0 and 1)."""
@@ -393,7 +433,7 @@ class Tape(object):
                 self._acc(a, self.b.concat_grad(g, a.shape, axis, 0))
             if b.needs_grad:
                 self._acc(b, self.b.concat_grad(g, b.shape, axis, 1))
-        return self._out(y, shape, [a, b], back)
+        return self._out(y, shape, [a, b], back, saved=[])
 
     def matmul(self, a, b, trans_a=False, trans_b=False):
         """gpu_ops/MatrixMult.py:57-86 (compute), :95-124 (gradient)."""
@@ -449,7 +489,7 @@ class Tape(object):
             self._acc(x, g)
             if bias.needs_grad:
                 self._acc(bias, self.b.reduce_sum_axis_zero(g, bias.shape))
-        return self._out(y, x.shape, [x, bias], back)
+        return self._out(y, x.shape, [x, bias], back, saved=[])
 
     def broadcast_like(self, x, shape):
         """gpu_ops/BroadcastTF.py:46-58 (numpy alignment from the right); gradient = reduce_sum
@@ -464,7 +504,7 @@ class Tape(object):
                 self._acc(x, self.b.reduce_sum(g, axes, x.shape))
             else:
                 self._acc(x, g)
-        return self._out(y, shape, [x], back)
+        return self._out(y, shape, [x], back, saved=[])
 
     def transpose(self, x, perm):
         """gpu_ops/Transpose.py:44-58 (compute), :60 (gradient: the inverse permutation)."""
@@ -474,7 +514,7 @@ class Tape(object):
         inv = [0] * len(perm)
         for i, p in enumerate(perm):
             inv[p] = i
-        return self._out(y, ys, [x], lambda g: self._acc(x, self.b.transpose(g, inv, x.shape)))
+        return self._out(y, ys, [x], lambda g: self._acc(x, self.b.transpose(g, inv, x.shape)), saved=[])
 
     def where(self, cond, a, b):
         """gpu_ops/Where.py:41-48 (compute), :50-55 (gradient: where(cond, g, 0) and where(cond, 0, g))."""
@@ -486,35 +526,39 @@ class Tape(object):
                 self._acc(a, self.b.where(cond.value, g, z, a.shape))
             if b.needs_grad:
                 self._acc(b, self.b.where(cond.value, z, g, a.shape))
-        return self._out(y, a.shape, [a, b], back)
+        return self._out(y, a.shape, [cond, a, b], back, saved=[cond])
 
     def one_hot(self, ids, classes):
         """gpu_ops/OneHot.py:44-46; no gradient."""
         ys = tuple(ids.shape) + (classes,)
-        return Var(self.b.one_hot(ids.value, ys), ys, False)
+        return self._out(self.b.one_hot(ids.value, ys), ys, [ids], None, saved=[])
 
     def embedding(self, table, ids):
         """gpu_ops/EmbeddingLookUp.py:41-42, gradient :48-49."""
         ys = tuple(ids.shape) + (table.shape[1],)
         y = self.b.embedding(table.value, ids.value, ys)
-        return self._out(y, ys, [table], lambda g: self._acc(table, self.b.embedding_grad(g, ids.value, table.shape)))
+        return self._out(y, ys, [table, ids], lambda g: self._acc(table, self.b.embedding_grad(g, ids.value, table.shape)),
+                         saved=[ids])
 
     def softmax_ce(self, logits, labels):
         """gpu_ops/SoftmaxCrossEntropy.py:46-67 (compute), :73 and :134-135 (gradient) with an adjoint of one."""
         assert len(logits.shape) == 2
         loss = self.b.softmax_ce(logits.value, labels.value)
-        return self._out(loss, (1,), [logits],
-                         lambda g: self._acc(logits, self.b.softmax_ce_grad(logits.value, labels.value, logits.shape)))
+        return self._out(loss, (1,), [logits, labels],
+                         lambda g: self._acc(logits, self.b.softmax_ce_grad(logits.value, labels.value, logits.shape)),
+                         saved=[logits, labels])
 
     # ---- reverse sweep
     def backward(self, loss):
         """Runs the recorded backward operators in reverse order; the loss adjoint is one
         (gpu_ops/executor.py:175), folded into softmax_ce's gradient."""
         loss.grad = True
-        for v, back in reversed(self._nodes):
-            if v.grad is None:
-                continue
-            back(v.grad)
-            if v is not loss:
-                v.grad = None      # interior gradients are dropped as soon as they are consumed
+        for node in reversed(self._nodes):
+            v = node.out
+            if node.back is not None and v.grad is not None:
+                self._before_backward(node)
+                node.back(v.grad)
+                if v is not loss:
+                    v.grad = None      # interior gradients are dropped as soon as they are consumed
+            self._after_backward(node)
         self._nodes = []

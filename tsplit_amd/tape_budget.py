@@ -1,0 +1,455 @@
+"""Training a branched graph (graph.Tape) under a device-memory budget.
+
+The reference's swapping executors decide per tensor of the dataflow graph what leaves the device
+after its forward use and comes back before its backward use (python/athena/gpu_ops/
+vdnnExecutor.py:202-330: offload on one copy stream, prefetch on another, DLEventRecord /
+DLEventSync around every move; the policy switch of examples/imagenet_resnet.py:139-154).  This
+module does that for the tape of graph.py, which runs the residual, multi-branch and attention
+graphs of the reference's examples:
+
+  record(build)       runs the graph builder without arithmetic and returns, per operator call, the
+                      size of its output, what it read, and what its backward operators read again;
+  plan(record, ...)   replays the executor's schedule on those sizes and, while the replayed peak
+                      exceeds the budget, sends away the largest value that sits idle at the moment
+                      of the peak (greedy, as planner.py does for layer lists);
+  BudgetedTape        a Tape that follows the plan: values without a later reader are dropped as the
+                      forward sweep passes their last use, planned values go to pinned host memory
+                      behind it and are fetched `lead` operators ahead of the backward sweep, and
+                      every value is dropped after the last backward operator that reads it.
+
+Schedule (replayed byte for byte by `replay`, measured against the pool by the tests):
+  forward  of operator t : its output is allocated; then every value whose last reader in the forward
+                           sweep was t and which no backward operator reads is released; a planned
+                           value whose last forward reader was t starts leaving, and is released
+                           after operator t + 1 has been issued (the host waits for the copy then);
+  backward of operator j : the planned values first read by operators j - lead .. j (in the order of
+                           the sweep) that are still away are allocated and start coming back; the
+                           host waits for those operator j reads; j's backward operators allocate
+                           the gradients of its inputs; then j's output gradient and every value
+                           whose last backward reader was j are released.
+Ordering between the streams goes through the host (DLEventSync), as in the reference: before a
+value leaves, the host waits for the operator that last read it; before memory for a returning value
+is taken from the pool, the host waits for the compute stream, so that no kernel still in flight
+reads memory the pool hands out again.
+
+The budget covers what the tape allocates: operator outputs, gradients, parameters and their
+gradients, inputs and constants.  The operator library's own scratch is outside it.
+"""
+import collections
+
+import numpy as np
+
+from . import graph
+from . import ndarray
+from .stream import create_event_handle, create_stream_handle
+
+
+def _bytes(shape):
+    n = 4
+    for s in shape:
+        n *= int(s)
+    return n
+
+
+class OpRecord(object):
+    """One operator call of a recorded graph.  Indices refer to operator calls (-1: a leaf)."""
+    __slots__ = ["bytes", "inputs", "saved", "has_backward", "grad_inputs", "leaf_grad_bytes"]
+
+    def __init__(self, nbytes, inputs, saved, has_backward, grad_inputs, leaf_grad_bytes):
+        self.bytes = nbytes                # of the output
+        self.inputs = inputs               # producers of the values the forward operator reads
+        self.saved = saved                 # producers of the values the backward operators read
+        self.has_backward = has_backward
+        self.grad_inputs = grad_inputs     # producers of the inputs that receive a gradient (operator outputs only)
+        self.leaf_grad_bytes = leaf_grad_bytes   # bytes of parameter gradients this operator's backward creates
+
+
+class _ShapeOnly(object):
+    """Backend that computes nothing: every primitive returns None."""
+
+    def __getattr__(self, name):
+        return lambda *a, **k: None
+
+
+class _Zeros(object):
+    trainable = {}
+
+    def get(self, name, shape, init, trainable=True):
+        return np.broadcast_to(np.float32(0), tuple(int(s) for s in shape))
+
+
+def record(build, inputs):
+    """Runs `build(tape, binder, cache)` (as graphbench.py's builders: cache maps input names to Vars)
+    on shapes only.  inputs: name -> shape.  -> (list of OpRecord, bytes of the leaves: inputs,
+    parameters, constants)."""
+    from .workloads import Binder
+    t = graph.Tape(_ShapeOnly())
+    b = Binder(t, _Zeros())
+    cache = {k: t.const(None, shape) for k, shape in inputs.items()}
+    loss, _ = build(t, b, cache)
+    ops = []
+    seen_param_grads = set()
+    for node in t._nodes:
+        leaf_grad = 0
+        for v in node.inputs:
+            if v.node < 0 and v.needs_grad and node.back is not None and id(v) not in seen_param_grads:
+                seen_param_grads.add(id(v))
+                leaf_grad += _bytes(v.shape)
+        ops.append(OpRecord(_bytes(node.out.shape), [v.node for v in node.inputs], [v.node for v in node.saved],
+                            node.back is not None,
+                            [v.node for v in node.inputs if v.node >= 0 and v.needs_grad] if node.back is not None else [],
+                            leaf_grad))
+    leaves = sum(_bytes(s) for s in inputs.values()) + sum(_bytes(v.shape) for v in b.vars.values())
+    leaves += sum(_bytes(shape) for _, shape in b._consts.values())
+    assert loss.node == len(ops) - 1
+    return ops, leaves
+
+
+class TapePlan(object):
+    def __init__(self, away, lead, peak_bytes, free_peak_bytes, budget_bytes, leaves_bytes):
+        self.away = frozenset(away)          # operator calls whose output leaves the device between the sweeps
+        self.lead = lead
+        self.peak_bytes = peak_bytes
+        self.free_peak_bytes = free_peak_bytes     # replayed peak with nothing sent away
+        self.budget_bytes = budget_bytes
+        self.leaves_bytes = leaves_bytes
+
+    def describe(self):
+        gib = float(1 << 30)
+        return {"away": len(self.away), "lead": self.lead, "peak_GiB": self.peak_bytes / gib,
+                "unplanned_peak_GiB": self.free_peak_bytes / gib,
+                "budget_GiB": None if self.budget_bytes is None else self.budget_bytes / gib}
+
+
+def _uses(ops):
+    """last forward reader and the backward readers of every operator's output"""
+    n = len(ops)
+    last_fwd = list(range(n))                 # at least its own producer
+    bwd = [[] for _ in range(n)]
+    for t, op in enumerate(ops):
+        for i in op.inputs:
+            if i >= 0:
+                last_fwd[i] = max(last_fwd[i], t)
+        if op.has_backward:
+            for i in op.saved:
+                if i >= 0:
+                    bwd[i].append(t)
+    return last_fwd, bwd
+
+
+def replay(ops, leaves_bytes, away=(), lead=3):
+    """Peak of the executor's schedule with `away` sent to the host.  -> (peak bytes, moment of the
+    peak, values resident and idle at that moment: list of (bytes, operator)).  A moment is an
+    operator index for the forward sweep and 2n - 1 - j for the backward of operator j."""
+    n = len(ops)
+    away = set(away)
+    last_fwd, bwd = _uses(ops)
+    first_bwd = [max(r) if r else -1 for r in bwd]       # the backward sweep descends: read first by the largest index
+    last_bwd = [min(r) if r else -1 for r in bwd]
+    live = leaves_bytes
+    resident = {}                                       # operator -> bytes of its value on the device
+    peak, peak_at, peak_set = live, -1, []
+    busy = set()
+
+    def note(moment):
+        nonlocal peak, peak_at, peak_set
+        if live > peak:
+            peak, peak_at = live, moment
+            peak_set = [(b, i) for i, b in resident.items() if i not in busy]
+
+    by_last_fwd = collections.defaultdict(list)
+    for i in range(n):
+        by_last_fwd[last_fwd[i]].append(i)
+    leaving = []                                        # values released after the next operator
+    # ---- forward
+    for t, op in enumerate(ops):
+        live += op.bytes
+        resident[t] = op.bytes
+        busy = set(i for i in op.inputs if i >= 0) | {t}
+        note(t)
+        for i in leaving:
+            live -= resident.pop(i)
+        leaving = []
+        for i in by_last_fwd[t]:
+            if not bwd[i]:
+                if i != n - 1:                          # the loss stays for the caller
+                    live -= resident.pop(i)
+            elif i in away:
+                leaving.append(i)
+    for i in leaving:
+        live -= resident.pop(i)
+    # ---- backward
+    grads = {}                                          # operator -> bytes of the gradient of its output
+    fetch_at = collections.defaultdict(list)
+    for i in away:
+        if bwd[i]:
+            fetch_at[min(n - 1, first_bwd[i] + lead)].append(i)
+    by_last_bwd = collections.defaultdict(list)
+    for i in range(n):
+        if bwd[i]:
+            by_last_bwd[last_bwd[i]].append(i)
+    param_grads = 0
+    for j in range(n - 1, -1, -1):
+        op = ops[j]
+        moment = 2 * n - 1 - j
+        for i in sorted(fetch_at[j], key=lambda i: -first_bwd[i]):
+            if i not in resident:
+                live += ops[i].bytes
+                resident[i] = ops[i].bytes
+        busy = set(i for i in op.saved if i >= 0)
+        note(moment)
+        if op.has_backward and (j == n - 1 or j in grads):
+            # every input that takes a gradient gets a new array; adding to an earlier one holds the
+            # sum and both terms for a moment
+            for i in op.grad_inputs:
+                extra = ops[i].bytes
+                live += extra
+                if i in grads:
+                    live += extra
+                    note(moment)
+                    live -= 2 * extra
+                else:
+                    grads[i] = extra
+                note(moment)
+            live += op.leaf_grad_bytes
+            param_grads += op.leaf_grad_bytes
+            note(moment)
+        if j in grads:
+            live -= grads.pop(j)
+        for i in by_last_bwd[j]:
+            if i in resident:
+                live -= resident.pop(i)
+    return peak, peak_at, peak_set
+
+
+def plan(ops, leaves_bytes, budget_bytes, lead=3, min_bytes=1 << 20):
+    """-> TapePlan.  Raises ValueError when the budget cannot be met by sending values away (a single
+    operator's operands, results and gradients do not fit)."""
+    free_peak, _, _ = replay(ops, leaves_bytes, (), lead)
+    away = set()
+    n = len(ops)
+    last_fwd, bwd = _uses(ops)
+    if budget_bytes is not None:
+        while True:
+            peak, at, idle = replay(ops, leaves_bytes, away, lead)
+            if peak <= budget_bytes:
+                break
+            # values that could be away at that moment: read again only in the backward sweep, after a gap
+            cands = []
+            for b, i in idle:
+                if i in away or not bwd[i] or b < min_bytes:
+                    continue
+                gone_from = last_fwd[i] + 2
+                back_at = 2 * n - 1 - min(n - 1, max(bwd[i]) + lead)
+                if gone_from <= at < back_at:
+                    cands.append((b, i))
+            if not cands:
+                raise ValueError("a step does not fit %.2f GiB: %.2f GiB are needed at once with everything "
+                                 "idle sent away" % (budget_bytes / float(1 << 30), peak / float(1 << 30)))
+            away.add(max(cands)[1])
+    peak, _, _ = replay(ops, leaves_bytes, away, lead)
+    return TapePlan(away, lead, peak, free_peak, budget_bytes, leaves_bytes)
+
+
+class BudgetedTape(graph.Tape):
+    """A Tape that executes `plan` (see the module description).  One instance per step; the streams
+    and the pinned host buffers live in `state`, shared by the steps (BudgetedTape.make_state)."""
+
+    class State(object):
+        def __init__(self, ctx):
+            self.ctx = ctx
+            self.host_ctx = ndarray.cpu(0)
+            self.out_stream = create_stream_handle(ctx)
+            self.in_stream = create_stream_handle(ctx)
+            self.host = {}           # operator -> pinned host array (kept across steps)
+            self.peak_used = 0       # largest `used` figure of the device pool seen after an operator
+            self.host_waits = 0
+
+    @staticmethod
+    def make_state(ctx):
+        return BudgetedTape.State(ctx)
+
+    def __init__(self, backend, tape_plan, ops, state, track_pool=False):
+        graph.Tape.__init__(self, backend)
+        self.plan, self.ops, self.state = tape_plan, ops, state
+        self.track_pool = track_pool
+        n = len(ops)
+        self.last_fwd, self.bwd = _uses(ops)
+        self.first_bwd = [max(r) if r else -1 for r in self.bwd]
+        self.last_bwd = [min(r) if r else -1 for r in self.bwd]
+        self.by_last_fwd = collections.defaultdict(list)
+        for i in range(n):
+            self.by_last_fwd[self.last_fwd[i]].append(i)
+        self.by_last_bwd = collections.defaultdict(list)
+        for i in range(n):
+            if self.bwd[i]:
+                self.by_last_bwd[self.last_bwd[i]].append(i)
+        self.fetch_at = collections.defaultdict(list)
+        for i in tape_plan.away:
+            if self.bwd[i]:
+                self.fetch_at[min(n - 1, self.first_bwd[i] + tape_plan.lead)].append(i)
+        self.leaving = []            # (operator, device array, copy-done event), released after the next operator
+        self.arriving = {}           # operator -> copy-done event
+        self.gone = set()
+
+    # ---- helpers
+    def _compute_stream(self):
+        return self.b.stream
+
+    def _host_wait_for_compute(self):
+        ev = create_event_handle(self.state.ctx)
+        ev.record(self._compute_stream())
+        ev.sync()
+        self.state.host_waits += 1
+
+    def _note_pool(self):
+        if self.track_pool:
+            from .gpu_memory_manager import pool_state
+            self.state.peak_used = max(self.state.peak_used, pool_state().used)
+
+    def _var(self, i):
+        return self._nodes[i].out
+
+    def _release_leaving(self):
+        for i, arr, ev in self.leaving:
+            ev.sync()                # the copy has left the device
+            self.state.host_waits += 1
+            del arr
+        self.leaving = []
+
+    # ---- hooks
+    def _after_forward(self, node):
+        t = node.index
+        assert t < len(self.ops) and _bytes(node.out.shape) == self.ops[t].bytes, "the graph differs from the recorded one"
+        self._note_pool()
+        self._release_leaving()
+        n = len(self.ops)
+        for i in self.by_last_fwd[t]:
+            v = self._var(i)
+            if not self.bwd[i]:
+                if i != n - 1:
+                    v.value = None
+            elif i in self.plan.away:
+                # the operator that read it last has been issued: wait for it, then copy out
+                self._host_wait_for_compute()
+                host = self.state.host.get(i)
+                if host is None or host.shape != v.shape:
+                    host = self.state.host[i] = ndarray.empty(v.shape, self.state.host_ctx)
+                v.value.copyto(host, self.state.out_stream)
+                ev = create_event_handle(self.state.ctx)
+                ev.record(self.state.out_stream)
+                self.leaving.append((i, v.value, ev))
+                v.value = None
+                self.gone.add(i)
+
+    def _fetch(self, i):
+        v = self._var(i)
+        self._host_wait_for_compute()          # nothing in flight reads memory the pool may hand out now
+        arr = ndarray.empty(v.shape, self.state.ctx)
+        self.state.host[i].copyto(arr, self.state.in_stream)
+        ev = create_event_handle(self.state.ctx)
+        ev.record(self.state.in_stream)
+        v.value = arr
+        self.arriving[i] = ev
+        self.gone.discard(i)
+
+    def _before_backward(self, node):
+        for i in (s.node for s in node.saved):
+            if i >= 0 and i in self.gone:      # (a value the plan fetches later than its reader needs it)
+                self._fetch(i)
+            ev = self.arriving.pop(i, None) if i >= 0 else None
+            if ev is not None:
+                ev.sync()
+                self.state.host_waits += 1
+
+    def backward(self, loss):
+        self._release_leaving()
+        n = len(self.ops)
+        assert len(self._nodes) == n, "the graph differs from the recorded one"
+        for i in sorted(self.fetch_at[n - 1], key=lambda i: -self.first_bwd[i]):     # planned for the first operator
+            if i in self.gone:
+                self._fetch(i)
+        graph.Tape.backward(self, loss)
+
+    def _after_backward(self, node):
+        # the sweep reaches operator j - 1 next: issue what the plan fetches there before its operators
+        j = node.index
+        self._note_pool()
+        for i in self.by_last_bwd[j]:
+            self._var(i).value = None
+        if j > 0:
+            for i in sorted(self.fetch_at[j - 1], key=lambda i: -self.first_bwd[i]):
+                if i in self.gone:
+                    self._fetch(i)
+
+
+class BudgetedRun(object):
+    """Trains a graph step after step under a plan: `build(tape, binder, cache)` as for record();
+    parameters come from `store` (workloads.ParamStore), inputs are numpy arrays uploaded once."""
+
+    def __init__(self, build, inputs, store, budget_bytes, ctx=None, lead=3, track_pool=False, min_bytes=1 << 20):
+        from . import stream, workloads
+        self.ctx = ctx or ndarray.gpu(0)
+        self.build = build
+        self.ops, self.leaves_bytes = record(build, {k: np.shape(v) for k, v in inputs.items()})
+        self.plan = plan(self.ops, self.leaves_bytes, budget_bytes, lead, min_bytes)
+        self.stream = stream.create_stream_handle(self.ctx)
+        self.backend = graph.GpuBackend(self.ctx, self.stream)
+        self.state = BudgetedTape.make_state(self.ctx)
+        self.track_pool = track_pool
+        self.binder = None
+        self.store = store
+        self.inputs = inputs
+        self.dev_inputs = None
+        self._workloads = workloads
+
+    def step(self, lr):
+        """One forward + backward + SGD step; returns the loss Var (its value stays on the device)."""
+        t = BudgetedTape(self.backend, self.plan, self.ops, self.state, self.track_pool)
+        if self.binder is None:
+            self.binder = self._workloads.Binder(t, self.store)
+            self.dev_inputs = {k: self.binder.input(v) for k, v in self.inputs.items()}
+        else:
+            self.binder.t, self.binder._n = t, 0
+            for v in self.binder.vars.values():
+                v.grad = None
+        loss, _ = self.build(t, self.binder, self.dev_inputs)
+        t.backward(loss)
+        self.binder.sgd_step(lr)
+        return loss
+
+    def sync(self):
+        self.backend.sync()
+
+
+def max_batch(build_for, input_shapes_for, budget_bytes, planned=True, lead=3, limit=1 << 12, min_bytes=1 << 20):
+    """Largest batch whose step fits `budget_bytes`: with `planned` the planner may send values to the
+    host, without it the replayed peak of the plain schedule must fit.  build_for(batch) -> builder,
+    input_shapes_for(batch) -> name -> shape.  The counterpart of the reference's batch-size sweeps per
+    policy (examples/imagenet_resnet.py:139-154).  -> (batch, TapePlan) or (0, None)."""
+    def fits(batch):
+        ops, leaves = record(build_for(batch), input_shapes_for(batch))
+        if any(op.bytes >= (1 << 33) for op in ops):      # tensors are limited to 2^31 elements
+            return None
+        try:
+            p = plan(ops, leaves, budget_bytes if planned else None, lead, min_bytes)
+        except ValueError:
+            return None
+        return p if p.peak_bytes <= budget_bytes else None
+
+    best, best_plan, hi = 0, None, 1
+    while hi <= limit:                 # double until it no longer fits
+        p = fits(hi)
+        if p is None:
+            break
+        best, best_plan = hi, p
+        hi *= 2
+    lo, hi = best, min(hi, limit + 1)
+    while hi - lo > 1:
+        mid = (lo + hi) // 2
+        p = fits(mid)
+        if p is None:
+            hi = mid
+        else:
+            lo, best, best_plan = mid, mid, p
+    return best, best_plan

@@ -1,0 +1,130 @@
+"""The branched example networks trained under device-memory budgets (one MI355X): the budgeted tape
+executor of tape_budget.py on ResNet-50 (batch 64), Inception-v4 (batch 32) and the Transformer (batch 32).
+
+    python -m tsplit_amd.tapebench --net resnet50|inception_v4|transformer [--fractions 0,0.75,0.5,0.35] [--steps 4] [--warmup 1]
+    python -m tsplit_amd.tapebench --net resnet50|inception_v4 --max-batch [--budgets 8,16]
+
+For every fraction f (0 = no limit) the budget is the leaves (parameters, their gradients' room is part
+of the replay, inputs, constants) plus f times what the operators' values and gradients take at the
+unplanned peak; the planner picks what leaves for pinned host memory, the executor trains on synthetic
+data.  One JSON object per budget: samples/s, the pool's measured peak over its level before the run,
+the replayed peak, values sent away, host waits per step.  With --max-batch the question is turned
+around, as in the reference's batch-size sweeps per policy (examples/imagenet_resnet.py:139-154): for
+every budget in GiB, the largest batch that trains with everything resident and the largest one the
+planner fits, and the measured throughput at the latter.
+"""
+import argparse
+import json
+import time
+
+import numpy as np
+
+
+def _net(name, batch=None):
+    """-> (builder(batch), numpy inputs(batch, rng), default batch, description)"""
+    from . import workloads
+    if name == "resnet50":
+        def build_for(n):
+            return lambda t, b, c: workloads.resnet(t, b, c["x"], c["y"])
+
+        def inputs_for(n, rng):
+            y = np.zeros((n, 1000), np.float32)
+            y[np.arange(n), rng.randint(0, 1000, n)] = 1
+            return {"x": rng.standard_normal((n, 3, 224, 224)).astype(np.float32), "y": y}
+        return build_for, inputs_for, 64, "ResNet-50, fp32 NCHW, 3x224x224, 1000 classes"
+    if name == "inception_v4":
+        def build_for(n):
+            return lambda t, b, c: workloads.inception_v4(t, b, c["x"], c["y"])
+
+        def inputs_for(n, rng):
+            y = np.zeros((n, 1000), np.float32)
+            y[np.arange(n), rng.randint(0, 1000, n)] = 1
+            return {"x": rng.standard_normal((n, 3, 299, 299)).astype(np.float32), "y": y}
+        return build_for, inputs_for, 32, "Inception-v4, fp32 NCHW, 3x299x299, 1000 classes"
+    if name == "transformer":
+        def cfg_for(n):
+            return workloads.TransformerConfig(batch=n, mask_value=0.0, embed_std=0.0002, pos_amplitude=0.003)
+
+        def build_for(n):
+            cfg = cfg_for(n)
+            return lambda t, b, c: workloads.transformer(t, b, cfg, c["xs"], c["yi"], c["yo"])
+
+        def inputs_for(n, rng):
+            cfg = cfg_for(n)
+            return {"xs": rng.randint(1, cfg.vocab, size=(n, cfg.len1)).astype(np.float32),
+                    "yi": rng.randint(1, cfg.vocab, size=(n, cfg.len2)).astype(np.float32),
+                    "yo": rng.randint(1, cfg.vocab, size=(n, cfg.len2)).astype(np.float32)}
+        return build_for, inputs_for, 32, "Transformer 6+6 blocks, d_model 512, 8 heads, FFN 2048, length 256, vocab 32000"
+    raise ValueError(name)
+
+
+def _measure(build, inputs, budget, steps, warmup, lr):
+    from . import tape_budget as tb, workloads
+    from .gpu_memory_manager import pool_state
+    base = pool_state().used
+    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(123), budget, track_pool=True)
+    for _ in range(warmup):
+        run.step(lr)
+    run.sync()
+    waits0 = run.state.host_waits
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = run.step(lr)
+    run.sync()
+    dt = (time.perf_counter() - t0) / steps
+    n = next(iter(inputs.values())).shape[0]
+    d = run.plan.describe()
+    gib = float(1 << 30)
+    return {"samples_per_s": n / dt, "ms_per_step": dt * 1e3, "measured_peak_GiB": (run.state.peak_used - base) / gib,
+            "planned_peak_GiB": d["peak_GiB"], "unplanned_peak_GiB": d["unplanned_peak_GiB"], "values_away": d["away"],
+            "away_GiB": sum(run.ops[i].bytes for i in run.plan.away) / gib,
+            "host_waits_per_step": (run.state.host_waits - waits0) / steps, "loss": float(loss.value.asnumpy()[0])}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--net", default="resnet50", choices=["resnet50", "inception_v4", "transformer"])
+    ap.add_argument("--fractions", default="0,0.75,0.5,0.35")
+    ap.add_argument("--budgets", default="8,16")
+    ap.add_argument("--batch", type=int, default=0)
+    ap.add_argument("--steps", type=int, default=4)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--lr", type=float, default=1e-4)
+    ap.add_argument("--max-batch", action="store_true")
+    a = ap.parse_args()
+    from . import tape_budget as tb
+    build_for, inputs_for, default_batch, desc = _net(a.net)
+    rng = np.random.RandomState(123)
+    if a.max_batch:
+        for b in [float(v) for v in a.budgets.split(",")]:
+            budget = int(b * (1 << 30))
+
+            one = {k: v.shape[1:] for k, v in inputs_for(1, np.random.RandomState(0)).items()}
+
+            def shapes_for(n):
+                return {k: (n,) + tail for k, tail in one.items()}
+            resident, _ = tb.max_batch(build_for, shapes_for, budget, planned=False)
+            planned, p = tb.max_batch(build_for, shapes_for, budget, planned=True)
+            row = {"net": a.net, "workload": desc, "budget_GiB": b, "max_batch_resident": resident, "max_batch_planned": planned}
+            if p is not None:
+                row.update(_measure(build_for(planned), inputs_for(planned, rng), budget, max(1, a.steps // 2), 1, a.lr))
+            print(json.dumps(row), flush=True)
+        return
+    n = a.batch or default_batch
+    inputs = inputs_for(n, rng)
+    build = build_for(n)
+    ops, leaves = tb.record(build, {k: v.shape for k, v in inputs.items()})
+    free_peak = tb.replay(ops, leaves)[0]
+    for f in [float(v) for v in a.fractions.split(",")]:
+        budget = None if f == 0 else leaves + int((free_peak - leaves) * f)
+        row = {"net": a.net, "workload": desc + ", batch %d" % n, "fraction": f,
+               "budget_GiB": None if budget is None else budget / float(1 << 30)}
+        try:
+            row.update(_measure(build, inputs, budget, a.steps, a.warmup, a.lr))
+        except ValueError as e:
+            row["error"] = str(e)
+        print(json.dumps(row), flush=True)
+
+
+if __name__ == "__main__":
+    main()
