@@ -180,11 +180,19 @@ class PlannedTrainer(object):
         self._reap(nbytes)
         if self.budget is not None and self.live + nbytes > self.budget:
             raise MemoryError("budget of %d bytes: %d live, %d more needed" % (self.budget, self.live, nbytes))
-        if reuse is not None:
-            reuse.malloc_itself()
-            arr = reuse
-        else:
-            arr = ndarray.empty(shape, self.ctx)
+        def take():
+            if reuse is not None:
+                reuse.malloc_itself()
+                return reuse
+            return ndarray.empty(shape, self.ctx)
+        try:
+            arr = take()
+        except RuntimeError:
+            # The pool itself is out (a capped pool, fragmented by releases still on their way): wait for
+            # every release that has been issued, then ask once more.
+            self.stall_events += 1
+            self._reap(force=True)
+            arr = take()
         self.live += nbytes
         self.peak = max(self.peak, self.live)
         return arr
