@@ -238,10 +238,20 @@ def main():
         # the GEMM kernels inside the Winograd calls, timed by the library with event pairs on the
         # compute stream around each launch; their work is the FLOP they execute
         wino_exec_flop = 0.0
-        for tag, grad in (("winograd_gemm", False), ("winograd_filter_grad_gemm", True)):
-            launches, ms, flop = L.winograd_gemm_times(filter_gradient=grad)
+        for tag, kind in (("winograd_gemm", 0), ("winograd_filter_grad_gemm", 1), ("winograd_gemm_shallow", 2)):
+            launches, ms, flop, nbytes = L.winograd_gemm_times(kind=kind)
             if launches:
                 wino_exec_flop += flop
+                if kind == 2:
+                    # 64 channels summed over: fewer than 19.7 executed FLOP per byte, so HBM bounds these launches
+                    k[tag] = {"calls": launches, "ms_total": ms, "ms_avg": ms / launches, "work": nbytes,
+                              "work_per_call": nbytes / launches, "rate": nbytes / (ms * 1e-3) / 1e9, "unit": "byte"}
+                    kernels[tag] = {"calls_per_step": launches / a.steps, "ms_per_step": ms / a.steps, "ms_avg": ms / launches,
+                                    "achieved": k[tag]["rate"], "unit": "GB/s", "frac": k[tag]["rate"] / PEAK_HBM_GBS,
+                                    "mfma_achieved_tflops": flop / (ms * 1e-3) / 1e12,
+                                    "note": "the forward / data-gradient GEMMs of the 64 -> 64 layer inside the *_winograd "
+                                            "calls: 16 executed FLOP per byte, bound by HBM; algorithmic bytes"}
+                    continue
                 k[tag] = {"calls": launches, "ms_total": ms, "ms_avg": ms / launches, "work": flop,
                           "work_per_call": flop / launches, "rate": flop / (ms * 1e-3) / 1e12, "unit": "flop"}
                 kernels[tag] = {"calls_per_step": launches / a.steps, "ms_per_step": ms / a.steps, "ms_avg": ms / launches,

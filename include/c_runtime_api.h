@@ -458,10 +458,15 @@ int TSplit_ConvTakesWinograd(int images, int in_channels, int out_channels, int 
  *      TSplit_WinogradGemmTiming(1) makes every such launch record an event pair on its stream
  *      (not while the stream is being recorded into a graph); (0) stops and forgets them.
  *      TSplit_WinogradGemmTimes waits for the launches of kind `which` (0: forward and data
- *      gradient, 1: filter gradient) and returns their count, summed milliseconds and summed
- *      executed FLOP (2 * 36 * rows * columns * depth per launch). ---- */
+ *      gradient, 1: filter gradient, 2: forward and data-gradient launches so shallow that memory
+ *      bounds them - fewer than 19.7 executed FLOP per byte moved, the ratio of the fp32 matrix
+ *      peak to the HBM peak; these are not part of kind 0) and returns their count, summed
+ *      milliseconds and summed executed FLOP (2 * 36 * rows * columns * depth per launch);
+ *      TSplit_WinogradGemmBytes returns their summed algorithmic bytes (both operands read once,
+ *      the result written once). ---- */
 int TSplit_WinogradGemmTiming(int on);
 int TSplit_WinogradGemmTimes(int which, double *launches, double *ms, double *flop);
+int TSplit_WinogradGemmBytes(int which, double *bytes);
 
 /* ---- Recorded steps.  NO counterpart in the reference (every step there is issued call by
  *      call from Python); for steps made of thousands of tiny kernels (recurrent nets, small

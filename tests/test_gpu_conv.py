@@ -163,9 +163,11 @@ def test_conv_winograd_choice(monkeypatch):
     assert L.conv_takes_winograd(16, 64, 128, 112, 112) and L.conv_takes_winograd(64, 512, 512, 14, 14)
     assert L.conv_takes_winograd(64, 256, 256, 56, 56, filter_gradient=True)
     assert L.conv_takes_winograd(16, 64, 128, 112, 112, filter_gradient=True)
-    assert L.conv_takes_winograd(16, 64, 64, 224, 224, filter_gradient=True)        # no transformed output to write: pays earlier
+    assert L.conv_takes_winograd(16, 64, 64, 224, 224, filter_gradient=True)
     assert not L.conv_takes_winograd(16, 32, 64, 224, 224, filter_gradient=True)
-    assert not L.conv_takes_winograd(64, 64, 64, 224, 224)           # too narrow: the transforms outweigh the GEMMs
+    # 64 channels on both sides are enough in every pass (tiles as wide as the produced channels)
+    assert L.conv_takes_winograd(64, 64, 64, 224, 224) and L.conv_takes_winograd(16, 64, 64, 224, 224, data_gradient=True)
+    assert not L.conv_takes_winograd(64, 32, 64, 224, 224) and not L.conv_takes_winograd(64, 64, 48, 224, 224)   # too narrow
     assert not L.conv_takes_winograd(2, 256, 256, 14, 14)            # too few tiles
     assert not L.conv_takes_winograd(64, 3, 64, 224, 224)
     monkeypatch.setenv("TSPLIT_CONV_WINOGRAD", "1")
@@ -241,11 +243,18 @@ def test_conv_micro_tensor_split_is_bit_identical(rng):
     np.testing.assert_array_equal(whole.asnumpy(), parts.asnumpy())
 
 
-def test_conv_full_size_properties(rng):
-    """Size-independent checks at a full VGG layer shape (64 x 64 x 224 x 224 -> 64, 236.8 GFLOP):
-    a delta filter copies one input channel (exact), and the adjoint identity
-    <conv(x,w),dy> = <x,bwd_data(w,dy)> = <w,bwd_filter(x,dy)> holds."""
+@pytest.mark.parametrize("winograd", ["0", None])
+def test_conv_full_size_properties(winograd, rng, monkeypatch):
+    """Size-independent checks at a full VGG layer shape (64 x 64 x 224 x 224 -> 64, 236.8 GFLOP), on the
+    direct kernels and with the routing the library chooses (the Winograd routine): a delta filter copies
+    one input channel (exactly on the direct kernels; to a few 1e-7 of the largest value through the
+    transforms), and the adjoint identity <conv(x,w),dy> = <x,bwd_data(w,dy)> = <w,bwd_filter(x,dy)> holds."""
     from tsplit_amd import gpu_links as L, ndarray
+    if winograd is None:
+        monkeypatch.delenv("TSPLIT_CONV_WINOGRAD", raising=False)
+        assert L.conv_takes_winograd(64, 64, 64, 224, 224)
+    else:
+        monkeypatch.setenv("TSPLIT_CONV_WINOGRAD", winograd)
     ctx = ndarray.gpu(0)
     shape = (64, 64, 224, 224)
     # build inputs on the host in float32 without large temporaries
@@ -257,7 +266,10 @@ def test_conv_full_size_properties(rng):
     y = ndarray.empty(shape, ctx)
     L.CuDNN_conv2d(gx, ndarray.array(w, ctx), y, 1, 1, 1)
     got = y.asnumpy()
-    assert np.array_equal(got, x[:, perm])
+    if winograd == "0":
+        assert np.array_equal(got, x[:, perm])
+    else:
+        assert_close(got, x[:, perm], 2e-6, "delta filter through the Winograd transforms")
     del got
     w2 = (rng.standard_normal(size=(64, 64, 3, 3)) / 24.0).astype(np.float32)
     gw2 = ndarray.array(w2, ctx)

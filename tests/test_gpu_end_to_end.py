@@ -172,8 +172,8 @@ def test_vgg16_224_natural_routing_every_operator_against_oracle():
     for imgs, c, o, hw in ((4, 64, 128, 112), (4, 128, 128, 112), (8, 128, 256, 56), (8, 256, 256, 56)):
         assert L.conv_takes_winograd(imgs, c, o, hw, hw, 3, 1, 1)
         assert L.conv_takes_winograd(imgs, c, o, hw, hw, 3, 1, 1, filter_gradient=True)
-        assert L.conv_takes_winograd(imgs, o, c, hw, hw, 3, 1, 1, data_gradient=True) or c == 64
-    assert not L.conv_takes_winograd(4, 64, 64, 224, 224, 3, 1, 1)
+        assert L.conv_takes_winograd(imgs, o, c, hw, hw, 3, 1, 1, data_gradient=True)
+    assert L.conv_takes_winograd(4, 64, 64, 224, 224, 3, 1, 1)
     lr, mom, eps = 0.01, 0.9, 0.01
     conv_idx = [i for i, l in enumerate(spec) if l[0] == "conv"]
     ctx = ndarray.gpu(0)

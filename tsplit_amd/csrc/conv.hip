@@ -2147,27 +2147,27 @@ inline bool winograd_shape(const ConvGeo &g) {
          static_cast<int64_t>(std::max(g.C, g.O)) * g.H * g.W < (1ll << 29);
 }
 
-// wide enough for the 36 GEMMs to outweigh the transforms (forward and data gradient write and read
-// back a transformed output as well, so they need more channels than the filter gradient, whose
-// GEMMs contract over the tiles), little of the 4x4 tiling hanging over the plane's edge, and
-// enough tiles to fill the chip
-inline bool winograd_wide(const ConvGeo &g, int widest) {
+// wide enough for the 36 GEMMs to outweigh the transforms (64 channels on both sides: with tiles as
+// wide as the produced channels even the 64 -> 64 layer at 224 x 224 runs a quarter faster than on the
+// direct kernels, forward and data gradient), little of the 4x4 tiling hanging over the plane's edge,
+// and enough tiles to fill the chip
+inline bool winograd_wide(const ConvGeo &g) {
   const int64_t covered = static_cast<int64_t>((g.H + 3) / 4) * ((g.W + 3) / 4) * 16;
-  return std::min(g.C, g.O) >= 64 && std::max(g.C, g.O) >= widest &&
-         covered * 3 <= static_cast<int64_t>(g.H) * g.W * 4 && static_cast<int64_t>(g.imgs) * covered >= 16 * 1024;
+  return std::min(g.C, g.O) >= 64 && covered * 3 <= static_cast<int64_t>(g.H) * g.W * 4 &&
+         static_cast<int64_t>(g.imgs) * covered >= 16 * 1024;
 }
 
 // forward and data gradient: the channels summed over are the GEMMs' K
 inline bool winograd_pays(const ConvGeo &g, int gathered) {
   const int forced = winograd_forced();
   if (!winograd_shape(g) || gathered % BK != 0 || forced == 0) return false;
-  return forced == 1 || winograd_wide(g, 128);
+  return forced == 1 || winograd_wide(g);
 }
 
 inline bool winograd_filter_grad_pays(const ConvGeo &g) {
   const int forced = winograd_forced();
   if (!winograd_shape(g) || forced == 0) return false;
-  return forced == 1 || winograd_wide(g, 64);
+  return forced == 1 || winograd_wide(g);
 }
 
 // ------------------------------------------------------------------ statistics of the output

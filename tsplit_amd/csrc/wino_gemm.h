@@ -20,7 +20,7 @@ struct Problem {
   const float *V;   // [36][depth][ld]
   float *M;         // [36][rows][ld]
   int rows, depth, ld;
-  int tm, tn;       // tiles of 128 rows / 128 columns
+  int tm, tn;       // tiles of BM rows / BN columns
 };
 
 // Persistent form: the grid is one resident round of blocks (blocks_per_cu on each CU) and every block
@@ -31,10 +31,19 @@ struct Problem {
 // that ends after its one tile holds its slot until the last store is acknowledged.)  The stores are
 // marked non-temporal: M is read next by another kernel, after the whole of it has been written.
 // Summation order is that of the one-tile-per-block engine: the results are the same bits.
-constexpr int kGemmBlocksPerCu = 4;   // resident blocks per compute unit: registers and LDS (4 x 40 KB) allow exactly four
-static __global__ __launch_bounds__(kThreads, 4) void wino_gemm_kernel(Problem p, int total) {
-  using ALoader = KContigBufLoader<128>;
-  using BLoader = MnContigBufLoader<128>;
+// Tiles are 128 x 128 (2 x 2 waves; four resident blocks per compute unit: registers and 4 x 40 KB of LDS
+// allow exactly four) or, for layers that produce at most 64 channels, 64 x 256 (1 x 4 waves, so that no
+// wave idles on rows that do not exist; 44 KB of LDS, three blocks).
+template <int BM, int BN>
+constexpr int gemm_blocks_per_cu() {
+  return BM == 128 ? 4 : 3;
+}
+template <int BM, int BN>
+static __global__ __launch_bounds__(kThreads, (gemm_blocks_per_cu<BM, BN>())) void wino_gemm_kernel(Problem p, int total) {
+  static_assert((BM == 128 && BN == 128) || (BM == 64 && BN == 256), "each of the 4 waves owns a 64x64 sub-tile");
+  constexpr int WN = BN / 64;
+  using ALoader = KContigBufLoader<BM>;
+  using BLoader = MnContigBufLoader<BN>;
   using ALds = typename ALoader::Lds;
   using BLds = typename BLoader::Lds;
   constexpr int kStage = ALds::kFloats + BLds::kFloats;
@@ -43,7 +52,7 @@ static __global__ __launch_bounds__(kThreads, 4) void wino_gemm_kernel(Problem p
   static_assert(4 * 32 * kPitch <= 2 * kStage, "staging areas fit the operand stages");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
+  const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
   const int M = p.rows, N = p.ld, K = p.depth;
   const int per_xi = p.tm * p.tn;
   // XCD-aware order: the dispatcher deals consecutive block ids to the 8 XCDs in turn, so XCD x owns
@@ -58,8 +67,8 @@ static __global__ __launch_bounds__(kThreads, 4) void wino_gemm_kernel(Problem p
     z = l / per_xi;
     const int rem = l - z * per_xi;
     const int tile_n = rem / p.tm;
-    m0 = (rem - tile_n * p.tm) * 128;
-    n0 = tile_n * 128;
+    m0 = (rem - tile_n * p.tm) * BM;
+    n0 = tile_n * BN;
   };
 
   ALoader la;
@@ -460,14 +469,23 @@ static __global__ __launch_bounds__(kThreads, NB) void wino_grad_gemm_kernel(Gra
   }
 }
 
-// One resident round of blocks: four on each of `cus` compute units (three were 3 % slower over the
-// launches of a VGG-16 step), never more blocks than tiles.
-inline void launch(const Problem &p, hipStream_t st, int cus) {
+// One resident round of blocks on `cus` compute units (with four per unit the 128 x 128 kernel ran 3 %
+// faster over the launches of a VGG-16 step than with three), never more blocks than tiles.
+template <int BM, int BN>
+inline void launch_tiles(Problem p, hipStream_t st, int cus) {
+  p.tm = (p.rows + BM - 1) / BM;
+  p.tn = (p.ld + BN - 1) / BN;
   const int total = p.tm * p.tn * kXi;
-  int grid = cus * kGemmBlocksPerCu / 8 * 8;
+  int grid = cus * gemm_blocks_per_cu<BM, BN>() / 8 * 8;
   if (grid > (total + 7) / 8 * 8) grid = (total + 7) / 8 * 8;
   if (grid < 8) grid = 8;
-  hipLaunchKernelGGL(wino_gemm_kernel, dim3(grid), dim3(kThreads), 0, st, p, total);
+  hipLaunchKernelGGL((wino_gemm_kernel<BM, BN>), dim3(grid), dim3(kThreads), 0, st, p, total);
+}
+inline void launch(const Problem &p, hipStream_t st, int cus) {
+  if (p.rows <= 64)
+    launch_tiles<64, 256>(p, st, cus);
+  else
+    launch_tiles<128, 128>(p, st, cus);
 }
 
 }  // namespace wg

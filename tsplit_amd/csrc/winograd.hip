@@ -356,8 +356,9 @@ __global__ __launch_bounds__(256) void wino_filter_grad_kernel(const float *__re
 // stream, so a benchmark can read the duration of these kernels inside its timed region.
 struct TimedLaunch {
   hipEvent_t begin, end;
-  int which;       // 0: forward / data-gradient GEMMs, 1: filter-gradient GEMMs
-  double flop;
+  int which;       // 0: forward / data-gradient GEMMs, 1: filter-gradient GEMMs, 2: forward / data-gradient
+                   // GEMMs so shallow that memory bounds them (below 19.7 FLOP per byte moved)
+  double flop, bytes;
 };
 std::mutex g_timing_mu;
 bool g_timing_on = false;
@@ -365,7 +366,7 @@ std::vector<TimedLaunch> g_timed;
 
 class GemmTiming {
  public:
-  GemmTiming(hipStream_t st, int which, double flop) : st_(st) {
+  GemmTiming(hipStream_t st, int which, double flop, double bytes) : st_(st) {
     std::lock_guard<std::mutex> lk(g_timing_mu);
     if (!g_timing_on) return;
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
@@ -377,6 +378,7 @@ class GemmTiming {
     }
     t_.which = which;
     t_.flop = flop;
+    t_.bytes = bytes;
     on_ = hipEventRecord(t_.begin, st) == hipSuccess;
   }
   ~GemmTiming() {
@@ -525,7 +527,10 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
     else
       hipLaunchKernelGGL(wino_input_kernel<false>, dim3((gi.ld + 255) / 256, gathered), dim3(256), 0, st, xr, V, gi);
     {
-      GemmTiming timed(st, 0, 2.0 * kXi * produced * static_cast<double>(gi.ld) * gathered);
+      // every operand read once, the result written once
+      const double flop = 2.0 * kXi * produced * static_cast<double>(gi.ld) * gathered;
+      const double bytes = 4.0 * kXi * (static_cast<double>(produced) * gathered + static_cast<double>(gathered + produced) * gi.ld);
+      GemmTiming timed(st, flop < 19.7 * bytes ? 2 : 0, flop, bytes);
       wg::launch(wg::Problem{U, V, M, produced, gathered, gi.ld, (produced + 127) / 128, (gi.ld + 127) / 128}, st,
                  compute_units());
     }
@@ -579,7 +584,8 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
       hipLaunchKernelGGL(wino_grad_kernel<false>, grid_y, dim3(256), 0, st, dyr, Y, gy);
     const int here = (gx.ld + kchunk - 1) / kchunk;
     {
-      GemmTiming timed(st, 1, 2.0 * kXi * O * static_cast<double>(gx.ld) * C);
+      GemmTiming timed(st, 1, 2.0 * kXi * O * static_cast<double>(gx.ld) * C,
+                       4.0 * kXi * (static_cast<double>(O) * C * here + static_cast<double>(O + C) * gx.ld));
       launch_grad_gemm(plan, wg::GradProblem{Y, V, part + static_cast<int64_t>(parts) * kXi * oc, O, C, gx.ld, kchunk, 0, 0},
                        here, st);
     }
@@ -607,6 +613,18 @@ extern "C" int TSplit_WinogradGemmTiming(int on) {
   }
   g_timed.clear();
   g_timing_on = on != 0;
+  return 0;
+}
+
+// The summed algorithmic bytes (every operand read once, the result written once) of the recorded launches
+// of kind `which`.
+extern "C" int TSplit_WinogradGemmBytes(int which, double *bytes) {
+  using namespace tsplit;
+  std::lock_guard<std::mutex> lk(g_timing_mu);
+  double total = 0;
+  for (const TimedLaunch &t : g_timed)
+    if (t.which == which) total += t.bytes;
+  if (bytes) *bytes = total;
   return 0;
 }
 

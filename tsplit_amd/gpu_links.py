@@ -421,13 +421,15 @@ def winograd_gemm_timing(on):
     check_call(_LIB.TSplit_WinogradGemmTiming(int(bool(on))))
 
 
-def winograd_gemm_times(filter_gradient=False):
-    """-> (launches, total ms, total executed FLOP) of the timed GEMM launches of the forward /
-    data-gradient routine, or of the filter-gradient routine."""
-    n, ms, flop = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
-    check_call(_LIB.TSplit_WinogradGemmTimes(int(bool(filter_gradient)), ctypes.byref(n), ctypes.byref(ms),
-                                             ctypes.byref(flop)))
-    return int(n.value), ms.value, flop.value
+def winograd_gemm_times(filter_gradient=False, kind=None):
+    """-> (launches, total ms, total executed FLOP, total algorithmic bytes) of the timed GEMM launches of
+    kind 0 (forward / data gradient), 1 (filter gradient) or 2 (forward / data-gradient launches that
+    memory bounds)."""
+    which = int(bool(filter_gradient)) if kind is None else int(kind)
+    n, ms, flop, nbytes = ctypes.c_double(), ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+    check_call(_LIB.TSplit_WinogradGemmTimes(which, ctypes.byref(n), ctypes.byref(ms), ctypes.byref(flop)))
+    check_call(_LIB.TSplit_WinogradGemmBytes(which, ctypes.byref(nbytes)))
+    return int(n.value), ms.value, flop.value, nbytes.value
 
 
 # ---- Fused BatchNorm + Relu (no counterpart in the reference's gpu_links) ----
