@@ -442,6 +442,17 @@ int TSplit_BatchNormFromStats(const DLArrayHandle input_X, const DLArrayHandle s
                               DLArrayHandle save_var_arr, int relu, DLStreamHandle stream_handle,
                               ProfilerHandle p);
 
+/* ---- Optimizer update of a whole model in one launch.  NO counterpart in the reference, whose
+ *      optimizer issues one SGDOptimizerUpdate / MomentumOptimizerUpdate per parameter
+ *      (python/athena/optimizer.py:95-176): dozens of launches, most of them on BatchNorm vectors
+ *      that cost a launch for nanoseconds of work.  params / grads / velocities are tables of `count`
+ *      array handles; velocities == NULL selects plain SGD, otherwise momentum (nesterov != 0: the
+ *      Nesterov form).  Per element the arithmetic is that of the single-parameter symbols (same
+ *      bits).  The table is kept in device memory per stream and uploaded again only when it changes. ---- */
+int TSplit_OptimizerUpdateMulti(DLArrayHandle *params, const DLArrayHandle *grads,
+                                DLArrayHandle *velocities, int count, float lr, float momentum,
+                                int nesterov, DLStreamHandle stream_handle);
+
 /* ---- Which routine a convolution takes.  NO counterpart in the reference (cuDNN's choice is
  *      internal there, src/ops/CudnnConv2d.cu:66).  Returns 1 when CuDNN_DLGpuConv2d (pass 0),
  *      CuDNN_DLGpuConv2d_Gradient_of_Data (pass 1) or CuDNN_DLGpuConv2d_Gradient_of_Filter (pass 2)

@@ -362,3 +362,49 @@ def test_fused_batchnorm_relu_needs_saved_statistics(ts):
     x, g, b, y = ts.empty((2, 3, 4, 4)), ts.empty((1, 3, 1, 1)), ts.empty((1, 3, 1, 1)), ts.empty((2, 3, 4, 4))
     with pytest.raises(Exception):
         ts.links.batch_norm_relu(x, g, b, y, None, None, 0.01, ts.stream)
+
+
+@pytest.mark.parametrize("kind", ["sgd", "momentum", "nesterov"])
+def test_optimizer_update_of_many_parameters_in_one_launch(ts, kind, rng):
+    """TSplit_OptimizerUpdateMulti against the per-parameter symbols (same bits) and the oracle, three
+    steps over parameters of awkward sizes: single values, tails of 1 - 3 elements, an array longer than
+    one block's share, a view that starts off a 16-byte boundary, an empty array."""
+    L, s = ts.links, ts.stream
+    shapes = [(1,), (3,), (5,), (1023,), (4096,), (4097,), (64, 3, 3, 3), (1, 512, 1, 1), (100003,), (300, 257)]
+    ps = [rng.normal(size=sh).astype(np.float32) for sh in shapes]
+    one, many = [ts.arr(p) for p in ps], [ts.arr(p) for p in ps]
+    vel_one, vel_many = [ts.arr(np.zeros_like(p)) for p in ps], [ts.arr(np.zeros_like(p)) for p in ps]
+    # an unaligned view: rows 1.. of a 5 x 3 array start 12 bytes into it
+    base_one, base_many = ts.arr(rng.normal(size=(5, 3))), None
+    base_many = ts.arr(base_one.asnumpy())
+    vb_one, vb_many = ts.arr(np.zeros((5, 3))), ts.arr(np.zeros((5, 3)))
+    for b in (base_one, base_many, vb_one, vb_many):
+        b.split_tensor(5)
+    views = lambda arr: [arr.sTensor[1], arr.sTensor[3]]
+    ref_p = [p.astype(np.float64) for p in ps] + [base_one.asnumpy()[1:2].astype(np.float64), base_one.asnumpy()[3:4].astype(np.float64)]
+    ref_v = [np.zeros_like(p) for p in ref_p]
+    lr, mom = 0.05, 0.9
+    for step in range(3):
+        gs = [rng.normal(size=p.shape).astype(np.float32) for p in ref_p]
+        g_dev = [ts.arr(g) for g in gs]
+        p_one, p_many = one + views(base_one), many + views(base_many)
+        v_one, v_many = vel_one + views(vb_one), vel_many + views(vb_many)
+        for p, g, v in zip(p_one, g_dev, v_one):
+            if kind == "sgd":
+                L.sgd_update(p, g, lr, s)
+            else:
+                L.momentum_update(p, g, v, lr, mom, kind == "nesterov", s)
+        L.optimizer_update_multi(p_many, g_dev, None if kind == "sgd" else v_many, lr, mom, kind == "nesterov", s)
+        for i, g in enumerate(gs):
+            if kind == "sgd":
+                ref_p[i] = O.sgd_update(ref_p[i], g, lr)
+            else:
+                ref_p[i], ref_v[i] = O.momentum_update(ref_p[i], g, ref_v[i], lr, mom, kind == "nesterov")
+    for a, b, r in zip(one + views(base_one), many + views(base_many), ref_p):
+        np.testing.assert_array_equal(b.asnumpy(), a.asnumpy())
+        assert_close(b.asnumpy(), r, TOL, "parameter after three updates")
+    for a, b in zip(vel_one, vel_many):
+        np.testing.assert_array_equal(b.asnumpy(), a.asnumpy())
+    # the rows of the 5 x 3 arrays that were not listed are untouched
+    np.testing.assert_array_equal(base_many.asnumpy()[[0, 2, 4]], base_one.asnumpy()[[0, 2, 4]])
+    L.optimizer_update_multi([], [], None, lr, stream=s)         # nothing to do

@@ -27,6 +27,7 @@ __all__ = [
     "embedding_lookup_gradient", "matrix_elementwise_divide", "matrix_elementwise_divide_const",
     "matrix_opposite", "matrix_sqrt", "matrix_rsqrt", "tanh", "sigmoid",
     "batch_norm_relu", "batch_norm_relu_gradient", "conv2d_batch_norm_stats", "batch_norm_from_stats",
+    "optimizer_update_multi",
     "CuDNN_Dropout", "CuDNN_Dropout_gradient", "CuSparse_Csrmv", "CuSparse_Csrmm",
 ]
 
@@ -222,6 +223,14 @@ def sgd_update(param, grad, lr, stream=None):
 def momentum_update(param, grad, velocity, lr, momentum, nesterov, stream=None):
     check_call(_LIB.MomentumOptimizerUpdate(_h(param), _h(grad), _h(velocity), ctypes.c_float(lr),
                                             ctypes.c_float(momentum), ctypes.c_bool(bool(nesterov)), _s(stream)))
+
+
+def optimizer_update_multi(params, grads, velocities, lr, momentum=0.0, nesterov=False, stream=None):
+    """SGD (velocities None) or momentum update of a list of parameters in one launch."""
+    n = len(params)
+    table = lambda arrs: (_nd.DLArrayHandle * n)(*[_h(a) for a in arrs])
+    check_call(_LIB.TSplit_OptimizerUpdateMulti(table(params), table(grads), table(velocities) if velocities is not None else None,
+                                                n, ctypes.c_float(lr), ctypes.c_float(momentum), int(bool(nesterov)), _s(stream)))
 
 
 def adagrad_update(param, grad, accumulation, lr, eps, stream=None):

@@ -117,7 +117,8 @@ def _out_shape(layer, s):
 
 class Trainer(object):
     def __init__(self, spec, params, input_shape, num_classes, ctx=None, optimizer=("sgd", 0.1),
-                 split=None, bn_eps=0.01, timer=None, fuse_bn_relu=False, conv_bn_stats=False):
+                 split=None, bn_eps=0.01, timer=None, fuse_bn_relu=False, conv_bn_stats=False,
+                 multi_tensor_update=False):
         self.spec = list(spec)
         # with fuse_bn_relu a ("bn", ...) layer directly followed by ("relu",) runs as ONE fused call
         # in each direction (symbols outside the reference's ABI); the Relu layer's own arrays are
@@ -132,6 +133,9 @@ class Trainer(object):
         if conv_bn_stats:
             self.stats_of = {li: None for li, l in enumerate(self.spec[:-1])
                              if l[0] == "conv" and self.spec[li + 1][0] == "bn"}
+        # with multi_tensor_update the optimizer updates every parameter in ONE launch (a symbol outside
+        # the reference's ABI) instead of one call per parameter
+        self.multi_tensor_update = multi_tensor_update
         # optional per-call timing hook: timer.begin(stream) / timer.end(stream, tag, work, unit)
         self.timer = timer
         self.ctx = ctx if ctx is not None else ndarray.gpu(0)
@@ -335,6 +339,16 @@ class Trainer(object):
 
     # ---------------------------------------------------------------- update
     def update(self):
+        if self.multi_tensor_update and self.optimizer[0] in ("sgd", "momentum"):
+            names = list(self.params)
+            total = sum(self._n(self.params[k].shape) for k in names)
+            ps, gs = [self.params[k] for k in names], [self.grads[k] for k in names]
+            if self.optimizer[0] == "sgd":
+                self._run("sgd_multi", 12.0 * total, "byte", L.optimizer_update_multi, ps, gs, None, self.optimizer[1], 0.0, False)
+            else:
+                self._run("momentum_multi", 20.0 * total, "byte", L.optimizer_update_multi, ps, gs,
+                          [self.state[k] for k in names], self.optimizer[1], self.optimizer[2], False)
+            return
         for name, p in self.params.items():
             g = self.grads[name]
             if self.optimizer[0] == "sgd":
