@@ -469,10 +469,10 @@ int TSplit_ConvTakesWinograd(int images, int in_channels, int out_channels, int 
  *      TSplit_WinogradGemmTiming(1) makes every such launch record an event pair on its stream
  *      (not while the stream is being recorded into a graph); (0) stops and forgets them.
  *      TSplit_WinogradGemmTimes waits for the launches of kind `which` (0: forward and data
- *      gradient, 1: filter gradient, 2: forward and data-gradient launches so shallow that memory
- *      bounds them - fewer than 19.7 executed FLOP per byte moved, the ratio of the fp32 matrix
- *      peak to the HBM peak; these are not part of kind 0) and returns their count, summed
- *      milliseconds and summed executed FLOP (2 * 36 * rows * columns * depth per launch);
+ *      gradient on 128 x 128 tiles, 1: filter gradient, 2: forward and data gradient of layers that
+ *      produce at most 64 channels, which run on 64 x 256 tiles: one kernel per kind) and returns
+ *      their count, summed milliseconds and summed executed FLOP (2 * 36 * rows * columns * depth
+ *      per launch);
  *      TSplit_WinogradGemmBytes returns their summed algorithmic bytes (both operands read once,
  *      the result written once). ---- */
 int TSplit_WinogradGemmTiming(int on);

@@ -356,8 +356,8 @@ __global__ __launch_bounds__(256) void wino_filter_grad_kernel(const float *__re
 // stream, so a benchmark can read the duration of these kernels inside its timed region.
 struct TimedLaunch {
   hipEvent_t begin, end;
-  int which;       // 0: forward / data-gradient GEMMs, 1: filter-gradient GEMMs, 2: forward / data-gradient
-                   // GEMMs so shallow that memory bounds them (below 19.7 FLOP per byte moved)
+  int which;       // 0: forward / data-gradient GEMMs on 128 x 128 tiles, 1: filter-gradient GEMMs,
+                   // 2: forward / data-gradient GEMMs on 64 x 256 tiles (at most 64 channels produced)
   double flop, bytes;
 };
 std::mutex g_timing_mu;
@@ -530,7 +530,7 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
       // every operand read once, the result written once
       const double flop = 2.0 * kXi * produced * static_cast<double>(gi.ld) * gathered;
       const double bytes = 4.0 * kXi * (static_cast<double>(produced) * gathered + static_cast<double>(gathered + produced) * gi.ld);
-      GemmTiming timed(st, flop < 19.7 * bytes ? 2 : 0, flop, bytes);
+      GemmTiming timed(st, produced <= 64 ? 2 : 0, flop, bytes);
       wg::launch(wg::Problem{U, V, M, produced, gathered, gi.ld, (produced + 127) / 128, (gi.ld + 127) / 128}, st,
                  compute_units());
     }
