@@ -1,5 +1,5 @@
 """The budgeted tape executor on the GPU: residual, multi-branch and attention graphs trained with
-part of their activations in pinned host memory.
+part of their activations in pinned host memory or dropped and computed again.
 
 Bars: losses of the budgeted run equal those of the plain tape on the same library bit for bit (the same
 operators run on the same values; only where the values wait differs); against the numpy oracle the
@@ -57,8 +57,9 @@ def _cases(rng):
     }
 
 
+@pytest.mark.parametrize("recompute", [False, True])
 @pytest.mark.parametrize("net", ["resnet", "inception", "transformer"])
-def test_budgeted_graph_tracks_the_plain_tape_and_the_oracle(net, rng):
+def test_budgeted_graph_tracks_the_plain_tape_and_the_oracle(net, recompute, rng):
     from tsplit_amd import graph, tape_budget as tb, workloads
     build, inputs, lr = _cases(rng)[net]
     steps = 3
@@ -70,14 +71,15 @@ def test_budgeted_graph_tracks_the_plain_tape_and_the_oracle(net, rng):
     for frac in (0.5, 0.6, 0.7, 0.8, 0.9):
         budget = leaves + int((free_peak - leaves) * frac)
         try:
-            plan = tb.plan(ops, leaves, budget, min_bytes=0)
+            plan = tb.plan(ops, leaves, budget, min_bytes=0, recompute=recompute)
             break
         except ValueError:
             continue
-    assert plan is not None and plan.away and plan.peak_bytes <= budget
+    assert plan is not None and (plan.away or plan.redo) and plan.peak_bytes <= budget
     assert net != "resnet" or frac == 0.5
-    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(5), budget, min_bytes=0)
-    assert run.plan.away == plan.away
+    assert bool(plan.redo) == recompute
+    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(5), budget, min_bytes=0, recompute=recompute)
+    assert run.plan.away == plan.away and run.plan.redo == plan.redo
     got = []
     for _ in range(steps):
         loss = run.step(lr)
@@ -100,7 +102,7 @@ def test_budgeted_graph_tracks_the_plain_tape_and_the_oracle(net, rng):
         # (and the Inception graph at a batch of three drifts the same way in its weights: 6e-3 after three steps)
         if net == "resnet" and k.endswith("weight"):
             assert_close(run.store.values[k].reshape(v.shape), v, 2e-3, k)
-    assert run.state.host_waits > 0
+    assert run.state.host_waits > 0 or not plan.away
 
 
 def test_pool_usage_stays_within_the_replayed_peak(rng):
@@ -115,9 +117,10 @@ def test_pool_usage_stays_within_the_replayed_peak(rng):
     ops, leaves = tb.record(build, {k: v.shape for k, v in inputs.items()})
     free_peak = tb.replay(ops, leaves)[0]
     peaks = {}
-    for tag, budget in (("free", None), ("half", leaves + (free_peak - leaves) // 2)):
+    half = leaves + (free_peak - leaves) // 2
+    for tag, budget, recompute in (("free", None, False), ("half", half, False), ("half recomputing", half, True)):
         base = pool_state().used
-        run = tb.BudgetedRun(build, inputs, workloads.ParamStore(3), budget, track_pool=True, min_bytes=0)
+        run = tb.BudgetedRun(build, inputs, workloads.ParamStore(3), budget, track_pool=True, min_bytes=0, recompute=recompute)
         for _ in range(2):
             run.step(0.01)
         run.sync()
@@ -125,6 +128,7 @@ def test_pool_usage_stays_within_the_replayed_peak(rng):
         # the pool rounds every block up and the executor's events, the loss seed and the library's
         # bookkeeping are small allocations of their own: 3 % and 2 MiB of slack
         assert peaks[tag] <= run.plan.peak_bytes * 1.03 + (2 << 20), (tag, peaks[tag], run.plan.peak_bytes)
-        assert peaks[tag] >= run.plan.peak_bytes * 0.9, (tag, peaks[tag], run.plan.peak_bytes)
+        # (the pool is read between operators, so moments inside a backward step escape it: a loose lower bound)
+        assert peaks[tag] >= run.plan.peak_bytes * 0.8, (tag, peaks[tag], run.plan.peak_bytes)
         del run
-    assert peaks["half"] < 0.65 * peaks["free"]
+    assert peaks["half"] < 0.65 * peaks["free"] and peaks["half recomputing"] < 0.65 * peaks["free"]

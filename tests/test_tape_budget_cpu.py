@@ -32,25 +32,48 @@ def test_record_lists_every_operator_with_its_readers(net):
     assert any(bwd[i] for i in range(len(ops))) and any(not bwd[i] for i in range(len(ops)))
 
 
+@pytest.mark.parametrize("recompute", [False, True])
 @pytest.mark.parametrize("net", sorted(SHAPES))
-def test_plan_meets_the_budget_by_sending_idle_values_away(net):
+def test_plan_meets_the_budget_by_taking_idle_values_off_the_device(net, recompute):
     build, shapes = SHAPES[net]
     ops, leaves = tb.record(build, shapes)
     free_peak, at, idle = tb.replay(ops, leaves)
     assert free_peak > leaves and 0 <= at < 2 * len(ops)
     last_fwd, bwd = tb._uses(ops)
-    previous = free_peak
     for frac in (0.9, 0.7, 0.55):
         budget = leaves + int((free_peak - leaves) * frac)
-        p = tb.plan(ops, leaves, budget, min_bytes=0)
+        p = tb.plan(ops, leaves, budget, min_bytes=0, recompute=recompute)
         assert p.peak_bytes <= budget and p.free_peak_bytes == free_peak
-        assert p.peak_bytes == tb.replay(ops, leaves, p.away, p.lead)[0]
-        assert all(bwd[i] for i in p.away)            # only values the backward sweep reads again are worth moving
-        assert p.peak_bytes <= previous
-        previous = p.peak_bytes
-    assert tb.plan(ops, leaves, None).away == frozenset()
+        assert p.peak_bytes == tb.replay(ops, leaves, p.away, p.lead, p.redo)[0]
+        last_fwd, need = tb._needs(ops, p.redo)
+        assert all(need[i] for i in p.away | p.redo)     # only values that are read again are worth taking off
+        assert not (p.away & p.redo) and all(ops[i].cheap for i in p.redo)
+        assert recompute or not p.redo
+    if recompute:
+        # what is computed again is never sent over the link as well, and less travels than without
+        moved = sum(ops[i].bytes for i in p.away)
+        q = tb.plan(ops, leaves, budget, min_bytes=0, recompute=False)
+        assert moved < sum(ops[i].bytes for i in q.away)
+    none = tb.plan(ops, leaves, None)
+    assert none.away == frozenset() and none.redo == frozenset()
     with pytest.raises(ValueError):
         tb.plan(ops, leaves, leaves + 1, min_bytes=0)
+
+
+def test_a_recomputed_value_keeps_its_inputs_until_it_has_been_rebuilt():
+    """Dropping a Relu output makes the BatchNorm output before it needed at the Relu output's first
+    backward reader, which is earlier in the sweep than the BatchNorm output's own reader."""
+    build, shapes = SHAPES["resnet"]
+    ops, leaves = tb.record(build, shapes)
+    last_fwd, bwd = tb._uses(ops)
+    # a cheap operator whose single input is an operator output that its own backward reads (Relu after BatchNorm)
+    i = next(k for k, op in enumerate(ops) if op.cheap and len(op.inputs) == 1 and op.inputs[0] >= 0 and bwd[k]
+             and ops[op.inputs[0]].cheap)
+    u = ops[i].inputs[0]
+    _, need = tb._needs(ops, {i})
+    assert max(need[u]) == max(bwd[i]) >= max(bwd[u])
+    _, need2 = tb._needs(ops, {i, u})           # chains: the convolution output before the BatchNorm as well
+    assert max(need2[ops[u].inputs[0]]) == max(bwd[i])
 
 
 def test_sending_a_value_away_frees_it_between_its_uses():
@@ -61,6 +84,8 @@ def test_sending_a_value_away_frees_it_between_its_uses():
     i = max((op.bytes, k) for k, op in enumerate(ops) if bwd[k])[1]
     base = tb.replay(ops, leaves)[0]
     assert tb.replay(ops, leaves, {i})[0] <= base
+    j = max((op.bytes, k) for k, op in enumerate(ops) if bwd[k] and op.cheap)[1]
+    assert tb.replay(ops, leaves, (), 3, {j})[0] <= base
 
 
 def test_max_batch_grows_with_the_budget_and_with_planning():

@@ -30,10 +30,13 @@ class Var(object):
 class Node(object):
     """One operator call: its output, the closure of its backward operators (None when no input
     needs a gradient), the Vars it read and the Vars its backward closure reads again."""
-    __slots__ = ["out", "back", "inputs", "saved", "index"]
+    __slots__ = ["out", "back", "inputs", "saved", "index", "redo"]
 
-    def __init__(self, out, back, inputs, saved, index):
+    def __init__(self, out, back, inputs, saved, index, redo=None):
         self.out, self.back, self.inputs, self.saved, self.index = out, back, tuple(inputs), tuple(saved), index
+        # for operators that are cheap to run again (one to three passes over HBM): a closure that
+        # computes the output once more from the inputs' current values, with the same bits
+        self.redo = redo
 
 
 SELF = object()      # in a `saved` list: the operator's own output
@@ -275,13 +278,13 @@ class Tape(object):
     def const(self, value, shape, name=None):
         return Var(value, shape, False, name)
 
-    def _out(self, value, shape, inputs, backward, saved=None):
+    def _out(self, value, shape, inputs, backward, saved=None, redo=None):
         """Registers an operator call.  `saved`: the Vars the backward closure reads (SELF for the
         output itself); by default the inputs.  A closure must read them as `var.value` when it
-        runs, so that an executor may move a value off the device in between."""
+        runs, so that an executor may move a value off the device in between.  `redo`: see Node."""
         v = Var(value, shape, any(i.needs_grad for i in inputs))
         saved = inputs if saved is None else [v if s is SELF else s for s in saved]
-        node = Node(v, backward if v.needs_grad else None, inputs, saved if v.needs_grad else (), len(self._nodes))
+        node = Node(v, backward if v.needs_grad else None, inputs, saved if v.needs_grad else (), len(self._nodes), redo)
         v.node = node.index
         self._nodes.append(node)
         self._after_forward(node)
@@ -318,19 +321,21 @@ class Tape(object):
     def batch_norm(self, x, gamma, beta, eps=0.01):
         """gpu_ops/BatchNorm.py:54-83 (compute), :166-227 (gradient node; statistics recomputed, no
         saved arrays); gamma / beta receive their gradients as in gpu_ops/BatchNorm2.py:104-114."""
-        y = self.b.bn(x.value, gamma.value, beta.value, x.shape, eps)
+        def fwd():
+            return self.b.bn(x.value, gamma.value, beta.value, x.shape, eps)
 
         def back(g):
             dx, dg, db = self.b.bn_grad(g, x.value, gamma.value, x.shape, eps)
             self._acc(x, dx)
             self._acc(gamma, dg)
             self._acc(beta, db)
-        return self._out(y, x.shape, [x, gamma, beta], back, saved=[x, gamma])
+        return self._out(fwd(), x.shape, [x, gamma, beta], back, saved=[x, gamma], redo=fwd)
 
     def relu(self, x):
         """gpu_ops/Relu.py:51,117."""
-        y = self.b.relu(x.value, x.shape)
-        return self._out(y, x.shape, [x], lambda g: self._acc(x, self.b.relu_grad(x.value, g, x.shape)))
+        def fwd():
+            return self.b.relu(x.value, x.shape)
+        return self._out(fwd(), x.shape, [x], lambda g: self._acc(x, self.b.relu_grad(x.value, g, x.shape)), redo=fwd)
 
     def max_pool(self, x, k, pad, stride):
         """gpu_ops/MaxPool.py:119 (compute), :146 (gradient)."""
@@ -353,32 +358,38 @@ class Tape(object):
     def add(self, a, b):
         """gpu_ops/AddElewise.py:54 (compute), :95 (gradient: both inputs receive the output gradient)."""
         assert a.shape == b.shape, (a.shape, b.shape)
-        y = self.b.add(a.value, b.value, a.shape)
+
+        def fwd():
+            return self.b.add(a.value, b.value, a.shape)
 
         def back(g):
             self._acc(a, g)
             self._acc(b, g)
-        return self._out(y, a.shape, [a, b], back, saved=[])
+        return self._out(fwd(), a.shape, [a, b], back, saved=[], redo=fwd)
 
     def scale(self, a, c):
         """gpu_ops/MultiplyConst.py:45 (compute), :63 (gradient: the output gradient times the constant)."""
-        y = self.b.mul_const(a.value, c, a.shape)
-        return self._out(y, a.shape, [a], lambda g: self._acc(a, self.b.mul_const(g, c, a.shape)), saved=[])
+        def fwd():
+            return self.b.mul_const(a.value, c, a.shape)
+        return self._out(fwd(), a.shape, [a], lambda g: self._acc(a, self.b.mul_const(g, c, a.shape)), saved=[], redo=fwd)
 
     def shift(self, a, c):
-        y = self.b.add_const(a.value, c, a.shape)
-        return self._out(y, a.shape, [a], lambda g: self._acc(a, g), saved=[])
+        def fwd():
+            return self.b.add_const(a.value, c, a.shape)
+        return self._out(fwd(), a.shape, [a], lambda g: self._acc(a, g), saved=[], redo=fwd)
 
     def mul(self, a, b):
         """gpu_ops/MultiplyElewise.py (compute; gradient: each input receives the other times the
         output gradient)."""
         assert a.shape == b.shape, (a.shape, b.shape)
-        y = self.b.mul(a.value, b.value, a.shape)
+
+        def fwd():
+            return self.b.mul(a.value, b.value, a.shape)
 
         def back(g):
             self._acc(a, self.b.mul(b.value, g, a.shape))
             self._acc(b, self.b.mul(a.value, g, a.shape))
-        return self._out(y, a.shape, [a, b], back)
+        return self._out(fwd(), a.shape, [a, b], back, redo=fwd)
 
     def sigmoid(self, x):
         """gpu_ops/Sigmoid.py:58-61: gradient s * (1 + -1 * s) * g, built from the same elementwise
@@ -418,22 +429,25 @@ class Tape(object):
             known = _prod([s for s in shape if s != -1])
             shape[shape.index(-1)] = _prod(a.shape) // known
         shape = tuple(shape)
-        y = self.b.reshape(a.value, shape)
-        return self._out(y, shape, [a], lambda g: self._acc(a, self.b.reshape(g, a.shape)), saved=[])
+        def fwd():
+            return self.b.reshape(a.value, shape)
+        return self._out(fwd(), shape, [a], lambda g: self._acc(a, self.b.reshape(g, a.shape)), saved=[], redo=fwd)
 
     def concat(self, a, b, axis):
         """gpu_ops/Concat.py:47-60 (compute), :65 (gradient: two concat_gradient nodes, idx 0 and 1)."""
         shape = list(a.shape)
         shape[axis] += b.shape[axis]
         shape = tuple(shape)
-        y = self.b.concat(a.value, b.value, shape, axis)
+        def fwd():
+            return self.b.concat(a.value, b.value, shape, axis)
+        y = fwd()
 
         def back(g):
             if a.needs_grad:
                 self._acc(a, self.b.concat_grad(g, a.shape, axis, 0))
             if b.needs_grad:
                 self._acc(b, self.b.concat_grad(g, b.shape, axis, 1))
-        return self._out(y, shape, [a, b], back, saved=[])
+        return self._out(y, shape, [a, b], back, saved=[], redo=fwd)
 
     def matmul(self, a, b, trans_a=False, trans_b=False):
         """gpu_ops/MatrixMult.py:57-86 (compute), :95-124 (gradient)."""
@@ -482,20 +496,23 @@ class Tape(object):
     def add_bias(self, x, bias):
         """x [rows, cols] + broadcast(bias [cols]) (gpu_ops/Broadcast.py:45-59, gradient :65 =
         reduce_sum_axis_zero)."""
-        bb = self.b.broadcast_to(bias.value, x.shape)
-        y = self.b.add(x.value, bb, x.shape)
+        def fwd():
+            return self.b.add(x.value, self.b.broadcast_to(bias.value, x.shape), x.shape)
 
         def back(g):
             self._acc(x, g)
             if bias.needs_grad:
                 self._acc(bias, self.b.reduce_sum_axis_zero(g, bias.shape))
-        return self._out(y, x.shape, [x, bias], back, saved=[])
+        return self._out(fwd(), x.shape, [x, bias], back, saved=[], redo=fwd)
 
     def broadcast_like(self, x, shape):
         """gpu_ops/BroadcastTF.py:46-58 (numpy alignment from the right); gradient = reduce_sum
         over the broadcast axes (gpu_ops/BroadcastShape.py:61)."""
         shape = tuple(shape)
-        y = self.b.broadcast_shape(x.value, shape)
+
+        def fwd():
+            return self.b.broadcast_shape(x.value, shape)
+        y = fwd()
         diff = len(shape) - len(x.shape)
         axes = [d for d in range(len(shape)) if d < diff or (x.shape[d - diff] == 1 and shape[d] != 1)]
 
@@ -504,21 +521,24 @@ class Tape(object):
                 self._acc(x, self.b.reduce_sum(g, axes, x.shape))
             else:
                 self._acc(x, g)
-        return self._out(y, shape, [x], back, saved=[])
+        return self._out(y, shape, [x], back, saved=[], redo=fwd)
 
     def transpose(self, x, perm):
         """gpu_ops/Transpose.py:44-58 (compute), :60 (gradient: the inverse permutation)."""
         perm = list(perm)
         ys = tuple(x.shape[p] for p in perm)
-        y = self.b.transpose(x.value, perm, ys)
+        def fwd():
+            return self.b.transpose(x.value, perm, ys)
         inv = [0] * len(perm)
         for i, p in enumerate(perm):
             inv[p] = i
-        return self._out(y, ys, [x], lambda g: self._acc(x, self.b.transpose(g, inv, x.shape)), saved=[])
+        return self._out(fwd(), ys, [x], lambda g: self._acc(x, self.b.transpose(g, inv, x.shape)), saved=[], redo=fwd)
 
     def where(self, cond, a, b):
         """gpu_ops/Where.py:41-48 (compute), :50-55 (gradient: where(cond, g, 0) and where(cond, 0, g))."""
-        y = self.b.where(cond.value, a.value, b.value, a.shape)
+        def fwd():
+            return self.b.where(cond.value, a.value, b.value, a.shape)
+        y = fwd()
 
         def back(g):
             z = self.b.zeros(a.shape)
@@ -526,7 +546,7 @@ class Tape(object):
                 self._acc(a, self.b.where(cond.value, g, z, a.shape))
             if b.needs_grad:
                 self._acc(b, self.b.where(cond.value, z, g, a.shape))
-        return self._out(y, a.shape, [cond, a, b], back, saved=[cond])
+        return self._out(y, a.shape, [cond, a, b], back, saved=[cond], redo=fwd)
 
     def one_hot(self, ids, classes):
         """gpu_ops/OneHot.py:44-46; no gradient."""
@@ -555,8 +575,8 @@ class Tape(object):
         loss.grad = True
         for node in reversed(self._nodes):
             v = node.out
+            self._before_backward(node)
             if node.back is not None and v.grad is not None:
-                self._before_backward(node)
                 node.back(v.grad)
                 if v is not loss:
                     v.grad = None      # interior gradients are dropped as soon as they are consumed

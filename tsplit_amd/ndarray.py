@@ -121,6 +121,9 @@ class NDArray(object):
     def merge(self):
         self.splitted = False
         self.in_gpu = True
+        # the views refer to this array and this array lists them: dropping the list breaks that cycle, so
+        # the array is freed when its last outside reference goes and not when the collector next runs
+        self.sTensor = []
 
     # ---- drop / re-acquire the data pointer, keeping the struct ----
     def delete_itself(self):

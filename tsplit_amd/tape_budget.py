@@ -10,23 +10,29 @@ graphs of the reference's examples:
   record(build)       runs the graph builder without arithmetic and returns, per operator call, the
                       size of its output, what it read, and what its backward operators read again;
   plan(record, ...)   replays the executor's schedule on those sizes and, while the replayed peak
-                      exceeds the budget, sends away the largest value that sits idle at the moment
-                      of the peak (greedy, as planner.py does for layer lists);
+                      exceeds the budget, takes the largest value that sits idle at the moment of the
+                      peak off the device (greedy, as planner.py does for layer lists): the output of
+                      an operator that is cheap to run again (BatchNorm, Relu, add, scale, concat: one
+                      to three passes over HBM) is dropped and computed again when the backward sweep
+                      needs it, any other value is sent to pinned host memory;
   BudgetedTape        a Tape that follows the plan: values without a later reader are dropped as the
-                      forward sweep passes their last use, planned values go to pinned host memory
-                      behind it and are fetched `lead` operators ahead of the backward sweep, and
-                      every value is dropped after the last backward operator that reads it.
+                      forward sweep passes their last use, values to be computed again likewise,
+                      values sent away go to pinned host memory behind the sweep and are fetched `lead`
+                      operators ahead of the backward sweep, and every value is dropped after the last
+                      backward operator (or recomputation) that reads it.
 
 Schedule (replayed byte for byte by `replay`, measured against the pool by the tests):
   forward  of operator t : its output is allocated; then every value whose last reader in the forward
                            sweep was t and which no backward operator reads is released; a planned
                            value whose last forward reader was t starts leaving, and is released
                            after operator t + 1 has been issued (the host waits for the copy then);
-  backward of operator j : the planned values first read by operators j - lead .. j (in the order of
-                           the sweep) that are still away are allocated and start coming back; the
-                           host waits for those operator j reads; j's backward operators allocate
-                           the gradients of its inputs; then j's output gradient and every value
-                           whose last backward reader was j are released.
+  backward of operator j : the values sent away that operators j - lead .. j need first (in the order
+                           of the sweep) are allocated and start coming back; the host waits for
+                           those operator j reads; dropped values operator j needs first are computed
+                           again, producers before consumers (a Relu output from the BatchNorm output
+                           from the kept convolution output), which gives the same bits; j's backward
+                           operators allocate the gradients of its inputs; then j's output gradient
+                           and every value whose last reader was j are released.
 Ordering between the streams goes through the host (DLEventSync), as in the reference: before a
 value leaves, the host waits for the operator that last read it; before memory for a returning value
 is taken from the pool, the host waits for the compute stream, so that no kernel still in flight
@@ -53,9 +59,10 @@ def _bytes(shape):
 
 class OpRecord(object):
     """One operator call of a recorded graph.  Indices refer to operator calls (-1: a leaf)."""
-    __slots__ = ["bytes", "inputs", "saved", "has_backward", "grad_inputs", "leaf_grad_bytes"]
+    __slots__ = ["bytes", "inputs", "saved", "has_backward", "grad_inputs", "leaf_grad_bytes", "cheap"]
 
-    def __init__(self, nbytes, inputs, saved, has_backward, grad_inputs, leaf_grad_bytes):
+    def __init__(self, nbytes, inputs, saved, has_backward, grad_inputs, leaf_grad_bytes, cheap=False):
+        self.cheap = cheap                 # the operator can compute its output again from its inputs
         self.bytes = nbytes                # of the output
         self.inputs = inputs               # producers of the values the forward operator reads
         self.saved = saved                 # producers of the values the backward operators read
@@ -98,7 +105,7 @@ def record(build, inputs):
         ops.append(OpRecord(_bytes(node.out.shape), [v.node for v in node.inputs], [v.node for v in node.saved],
                             node.back is not None,
                             [v.node for v in node.inputs if v.node >= 0 and v.needs_grad] if node.back is not None else [],
-                            leaf_grad))
+                            leaf_grad, node.redo is not None))
     leaves = sum(_bytes(s) for s in inputs.values()) + sum(_bytes(v.shape) for v in b.vars.values())
     leaves += sum(_bytes(shape) for _, shape in b._consts.values())
     assert loss.node == len(ops) - 1
@@ -106,8 +113,9 @@ def record(build, inputs):
 
 
 class TapePlan(object):
-    def __init__(self, away, lead, peak_bytes, free_peak_bytes, budget_bytes, leaves_bytes):
+    def __init__(self, away, lead, peak_bytes, free_peak_bytes, budget_bytes, leaves_bytes, redo=()):
         self.away = frozenset(away)          # operator calls whose output leaves the device between the sweeps
+        self.redo = frozenset(redo)          # operator calls whose output is dropped and computed again
         self.lead = lead
         self.peak_bytes = peak_bytes
         self.free_peak_bytes = free_peak_bytes     # replayed peak with nothing sent away
@@ -116,7 +124,7 @@ class TapePlan(object):
 
     def describe(self):
         gib = float(1 << 30)
-        return {"away": len(self.away), "lead": self.lead, "peak_GiB": self.peak_bytes / gib,
+        return {"away": len(self.away), "recomputed": len(self.redo), "lead": self.lead, "peak_GiB": self.peak_bytes / gib,
                 "unplanned_peak_GiB": self.free_peak_bytes / gib,
                 "budget_GiB": None if self.budget_bytes is None else self.budget_bytes / gib}
 
@@ -137,15 +145,33 @@ def _uses(ops):
     return last_fwd, bwd
 
 
-def replay(ops, leaves_bytes, away=(), lead=3):
-    """Peak of the executor's schedule with `away` sent to the host.  -> (peak bytes, moment of the
-    peak, values resident and idle at that moment: list of (bytes, operator)).  A moment is an
-    operator index for the forward sweep and 2n - 1 - j for the backward of operator j."""
-    n = len(ops)
-    away = set(away)
+def _needs(ops, redo):
+    """When, in the backward sweep, every value must be on the device: need[i] lists the operators
+    during whose backward step value i is read - by their backward operators, or by the recomputation
+    of a dropped value, which happens in the step of that value's first reader.  The sweep descends,
+    so max(need[i]) is the first moment and min(need[i]) the last."""
     last_fwd, bwd = _uses(ops)
-    first_bwd = [max(r) if r else -1 for r in bwd]       # the backward sweep descends: read first by the largest index
-    last_bwd = [min(r) if r else -1 for r in bwd]
+    need = [list(r) for r in bwd]
+    for c in sorted(redo, reverse=True):      # consumers before producers
+        if not need[c]:
+            continue                          # nobody reads it again: it is simply dropped
+        t = max(need[c])
+        for u in set(ops[c].inputs):
+            if u >= 0:
+                need[u].append(t)
+    return last_fwd, need
+
+
+def replay(ops, leaves_bytes, away=(), lead=3, redo=()):
+    """Peak of the executor's schedule with `away` sent to the host and `redo` dropped and computed
+    again.  -> (peak bytes, moment of the peak, values resident and idle at that moment: list of
+    (bytes, operator)).  A moment is an operator index for the forward sweep and 2n - 1 - j for the
+    backward step of operator j."""
+    n = len(ops)
+    away, redo = set(away), set(redo)
+    last_fwd, need = _needs(ops, redo)
+    first = [max(r) if r else -1 for r in need]
+    last = [min(r) if r else -1 for r in need]
     live = leaves_bytes
     resident = {}                                       # operator -> bytes of its value on the device
     peak, peak_at, peak_set = live, -1, []
@@ -171,7 +197,7 @@ def replay(ops, leaves_bytes, away=(), lead=3):
             live -= resident.pop(i)
         leaving = []
         for i in by_last_fwd[t]:
-            if not bwd[i]:
+            if not need[i] or i in redo:
                 if i != n - 1:                          # the loss stays for the caller
                     live -= resident.pop(i)
             elif i in away:
@@ -182,21 +208,30 @@ def replay(ops, leaves_bytes, away=(), lead=3):
     grads = {}                                          # operator -> bytes of the gradient of its output
     fetch_at = collections.defaultdict(list)
     for i in away:
-        if bwd[i]:
-            fetch_at[min(n - 1, first_bwd[i] + lead)].append(i)
-    by_last_bwd = collections.defaultdict(list)
+        if need[i]:
+            fetch_at[min(n - 1, first[i] + lead)].append(i)
+    redo_at = collections.defaultdict(list)
+    for i in redo:
+        if need[i]:
+            redo_at[first[i]].append(i)
+    by_last = collections.defaultdict(list)
     for i in range(n):
-        if bwd[i]:
-            by_last_bwd[last_bwd[i]].append(i)
-    param_grads = 0
+        if need[i]:
+            by_last[last[i]].append(i)
     for j in range(n - 1, -1, -1):
         op = ops[j]
         moment = 2 * n - 1 - j
-        for i in sorted(fetch_at[j], key=lambda i: -first_bwd[i]):
+        for i in sorted(fetch_at[j], key=lambda i: -first[i]):
             if i not in resident:
                 live += ops[i].bytes
                 resident[i] = ops[i].bytes
         busy = set(i for i in op.saved if i >= 0)
+        for i in sorted(redo_at[j]):                    # producers before consumers
+            busy |= set(u for u in ops[i].inputs if u >= 0) | {i}
+            if i not in resident:
+                live += ops[i].bytes
+                resident[i] = ops[i].bytes
+                note(moment)
         note(moment)
         if op.has_backward and (j == n - 1 or j in grads):
             # every input that takes a gradient gets a new array; adding to an earlier one holds the
@@ -212,43 +247,57 @@ def replay(ops, leaves_bytes, away=(), lead=3):
                     grads[i] = extra
                 note(moment)
             live += op.leaf_grad_bytes
-            param_grads += op.leaf_grad_bytes
             note(moment)
         if j in grads:
             live -= grads.pop(j)
-        for i in by_last_bwd[j]:
+        for i in by_last[j]:
             if i in resident:
                 live -= resident.pop(i)
     return peak, peak_at, peak_set
 
 
-def plan(ops, leaves_bytes, budget_bytes, lead=3, min_bytes=1 << 20):
-    """-> TapePlan.  Raises ValueError when the budget cannot be met by sending values away (a single
-    operator's operands, results and gradients do not fit)."""
+def plan(ops, leaves_bytes, budget_bytes, lead=3, min_bytes=1 << 20, recompute=True):
+    """-> TapePlan.  Raises ValueError when the budget cannot be met (a single operator's operands,
+    results and gradients do not fit with everything idle off the device)."""
     free_peak, _, _ = replay(ops, leaves_bytes, (), lead)
-    away = set()
+    away, redo, banned = set(), set(), set()
     n = len(ops)
-    last_fwd, bwd = _uses(ops)
     if budget_bytes is not None:
         while True:
-            peak, at, idle = replay(ops, leaves_bytes, away, lead)
+            peak, at, idle = replay(ops, leaves_bytes, away, lead, redo)
             if peak <= budget_bytes:
                 break
-            # values that could be away at that moment: read again only in the backward sweep, after a gap
+            last_fwd, need = _needs(ops, redo)
+            # values that could be off the device at that moment: read again only later in the backward
+            # sweep, after a gap
             cands = []
             for b, i in idle:
-                if i in away or not bwd[i] or b < min_bytes:
+                if i in away or i in redo or not need[i] or b < min_bytes:
                     continue
-                gone_from = last_fwd[i] + 2
-                back_at = 2 * n - 1 - min(n - 1, max(bwd[i]) + lead)
+                gone_from = last_fwd[i] + 1
+                cheap = recompute and ops[i].cheap and (i, "redo") not in banned
+                back_at = 2 * n - 1 - (max(need[i]) if cheap else min(n - 1, max(need[i]) + lead))
+                if not cheap:
+                    gone_from += 1                      # a copy takes one more operator to leave
+                    if (i, "away") in banned:
+                        continue
                 if gone_from <= at < back_at:
-                    cands.append((b, i))
+                    cands.append((b, i, cheap))
             if not cands:
                 raise ValueError("a step does not fit %.2f GiB: %.2f GiB are needed at once with everything "
-                                 "idle sent away" % (budget_bytes / float(1 << 30), peak / float(1 << 30)))
-            away.add(max(cands)[1])
-    peak, _, _ = replay(ops, leaves_bytes, away, lead)
-    return TapePlan(away, lead, peak, free_peak, budget_bytes, leaves_bytes)
+                                 "idle off the device" % (budget_bytes / float(1 << 30), peak / float(1 << 30)))
+            # a value that can be computed again goes before one that has to travel, the larger first
+            b, i, cheap = max(cands, key=lambda c: (c[2], c[0], c[1]))
+            trial_away, trial_redo = (away, redo | {i}) if cheap else (away | {i}, redo)
+            new_peak, new_at, _ = replay(ops, leaves_bytes, trial_away, lead, trial_redo)
+            if new_peak > peak or (new_peak == peak and new_at == at):
+                # keeping this value's inputs for the recomputation (or the move itself) does not help
+                # here: try the other way, then other values
+                banned.add((i, "redo" if cheap else "away"))
+                continue
+            away, redo = set(trial_away), set(trial_redo)
+    peak, _, _ = replay(ops, leaves_bytes, away, lead, redo)
+    return TapePlan(away, lead, peak, free_peak, budget_bytes, leaves_bytes, redo)
 
 
 class BudgetedTape(graph.Tape):
@@ -274,23 +323,28 @@ class BudgetedTape(graph.Tape):
         self.plan, self.ops, self.state = tape_plan, ops, state
         self.track_pool = track_pool
         n = len(ops)
-        self.last_fwd, self.bwd = _uses(ops)
-        self.first_bwd = [max(r) if r else -1 for r in self.bwd]
-        self.last_bwd = [min(r) if r else -1 for r in self.bwd]
+        self.last_fwd, self.need = _needs(ops, tape_plan.redo)
+        self.first = [max(r) if r else -1 for r in self.need]
+        self.last = [min(r) if r else -1 for r in self.need]
         self.by_last_fwd = collections.defaultdict(list)
         for i in range(n):
             self.by_last_fwd[self.last_fwd[i]].append(i)
-        self.by_last_bwd = collections.defaultdict(list)
+        self.by_last = collections.defaultdict(list)
         for i in range(n):
-            if self.bwd[i]:
-                self.by_last_bwd[self.last_bwd[i]].append(i)
+            if self.need[i]:
+                self.by_last[self.last[i]].append(i)
         self.fetch_at = collections.defaultdict(list)
         for i in tape_plan.away:
-            if self.bwd[i]:
-                self.fetch_at[min(n - 1, self.first_bwd[i] + tape_plan.lead)].append(i)
+            if self.need[i]:
+                self.fetch_at[min(n - 1, self.first[i] + tape_plan.lead)].append(i)
+        self.redo_at = collections.defaultdict(list)
+        for i in tape_plan.redo:
+            if self.need[i]:
+                self.redo_at[self.first[i]].append(i)
         self.leaving = []            # (operator, device array, copy-done event), released after the next operator
         self.arriving = {}           # operator -> copy-done event
-        self.gone = set()
+        self.gone = set()            # values in host memory only
+        self.recomputed = 0
 
     # ---- helpers
     def _compute_stream(self):
@@ -326,9 +380,9 @@ class BudgetedTape(graph.Tape):
         n = len(self.ops)
         for i in self.by_last_fwd[t]:
             v = self._var(i)
-            if not self.bwd[i]:
+            if not self.need[i] or i in self.plan.redo:
                 if i != n - 1:
-                    v.value = None
+                    v.value = None       # nobody reads it again, or it will be computed again
             elif i in self.plan.away:
                 # the operator that read it last has been issued: wait for it, then copy out
                 self._host_wait_for_compute()
@@ -353,20 +407,34 @@ class BudgetedTape(graph.Tape):
         self.arriving[i] = ev
         self.gone.discard(i)
 
+    def _ensure(self, i):
+        """Value i is on the device and complete when this returns."""
+        if i in self.gone:                     # (a value the plan fetches later than this reader needs it)
+            self._fetch(i)
+        ev = self.arriving.pop(i, None)
+        if ev is not None:
+            ev.sync()
+            self.state.host_waits += 1
+        if self._var(i).value is None and i in self.plan.redo:
+            node = self._nodes[i]
+            for u in node.inputs:
+                if u.node >= 0:
+                    self._ensure(u.node)
+            node.out.value = node.redo()
+            self.recomputed += 1
+
     def _before_backward(self, node):
-        for i in (s.node for s in node.saved):
-            if i >= 0 and i in self.gone:      # (a value the plan fetches later than its reader needs it)
-                self._fetch(i)
-            ev = self.arriving.pop(i, None) if i >= 0 else None
-            if ev is not None:
-                ev.sync()
-                self.state.host_waits += 1
+        for i in sorted(self.redo_at[node.index]):      # producers before consumers
+            self._ensure(i)
+        for s in node.saved:
+            if s.node >= 0:
+                self._ensure(s.node)
 
     def backward(self, loss):
         self._release_leaving()
         n = len(self.ops)
         assert len(self._nodes) == n, "the graph differs from the recorded one"
-        for i in sorted(self.fetch_at[n - 1], key=lambda i: -self.first_bwd[i]):     # planned for the first operator
+        for i in sorted(self.fetch_at[n - 1], key=lambda i: -self.first[i]):     # planned for the first operator
             if i in self.gone:
                 self._fetch(i)
         graph.Tape.backward(self, loss)
@@ -375,10 +443,10 @@ class BudgetedTape(graph.Tape):
         # the sweep reaches operator j - 1 next: issue what the plan fetches there before its operators
         j = node.index
         self._note_pool()
-        for i in self.by_last_bwd[j]:
+        for i in self.by_last[j]:
             self._var(i).value = None
         if j > 0:
-            for i in sorted(self.fetch_at[j - 1], key=lambda i: -self.first_bwd[i]):
+            for i in sorted(self.fetch_at[j - 1], key=lambda i: -self.first[i]):
                 if i in self.gone:
                     self._fetch(i)
 
@@ -387,12 +455,13 @@ class BudgetedRun(object):
     """Trains a graph step after step under a plan: `build(tape, binder, cache)` as for record();
     parameters come from `store` (workloads.ParamStore), inputs are numpy arrays uploaded once."""
 
-    def __init__(self, build, inputs, store, budget_bytes, ctx=None, lead=3, track_pool=False, min_bytes=1 << 20):
+    def __init__(self, build, inputs, store, budget_bytes, ctx=None, lead=3, track_pool=False, min_bytes=1 << 20,
+                 recompute=True):
         from . import stream, workloads
         self.ctx = ctx or ndarray.gpu(0)
         self.build = build
         self.ops, self.leaves_bytes = record(build, {k: np.shape(v) for k, v in inputs.items()})
-        self.plan = plan(self.ops, self.leaves_bytes, budget_bytes, lead, min_bytes)
+        self.plan = plan(self.ops, self.leaves_bytes, budget_bytes, lead, min_bytes, recompute)
         self.stream = stream.create_stream_handle(self.ctx)
         self.backend = graph.GpuBackend(self.ctx, self.stream)
         self.state = BudgetedTape.make_state(self.ctx)
@@ -422,7 +491,8 @@ class BudgetedRun(object):
         self.backend.sync()
 
 
-def max_batch(build_for, input_shapes_for, budget_bytes, planned=True, lead=3, limit=1 << 12, min_bytes=1 << 20):
+def max_batch(build_for, input_shapes_for, budget_bytes, planned=True, lead=3, limit=1 << 12, min_bytes=1 << 20,
+              recompute=True):
     """Largest batch whose step fits `budget_bytes`: with `planned` the planner may send values to the
     host, without it the replayed peak of the plain schedule must fit.  build_for(batch) -> builder,
     input_shapes_for(batch) -> name -> shape.  The counterpart of the reference's batch-size sweeps per
@@ -432,7 +502,7 @@ def max_batch(build_for, input_shapes_for, budget_bytes, planned=True, lead=3, l
         if any(op.bytes >= (1 << 33) for op in ops):      # tensors are limited to 2^31 elements
             return None
         try:
-            p = plan(ops, leaves, budget_bytes if planned else None, lead, min_bytes)
+            p = plan(ops, leaves, budget_bytes if planned else None, lead, min_bytes, recompute)
         except ValueError:
             return None
         return p if p.peak_bytes <= budget_bytes else None

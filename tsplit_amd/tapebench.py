@@ -1,13 +1,13 @@
 """The branched example networks trained under device-memory budgets (one MI355X): the budgeted tape
 executor of tape_budget.py on ResNet-50 (batch 64), Inception-v4 (batch 32) and the Transformer (batch 32).
 
-    python -m tsplit_amd.tapebench --net resnet50|inception_v4|transformer [--fractions 0,0.75,0.5,0.35] [--steps 4] [--warmup 1]
-    python -m tsplit_amd.tapebench --net resnet50|inception_v4 --max-batch [--budgets 8,16]
+    python -m tsplit_amd.tapebench --net resnet50|inception_v4|transformer [--fractions 0,0.75,0.5,0.35] [--steps 4] [--warmup 1] [--no-recompute]
+    python -m tsplit_amd.tapebench --net resnet50|inception_v4 --max-batch [--budgets 8,16] [--no-recompute]
 
 For every fraction f (0 = no limit) the budget is the leaves (parameters, their gradients' room is part
 of the replay, inputs, constants) plus f times what the operators' values and gradients take at the
-unplanned peak; the planner picks what leaves for pinned host memory, the executor trains on synthetic
-data.  One JSON object per budget: samples/s, the pool's measured peak over its level before the run,
+unplanned peak; the planner picks what is dropped and computed again and what leaves for pinned host memory
+(only the latter with --no-recompute), the executor trains on synthetic data.  One JSON object per budget: samples/s, the pool's measured peak over its level before the run,
 the replayed peak, values sent away, host waits per step.  With --max-batch the question is turned
 around, as in the reference's batch-size sweeps per policy (examples/imagenet_resnet.py:139-154): for
 every budget in GiB, the largest batch that trains with everything resident and the largest one the
@@ -58,11 +58,11 @@ def _net(name, batch=None):
     raise ValueError(name)
 
 
-def _measure(build, inputs, budget, steps, warmup, lr):
+def _measure(build, inputs, budget, steps, warmup, lr, recompute=True):
     from . import tape_budget as tb, workloads
     from .gpu_memory_manager import pool_state
     base = pool_state().used
-    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(123), budget, track_pool=True)
+    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(123), budget, track_pool=True, recompute=recompute)
     for _ in range(warmup):
         run.step(lr)
     run.sync()
@@ -77,7 +77,8 @@ def _measure(build, inputs, budget, steps, warmup, lr):
     gib = float(1 << 30)
     return {"samples_per_s": n / dt, "ms_per_step": dt * 1e3, "measured_peak_GiB": (run.state.peak_used - base) / gib,
             "planned_peak_GiB": d["peak_GiB"], "unplanned_peak_GiB": d["unplanned_peak_GiB"], "values_away": d["away"],
-            "away_GiB": sum(run.ops[i].bytes for i in run.plan.away) / gib,
+            "away_GiB": sum(run.ops[i].bytes for i in run.plan.away) / gib, "values_recomputed": len(run.plan.redo),
+            "recomputed_GiB": sum(run.ops[i].bytes for i in run.plan.redo) / gib,
             "host_waits_per_step": (run.state.host_waits - waits0) / steps, "loss": float(loss.value.asnumpy()[0])}
 
 
@@ -91,6 +92,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--lr", type=float, default=1e-4)
     ap.add_argument("--max-batch", action="store_true")
+    ap.add_argument("--no-recompute", action="store_true", help="the plan may only send values to the host")
     a = ap.parse_args()
     from . import tape_budget as tb
     build_for, inputs_for, default_batch, desc = _net(a.net)
@@ -104,10 +106,12 @@ def main():
             def shapes_for(n):
                 return {k: (n,) + tail for k, tail in one.items()}
             resident, _ = tb.max_batch(build_for, shapes_for, budget, planned=False)
-            planned, p = tb.max_batch(build_for, shapes_for, budget, planned=True)
-            row = {"net": a.net, "workload": desc, "budget_GiB": b, "max_batch_resident": resident, "max_batch_planned": planned}
+            planned, p = tb.max_batch(build_for, shapes_for, budget, planned=True, recompute=not a.no_recompute)
+            row = {"net": a.net, "workload": desc, "budget_GiB": b, "recompute": not a.no_recompute,
+                   "max_batch_resident": resident, "max_batch_planned": planned}
             if p is not None:
-                row.update(_measure(build_for(planned), inputs_for(planned, rng), budget, max(1, a.steps // 2), 1, a.lr))
+                row.update(_measure(build_for(planned), inputs_for(planned, rng), budget, max(1, a.steps // 2), 1, a.lr,
+                                    not a.no_recompute))
             print(json.dumps(row), flush=True)
         return
     n = a.batch or default_batch
@@ -118,9 +122,9 @@ def main():
     for f in [float(v) for v in a.fractions.split(",")]:
         budget = None if f == 0 else leaves + int((free_peak - leaves) * f)
         row = {"net": a.net, "workload": desc + ", batch %d" % n, "fraction": f,
-               "budget_GiB": None if budget is None else budget / float(1 << 30)}
+               "budget_GiB": None if budget is None else budget / float(1 << 30), "recompute": not a.no_recompute}
         try:
-            row.update(_measure(build, inputs, budget, a.steps, a.warmup, a.lr))
+            row.update(_measure(build, inputs, budget, a.steps, a.warmup, a.lr, not a.no_recompute))
         except ValueError as e:
             row["error"] = str(e)
         print(json.dumps(row), flush=True)
