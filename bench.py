@@ -33,6 +33,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS_FP32_MFMA = 157.3
+PEAK_TFLOPS_BF16_MFMA = 2500.0   # dense bf16 matrix peak
 PEAK_HBM_GBS = 8000.0
 # Kernel names (as rocprofv3 prints them) behind the operator classes that can be the step's largest
 # single kernel; their HBM bytes per launch are read from the counter summary under profiles/.
@@ -180,6 +181,10 @@ def main():
                     help="run every BatchNorm+Relu pair through the fused symbols, let every convolution hand its "
                          "output's statistics to the BatchNorm behind it and update all parameters in one launch "
                          "(symbols outside the reference's ABI)")
+    ap.add_argument("--split-bf16", action="store_true",
+                    help="opt-in, outside the reference's ABI and outside the default path's fp32 matrix instructions: the "
+                         "Winograd GEMMs of layers with more than 64 channels on both sides take each fp32 product as six "
+                         "bf16 x bf16 products of the operands' exact three-term splits, accumulated in fp32")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build is single-GPU by design (no collectives, no sharding); run with --gpus 1. "
@@ -192,6 +197,7 @@ def main():
     if a.no_split:
         split = {}
     timer = None if a.no_events else EventTimer(ctx, chained=True)
+    L.split_bf16(a.split_bf16)
     t = trainer.Trainer(spec, params, x.shape, 1000, ctx, optimizer=("momentum", 1e-4, 0.9), split=split, timer=timer,
                         fuse_bn_relu=a.fused, conv_bn_stats=a.fused, multi_tensor_update=a.fused)
     gx, gy = ndarray.array(x, ctx), ndarray.array(labels, ctx)      # resident before timing
@@ -213,11 +219,13 @@ def main():
         "metric": "train samples/s, fp32, 1 MI355X; conv MFMA util %; BN/relu HBM GB/s",
         "value": a.batch * a.steps / dt, "unit": "samples/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": "f32 (Winograd GEMM products of wide layers as six bf16 x bf16 terms of exact operand splits, fp32 accumulation)"
+                 if a.split_bf16 else "f32", "data": "synthetic",
         "config": {"workload": "VGG-16 training step (fwd+bwd+momentum SGD), fp32 NCHW, batch %d, 3x224x224, "
                                "1000 classes, He init, %s%s" % (a.batch, "4 batch micro-tensors on the 4 largest conv layers"
                                                                 if split else "no micro-tensor split",
-                                                                ", BatchNorm+Relu pairs fused, BatchNorm statistics from the convolutions' epilogues, one optimizer launch" if a.fused else ""),
+                                                                (", BatchNorm+Relu pairs fused, BatchNorm statistics from the convolutions' epilogues, one optimizer launch" if a.fused else "")
+                                                                + (", split-bf16 products in the wide layers' Winograd GEMMs" if a.split_bf16 else "")),
                    "global_batch": a.batch, "final_loss": loss},
     }
     if timer:
@@ -257,15 +265,30 @@ def main():
                     kernels[tag]["hbm_frac"] = kernels[tag]["hbm_achieved_gbs"] / PEAK_HBM_GBS
                     kernels[tag]["note"] = ("the forward / data-gradient GEMMs of the layers that produce 64 channels (64 x 256 "
                                             "tiles) inside the *_winograd calls; executed FLOP, and algorithmic bytes for hbm_*")
+        # the same GEMMs with split-bf16 products: six bf16 matrix instructions per fp32-equivalent product, so
+        # the executed work is six times the GEMM's FLOP and the peak is the bf16 matrix peak
+        for tag, kind in (("winograd_gemm_split_bf16", 3), ("winograd_filter_grad_gemm_split_bf16", 4)):
+            launches, ms, flop, nbytes = L.winograd_gemm_times(kind=kind)
+            if launches:
+                k[tag] = {"calls": launches, "ms_total": ms, "ms_avg": ms / launches, "work": 6 * flop,
+                          "work_per_call": 6 * flop / launches, "rate": 6 * flop / (ms * 1e-3) / 1e12, "unit": "flop",
+                          "peak": PEAK_TFLOPS_BF16_MFMA}
+                kernels[tag] = {"calls_per_step": launches / a.steps, "ms_per_step": ms / a.steps, "ms_avg": ms / launches,
+                                "achieved": k[tag]["rate"], "unit": "TFLOP/s", "frac": k[tag]["rate"] / PEAK_TFLOPS_BF16_MFMA,
+                                "fp32_equivalent_tflops": flop / (ms * 1e-3) / 1e12,
+                                "hbm_achieved_gbs": nbytes / (ms * 1e-3) / 1e9, "hbm_frac": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                "note": "one kernel inside the *_winograd calls above; executed bf16 FLOP (six products per "
+                                        "fp32-equivalent product) against the bf16 matrix peak, and algorithmic bytes for hbm_*"}
         L.winograd_gemm_timing(False)
         kernels = dict(sorted(kernels.items(), key=lambda kv: -kv[1]["ms_per_step"]))
         dom = next(tag for tag in kernels if not tag.endswith("_winograd"))
         dd = k[dom]
+        dom_peak = dd.get("peak", PEAK_TFLOPS_FP32_MFMA if dd["unit"] == "flop" else PEAK_HBM_GBS)
         out["roofline"] = {"kernel": dom, "bound": "mfma" if dd["unit"] == "flop" else "hbm",
-                           "achieved": dd["rate"], "peak": PEAK_TFLOPS_FP32_MFMA if dd["unit"] == "flop" else PEAK_HBM_GBS,
+                           "achieved": dd["rate"], "peak": dom_peak,
                            "unit": "TFLOP/s" if dd["unit"] == "flop" else "GB/s",
-                           "frac": dd["rate"] / (PEAK_TFLOPS_FP32_MFMA if dd["unit"] == "flop" else PEAK_HBM_GBS),
-                           "traffic": traffic_bytes_per_launch(dom) if split and a.batch == 64 and not a.fused else None,
+                           "frac": dd["rate"] / dom_peak,
+                           "traffic": traffic_bytes_per_launch(dom) if split and a.batch == 64 and not a.fused and not a.split_bf16 else None,
                            "per_launch": dd["work_per_call"], "ms_avg": dd["ms_avg"]}
         # Conv utilisation, two ways.  The thin first layer (Cin*kH*kW = 27) is timed in bytes because
         # HBM bounds it, so its FLOP (forward and filter gradient) are added to both counts.
@@ -287,7 +310,8 @@ def main():
             return 100.0 * flop / (ms * 1e-3) / 1e12 / PEAK_TFLOPS_FP32_MFMA if ms > 0 else None
         # executed: what the matrix pipe really multiplies (the Winograd calls count with their 36 GEMMs'
         # FLOP, the direct kernels with the algorithm's) over ALL conv time, transforms included
-        out["conv_mfma_util_executed_pct"] = pct(direct_flop + thin_flop + wino_exec_flop, conv_ms)
+        # (with split-bf16 products part of the work runs on the bf16 matrix instruction: no single peak applies)
+        out["conv_mfma_util_executed_pct"] = None if a.split_bf16 else pct(direct_flop + thin_flop + wino_exec_flop, conv_ms)
         # direct-equivalent: the direct algorithm's FLOP count of every layer over the same time; above 100
         # because the Winograd layers execute a quarter of it.  A throughput figure, not a utilisation
         out["conv_direct_equivalent_pct"] = pct(equivalent_flop, conv_ms)

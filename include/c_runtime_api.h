@@ -470,7 +470,8 @@ int TSplit_ConvTakesWinograd(int images, int in_channels, int out_channels, int 
  *      (not while the stream is being recorded into a graph); (0) stops and forgets them.
  *      TSplit_WinogradGemmTimes waits for the launches of kind `which` (0: forward and data
  *      gradient on 128 x 128 tiles, 1: filter gradient, 2: forward and data gradient of layers that
- *      produce at most 64 channels, which run on 64 x 256 tiles: one kernel per kind) and returns
+ *      produce at most 64 channels, which run on 64 x 256 tiles, 3 / 4: forward and data gradient /
+ *      filter gradient with split-bf16 products, see TSplit_SplitBf16: one kernel per kind) and returns
  *      their count, summed milliseconds and summed executed FLOP (2 * 36 * rows * columns * depth
  *      per launch);
  *      TSplit_WinogradGemmBytes returns their summed algorithmic bytes (both operands read once,
@@ -478,6 +479,17 @@ int TSplit_ConvTakesWinograd(int images, int in_channels, int out_channels, int 
 int TSplit_WinogradGemmTiming(int on);
 int TSplit_WinogradGemmTimes(int which, double *launches, double *ms, double *flop);
 int TSplit_WinogradGemmBytes(int which, double *bytes);
+
+/* ---- Split-bf16 products in the Winograd routine's GEMMs.  NO counterpart in the reference; opt-in,
+ *      off by default (every product of the default path is an fp32 matrix instruction).  With
+ *      TSplit_SplitBf16(1, NULL) the GEMMs of 3x3 layers with more than 64 channels on both sides
+ *      split each fp32 operand exactly into three bf16 terms, a = a1 + a2 + a3, and take a product as
+ *      the six bf16 x bf16 products a_i b_j with i + j <= 4, accumulated in fp32 by the bf16 matrix
+ *      instruction; what is left out is below 2^-23 of the product, the rounding of one fp32
+ *      multiplication.  Operands and results stay fp32 in memory.  Affects calls issued afterwards, on
+ *      every stream; `was` (may be NULL) receives the previous setting.  The environment variable
+ *      TSPLIT_SPLIT_BF16=1 turns it on from the start. ---- */
+int TSplit_SplitBf16(int on, int *was);
 
 /* ---- Recorded steps.  NO counterpart in the reference (every step there is issued call by
  *      call from Python); for steps made of thousands of tiny kernels (recurrent nets, small

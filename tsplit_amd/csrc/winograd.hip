@@ -21,13 +21,14 @@
 // differ from the directly summed one by a few 1e-6 of the output's magnitude.
 #include <algorithm>
 #include <cstdlib>
+#include <atomic>
 #include <mutex>
 #include <vector>
 
 #include "common.h"
 #include "mfma_gemm.h"
 #include "reduce.h"
-#include "wino_gemm.h"
+#include "wino_gemm_split.h"
 
 namespace tsplit {
 using namespace mg;
@@ -357,7 +358,8 @@ __global__ __launch_bounds__(256) void wino_filter_grad_kernel(const float *__re
 struct TimedLaunch {
   hipEvent_t begin, end;
   int which;       // 0: forward / data-gradient GEMMs on 128 x 128 tiles, 1: filter-gradient GEMMs,
-                   // 2: forward / data-gradient GEMMs on 64 x 256 tiles (at most 64 channels produced)
+                   // 2: forward / data-gradient GEMMs on 64 x 256 tiles (at most 64 channels produced),
+                   // 3 / 4: forward / data-gradient and filter-gradient GEMMs in split bf16
   double flop, bytes;
 };
 std::mutex g_timing_mu;
@@ -393,6 +395,19 @@ class GemmTiming {
   TimedLaunch t_{};
   bool on_ = false;
 };
+
+// Opt-in: the GEMMs of layers with more than 64 channels on both sides take their products in split bf16
+// (wino_gemm_split.h).  -1 until asked: the environment variable TSPLIT_SPLIT_BF16 then gives the first value.
+std::atomic<int> g_split_bf16{-1};
+inline bool split_bf16() {
+  int v = g_split_bf16.load(std::memory_order_relaxed);
+  if (v < 0) {
+    const char *e = std::getenv("TSPLIT_SPLIT_BF16");
+    v = e && std::atoi(e) != 0 ? 1 : 0;
+    g_split_bf16.store(v, std::memory_order_relaxed);
+  }
+  return v != 0;
+}
 
 // compute units of the current device and resident blocks of the GEMM kernel on each, asked once
 inline int compute_units() {
@@ -459,13 +474,16 @@ inline GradPlan plan_grad_gemm(int O, int C, int ld, int cus) {
 }
 
 // `here` ranges of p.kchunk cover p.ld; partial sum z = range * 36 + xi goes to p.out + z * rows * cols
-inline void launch_grad_gemm(const GradPlan &g, wg::GradProblem p, int here, hipStream_t st) {
+inline void launch_grad_gemm(const GradPlan &g, wg::GradProblem p, int here, hipStream_t st, bool split) {
   p.tm = g.tm;
   p.tn = g.tn;
   const int units = g.tm * g.tn * kXi * here;
   if (g.grid > 0) {
     const int grid = std::min(g.grid, (units + 7) / 8 * 8);
-    hipLaunchKernelGGL((wg::wino_grad_gemm_kernel<kGradBlocksPerCu>), dim3(grid), dim3(kThreads), 0, st, p, units);
+    if (split)
+      hipLaunchKernelGGL((wg::wino_grad_gemm_split_kernel<kGradBlocksPerCu>), dim3(grid), dim3(kThreads), 0, st, p, units);
+    else
+      hipLaunchKernelGGL((wg::wino_grad_gemm_kernel<kGradBlocksPerCu>), dim3(grid), dim3(kThreads), 0, st, p, units);
     return;
   }
   const TileGrid tg{g.tm, g.tn, units};
@@ -530,9 +548,13 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
       // every operand read once, the result written once
       const double flop = 2.0 * kXi * produced * static_cast<double>(gi.ld) * gathered;
       const double bytes = 4.0 * kXi * (static_cast<double>(produced) * gathered + static_cast<double>(gathered + produced) * gi.ld);
-      GemmTiming timed(st, produced <= 64 ? 2 : 0, flop, bytes);
-      wg::launch(wg::Problem{U, V, M, produced, gathered, gi.ld, (produced + 127) / 128, (gi.ld + 127) / 128}, st,
-                 compute_units());
+      const bool split = produced > 64 && (gathered & 7) == 0 && split_bf16();
+      GemmTiming timed(st, split ? 3 : produced <= 64 ? 2 : 0, flop, bytes);
+      const wg::Problem gemm{U, V, M, produced, gathered, gi.ld, 0, 0};
+      if (split)
+        wg::launch_split(gemm, st, compute_units());
+      else
+        wg::launch(gemm, st, compute_units());
     }
     const dim3 grid_out((go.tiles + 255) / 256, produced);
     float *yr = y + static_cast<int64_t>(first) * produced * H * W;
@@ -584,10 +606,11 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
       hipLaunchKernelGGL(wino_grad_kernel<false>, grid_y, dim3(256), 0, st, dyr, Y, gy);
     const int here = (gx.ld + kchunk - 1) / kchunk;
     {
-      GemmTiming timed(st, 1, 2.0 * kXi * O * static_cast<double>(gx.ld) * C,
+      const bool split = plan.grid > 0 && split_bf16();
+      GemmTiming timed(st, split ? 4 : 1, 2.0 * kXi * O * static_cast<double>(gx.ld) * C,
                        4.0 * kXi * (static_cast<double>(O) * C * here + static_cast<double>(O + C) * gx.ld));
       launch_grad_gemm(plan, wg::GradProblem{Y, V, part + static_cast<int64_t>(parts) * kXi * oc, O, C, gx.ld, kchunk, 0, 0},
-                       here, st);
+                       here, st, split);
     }
     parts += here;
   }
@@ -602,6 +625,15 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
 }
 
 }  // namespace tsplit
+
+// Switches the split-bf16 products of the Winograd routine's GEMMs on or off (off unless the environment
+// variable TSPLIT_SPLIT_BF16 says otherwise); `was`, if given, receives the previous setting.
+extern "C" int TSplit_SplitBf16(int on, int *was) {
+  const bool before = tsplit::split_bf16();
+  tsplit::g_split_bf16.store(on != 0 ? 1 : 0, std::memory_order_relaxed);
+  if (was) *was = before ? 1 : 0;
+  return 0;
+}
 
 // Switches the timing of the Winograd routine's GEMM launches on or off (and forgets what was recorded).
 extern "C" int TSplit_WinogradGemmTiming(int on) {

@@ -430,10 +430,19 @@ def winograd_gemm_timing(on):
     check_call(_LIB.TSplit_WinogradGemmTiming(int(bool(on))))
 
 
+def split_bf16(on):
+    """Switches the split-bf16 products of the Winograd routine's GEMMs on or off (off by default); returns
+    the previous setting."""
+    was = ctypes.c_int()
+    check_call(_LIB.TSplit_SplitBf16(int(bool(on)), ctypes.byref(was)))
+    return bool(was.value)
+
+
 def winograd_gemm_times(filter_gradient=False, kind=None):
     """-> (launches, total ms, total executed FLOP, total algorithmic bytes) of the timed GEMM launches of
-    kind 0 (forward / data gradient on 128 x 128 tiles), 1 (filter gradient) or 2 (forward / data gradient
-    of layers that produce at most 64 channels, on 64 x 256 tiles)."""
+    kind 0 (forward / data gradient on 128 x 128 tiles), 1 (filter gradient), 2 (forward / data gradient
+    of layers that produce at most 64 channels, on 64 x 256 tiles), 3 / 4 (forward and data gradient /
+    filter gradient with split-bf16 products)."""
     which = int(bool(filter_gradient)) if kind is None else int(kind)
     n, ms, flop, nbytes = ctypes.c_double(), ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
     check_call(_LIB.TSplit_WinogradGemmTimes(which, ctypes.byref(n), ctypes.byref(ms), ctypes.byref(flop)))

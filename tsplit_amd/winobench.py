@@ -1,13 +1,15 @@
 """The 3x3 / stride 1 / pad 1 layers of VGG-16 one by one on one MI355X: every pass on the direct kernels
 and through the Winograd routine, with the time and rate of the GEMM launch inside the routine.
 
-    python -m tsplit_amd.winobench [--iters 10]
+    python -m tsplit_amd.winobench [--iters 10] [--split-bf16]
 
 Shapes are those of the benchmark step (batch 64; the 224x224 and 112x112 layers as micro-tensors of 16
 images).  A call is timed over `iters` back-to-back launches between two HIP events after two untimed
 ones; the GEMM inside a Winograd call by the library's own event pairs (TSplit_WinogradGemmTiming).
 "direct-equivalent" rates count the direct algorithm's FLOP, of which the routine executes a quarter;
 GEMM rates count executed FLOP (2 * 36 * rows * tiles * depth) against the 157.3 TFLOP/s fp32 matrix peak.
+With --split-bf16 the GEMMs of layers with more than 64 channels on both sides take their products as six
+bf16 x bf16 terms (TSplit_SplitBf16); their rate is then the fp32-equivalent one (the same FLOP count).
 Prints one JSON object per layer and pass and a final table.
 """
 import argparse
@@ -23,10 +25,12 @@ LAYERS = [(16, 64, 64, 224), (16, 64, 128, 112), (16, 128, 128, 112), (64, 128, 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--iters", type=int, default=10)
+    ap.add_argument("--split-bf16", action="store_true")
     a = ap.parse_args()
     from . import gpu_links as L, ndarray, stream
     from .timing import EventTimer
     ctx = ndarray.gpu(0)
+    L.split_bf16(a.split_bf16)
     st = stream.create_stream_handle(ctx)
     timer = EventTimer(ctx)
     rng = np.random.RandomState(0)
@@ -62,7 +66,7 @@ def main():
                 fn()
             st.sync()
             launches = ms = gf = 0
-            for k in ((1,) if kind == 1 else (0, 2)):
+            for k in ((1, 4) if kind == 1 else (0, 2, 3)):
                 ln, m, f, _ = L.winograd_gemm_times(kind=k)
                 launches, ms, gf = launches + ln, ms + m, gf + f
             L.winograd_gemm_timing(False)
@@ -80,6 +84,9 @@ def main():
             r["winograd_us"], r["direct_tflops_direct_equivalent"], r["winograd_tflops_direct_equivalent"], r["gemm_us"],
             r["gemm_tflops_executed"]))
     print("(* rate of the direct algorithm's FLOP count)")
+    if a.split_bf16:
+        print("(split-bf16 products in the GEMMs of layers with more than 64 channels on both sides: GEMM TF is the "
+              "fp32-equivalent rate)")
 
 
 if __name__ == "__main__":
