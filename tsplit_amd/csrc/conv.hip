@@ -2031,6 +2031,7 @@ struct ThinParams {
   int C, H, W, O, Opad, kH, kW, ph, pw, s, oH, oW, K;   // Opad: O rounded up to the channels per thread
   FastDiv plane, width;              // oH*oW, oW
   int64_t n_total;                   // imgs * oH * oW
+  int64_t x_bytes;
 };
 
 __global__ __launch_bounds__(256) void filter_thin_kernel(const float *__restrict__ w, float *__restrict__ out, int O,
@@ -2098,6 +2099,106 @@ __global__ __launch_bounds__(256) void conv_thin_fwd_kernel(ThinParams P, const 
     if (og * kThinChans + o < P.O) __builtin_nontemporal_store(acc[o], yo + static_cast<int64_t>(o) * P.plane.d);
 }
 
+// The same layer class on the matrix pipes, without LDS staging and without barriers: y[oc][pos] = sum over k of
+// w[oc][k] patch[k][pos] as 32 x 32 x 2 MFMAs whose operands come straight from memory in the instruction's
+// own layout.  A wave takes 64 consecutive output positions (two column tiles) and 64 output channels (two
+// row tiles).  Lane l supplies, for MFMA j, the filter value w[32 t + l % 32][2 j + l / 32] (kept in
+// registers for the whole wave: the filter is 64 x 27 numbers) and the input value of position l % 32 under
+// reduction index 2 j + l / 32 (a gather from x, which stays in L2: 32 consecutive positions are 128
+// consecutive bytes of an image row); the result's lanes 0 - 31 hold 32 consecutive positions of one output
+// channel, so every store instruction writes two whole 128-byte lines.  The multiplications take a quarter
+// of the time it takes to write y: the kernel is bound by that write.
+template <int kRowTiles, int kSteps, bool kAllRows>
+__global__ __launch_bounds__(256) void conv_thin_mfma_kernel(ThinParams P, const float *__restrict__ x,
+                                                             const float *__restrict__ w, float *__restrict__ y) {
+  __shared__ int tab[2 * kSteps][4];     // per reduction index: kh, kw, offset inside one image of x
+  if (threadIdx.x < 2 * kSteps) {
+    const int k = threadIdx.x < P.K ? threadIdx.x : 0;
+    const int taps = P.kH * P.kW;
+    const int c = k / taps, t = k - c * taps;
+    const int kh = t / P.kW, kw = t - kh * P.kW;
+    tab[threadIdx.x][0] = kh;
+    tab[threadIdx.x][1] = kw;
+    tab[threadIdx.x][2] = (c * P.H + kh) * P.W + kw;
+    tab[threadIdx.x][3] = threadIdx.x < P.K ? 1 : 0;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
+  const int oc0 = blockIdx.y * (32 * kRowTiles);
+  // Both operands come through buffer loads: an element that does not exist (a channel beyond O, an index
+  // beyond K, a tap outside the image, a position beyond the last one) gets an offset beyond the buffer and
+  // reads as zero, without a branch.
+  const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(w), 0, P.O * P.K * 4, mg::kBufFlags);
+  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(x), 0, static_cast<int>(P.x_bytes), mg::kBufFlags);
+  float wa[kRowTiles][kSteps];
+#pragma unroll
+  for (int t = 0; t < kRowTiles; ++t)
+#pragma unroll
+    for (int j = 0; j < kSteps; ++j) {
+      const int oc = oc0 + 32 * t + col, k = 2 * j + half;
+      const unsigned off = oc < P.O && k < P.K ? static_cast<unsigned>(oc * P.K + k) * 4u : mg::kOobOffset;
+      wa[t][j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rw, off, 0, 0));
+    }
+  const int64_t n0 = (static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6)) * 64;
+  if (n0 >= P.n_total) return;
+  // the gathered inputs of this lane's two positions, all loads in flight together
+  float xb[2][kSteps];
+  uint32_t img[2], pos[2];
+  bool ok[2];
+#pragma unroll
+  for (int pt = 0; pt < 2; ++pt) {
+    const int64_t n = n0 + 32 * pt + col;
+    ok[pt] = n < P.n_total;
+    const uint32_t nn = ok[pt] ? static_cast<uint32_t>(n) : 0u;
+    img[pt] = P.plane.div(nn);
+    pos[pt] = nn - img[pt] * P.plane.d;
+    const uint32_t oh = P.width.div(pos[pt]), ow = pos[pt] - oh * P.width.d;
+    const int ih0 = static_cast<int>(oh) * P.s - P.ph, iw0 = static_cast<int>(ow) * P.s - P.pw;
+    const int base = static_cast<int>(img[pt]) * (P.C * P.H * P.W) + ih0 * P.W + iw0;   // below 2^29 elements
+#pragma unroll
+    for (int j = 0; j < kSteps; ++j) {
+      const int4 e = *reinterpret_cast<const int4 *>(tab[2 * j + half]);
+      const bool in = ok[pt] && e.w != 0 && static_cast<unsigned>(ih0 + e.x) < static_cast<unsigned>(P.H) &&
+                      static_cast<unsigned>(iw0 + e.y) < static_cast<unsigned>(P.W);
+      const unsigned off = in ? static_cast<unsigned>(base + e.z) * 4u : mg::kOobOffset;
+      xb[pt][j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rx, off, 0, 0));
+    }
+  }
+  mg::acc16 acc[kRowTiles][2];
+#pragma unroll
+  for (int t = 0; t < kRowTiles; ++t)
+#pragma unroll
+    for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[t][pt][e] = 0.f;
+#pragma unroll
+  for (int j = 0; j < kSteps; ++j)
+#pragma unroll
+    for (int t = 0; t < kRowTiles; ++t)
+#pragma unroll
+      for (int pt = 0; pt < 2; ++pt)
+        acc[t][pt] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[t][j], xb[pt][j], acc[t][pt], 0, 0, 0);
+  // element e of a lane: output channel 32 t + 8 (e / 4) + 4 (lane / 32) + e % 4, position of the lane
+#pragma unroll
+  for (int pt = 0; pt < 2; ++pt) {
+    if (!ok[pt]) continue;
+    float *yo = y + static_cast<int64_t>(img[pt]) * P.O * P.plane.d + pos[pt];
+#pragma unroll
+    for (int t = 0; t < kRowTiles; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int oc = oc0 + 32 * t + 8 * (e >> 2) + 4 * half + (e & 3);
+        if (kAllRows || oc < P.O) __builtin_nontemporal_store(acc[t][pt][e], yo + static_cast<int64_t>(oc) * P.plane.d);
+      }
+  }
+}
+
+// from 32 output channels on, the matrix-pipe form (TSPLIT_CONV_THIN_MFMA=0 keeps the vector-ALU kernel)
+inline bool thin_on_matrix_pipes(const ConvGeo &g) {
+  const char *e = std::getenv("TSPLIT_CONV_THIN_MFMA");
+  return g.O >= 32 && static_cast<int64_t>(g.imgs) * g.C * g.H * g.W < (1ll << 29) && !(e && e[0] == '0');
+}
+
 inline bool thin_fwd_ok(const ConvGeo &g) {
   return g.C * g.kH * g.kW <= kThinMaxK && static_cast<int64_t>(g.imgs) * g.oH * g.oW < (1ll << 31);
 }
@@ -2107,9 +2208,13 @@ int launch_conv_thin_fwd(const ConvGeo &g, const float *x, const float *w, float
   P.K = g.C * g.kH * g.kW;
   const int chans = g.O > 16 ? 32 : 16;
   P.Opad = (g.O + chans - 1) / chans * chans;
-  float *wt = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(P.K) * P.Opad * 4));
-  TS_REQUIRE(wt, "conv: no scratch memory for the re-laid filter");
-  hipLaunchKernelGGL(filter_thin_kernel, dim3((P.K * P.Opad + 255) / 256), dim3(256), 0, st, w, wt, g.O, P.Opad, P.K);
+  const bool mfma = thin_on_matrix_pipes(g);
+  float *wt = nullptr;
+  if (!mfma) {
+    wt = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(P.K) * P.Opad * 4));
+    TS_REQUIRE(wt, "conv: no scratch memory for the re-laid filter");
+    hipLaunchKernelGGL(filter_thin_kernel, dim3((P.K * P.Opad + 255) / 256), dim3(256), 0, st, w, wt, g.O, P.Opad, P.K);
+  }
   P.C = g.C;
   P.H = g.H;
   P.W = g.W;
@@ -2124,6 +2229,20 @@ int launch_conv_thin_fwd(const ConvGeo &g, const float *x, const float *w, float
   P.plane = FastDiv(g.oH * g.oW);
   P.width = FastDiv(g.oW);
   P.n_total = static_cast<int64_t>(g.imgs) * g.oH * g.oW;
+  if (mfma) {
+    const dim3 grid_m(static_cast<unsigned>((P.n_total + 255) / 256), static_cast<unsigned>((g.O + 63) / 64));
+    P.x_bytes = static_cast<int64_t>(g.imgs) * g.C * g.H * g.W * 4;
+    const bool all = g.O % 64 == 0;   // every row tile is whole: the stores need no channel check
+    if (P.K <= 28 && all)
+      hipLaunchKernelGGL((conv_thin_mfma_kernel<2, 14, true>), grid_m, dim3(256), 0, st, P, x, w, y);
+    else if (P.K <= 28)
+      hipLaunchKernelGGL((conv_thin_mfma_kernel<2, 14, false>), grid_m, dim3(256), 0, st, P, x, w, y);
+    else if (all)
+      hipLaunchKernelGGL((conv_thin_mfma_kernel<2, 16, true>), grid_m, dim3(256), 0, st, P, x, w, y);
+    else
+      hipLaunchKernelGGL((conv_thin_mfma_kernel<2, 16, false>), grid_m, dim3(256), 0, st, P, x, w, y);
+    return 0;
+  }
   const unsigned groups = static_cast<unsigned>(P.Opad / chans);
   const dim3 grid(static_cast<unsigned>((P.n_total + 63) / 64), (groups + 3) / 4);
   if (chans == 32)
