@@ -480,15 +480,15 @@ int TSplit_WinogradGemmTiming(int on);
 int TSplit_WinogradGemmTimes(int which, double *launches, double *ms, double *flop);
 int TSplit_WinogradGemmBytes(int which, double *bytes);
 
-/* ---- Split-bf16 products in the Winograd routine's GEMMs.  NO counterpart in the reference; opt-in,
- *      off by default (every product of the default path is an fp32 matrix instruction).  With
- *      TSplit_SplitBf16(1, NULL) the GEMMs of 3x3 layers with more than 64 channels on both sides
- *      split each fp32 operand exactly into three bf16 terms, a = a1 + a2 + a3, and take a product as
- *      the six bf16 x bf16 products a_i b_j with i + j <= 4, accumulated in fp32 by the bf16 matrix
- *      instruction; what is left out is below 2^-23 of the product, the rounding of one fp32
- *      multiplication.  Operands and results stay fp32 in memory.  Affects calls issued afterwards, on
- *      every stream; `was` (may be NULL) receives the previous setting.  The environment variable
- *      TSPLIT_SPLIT_BF16=1 turns it on from the start. ---- */
+/* ---- Split-bf16 products in the Winograd routine's GEMMs and in DLGpuMatrixMultiply.  NO counterpart in
+ *      the reference; opt-in, off by default (every product of the default path is an fp32 matrix
+ *      instruction).  With TSplit_SplitBf16(1, NULL) the GEMMs of 3x3 layers with more than 64 channels on
+ *      both sides and the matrix products whose depth is a multiple of 4 split each fp32 operand exactly
+ *      into three bf16 terms, a = a1 + a2 + a3, and take a product as the six bf16 x bf16 products a_i b_j
+ *      with i + j <= 4, accumulated in fp32 by the bf16 matrix instruction; what is left out is below
+ *      2^-23 of the product, the rounding of one fp32 multiplication.  Operands and results stay fp32 in
+ *      memory.  Affects calls issued afterwards, on every stream; `was` (may be NULL) receives the
+ *      previous setting.  The environment variable TSPLIT_SPLIT_BF16=1 turns it on from the start. ---- */
 int TSplit_SplitBf16(int on, int *was);
 
 /* ---- Recorded steps.  NO counterpart in the reference (every step there is issued call by

@@ -1,4 +1,5 @@
-"""The opt-in split-bf16 products of the Winograd routine's GEMMs (TSplit_SplitBf16), through the C ABI.
+"""The opt-in split-bf16 products of the Winograd routine's GEMMs and of the matrix products (TSplit_SplitBf16),
+through the C ABI.
 
 Bars: with the switch on, the three convolutions of wide 3x3 layers meet the float64 oracle within the
 convolution tolerance (2e-3 max relative error, and below 1e-4 as the fp32 path does), their error against
@@ -114,6 +115,58 @@ def test_operands_with_extreme_exponents(split, monkeypatch):
         y = nd.empty(x.shape, ctx)
         L.CuDNN_conv2d(nd.array(xs, ctx), nd.array(w, ctx), y, 1, 1, 1)
         assert_close(y.asnumpy() / np.float32(scale), O.conv2d(x, w, 1, 1, 1), 1e-4, f"scale {scale}")
+
+
+MATMULS = [
+    # M, K, N
+    (64, 4096, 1000),      # a fully-connected layer at batch 64: one row tile half empty, the depth cut into ranges
+    (200, 72, 300),        # ragged rows and columns, a depth that is a multiple of 4 only
+    (256, 512, 2048),      # whole tiles
+    (130, 20, 70),         # one full and one partial k-step
+]
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("shape", MATMULS)
+def test_matrix_product_with_split_terms(shape, ta, tb, rng, split):
+    """DLGpuMatrixMultiply in its four transpose forms: against float64 no further off than 1.5 times the fp32
+    matrix instruction's own error (relative to the sum of the products' magnitudes), inside the 2e-3 tolerance."""
+    from tsplit_amd import ndarray as nd
+    L, ctx = split, nd.gpu(0)
+    M, K, N = shape
+    a = rng.normal(size=(K, M) if ta else (M, K)).astype(np.float32)
+    b = rng.normal(size=(N, K) if tb else (K, N)).astype(np.float32)
+    a64, b64 = (a.T if ta else a).astype(np.float64), (b.T if tb else b).astype(np.float64)
+    ref, mag = a64 @ b64, np.abs(a64) @ np.abs(b64)
+    ga, gb = nd.array(a, ctx), nd.array(b, ctx)
+    outs = []
+    for on in (False, True):
+        L.split_bf16(on)
+        c = nd.empty((M, N), ctx)
+        L.matrix_multiply(ga, ta, gb, tb, c)
+        outs.append(c.asnumpy())
+    L.split_bf16(False)
+    e_plain, e_split = [(np.abs(o - ref) / mag).max() for o in outs]
+    assert_close(outs[1], ref, TOL, f"matmul {shape} ta={ta} tb={tb}")
+    assert e_split <= 1.5 * e_plain + 1e-8, (e_split, e_plain)
+    assert not np.array_equal(outs[0], outs[1])      # the split kernel did run
+
+
+def test_matrix_product_outside_the_switch_keeps_its_bits(rng, split):
+    """A depth that is not a multiple of 4 stays on the fp32 kernels."""
+    from tsplit_amd import ndarray as nd
+    L, ctx = split, nd.gpu(0)
+    a, b = rng.normal(size=(70, 30)).astype(np.float32), rng.normal(size=(30, 90)).astype(np.float32)
+    ga, gb = nd.array(a, ctx), nd.array(b, ctx)
+    outs = []
+    for on in (False, True):
+        L.split_bf16(on)
+        c = nd.empty((70, 90), ctx)
+        L.matrix_multiply(ga, False, gb, False, c)
+        outs.append(c.asnumpy())
+    L.split_bf16(False)
+    np.testing.assert_array_equal(outs[0], outs[1])
 
 
 def _onehot(lab, n):

@@ -27,6 +27,9 @@ inline float mib(int64_t elems) { return static_cast<float>(elems) * 4.0f / (102
 // that stream without waiting; ops on different streams never share one.
 void *scratch_get(hipStream_t stream, int slot, size_t bytes);
 
+// whether contractions take their products in split bf16 (TSplit_SplitBf16; winograd.hip)
+bool split_bf16_enabled();
+
 // Where a convolution leaves per-channel partial sums of its output for a BatchNorm that follows:
 // partial k of channel c is the pair (sum, sum of squares) at part[(k * channels + c) * 2]; `used`
 // counts the partials written so far (a call may run as several launches).

@@ -11,6 +11,7 @@
 // batches already give thousands of tiles); narrow outputs (N <= 64) use 256x64 tiles.
 #include "common.h"
 #include "mfma_gemm.h"
+#include "gemm_split.h"
 
 namespace tsplit {
 namespace {
@@ -59,6 +60,32 @@ int launch_gemm(const float *A, int64_t lda, const float *B, int64_t ldb, float 
   return 0;
 }
 
+// the same product with split-bf16 terms (opt-in): 128 x 128 tiles whatever M, the split-K plan and fold of above
+template <bool TA, bool TB>
+int launch_gemm_split(const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int M, int N, int K,
+                      hipStream_t s, int64_t *ws_elems) {
+  using AL = typename std::conditional<TA, SplitMnContigLoader, SplitKContigLoader>::type;
+  using BL = typename std::conditional<TB, SplitKContigLoader, SplitMnContigLoader>::type;
+  const typename AL::Params ap{A, lda, M, K};
+  const typename BL::Params bp{B, ldb, N, K};
+  const int tm = (M + 127) / 128, tn = (N + 127) / 128;
+  int S, kchunk;
+  plan_splitk(tm * tn, K, 64, 3, S, kchunk);
+  float *out = C;
+  const int64_t mn = static_cast<int64_t>(M) * N;
+  if (S > 1) {
+    out = static_cast<float *>(scratch_get(s, 2, static_cast<size_t>(S) * mn * 4));
+    TS_REQUIRE(out, "DLGpuMatrixMultiply: no scratch memory for split-K");
+    *ws_elems = S * mn;
+  }
+  hipLaunchKernelGGL((mfma_gemm_split_kernel<AL, BL>), dim3(grid_blocks(tm, tn, S)), dim3(kThreads), 0, s, ap, bp, out, mn,
+                     M, N, K, kchunk, TileGrid{tm, tn, tm * tn * S});
+  if (S > 1)
+    hipLaunchKernelGGL(splitk_fold_kernel, dim3(static_cast<unsigned>((mn + 255) / 256)), dim3(256), 0, s, out, C, mn,
+                       mn, S);
+  return 0;
+}
+
 template <int BM, int BN, int WM, int WN, bool TA, bool TB>
 int launch_gemm_any(const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int M, int N, int K,
                     hipStream_t s, int64_t *ws) {
@@ -71,6 +98,11 @@ int launch_gemm_any(const float *A, int64_t lda, const float *B, int64_t ldb, fl
 template <bool TA, bool TB>
 int dispatch_tile(const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int M, int N, int K,
                   hipStream_t s, int64_t *ws) {
+  // split-bf16 products where asked for: K a multiple of 4 (a loaded word lies inside a row or outside it) and
+  // both operands within reach of 32-bit byte offsets
+  if (split_bf16_enabled() && K % 4 == 0 && K >= BK && K < (1 << 29) &&
+      dense_fits_buffer(stored_rows(TA, M, K), lda, TA ? BK : 128) && dense_fits_buffer(stored_rows(!TB, N, K), ldb, TB ? 128 : BK))
+    return launch_gemm_split<TA, TB>(A, lda, B, ldb, C, M, N, K, s, ws);
   if (M <= 64) return launch_gemm_any<64, 256, 1, 4, TA, TB>(A, lda, B, ldb, C, M, N, K, s, ws);
   return launch_gemm_any<128, 128, 2, 2, TA, TB>(A, lda, B, ldb, C, M, N, K, s, ws);
 }

@@ -396,19 +396,6 @@ class GemmTiming {
   bool on_ = false;
 };
 
-// Opt-in: the GEMMs of layers with more than 64 channels on both sides take their products in split bf16
-// (wino_gemm_split.h).  -1 until asked: the environment variable TSPLIT_SPLIT_BF16 then gives the first value.
-std::atomic<int> g_split_bf16{-1};
-inline bool split_bf16() {
-  int v = g_split_bf16.load(std::memory_order_relaxed);
-  if (v < 0) {
-    const char *e = std::getenv("TSPLIT_SPLIT_BF16");
-    v = e && std::atoi(e) != 0 ? 1 : 0;
-    g_split_bf16.store(v, std::memory_order_relaxed);
-  }
-  return v != 0;
-}
-
 // compute units of the current device and resident blocks of the GEMM kernel on each, asked once
 inline int compute_units() {
   static const int n = [] {
@@ -517,6 +504,20 @@ inline int run_images(int imgs, int per_img, int chans_a, int chans_b) {
 
 }  // namespace
 
+// Opt-in: the Winograd GEMMs of layers with more than 64 channels on both sides and the matrix products take
+// their products in split bf16 (wino_gemm_split.h, gemm_split.h).  -1 until asked: the environment variable
+// TSPLIT_SPLIT_BF16 then gives the first value.
+std::atomic<int> g_split_bf16{-1};
+bool split_bf16_enabled() {
+  int v = g_split_bf16.load(std::memory_order_relaxed);
+  if (v < 0) {
+    const char *e = std::getenv("TSPLIT_SPLIT_BF16");
+    v = e && std::atoi(e) != 0 ? 1 : 0;
+    g_split_bf16.store(v, std::memory_order_relaxed);
+  }
+  return v != 0;
+}
+
 // y[n][produced][H][W] = conv3x3(x[n][gathered][H][W], filter), stride 1, pad 1.  `rotated` selects
 // the data-gradient reading of the filter (stored [gathered][produced][3][3], rotated 180 degrees).
 // With a sink, every block of the output transform adds one partial (sum, sum of squares) per channel.
@@ -548,7 +549,7 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
       // every operand read once, the result written once
       const double flop = 2.0 * kXi * produced * static_cast<double>(gi.ld) * gathered;
       const double bytes = 4.0 * kXi * (static_cast<double>(produced) * gathered + static_cast<double>(gathered + produced) * gi.ld);
-      const bool split = produced > 64 && (gathered & 7) == 0 && split_bf16();
+      const bool split = produced > 64 && (gathered & 7) == 0 && split_bf16_enabled();
       GemmTiming timed(st, split ? 3 : produced <= 64 ? 2 : 0, flop, bytes);
       const wg::Problem gemm{U, V, M, produced, gathered, gi.ld, 0, 0};
       if (split)
@@ -606,7 +607,7 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
       hipLaunchKernelGGL(wino_grad_kernel<false>, grid_y, dim3(256), 0, st, dyr, Y, gy);
     const int here = (gx.ld + kchunk - 1) / kchunk;
     {
-      const bool split = plan.grid > 0 && split_bf16();
+      const bool split = plan.grid > 0 && split_bf16_enabled();
       GemmTiming timed(st, split ? 4 : 1, 2.0 * kXi * O * static_cast<double>(gx.ld) * C,
                        4.0 * kXi * (static_cast<double>(O) * C * here + static_cast<double>(O + C) * gx.ld));
       launch_grad_gemm(plan, wg::GradProblem{Y, V, part + static_cast<int64_t>(parts) * kXi * oc, O, C, gx.ld, kchunk, 0, 0},
@@ -626,10 +627,10 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
 
 }  // namespace tsplit
 
-// Switches the split-bf16 products of the Winograd routine's GEMMs on or off (off unless the environment
+// Switches the split-bf16 products of the Winograd routine's GEMMs and of the matrix products on or off (off unless the environment
 // variable TSPLIT_SPLIT_BF16 says otherwise); `was`, if given, receives the previous setting.
 extern "C" int TSplit_SplitBf16(int on, int *was) {
-  const bool before = tsplit::split_bf16();
+  const bool before = tsplit::split_bf16_enabled();
   tsplit::g_split_bf16.store(on != 0 ? 1 : 0, std::memory_order_relaxed);
   if (was) *was = before ? 1 : 0;
   return 0;

@@ -1,9 +1,10 @@
 """Times one training step (forward, backward, SGD) of the branched example networks at the
 sizes of the reference's benchmark configurations, on one MI355X through the C ABI.
 
-    python -m tsplit_amd.graphbench --net resnet50|resnet101|inception_v4|transformer|lstm|mlp|vgg19 [--steps 5] [--warmup 2] [--record]
+    python -m tsplit_amd.graphbench --net resnet50|resnet101|inception_v4|transformer|lstm|mlp|vgg19 [--steps 5] [--warmup 2] [--record] [--split-bf16]
 
---record issues the step once into a HIP graph after the warm-up and times replays of that graph
+--split-bf16 turns on the opt-in split-bf16 products of the matrix products and the Winograd GEMMs
+(TSplit_SplitBf16).  --record issues the step once into a HIP graph after the warm-up and times replays of that graph
 (one host call per step) instead of Python issuing every operator again.
 
 Prints one JSON object: samples/s, ms/step, final loss, operator calls per step.  Synthetic
@@ -25,9 +26,11 @@ def main():
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--lr", type=float, default=1e-4)
     ap.add_argument("--record", action="store_true", help="record the step into a graph and time its replays")
+    ap.add_argument("--split-bf16", action="store_true")
     a = ap.parse_args()
-    from . import graph, ndarray, stream, workloads
+    from . import gpu_links, graph, ndarray, stream, workloads
     ctx = ndarray.gpu(0)
+    gpu_links.split_bf16(a.split_bf16)
     if a.net in ("mlp", "vgg19"):
         return layer_list(a, ctx)
     st = stream.create_stream_handle(ctx)
@@ -165,7 +168,9 @@ def layer_list(a, ctx):
     dt = time.perf_counter() - t0
     print(json.dumps({"net": a.net, "workload": desc, "samples_per_s": n * steps / dt,
                       "ms_per_step": dt / steps * 1e3, "steps": steps, "warmup": a.warmup, "final_loss": t.loss_value(),
-                      "recorded": bool(a.record), "dtype": "f32", "data": "synthetic"}))
+                      "recorded": bool(a.record),
+                      "dtype": "f32 (matrix products and Winograd GEMMs as six bf16 x bf16 terms of exact operand splits, fp32 accumulation)"
+                      if a.split_bf16 else "f32", "data": "synthetic"}))
 
 
 if __name__ == "__main__":
