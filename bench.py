@@ -181,9 +181,9 @@ def main():
     ap.add_argument("--no-split", action="store_true")
     ap.add_argument("--no-events", action="store_true", help="time the steps without per-launch events")
     ap.add_argument("--fused", action="store_true",
-                    help="run every BatchNorm+Relu pair through the fused symbols, let every convolution hand its "
-                         "output's statistics to the BatchNorm behind it and update all parameters in one launch "
-                         "(symbols outside the reference's ABI)")
+                    help="run every BatchNorm+Relu pair (and the max pooling behind it, where one follows) through the fused "
+                         "symbols, let every convolution hand its output's statistics to the BatchNorm behind it and "
+                         "update all parameters in one launch (symbols outside the reference's ABI)")
     ap.add_argument("--split-bf16", action="store_true",
                     help="opt-in, outside the reference's ABI and outside the default path's fp32 matrix instructions: the "
                          "Winograd GEMMs of layers with more than 64 channels on both sides take each fp32 product as six "
@@ -202,7 +202,7 @@ def main():
     timer = None if a.no_events else EventTimer(ctx, chained=True)
     L.split_bf16(a.split_bf16)
     t = trainer.Trainer(spec, params, x.shape, 1000, ctx, optimizer=("momentum", 1e-4, 0.9), split=split, timer=timer,
-                        fuse_bn_relu=a.fused, conv_bn_stats=a.fused, multi_tensor_update=a.fused)
+                        fuse_bn_relu=a.fused, conv_bn_stats=a.fused, multi_tensor_update=a.fused, fuse_max_pool=a.fused)
     gx, gy = ndarray.array(x, ctx), ndarray.array(labels, ctx)      # resident before timing
     for _ in range(a.warmup):
         t.step(gx, gy)
@@ -239,7 +239,7 @@ def main():
         "config": {"workload": "VGG-16 training step (fwd+bwd+momentum SGD), fp32 NCHW, batch %d, 3x224x224, "
                                "1000 classes, He init, %s%s" % (a.batch, "4 batch micro-tensors on the 4 largest conv layers"
                                                                 if split else "no micro-tensor split",
-                                                                (", BatchNorm+Relu pairs fused, BatchNorm statistics from the convolutions' epilogues, one optimizer launch" if a.fused else "")
+                                                                (", BatchNorm+Relu pairs fused (with the max pooling behind them where one follows), BatchNorm statistics from the convolutions' epilogues, one optimizer launch" if a.fused else "")
                                                                 + (", split-bf16 products in the wide layers' Winograd GEMMs" if a.split_bf16 else "")),
                    "global_batch": a.batch, "final_loss": loss},
     }

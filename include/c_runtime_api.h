@@ -442,6 +442,35 @@ int TSplit_BatchNormFromStats(const DLArrayHandle input_X, const DLArrayHandle s
                               DLArrayHandle save_var_arr, int relu, DLStreamHandle stream_handle,
                               ProfilerHandle p);
 
+/* ---- BatchNorm + Relu + max pooling as one call each way.  NO counterpart in the reference, where the three
+ *      nodes that end a VGG stage are three calls (src/ops/CudnnBn.cu:12-210, src/ops/Relu.cu,
+ *      src/ops/CudnnMaxPool.cu:6-210) and the activation in front of the pooling is written, read back by
+ *      the pooling and kept for its gradient; for hosts that know the three follow one another.  2x2
+ *      windows, stride 2, no padding; H and W of input_X even.  The forward calls read input_X
+ *      [N][C][H][W] once and write only output_Y [N][C][H/2][W/2] (values equal those of the three calls);
+ *      TSplit_BatchNormReluMaxPool takes the batch statistics from input_X itself (one more read),
+ *      TSplit_BatchNormReluMaxPoolFromStats from rows 0 .. slots-1 of `stats` as
+ *      TSplit_BatchNormFromStats does.  Both save arrays are required.
+ *      TSplit_BatchNormReluMaxPool_gradient takes the pooled tensor's gradient gradient_Y
+ *      [N][C][H/2][W/2] and input_X: a window's gradient goes to the first maximum of Relu(BN(input_X))
+ *      in row-major order (the tie rule of the pooling gradient), is gated with the reference's Relu
+ *      derivative there, and the BatchNorm gradient is taken; gradient_X [N][C][H][W]. ---- */
+int TSplit_BatchNormReluMaxPool(const DLArrayHandle input_X, const DLArrayHandle bn_scale,
+                                const DLArrayHandle bn_bias, DLArrayHandle output_Y, float eps,
+                                DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                                DLStreamHandle stream_handle, ProfilerHandle p);
+int TSplit_BatchNormReluMaxPoolFromStats(const DLArrayHandle input_X, const DLArrayHandle stats, int slots,
+                                         const DLArrayHandle bn_scale, const DLArrayHandle bn_bias,
+                                         DLArrayHandle output_Y, float eps, DLArrayHandle save_mean_arr,
+                                         DLArrayHandle save_var_arr, DLStreamHandle stream_handle,
+                                         ProfilerHandle p);
+int TSplit_BatchNormReluMaxPool_gradient(const DLArrayHandle gradient_Y, const DLArrayHandle input_X,
+                                         const DLArrayHandle bn_scale, const DLArrayHandle bn_bias,
+                                         DLArrayHandle gradient_X, DLArrayHandle gradient_bn_scale,
+                                         DLArrayHandle gradient_bn_bias, float eps,
+                                         DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                                         DLStreamHandle stream_handle, ProfilerHandle p);
+
 /* ---- Optimizer update of a whole model in one launch.  NO counterpart in the reference, whose
  *      optimizer issues one SGDOptimizerUpdate / MomentumOptimizerUpdate per parameter
  *      (python/athena/optimizer.py:95-176): dozens of launches, most of them on BatchNorm vectors

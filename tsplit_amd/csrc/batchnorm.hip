@@ -613,6 +613,202 @@ inline bool plane_major_ok(const Plan &pl, const DLArray *x, PlaneGeo &pg, unsig
   return true;
 }
 
+// ---------------------------------------------------------------- BatchNorm + Relu + 2x2 / stride 2 max pooling
+// One pass each way for the three nodes that end a VGG stage: the forward pass reads the BatchNorm's input and
+// writes only the pooled tensor (the activation in front of the pooling is never written: 5 B per element
+// instead of the 13 of BatchNorm+Relu and pooling on their own), the gradient reads that input and the
+// pooled gradient twice and writes the input's gradient (14 B per element instead of 29).  A thread owns the
+// 2x2 windows under VECW consecutive columns of two rows (VECW = 4: two windows, 16-byte loads; 2: one window).
+// Element (plane, h, w) of x at x[(plane * H + h) * W + w], plane = image * C + channel; H and W even.
+struct PoolGeo {
+  FastDiv wq;       // words per row: W / VECW
+  FastDiv rows;     // pooled rows per plane: H / 2
+  FastDiv chans;    // C
+  uint32_t words;   // words of the whole array: N * C * (H / 2) * (W / VECW)
+  int H, W;
+};
+template <int VECW>
+struct PoolWord;
+template <>
+struct PoolWord<4> {
+  using In = f32x4;
+  using Out = float __attribute__((ext_vector_type(2)));
+};
+template <>
+struct PoolWord<2> {
+  using In = float __attribute__((ext_vector_type(2)));
+  using Out = float;
+};
+// word i -> its plane, channel and the offsets of its top row in x and of its pooled values
+template <int VECW>
+__device__ __forceinline__ void pool_locate(const PoolGeo &g, uint32_t i, uint32_t &c, int64_t &top, int64_t &pooled) {
+  const uint32_t row = g.wq.div(i), q = i - row * g.wq.d;       // row = plane * (H / 2) + pooled row
+  const uint32_t plane = g.rows.div(row), ph = row - plane * g.rows.d;
+  c = plane - g.chans.div(plane) * g.chans.d;
+  top = (static_cast<int64_t>(plane) * g.H + 2 * ph) * g.W + VECW * q;
+  pooled = static_cast<int64_t>(row) * (g.W / 2) + (VECW / 2) * q;
+}
+__device__ __forceinline__ float max4(float a, float b, float c, float d) { return fmaxf(fmaxf(a, b), fmaxf(c, d)); }
+
+template <int VECW>
+__global__ __launch_bounds__(kThreads) void bn_relu_pool_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                const float *__restrict__ coef, PoolGeo g) {
+  using In = typename PoolWord<VECW>::In;
+  using Out = typename PoolWord<VECW>::Out;
+  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= g.words) return;
+  uint32_t c;
+  int64_t top, pooled;
+  pool_locate<VECW>(g, i, c, top, pooled);
+  const float a = coef[2 * c], b = coef[2 * c + 1];
+  const In r0 = __builtin_nontemporal_load(reinterpret_cast<const In *>(x + top));
+  const In r1 = __builtin_nontemporal_load(reinterpret_cast<const In *>(x + top + g.W));
+  if constexpr (VECW == 4) {
+    const f32x4 z0 = relu_w(axpb(r0, a, b)), z1 = relu_w(axpb(r1, a, b));
+    const Out o = {max4(z0.x, z0.y, z1.x, z1.y), max4(z0.z, z0.w, z1.z, z1.w)};
+    __builtin_nontemporal_store(o, reinterpret_cast<Out *>(y + pooled));
+  } else {
+    const float o = max4(relu1(a * r0.x + b), relu1(a * r0.y + b), relu1(a * r1.x + b), relu1(a * r1.y + b));
+    __builtin_nontemporal_store(o, y + pooled);
+  }
+}
+
+// The gradient that reaches the BatchNorm's output through pooling and Relu, for the 2x2 window with the
+// BatchNorm outputs (z00 z01 / z10 z11): the pooled gradient goes to the first maximum of relu(z) in
+// row-major order (the pooling gradient's tie rule), times the Relu gradient's factor there.
+__device__ __forceinline__ void pool_route(float z00, float z01, float z10, float z11, float dyp, float &g00, float &g01,
+                                           float &g10, float &g11) {
+  const float r00 = relu1(z00), r01 = relu1(z01), r10 = relu1(z10), r11 = relu1(z11);
+  const float m = max4(r00, r01, r10, r11);
+  const int at = r00 == m ? 0 : r01 == m ? 1 : r10 == m ? 2 : 3;
+  g00 = at == 0 ? dyp * gate1(z00) : 0.f;
+  g01 = at == 1 ? dyp * gate1(z01) : 0.f;
+  g10 = at == 2 ? dyp * gate1(z10) : 0.f;
+  g11 = at == 3 ? dyp * gate1(z11) : 0.f;
+}
+// one word: the gradients g0 (top row), g1 (bottom row) behind the loaded rows r0, r1
+template <int VECW>
+__device__ __forceinline__ void pool_word_grads(const typename PoolWord<VECW>::In &r0, const typename PoolWord<VECW>::In &r1,
+                                                const typename PoolWord<VECW>::Out &dyp, float a, float b,
+                                                typename PoolWord<VECW>::In &g0, typename PoolWord<VECW>::In &g1) {
+  float t[8];   // a vector's elements cannot be bound to references
+  if constexpr (VECW == 4) {
+    pool_route(a * r0.x + b, a * r0.y + b, a * r1.x + b, a * r1.y + b, dyp.x, t[0], t[1], t[4], t[5]);
+    pool_route(a * r0.z + b, a * r0.w + b, a * r1.z + b, a * r1.w + b, dyp.y, t[2], t[3], t[6], t[7]);
+    g0 = f32x4{t[0], t[1], t[2], t[3]};
+    g1 = f32x4{t[4], t[5], t[6], t[7]};
+  } else {
+    pool_route(a * r0.x + b, a * r0.y + b, a * r1.x + b, a * r1.y + b, dyp, t[0], t[1], t[2], t[3]);
+    g0 = typename PoolWord<VECW>::In{t[0], t[1]};
+    g1 = typename PoolWord<VECW>::In{t[2], t[3]};
+  }
+}
+
+// partials per block (split s of channel c): sum g, sum g*x, 0, 0 in the layout of bn_bwd_reduce_kernel;
+// word j of a channel: image j / wpp, pooled row and column word from the rest
+template <int VECW>
+__global__ __launch_bounds__(kThreads) void bn_pool_bwd_reduce_kernel(const float *__restrict__ dyp, const float *__restrict__ x,
+                                                                      double *__restrict__ part, PoolGeo g, FastDiv per_plane,
+                                                                      uint32_t words_c, uint32_t chunk, int S,
+                                                                      const float *__restrict__ gamma,
+                                                                      const float *__restrict__ beta,
+                                                                      const float *__restrict__ save_mean,
+                                                                      const float *__restrict__ save_istd) {
+  using In = typename PoolWord<VECW>::In;
+  using Out = typename PoolWord<VECW>::Out;
+  __shared__ double sm[2 * kWaves];
+  const int c = blockIdx.y, s = blockIdx.x;
+  // the same float expressions as the forward pass, so that the sign of a*x + b is the same
+  const double ad = static_cast<double>(gamma[c]) * static_cast<double>(save_istd[c]);
+  const float a = static_cast<float>(ad);
+  const float b = static_cast<float>(static_cast<double>(beta[c]) - static_cast<double>(save_mean[c]) * ad);
+  const uint32_t wpp = per_plane.d;
+  const uint32_t begin = s * chunk, end = min(begin + chunk, words_c);
+  float sg = 0.f, sgx = 0.f;
+  for (uint32_t j = begin + threadIdx.x; j < end; j += kThreads) {
+    const uint32_t n = per_plane.div(j), rest = j - n * wpp;
+    const uint32_t ph = g.wq.div(rest), q = rest - ph * g.wq.d;
+    const int64_t plane = static_cast<int64_t>(n) * g.chans.d + c;
+    const int64_t top = (plane * g.H + 2 * ph) * g.W + VECW * q;
+    const int64_t pooled = (plane * g.rows.d + ph) * (g.W / 2) + (VECW / 2) * q;
+    const In r0 = *reinterpret_cast<const In *>(x + top), r1 = *reinterpret_cast<const In *>(x + top + g.W);
+    const Out d = *reinterpret_cast<const Out *>(dyp + pooled);
+    In g0, g1;
+    pool_word_grads<VECW>(r0, r1, d, a, b, g0, g1);
+    if constexpr (VECW == 4) {
+      sg += (g0.x + g0.y) + (g0.z + g0.w) + (g1.x + g1.y) + (g1.z + g1.w);
+      sgx += (g0.x * r0.x + g0.y * r0.y) + (g0.z * r0.z + g0.w * r0.w) + (g1.x * r1.x + g1.y * r1.y) + (g1.z * r1.z + g1.w * r1.w);
+    } else {
+      sg += (g0.x + g0.y) + (g1.x + g1.y);
+      sgx += (g0.x * r0.x + g0.y * r0.y) + (g1.x * r1.x + g1.y * r1.y);
+    }
+  }
+  sg = wave_sum(sg);
+  sgx = wave_sum(sgx);
+  const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+  if (lane == 0) {
+    sm[w] = static_cast<double>(sg);
+    sm[kWaves + w] = static_cast<double>(sgx);
+  }
+  __syncthreads();
+  if (threadIdx.x < 4) {
+    double r = 0.0;
+    if (threadIdx.x < 2) {
+      r = sm[threadIdx.x * kWaves];
+#pragma unroll
+      for (int k = 1; k < kWaves; ++k) r += sm[threadIdx.x * kWaves + k];
+    }
+    part[(static_cast<int64_t>(c) * S + s) * 4 + threadIdx.x] = r;
+  }
+}
+
+// dx = k1*g + k2*x + k3 in the order of memory; coef[5c ..] as bn_bwd_coef_kernel<true> leaves them
+template <int VECW>
+__global__ __launch_bounds__(kThreads) void bn_pool_bwd_dx_kernel(const float *__restrict__ dyp, const float *__restrict__ x,
+                                                                  float *__restrict__ dx, const float *__restrict__ coef,
+                                                                  PoolGeo g) {
+  using In = typename PoolWord<VECW>::In;
+  using Out = typename PoolWord<VECW>::Out;
+  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= g.words) return;
+  uint32_t c;
+  int64_t top, pooled;
+  pool_locate<VECW>(g, i, c, top, pooled);
+  const float k1 = coef[5 * c], k2 = coef[5 * c + 1], k3 = coef[5 * c + 2], a = coef[5 * c + 3], b = coef[5 * c + 4];
+  const In r0 = __builtin_nontemporal_load(reinterpret_cast<const In *>(x + top));
+  const In r1 = __builtin_nontemporal_load(reinterpret_cast<const In *>(x + top + g.W));
+  const Out d = __builtin_nontemporal_load(reinterpret_cast<const Out *>(dyp + pooled));
+  In g0, g1;
+  pool_word_grads<VECW>(r0, r1, d, a, b, g0, g1);
+  In o0, o1;
+  if constexpr (VECW == 4) {
+    o0 = lin2(g0, r0, k1, k2, k3);
+    o1 = lin2(g1, r1, k1, k2, k3);
+  } else {
+    o0 = In{k1 * g0.x + k2 * r0.x + k3, k1 * g0.y + k2 * r0.y + k3};
+    o1 = In{k1 * g1.x + k2 * r1.x + k3, k1 * g1.y + k2 * r1.y + k3};
+  }
+  __builtin_nontemporal_store(o0, reinterpret_cast<In *>(dx + top));
+  __builtin_nontemporal_store(o1, reinterpret_cast<In *>(dx + top + g.W));
+}
+
+// VECW and the geometry for x[N][C][H][W]; false when H or W is odd or the words do not fit 32 bits
+inline bool make_pool_geo(const DLArray *x, bool aligned, int &vecw, PoolGeo &g) {
+  if (x->ndim != 4) return false;
+  const int64_t N = x->shape[0], C = x->shape[1], H = x->shape[2], W = x->shape[3];
+  if (N <= 0 || C <= 0 || H < 2 || W < 2 || (H & 1) || (W & 1) || C > 65535) return false;
+  vecw = (W % 4 == 0 && aligned) ? 4 : 2;
+  const int64_t words = N * C * (H / 2) * (W / vecw);
+  if (words >= (1ll << 32) - kThreads || N * (H / 2) * (W / vecw) >= (1ll << 31)) return false;
+  g.wq = FastDiv(static_cast<uint32_t>(W / vecw));
+  g.rows = FastDiv(static_cast<uint32_t>(H / 2));
+  g.chans = FastDiv(static_cast<uint32_t>(C));
+  g.words = static_cast<uint32_t>(words);
+  g.H = static_cast<int>(H);
+  g.W = static_cast<int>(W);
+  return true;
+}
+
 inline const float *cf(const DLArray *a) { return static_cast<const float *>(a->data); }
 inline float *mf(DLArray *a) { return static_cast<float *>(a->data); }
 
@@ -912,6 +1108,150 @@ int TSplit_BatchNormRelu_gradient(const DLArrayHandle gradient_Y, const DLArrayH
                                   DLStreamHandle stream_handle, ProfilerHandle p) {
   return bn_backward("TSplit_BatchNormRelu_gradient", true, gradient_Y, input_X, bn_scale, bn_bias, gradient_X,
                      gradient_bn_scale, gradient_bn_bias, eps, save_mean_arr, save_var_arr, stream_handle, p);
+}
+
+// ---- BatchNorm + Relu + 2x2 / stride 2 max pooling as one call each way (outside the reference's ABI) ----
+static int bn_relu_pool_forward(const char *who, const DLArrayHandle input_X, const DLArrayHandle stats, int slots,
+                                const DLArrayHandle bn_scale, const DLArrayHandle bn_bias, DLArrayHandle output_Y, float eps,
+                                DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr, DLStreamHandle stream_handle,
+                                ProfilerHandle p) {
+  TS_REQUIRE(input_X && bn_scale && bn_bias && output_Y && save_mean_arr && save_var_arr, "%s: NULL array", who);
+  TS_REQUIRE(input_X->ndim == 4 && output_Y->ndim == 4, "%s: input and output must be 4-D NCHW", who);
+  const int64_t N = input_X->shape[0], C = input_X->shape[1], H = input_X->shape[2], W = input_X->shape[3];
+  TS_REQUIRE(H % 2 == 0 && W % 2 == 0, "%s: height and width must be even, got %lld x %lld", who, (long long)H, (long long)W);
+  TS_REQUIRE(output_Y->shape[0] == N && output_Y->shape[1] == C && output_Y->shape[2] == H / 2 && output_Y->shape[3] == W / 2,
+             "%s: the output must be [N][C][H/2][W/2]", who);
+  TS_REQUIRE(numel(bn_scale) == C && numel(bn_bias) == C, "%s: scale/bias must hold C=%lld elements", who, (long long)C);
+  TS_REQUIRE(numel(save_mean_arr) == C && numel(save_var_arr) == C, "%s: the save arrays must hold C elements", who);
+  if (stats) {
+    TS_REQUIRE(slots >= 1 && numel(stats) >= static_cast<int64_t>(slots) * C * 4, "%s: stats must hold slots * C * 4 floats", who);
+    TS_REQUIRE((reinterpret_cast<uintptr_t>(stats->data) & 7) == 0, "%s: stats must be 8-byte aligned", who);
+  }
+  hipStream_t s = stream_of(stream_handle);
+  ProfileScope ps(p, s, numel(input_X) + 2 * C, numel(output_Y), 0);
+  if (numel(input_X) == 0) return ps.finish();
+  int vecw = 2;
+  PoolGeo pg;
+  TS_REQUIRE(make_pool_geo(input_X, aligned16(input_X->data) && (reinterpret_cast<uintptr_t>(output_Y->data) & 7) == 0, vecw, pg),
+             "%s: unsupported shape", who);
+  const double inv_m = 1.0 / static_cast<double>(N * H * W);
+  const unsigned Cu = static_cast<unsigned>(C);
+  float *coef = nullptr;
+  if (stats) {
+    coef = static_cast<float *>(scratch_get(s, 1, static_cast<size_t>(C) * 2 * sizeof(float)));
+    TS_REQUIRE(coef, "%s: no scratch memory", who);
+    hipLaunchKernelGGL(bn_coef_kernel<true>, dim3(Cu), dim3(kThreads), 0, s, static_cast<const double *>(stats->data), slots,
+                       static_cast<int64_t>(1), C, cf(bn_scale), cf(bn_bias), eps, inv_m, coef, mf(save_mean_arr),
+                       mf(save_var_arr));
+  } else {
+    Plan st;
+    TS_REQUIRE(make_plan(input_X, aligned16(input_X->data), kStatsWords, 16384, st), "%s: unsupported shape", who);
+    double *part = static_cast<double *>(scratch_get(s, 1, static_cast<size_t>(C) * st.S * 2 * sizeof(double) +
+                                                               static_cast<size_t>(C) * 2 * sizeof(float)));
+    TS_REQUIRE(part, "%s: no scratch memory", who);
+    coef = reinterpret_cast<float *>(part + static_cast<size_t>(C) * st.S * 2);
+    const dim3 gs(st.S, Cu);
+    if (st.vec == 4)
+      hipLaunchKernelGGL(bn_stats_kernel<4>, gs, dim3(kThreads), 0, s, cf(input_X), part, st.g, st.S);
+    else
+      hipLaunchKernelGGL(bn_stats_kernel<1>, gs, dim3(kThreads), 0, s, cf(input_X), part, st.g, st.S);
+    hipLaunchKernelGGL(bn_coef_kernel<true>, dim3(Cu), dim3(kThreads), 0, s, static_cast<const double *>(part), st.S,
+                       static_cast<int64_t>(st.S), static_cast<int64_t>(1), cf(bn_scale), cf(bn_bias), eps, inv_m, coef,
+                       mf(save_mean_arr), mf(save_var_arr));
+  }
+  const unsigned blocks = (pg.words + kThreads - 1) / kThreads;
+  if (vecw == 4)
+    hipLaunchKernelGGL(bn_relu_pool_kernel<4>, dim3(blocks), dim3(kThreads), 0, s, cf(input_X), mf(output_Y),
+                       static_cast<const float *>(coef), pg);
+  else
+    hipLaunchKernelGGL(bn_relu_pool_kernel<2>, dim3(blocks), dim3(kThreads), 0, s, cf(input_X), mf(output_Y),
+                       static_cast<const float *>(coef), pg);
+  return ps.finish();
+}
+
+// BatchNorm + Relu + max pooling (2x2 windows, stride 2, no padding) forward: output_Y [N][C][H/2][W/2] from
+// input_X [N][C][H][W] (H, W even); the save arrays as TSplit_BatchNormRelu leaves them.
+int TSplit_BatchNormReluMaxPool(const DLArrayHandle input_X, const DLArrayHandle bn_scale, const DLArrayHandle bn_bias,
+                                DLArrayHandle output_Y, float eps, DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                                DLStreamHandle stream_handle, ProfilerHandle p) {
+  return bn_relu_pool_forward("TSplit_BatchNormReluMaxPool", input_X, nullptr, 0, bn_scale, bn_bias, output_Y, eps,
+                              save_mean_arr, save_var_arr, stream_handle, p);
+}
+
+// The same with the batch statistics taken from rows 0 .. slots-1 of `stats` (as TSplit_BatchNormFromStats).
+int TSplit_BatchNormReluMaxPoolFromStats(const DLArrayHandle input_X, const DLArrayHandle stats, int slots,
+                                         const DLArrayHandle bn_scale, const DLArrayHandle bn_bias, DLArrayHandle output_Y,
+                                         float eps, DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                                         DLStreamHandle stream_handle, ProfilerHandle p) {
+  const char *who = "TSplit_BatchNormReluMaxPoolFromStats";
+  TS_REQUIRE(stats, "%s: NULL array", who);
+  return bn_relu_pool_forward(who, input_X, stats, slots, bn_scale, bn_bias, output_Y, eps, save_mean_arr, save_var_arr,
+                              stream_handle, p);
+}
+
+// Their gradient: gradient_Y is the pooled tensor's gradient [N][C][H/2][W/2], input_X the BatchNorm's input,
+// gradient_X its gradient; the statistics are those the forward call saved.
+int TSplit_BatchNormReluMaxPool_gradient(const DLArrayHandle gradient_Y, const DLArrayHandle input_X,
+                                         const DLArrayHandle bn_scale, const DLArrayHandle bn_bias, DLArrayHandle gradient_X,
+                                         DLArrayHandle gradient_bn_scale, DLArrayHandle gradient_bn_bias, float eps,
+                                         DLArrayHandle save_mean_arr, DLArrayHandle save_var_arr,
+                                         DLStreamHandle stream_handle, ProfilerHandle p) {
+  const char *who = "TSplit_BatchNormReluMaxPool_gradient";
+  TS_REQUIRE(gradient_Y && input_X && bn_scale && bn_bias && gradient_X && save_mean_arr && save_var_arr, "%s: NULL array", who);
+  TS_REQUIRE(input_X->ndim == 4 && gradient_Y->ndim == 4, "%s: arrays must be 4-D NCHW", who);
+  const int64_t N = input_X->shape[0], C = input_X->shape[1], H = input_X->shape[2], W = input_X->shape[3];
+  TS_REQUIRE(H % 2 == 0 && W % 2 == 0, "%s: height and width must be even, got %lld x %lld", who, (long long)H, (long long)W);
+  TS_REQUIRE(gradient_Y->shape[0] == N && gradient_Y->shape[1] == C && gradient_Y->shape[2] == H / 2 &&
+                 gradient_Y->shape[3] == W / 2, "%s: the pooled gradient must be [N][C][H/2][W/2]", who);
+  TS_REQUIRE(numel(gradient_X) == numel(input_X), "%s: x and dx sizes differ", who);
+  TS_REQUIRE(numel(bn_scale) == C && numel(bn_bias) == C && numel(save_mean_arr) == C && numel(save_var_arr) == C,
+             "%s: scale, bias and the saved statistics must hold C elements", who);
+  TS_REQUIRE(!gradient_bn_scale || numel(gradient_bn_scale) == C, "%s: dscale must hold C elements", who);
+  TS_REQUIRE(!gradient_bn_bias || numel(gradient_bn_bias) == C, "%s: dbias must hold C elements", who);
+  hipStream_t s = stream_of(stream_handle);
+  int vecw = 2;
+  PoolGeo pg;
+  const bool al = aligned16(input_X->data) && aligned16(gradient_X->data) && (reinterpret_cast<uintptr_t>(gradient_Y->data) & 7) == 0;
+  TS_REQUIRE(make_pool_geo(input_X, al, vecw, pg), "%s: unsupported shape", who);
+  // a channel's words, cut into S ranges of whole blocks' worth
+  const uint32_t wpp = static_cast<uint32_t>((H / 2) * (W / vecw));
+  const uint32_t words_c = static_cast<uint32_t>(N) * wpp;
+  int64_t S = (words_c + kStatsWords / 2 - 1) / (kStatsWords / 2);
+  const int64_t cap = 16384 / C > 0 ? 16384 / C : 1;
+  if (S > cap) S = cap;
+  if (S < 1) S = 1;
+  uint32_t chunk = static_cast<uint32_t>((words_c + S - 1) / S);
+  chunk = (chunk + kThreads - 1) / kThreads * kThreads;
+  S = (words_c + chunk - 1) / chunk;
+  double *part = static_cast<double *>(scratch_get(s, 1, static_cast<size_t>(C) * S * 4 * sizeof(double) +
+                                                             static_cast<size_t>(C) * 5 * sizeof(float)));
+  TS_REQUIRE(part, "%s: no scratch memory", who);
+  float *coef = reinterpret_cast<float *>(part + static_cast<size_t>(C) * S * 4);
+  ProfileScope ps(p, s, 2 * numel(input_X) + 2 * numel(gradient_Y) + C, numel(gradient_X) + 2 * C, C * S * 8);
+  if (numel(input_X) == 0) return ps.finish();
+  const double inv_m = 1.0 / static_cast<double>(N * H * W);
+  const unsigned Cu = static_cast<unsigned>(C);
+  const dim3 gr(static_cast<unsigned>(S), Cu);
+  const unsigned blocks = (pg.words + kThreads - 1) / kThreads;
+  float *dg = gradient_bn_scale ? mf(gradient_bn_scale) : nullptr;
+  float *db = gradient_bn_bias ? mf(gradient_bn_bias) : nullptr;
+#define BN_POOL_BWD(V)                                                                                               \
+  do {                                                                                                               \
+    hipLaunchKernelGGL(bn_pool_bwd_reduce_kernel<V>, gr, dim3(kThreads), 0, s, cf(gradient_Y), cf(input_X), part, pg, \
+                       FastDiv(wpp), words_c, chunk, static_cast<int>(S), cf(bn_scale), cf(bn_bias),                 \
+                       cf(save_mean_arr), cf(save_var_arr));                                                         \
+    hipLaunchKernelGGL(bn_bwd_coef_kernel<true>, dim3(Cu), dim3(kThreads), 0, s, static_cast<const double *>(part),  \
+                       static_cast<int>(S), cf(bn_scale), cf(bn_bias), eps, inv_m, cf(save_mean_arr),                \
+                       cf(save_var_arr), coef, dg, db);                                                              \
+    hipLaunchKernelGGL(bn_pool_bwd_dx_kernel<V>, dim3(blocks), dim3(kThreads), 0, s, cf(gradient_Y), cf(input_X),    \
+                       mf(gradient_X), static_cast<const float *>(coef), pg);                                        \
+  } while (0)
+  if (vecw == 4)
+    BN_POOL_BWD(4);
+  else
+    BN_POOL_BWD(2);
+#undef BN_POOL_BWD
+  return ps.finish();
 }
 
 }  // extern "C"

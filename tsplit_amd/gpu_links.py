@@ -457,6 +457,27 @@ def batch_norm_relu(in_arr, bn_scale_arr, bn_bias_arr, out_arr, save_mean, save_
                                          ctypes.c_float(eps), _h(save_mean), _h(save_var), _s(stream), _p(profiler)))
 
 
+def batch_norm_relu_max_pool(in_arr, bn_scale_arr, bn_bias_arr, out_arr, save_mean, save_var, eps=0.01, stats=None, slots=0,
+                             stream=None, profiler=None):
+    """BatchNorm + Relu + 2x2 / stride 2 max pooling forward in one call: out_arr is the pooled tensor.  With
+    `stats` (rows 0 .. slots-1 of a convolution's sums) the batch statistics come from there."""
+    if stats is None:
+        check_call(_LIB.TSplit_BatchNormReluMaxPool(_h(in_arr), _h(bn_scale_arr), _h(bn_bias_arr), _h(out_arr),
+                                                    ctypes.c_float(eps), _h(save_mean), _h(save_var), _s(stream), _p(profiler)))
+    else:
+        check_call(_LIB.TSplit_BatchNormReluMaxPoolFromStats(_h(in_arr), _h(stats), int(slots), _h(bn_scale_arr),
+                                                             _h(bn_bias_arr), _h(out_arr), ctypes.c_float(eps), _h(save_mean),
+                                                             _h(save_var), _s(stream), _p(profiler)))
+
+
+def batch_norm_relu_max_pool_gradient(gradient_pooled, in_arr, bn_scale_arr, bn_bias_arr, gradient_in, gradient_scale,
+                                      gradient_bias, save_mean, save_var, eps=0.01, stream=None, profiler=None):
+    check_call(_LIB.TSplit_BatchNormReluMaxPool_gradient(_h(gradient_pooled), _h(in_arr), _h(bn_scale_arr), _h(bn_bias_arr),
+                                                         _h(gradient_in), _h(gradient_scale), _h(gradient_bias),
+                                                         ctypes.c_float(eps), _h(save_mean), _h(save_var), _s(stream),
+                                                         _p(profiler)))
+
+
 def conv2d_batch_norm_stats(in_arr_x, in_arr_f, out_arr, stats, slot, padding=0, padding2=None, stride=1, stream=None,
                             profiler=None):
     """CuDNN_conv2d that also writes the per-channel (sum, sum of squares) of out_arr into row `slot` of

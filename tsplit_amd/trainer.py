@@ -118,7 +118,7 @@ def _out_shape(layer, s):
 class Trainer(object):
     def __init__(self, spec, params, input_shape, num_classes, ctx=None, optimizer=("sgd", 0.1),
                  split=None, bn_eps=0.01, timer=None, fuse_bn_relu=False, conv_bn_stats=False,
-                 multi_tensor_update=False):
+                 multi_tensor_update=False, fuse_max_pool=False):
         self.spec = list(spec)
         # with fuse_bn_relu a ("bn", ...) layer directly followed by ("relu",) runs as ONE fused call
         # in each direction (symbols outside the reference's ABI); the Relu layer's own arrays are
@@ -126,6 +126,11 @@ class Trainer(object):
         self.fused = set()
         if fuse_bn_relu:
             self.fused = {li for li, l in enumerate(self.spec[:-1]) if l[0] == "bn" and self.spec[li + 1][0] == "relu"}
+        # with fuse_max_pool a fused pair directly followed by ("maxpool", 2, 0, 2) on planes of even height and
+        # width runs as ONE call each way together with the pooling (symbols outside the reference's ABI): the
+        # activation in front of the pooling is never written (filled in below, where the shapes are known)
+        self.fused_pool = set()
+        want_pool = bool(fuse_max_pool and fuse_bn_relu)
         # with conv_bn_stats a ("conv", ...) layer directly followed by ("bn", ...) hands the BatchNorm its
         # batch statistics (one row of sums per micro-tensor; symbols outside the reference's ABI), so
         # the BatchNorm reads the convolution's output once instead of twice
@@ -156,9 +161,13 @@ class Trainer(object):
         s = tuple(input_shape)
         self.shapes = [s]
         for li, layer in enumerate(self.spec):
+            if (want_pool and li in self.fused and li + 2 < len(self.spec) and tuple(self.spec[li + 2]) == ("maxpool", 2, 0, 2)
+                    and s[2] % 2 == 0 and s[3] % 2 == 0):
+                self.fused_pool.add(li)
             s = _out_shape(layer, s)
             self.shapes.append(s)
-            unused = li in self.fused          # the BN output of a fused pair never exists
+            # the BN output of a fused pair never exists, nor the Relu output in front of a fused pooling
+            unused = li in self.fused or (layer[0] == "relu" and li - 1 in self.fused_pool)
             self.acts.append(None if unused else ndarray.empty(s, self.ctx))
             self.dacts.append(None if unused else ndarray.empty(s, self.ctx))
             if layer[0] == "bn":
@@ -226,6 +235,15 @@ class Trainer(object):
                         self._run(tag, 4.0 * (n(xa.shape) + n(w.shape) + n(ya.shape)), "byte", call, *args)
                     else:
                         self._run(tag, 2.0 * n(ya.shape) * cin * k * k, "flop", call, *args)
+            elif kind == "bn" and li in self.fused_pool:
+                name = layer[1]
+                sm, sv = self.saved[li]
+                pooled = self.acts[li + 3]
+                from_stats = li - 1 in self.stats_of
+                self._run("bn_relu_pool_fwd_from_stats" if from_stats else "bn_relu_pool_fwd", 4.0 * (n(a.shape) + n(pooled.shape)),
+                          "byte", L.batch_norm_relu_max_pool, a, self.params[name + "_scale"], self.params[name + "_bias"],
+                          pooled, sm, sv, self.eps, self.stats_of[li - 1] if from_stats else None,
+                          self.split.get(li - 1, 1) if from_stats else 0)
             elif kind == "bn" and li - 1 in self.stats_of:
                 name = layer[1]
                 sm, sv = self.saved[li]
@@ -249,6 +267,8 @@ class Trainer(object):
                 pass
             elif kind == "relu":
                 self._run("relu_fwd", 8.0 * n(a.shape), "byte", L.relu, a, out)
+            elif kind == "maxpool" and li - 2 in self.fused_pool:
+                pass
             elif kind == "maxpool":
                 _, k, pad, stride = layer
                 self._run("maxpool_fwd", 4.0 * (n(a.shape) + n(out.shape)), "byte", L.CuDNN_max_pooling2d, a, k, k, out,
@@ -303,6 +323,13 @@ class Trainer(object):
                         self._run("conv_bwd_data_winograd" if wino else "conv_bwd_data_" + self._tile(cin),
                                   2.0 * n(ga.shape) * cin * k * k, "flop",
                                   L.CuDNN_conv2d_gradient_of_data, w, ga, gi, pad, pad, stride)
+            elif kind == "bn" and li in self.fused_pool:
+                name = layer[1]
+                sm, sv = self.saved[li]
+                gp = self.dacts[li + 3]      # the gradient behind the pooling
+                self._run("bn_relu_pool_bwd", 4.0 * (2 * n(a.shape) + n(gp.shape)), "byte", L.batch_norm_relu_max_pool_gradient,
+                          gp, a, self.params[name + "_scale"], self.params[name + "_bias"], g_in,
+                          self.grads[name + "_scale"], self.grads[name + "_bias"], sm, sv, self.eps)
             elif kind == "bn" and li in self.fused:
                 name = layer[1]
                 sm, sv = self.saved[li]
@@ -320,6 +347,8 @@ class Trainer(object):
                 pass
             elif kind == "relu":
                 self._run("relu_bwd", 12.0 * n(a.shape), "byte", L.relu_gradient, a, g_out, g_in)
+            elif kind == "maxpool" and li - 2 in self.fused_pool:
+                pass
             elif kind == "maxpool":
                 _, k, pad, stride = layer
                 self._run("maxpool_bwd", 4.0 * (2 * n(a.shape) + n(g_out.shape)), "byte",
