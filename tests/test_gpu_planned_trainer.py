@@ -26,11 +26,16 @@ def _data(rng):
     return x, labels
 
 
+def _fuse(fused):
+    """False: the layers as they are; True: BatchNorm+Relu pairs merged; "pool": and the pooling behind them."""
+    return planner.fuse_spec(SPEC, pool=fused == "pool", input_shape=IN) if fused else SPEC
+
+
 def _plain_losses(spec_fused, steps, rng_seed=5):
     from tsplit_amd import ndarray
     rng = np.random.RandomState(rng_seed)
     params = trainer.init_params(SPEC, seed=3)
-    t = trainer.Trainer(SPEC, params, IN, 10, optimizer=OPT, fuse_bn_relu=spec_fused)
+    t = trainer.Trainer(SPEC, params, IN, 10, optimizer=OPT, fuse_bn_relu=bool(spec_fused), fuse_max_pool=spec_fused == "pool")
     x, labels = _data(rng)
     gx, gl = ndarray.array(x, t.ctx), ndarray.array(labels, t.ctx)
     out = []
@@ -94,9 +99,9 @@ def _planned(spec, budget_frac, steps, piece_bytes=64 << 10, rng_seed=5, allow_r
     return out, {k: v.asnumpy() for k, v in t.params.items()}, t, plan, free
 
 
-@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("fused", [False, True, "pool"])
 def test_unlimited_budget_equals_plain_trainer(fused):
-    spec = planner.fuse_spec(SPEC) if fused else SPEC
+    spec = _fuse(fused)
     want, wp = _plain_losses(fused, 4)
     got, gp, t, plan, _ = _planned(spec, None, 4)
     assert not plan.swap
@@ -114,10 +119,10 @@ def test_unlimited_budget_equals_plain_trainer(fused):
     assert t2.peak == plan.peak_bytes and got2 == want
 
 
-@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("fused", [False, True, "pool"])
 @pytest.mark.parametrize("frac", [0.6, 0.1])
 def test_budget_is_met_and_results_do_not_change(fused, frac):
-    spec = planner.fuse_spec(SPEC) if fused else SPEC
+    spec = _fuse(fused)
     want, wp = _plain_losses(fused, 4)
     got, gp, t, plan, free = _planned(spec, frac, 4)
     assert plan.swap and plan.budget_bytes < free.peak_bytes
@@ -137,13 +142,13 @@ def test_impossible_budget_is_refused():
         make_plan(SPEC, IN, 10, 64 << 10, OPT)
 
 
-@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("fused", [False, True, "pool"])
 @pytest.mark.parametrize("frac", [0.6, 0.3, 0.1])
 def test_recomputation_meets_the_budget_with_the_same_bits(fused, frac):
     """With recomputation allowed the plan drops BatchNorm / Relu outputs and computes them again in the
     backward sweep; computing a tensor again gives the bits it had, so the results equal the plain
     trainer's exactly wherever no convolution is split, and the executor's peak is the replayed one."""
-    spec = planner.fuse_spec(SPEC) if fused else SPEC
+    spec = _fuse(fused)
     want, wp = _plain_losses(fused, 4)
     got, gp, t, plan, free = _planned(spec, frac, 4, allow_recompute=True)
     assert plan.recompute and plan.budget_bytes < free.peak_bytes

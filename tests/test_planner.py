@@ -18,6 +18,26 @@ def test_fuse_spec_merges_bn_relu_pairs_only():
     assert planner.layer_shapes(f, IN)[-1] == (4, 10)
 
 
+def test_fuse_spec_takes_the_pooling_behind_a_pair_where_the_planes_are_even():
+    f = planner.fuse_spec(SMALL, pool=True, input_shape=IN)
+    assert [l[0] for l in f] == ["conv", "bnrelu", "conv", "bnrelupool", "flatten", "fc"]
+    assert f[3] == ("bnrelupool", "c2_bn", 8)
+    assert planner.layer_shapes(f, IN)[4] == (4, 8, 8, 8) and planner.layer_shapes(f, IN)[-1] == (4, 10)
+    # odd planes, other windows or a pooling that does not follow directly stay as they are
+    odd = planner.fuse_spec(SMALL, pool=True, input_shape=(4, 3, 15, 15))
+    assert [l[0] for l in odd] == ["conv", "bnrelu", "conv", "bnrelu", "maxpool", "flatten", "fc"]
+    other = [("bn", "x", 4), ("relu",), ("maxpool", 3, 1, 2)]
+    assert [l[0] for l in planner.fuse_spec(other, pool=True, input_shape=(2, 4, 8, 8))] == ["bnrelu", "maxpool"]
+    # the activation in front of the pooling never exists: VGG-16 at batch 64 holds 1.57 GB less
+    spec = trainer.vgg16_spec(1000, 224)
+    shape = (64, 3, 224, 224)
+    pairs = planner.plan_memory(planner.fuse_spec(spec), shape, None, 0)
+    ends = planner.plan_memory(planner.fuse_spec(spec, pool=True, input_shape=shape), shape, None, 0)
+    shapes = planner.layer_shapes(spec, shape)
+    pre_pool = sum(planner.tensor_bytes(shapes)[i] for i, l in enumerate(spec) if l[0] == "maxpool")
+    assert pairs.peak_bytes - ends.peak_bytes >= pre_pool > 1.5e9
+
+
 def test_simulate_without_swapping_holds_every_activation_at_the_turn():
     shapes = planner.layer_shapes(SMALL, IN)
     size = planner.tensor_bytes(shapes)

@@ -1,7 +1,7 @@
 """VGG-16 training throughput under device-memory budgets (one MI355X).
 
-    python -m tsplit_amd.planbench [--budgets 0,8,7,6.5] [--fused] [--recompute] [--steps 5] [--warmup 2] [--batch 64]
-    python -m tsplit_amd.planbench --max-batch [--budgets 8,16] [--fused] [--recompute]
+    python -m tsplit_amd.planbench [--budgets 0,8,7,6.5] [--fused] [--fused-pool] [--recompute] [--steps 5] [--warmup 2] [--batch 64]
+    python -m tsplit_amd.planbench --max-batch [--budgets 8,16] [--fused] [--fused-pool] [--recompute]
 
 For every budget (GiB; 0 = no limit) the planner chooses which activations leave for pinned
 host memory (and, with --recompute, which BatchNorm / Relu outputs are dropped and computed again in
@@ -23,6 +23,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--budgets", default="0,8,7,6.5")
     ap.add_argument("--fused", action="store_true")
+    ap.add_argument("--fused-pool", action="store_true", help="with --fused: the max pooling behind a BatchNorm+Relu pair joins it")
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--batch", type=int, default=64)
@@ -34,7 +35,7 @@ def main():
     spec = trainer.vgg16_spec(1000, 224)
     params = trainer.init_params(spec, seed=123)
     if a.fused:
-        spec = planner.fuse_spec(spec)
+        spec = planner.fuse_spec(spec, pool=a.fused_pool, input_shape=(a.batch, 3, 224, 224))
     opt = ("momentum", 1e-4, 0.9)
     if a.max_batch:
         return max_batch_sweep(a, spec, params, opt)
@@ -60,7 +61,7 @@ def main():
             t.step(gx, gl)
         dt = (time.perf_counter() - t0) / a.steps
         d = plan.describe()
-        print(json.dumps({"budget_GiB": b, "fused_bn_relu": a.fused, "recompute": a.recompute, "samples_per_s": a.batch / dt, "ms_per_step": dt * 1e3,
+        print(json.dumps({"budget_GiB": b, "fused_bn_relu": a.fused, "fused_max_pool": bool(a.fused and a.fused_pool), "recompute": a.recompute, "samples_per_s": a.batch / dt, "ms_per_step": dt * 1e3,
                           "measured_peak_GiB": t.peak / planner.GiB, "planned_peak_GiB": d["peak_GiB"],
                           "estimated_ms_per_step": d["est_step_ms"],
                           "tensors_swapped": len(plan.swap), "swapped_GiB": sum(4 * int(np.prod(t.shapes[j])) for j in plan.swap) / planner.GiB,
@@ -78,7 +79,7 @@ def max_batch_sweep(a, spec, params, opt):
         budget = int(b * (1 << 30))
         resident, _ = max_batch(spec, (3, 224, 224), 1000, budget, opt, swap=False)
         planned, plan = max_batch(spec, (3, 224, 224), 1000, budget, opt, swap=True, allow_recompute=a.recompute)
-        row = {"budget_GiB": b, "fused_bn_relu": a.fused, "recompute": a.recompute, "max_batch_resident": resident,
+        row = {"budget_GiB": b, "fused_bn_relu": a.fused, "fused_max_pool": bool(a.fused and a.fused_pool), "recompute": a.recompute, "max_batch_resident": resident,
                "max_batch_planned": planned}
         if plan is not None:
             in_shape = (planned, 3, 224, 224)

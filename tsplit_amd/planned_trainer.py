@@ -36,7 +36,7 @@ def fixed_bytes(spec, input_shape, num_classes, optimizer, split=()):
     shapes = param_shapes(spec)
     params = sum(4 * int(np.prod(s)) for s in shapes.values())
     total = params * (3 if optimizer[0] == "momentum" else 2)
-    total += sum(2 * 4 * l[2] for l in spec if l[0] in ("bn", "bnrelu"))
+    total += sum(2 * 4 * l[2] for l in spec if l[0] in ("bn", "bnrelu", "bnrelupool"))
     total += sum(4 * int(np.prod(shapes[spec[li][1] + "_weight"])) for li in split)
     total += 8 + 4 * input_shape[0] * num_classes
     return total
@@ -125,7 +125,7 @@ class PlannedTrainer(object):
             self.state = {k: self._own(ndarray.array(np.zeros(v.shape, np.float32), self.ctx)) for k, v in params.items()}
         self.saved = {}
         for li, layer in enumerate(self.spec):
-            if layer[0] in ("bn", "bnrelu"):
+            if layer[0] in ("bn", "bnrelu", "bnrelupool"):
                 c = layer[2]
                 self.saved[li] = (self._own(ndarray.empty((1, c, 1, 1), self.ctx)),
                                   self._own(ndarray.empty((1, c, 1, 1), self.ctx)))
@@ -264,6 +264,10 @@ class PlannedTrainer(object):
                 sm, sv = self.saved[li]
                 L.batch_norm_relu(a, self.params[layer[1] + "_scale"], self.params[layer[1] + "_bias"], out, sm, sv,
                                   self.eps, self.stream)
+            elif kind == "bnrelupool":
+                sm, sv = self.saved[li]
+                L.batch_norm_relu_max_pool(a, self.params[layer[1] + "_scale"], self.params[layer[1] + "_bias"], out, sm, sv,
+                                           self.eps, stream=self.stream)
             elif kind == "bn":
                 sm, sv = self.saved[li]
                 L.CuDNN_Batch_Normalization(a, self.params[layer[1] + "_scale"], self.params[layer[1] + "_bias"], out,
@@ -306,6 +310,10 @@ class PlannedTrainer(object):
             sm, sv = self.saved[j - 1]
             L.batch_norm_relu(src, self.params[layer[1] + "_scale"], self.params[layer[1] + "_bias"], out, sm, sv,
                               self.eps, self.stream)
+        elif kind == "bnrelupool":
+            sm, sv = self.saved[j - 1]
+            L.batch_norm_relu_max_pool(src, self.params[layer[1] + "_scale"], self.params[layer[1] + "_bias"], out, sm, sv,
+                                       self.eps, stream=self.stream)
         elif kind == "bn":
             sm, sv = self.saved[j - 1]
             L.CuDNN_Batch_Normalization(src, self.params[layer[1] + "_scale"], self.params[layer[1] + "_bias"], out,
@@ -363,6 +371,12 @@ class PlannedTrainer(object):
                     L.batch_norm_relu_gradient(g_out, a, self.params[name + "_scale"], self.params[name + "_bias"], g_in,
                                                self.grads[name + "_scale"], self.grads[name + "_bias"], sm, sv, self.eps,
                                                self.stream)
+                elif kind == "bnrelupool":
+                    sm, sv = self.saved[li]
+                    name = layer[1]
+                    L.batch_norm_relu_max_pool_gradient(g_out, a, self.params[name + "_scale"], self.params[name + "_bias"],
+                                                        g_in, self.grads[name + "_scale"], self.grads[name + "_bias"], sm, sv,
+                                                        self.eps, self.stream)
                 elif kind == "bn":
                     sm, sv = self.saved[li]
                     name = layer[1]

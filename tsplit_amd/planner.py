@@ -12,7 +12,9 @@ Model.  Tensor j is the input of layer j (tensor 0 is the batch, tensor L the lo
 tensor is needed again in the backward sweep (by the layer that consumed it, and a max-pool's
 output also by the pool itself).  A BatchNorm directly followed by a Relu may be merged into one
 "bnrelu" layer (`fuse_spec`), which runs on the fused entry points and never materialises the
-BatchNorm output.  The executor (`tsplit_amd.planned_trainer`) follows this
+BatchNorm output; with a 2x2 / stride 2 max pooling behind the pair the three may be merged into one
+"bnrelupool" layer, which never materialises the activation in front of the pooling either and does not
+need its own output in the backward sweep.  The executor (`tsplit_amd.planned_trainer`) follows this
 schedule, which `simulate` replays byte for byte:
 
   forward  of layer i : allocate tensor i+1, run; then a swapped tensor i starts leaving
@@ -52,15 +54,29 @@ class CostModel(object):
     event wait costs the compute stream (the host has to catch up with its launches afterwards;
     a swapped tensor brings one such wait on the way out and one on the way in)."""
 
-    def __init__(self, conv_tflops=110.0, conv_tflops_narrow=90.0, matmul_tflops=65.0, stream_gbs=5500.0,
-                 link_gbs=55.0, host_wait_ms=0.2, conv_tflops_winograd=240.0):
+    def __init__(self, conv_tflops=110.0, conv_tflops_narrow=90.0, matmul_tflops=45.0, stream_gbs=5900.0,
+                 link_gbs=55.0, host_wait_ms=0.2, thin_gbs=2900.0):
         self.host_wait_ms = host_wait_ms
-        self.conv_tflops_winograd = conv_tflops_winograd
         self.conv_tflops = conv_tflops
         self.conv_tflops_narrow = conv_tflops_narrow
         self.matmul_tflops = matmul_tflops
         self.stream_gbs = stream_gbs
         self.link_gbs = link_gbs
+        self.thin_gbs = thin_gbs
+
+    @staticmethod
+    def winograd_tflops(cin, cout, plane):
+        """Rate of the direct algorithm's FLOP count of a 3x3 / stride 1 / pad 1 layer under the Winograd routine
+        (all three passes together), as measured layer by layer on the VGG-16 shapes: the transforms' share
+        falls and the GEMMs' depth grows with the channel count; the 14 x 14 planes leave a sparse last round."""
+        lo, hi = min(cin, cout), max(cin, cout)
+        if lo < 128:
+            return 125.0 if hi < 128 else 157.0
+        if lo < 256:
+            return 207.0 if hi < 256 else 255.0
+        if lo < 512:
+            return 311.0
+        return 368.0 if plane >= 28 else 231.0
 
     def copy_ms(self, nbytes):
         return nbytes / (self.link_gbs * 1e9) * 1e3
@@ -72,16 +88,19 @@ class CostModel(object):
         if kind == "conv":
             _, _, cin, cout, k, pad, stride = layer
             flop = 2.0 * n_out * cin * k * k
-            rate = self.conv_tflops if min(cin, cout) > 64 else self.conv_tflops_narrow
-            if (k, pad, stride) == (3, 1, 1) and min(cin, cout) >= 64 and max(cin, cout) >= 128:
-                rate = self.conv_tflops_winograd     # wide 3x3 layers run through the Winograd routine
             passes = (1 if first else 2) if backward else 1
+            if cin * k * k <= 32:      # a first layer on 3 channels: bound by writing (reading) the wide side
+                return passes * 4.0 * (n_in + n_out) / (self.thin_gbs * 1e9) * 1e3
+            rate = self.conv_tflops if min(cin, cout) > 64 else self.conv_tflops_narrow
+            if (k, pad, stride) == (3, 1, 1) and min(cin, cout) >= 64:
+                rate = self.winograd_tflops(cin, cout, out_shape[2])     # wide 3x3 layers run through the Winograd routine
             return passes * flop / (rate * 1e12) * 1e3
         if kind == "fc":
             flop = 2.0 * in_shape[0] * layer[2] * layer[3]
             return (2 if backward and not first else 1) * flop / (self.matmul_tflops * 1e12) * 1e3
         moved = {"bn": (20.0 if backward else 12.0) * n_in, "relu": (12.0 if backward else 8.0) * n_in,
                  "bnrelu": (20.0 if backward else 12.0) * n_in,
+                 "bnrelupool": (14.0 if backward else 9.0) * n_in,
                  "maxpool": 4.0 * ((2 * n_in + n_out) if backward else (n_in + n_out)),
                  "flatten": 0.0}[kind]
         return moved / (self.stream_gbs * 1e9) * 1e3
@@ -91,7 +110,7 @@ IN_PLACE_BACKWARD = ("relu", "bn", "bnrelu")   # the input gradient may overwrit
 NEEDS_OUTPUT_BACKWARD = ("maxpool",)           # CuDNN_DLGpuMax_Pooling2d_gradient takes y as well as x
 # layers whose output is cheap to compute again from their input (two or three passes over HBM):
 # such an output may be dropped after its forward use and recomputed when the backward sweep needs it
-CHEAP_TO_REDO = ("relu", "bn", "bnrelu")
+CHEAP_TO_REDO = ("relu", "bn", "bnrelu", "bnrelupool")
 
 
 class MemoryPlan(object):
@@ -120,11 +139,19 @@ class MemoryPlan(object):
                 "budget_GiB": None if self.budget_bytes is None else self.budget_bytes / GiB}
 
 
-def fuse_spec(spec):
-    """("bn", name, C), ("relu",) -> ("bnrelu", name, C)."""
+def fuse_spec(spec, pool=False, input_shape=None):
+    """("bn", name, C), ("relu",) -> ("bnrelu", name, C); with `pool` (and the net's input shape, to know the
+    planes) a pair followed by ("maxpool", 2, 0, 2) on planes of even height and width ->
+    ("bnrelupool", name, C)."""
+    shapes = layer_shapes(spec, input_shape) if pool else None
     out, i = [], 0
     while i < len(spec):
         if spec[i][0] == "bn" and i + 1 < len(spec) and spec[i + 1][0] == "relu":
+            if (pool and i + 2 < len(spec) and tuple(spec[i + 2]) == ("maxpool", 2, 0, 2) and shapes[i][2] % 2 == 0
+                    and shapes[i][3] % 2 == 0):
+                out.append(("bnrelupool",) + tuple(spec[i][1:]))
+                i += 3
+                continue
             out.append(("bnrelu",) + tuple(spec[i][1:]))
             i += 2
         else:

@@ -70,7 +70,7 @@ def param_shapes(spec):
         if layer[0] == "conv":
             _, name, cin, cout, k, _, _ = layer
             shapes[name + "_weight"] = (cout, cin, k, k)
-        elif layer[0] in ("bn", "bnrelu"):
+        elif layer[0] in ("bn", "bnrelu", "bnrelupool"):
             _, name, c = layer
             shapes[name + "_scale"] = (1, c, 1, 1)
             shapes[name + "_bias"] = (1, c, 1, 1)
@@ -105,6 +105,8 @@ def _out_shape(layer, s):
         return (s[0], cout, (s[2] + 2 * pad - k) // stride + 1, (s[3] + 2 * pad - k) // stride + 1)
     if kind in ("bn", "relu", "bnrelu"):
         return s
+    if kind == "bnrelupool":       # BatchNorm + Relu + 2x2 / stride 2 max pooling as one layer
+        return (s[0], s[1], s[2] // 2, s[3] // 2)
     if kind == "maxpool":
         _, k, pad, stride = layer
         return (s[0], s[1], (s[2] + 2 * pad - k) // stride + 1, (s[3] + 2 * pad - k) // stride + 1)
