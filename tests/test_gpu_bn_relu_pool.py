@@ -127,6 +127,16 @@ def test_argument_errors():
         L.batch_norm_relu_max_pool(x, g, g, nd.empty((2, 4, 3, 3), ctx), s1, s2)        # wrong pooled shape
     with pytest.raises(Exception):
         L.batch_norm_relu_max_pool_gradient(nd.empty((2, 4, 3, 3), ctx), x, g, g, nd.empty((2, 4, 6, 8), ctx), s1, s2, s1, s2)
+    # statistics over an empty batch are refused, as the BatchNorm entry points refuse them
+    e, pe = nd.empty((0, 4, 6, 8), ctx), nd.empty((0, 4, 3, 4), ctx)
+    with pytest.raises(Exception):
+        L.batch_norm_relu_max_pool(e, g, g, pe, s1, s2)
+    with pytest.raises(Exception):
+        L.batch_norm_relu_max_pool_gradient(pe, e, g, g, nd.empty((0, 4, 6, 8), ctx), s1, s2, s1, s2)
+    # and the library still works
+    p = nd.empty((2, 4, 3, 4), ctx)
+    L.batch_norm_relu_max_pool(x, g, g, p, s1, s2)
+    np.testing.assert_allclose(p.asnumpy(), 1.0)      # zeros normalise to zero, plus a bias of one
 
 
 def _onehot(lab, n):

@@ -1127,9 +1127,10 @@ static int bn_relu_pool_forward(const char *who, const DLArrayHandle input_X, co
     TS_REQUIRE(slots >= 1 && numel(stats) >= static_cast<int64_t>(slots) * C * 4, "%s: stats must hold slots * C * 4 floats", who);
     TS_REQUIRE((reinterpret_cast<uintptr_t>(stats->data) & 7) == 0, "%s: stats must be 8-byte aligned", who);
   }
+  TS_REQUIRE(numel(input_X) > 0, "%s: batch statistics of an empty tensor", who);
+  TS_REQUIRE((reinterpret_cast<uintptr_t>(input_X->data) & 7) == 0, "%s: the input must be 8-byte aligned", who);
   hipStream_t s = stream_of(stream_handle);
   ProfileScope ps(p, s, numel(input_X) + 2 * C, numel(output_Y), 0);
-  if (numel(input_X) == 0) return ps.finish();
   int vecw = 2;
   PoolGeo pg;
   TS_REQUIRE(make_pool_geo(input_X, aligned16(input_X->data) && (reinterpret_cast<uintptr_t>(output_Y->data) & 7) == 0, vecw, pg),
@@ -1208,7 +1209,10 @@ int TSplit_BatchNormReluMaxPool_gradient(const DLArrayHandle gradient_Y, const D
              "%s: scale, bias and the saved statistics must hold C elements", who);
   TS_REQUIRE(!gradient_bn_scale || numel(gradient_bn_scale) == C, "%s: dscale must hold C elements", who);
   TS_REQUIRE(!gradient_bn_bias || numel(gradient_bn_bias) == C, "%s: dbias must hold C elements", who);
+  TS_REQUIRE(numel(input_X) > 0, "%s: batch statistics of an empty tensor", who);
   hipStream_t s = stream_of(stream_handle);
+  TS_REQUIRE(((reinterpret_cast<uintptr_t>(input_X->data) | reinterpret_cast<uintptr_t>(gradient_X->data)) & 7) == 0,
+             "%s: x and dx must be 8-byte aligned", who);
   int vecw = 2;
   PoolGeo pg;
   const bool al = aligned16(input_X->data) && aligned16(gradient_X->data) && (reinterpret_cast<uintptr_t>(gradient_Y->data) & 7) == 0;
@@ -1228,7 +1232,6 @@ int TSplit_BatchNormReluMaxPool_gradient(const DLArrayHandle gradient_Y, const D
   TS_REQUIRE(part, "%s: no scratch memory", who);
   float *coef = reinterpret_cast<float *>(part + static_cast<size_t>(C) * S * 4);
   ProfileScope ps(p, s, 2 * numel(input_X) + 2 * numel(gradient_Y) + C, numel(gradient_X) + 2 * C, C * S * 8);
-  if (numel(input_X) == 0) return ps.finish();
   const double inv_m = 1.0 / static_cast<double>(N * H * W);
   const unsigned Cu = static_cast<unsigned>(C);
   const dim3 gr(static_cast<unsigned>(S), Cu);
