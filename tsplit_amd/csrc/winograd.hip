@@ -49,9 +49,9 @@ __device__ __forceinline__ void g_rows(float g0, float g1, float g2, float u[6])
 
 // U[xi][o][c], o over the produced channels, c over the gathered ones.  Forward: the filter is
 // stored [o][c][3][3].  Data gradient: stored [c][o][3][3] and read rotated by 180 degrees.
-__global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restrict__ w, float *__restrict__ U, int produced,
-                                                          int gathered, bool rotated) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
+__device__ __forceinline__ void wino_filter_block(const float *__restrict__ w, float *__restrict__ U, int produced, int gathered,
+                                                  bool rotated, int bx) {
+  const int i = bx * 256 + threadIdx.x;
   if (i >= produced * gathered) return;
   const int o = i / gathered, c = i - o * gathered;
   const float *g = w + (rotated ? static_cast<int64_t>(c) * produced + o : static_cast<int64_t>(o) * gathered + c) * 9;
@@ -69,6 +69,16 @@ __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restric
     for (int q = 0; q < 6; ++q) U[static_cast<int64_t>(r * 6 + q) * produced * gathered + i] = u[q];
   }
 }
+// A filter transform that rides in the first rows of another kernel's grid (the input transform of a call's
+// first run: neither depends on the other, and a launch of its own would cost its ramp and tail).
+struct FilterJob {
+  const float *w;
+  float *U;
+  int produced, gathered;
+  bool rotated;
+  int blocks;   // blocks of 256 filter elements; 0: nothing to do
+  int rows;     // grid rows (of the host kernel's width) they take
+};
 
 // ---------------------------------------------------------------- input transform
 // rows of B^T applied to (d0 .. d5)
@@ -90,15 +100,14 @@ struct WinoGeo {
   bool quads;     // output rows may be stored as aligned 16-byte quads
 };
 
-// one thread per (channel, tile): grid (ceil(ld / 256), chans).  With QUADS (W a multiple of 4, planes
+// one thread per (channel, tile).  With QUADS (W a multiple of 4, planes
 // 16-byte aligned) a thread loads the aligned quad of each of its six rows and takes the two columns
 // beside it from the neighbouring lanes, which hold the neighbouring tiles of the same tile row; at
 // a wave's ends those come from memory, at the plane's edges they are the zero padding.
 template <bool QUADS>
-__global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict__ x, float *__restrict__ V, WinoGeo g) {
+__device__ __forceinline__ void wino_input_block(const float *__restrict__ x, float *__restrict__ V, const WinoGeo &g, int c) {
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= g.ld) return;
-  const int c = blockIdx.y;
   float *out = V + static_cast<int64_t>(c) * g.ld + t;
   const int64_t plane_stride = static_cast<int64_t>(g.chans) * g.ld;
   if (t >= g.tiles) {   // padding columns of the GEMMs: defined, and never read back
@@ -158,6 +167,18 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
 #pragma unroll
     for (int q = 0; q < 6; ++q) out[(r * 6 + q) * plane_stride] = v[q];
   }
+}
+// grid (ceil(ld / 256), job.rows + chans): the first job.rows rows are the filter transform's
+template <bool QUADS>
+__global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict__ x, float *__restrict__ V, WinoGeo g,
+                                                         FilterJob job) {
+  const int row = blockIdx.y;
+  if (row < job.rows) {
+    const int fb = row * gridDim.x + blockIdx.x;
+    if (fb < job.blocks) wino_filter_block(job.w, job.U, job.produced, job.gathered, job.rotated, fb);
+    return;
+  }
+  wino_input_block<QUADS>(x, V, g, row - job.rows);
 }
 
 // ---------------------------------------------------------------- output transform
@@ -256,10 +277,9 @@ __device__ __forceinline__ void a_rows(const float d[4], float o[6]) {
 
 // Y[xi][o][t] = (A dy A^T)[xi] of the 4x4 output tile t, channel o (zero beyond the plane's edge)
 template <bool QUADS>
-__global__ __launch_bounds__(256) void wino_grad_kernel(const float *__restrict__ dy, float *__restrict__ Y, WinoGeo g) {
+__device__ __forceinline__ void wino_grad_block(const float *__restrict__ dy, float *__restrict__ Y, const WinoGeo &g, int o) {
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= g.ld) return;
-  const int o = blockIdx.y;
   float *out = Y + static_cast<int64_t>(o) * g.ld + t;
   const int64_t plane_stride = static_cast<int64_t>(g.chans) * g.ld;
   if (t >= g.tiles) {   // padding of the reduction: contributes nothing
@@ -306,6 +326,17 @@ __global__ __launch_bounds__(256) void wino_grad_kernel(const float *__restrict_
     for (int q = 0; q < 6; ++q) out[(r * 6 + q) * plane_stride] = v[q];
   }
 }
+// Both transforms of a filter-gradient run in one launch, grid (ceil(ld / 256), gx.chans + gy.chans): rows
+// below gx.chans transform a channel of x, the others a channel of dy (the two share nothing but the tiling)
+template <bool QUADS_X, bool QUADS_Y>
+__global__ __launch_bounds__(256) void wino_grad_pair_kernel(const float *__restrict__ x, float *__restrict__ V, WinoGeo gx,
+                                                             const float *__restrict__ dy, float *__restrict__ Y, WinoGeo gy) {
+  const int row = blockIdx.y;
+  if (row < gx.chans)
+    wino_input_block<QUADS_X>(x, V, gx, row);
+  else
+    wino_grad_block<QUADS_Y>(dy, Y, gy, row - gx.chans);
+}
 
 // rows of G^T applied to (u0 .. u5)
 __device__ __forceinline__ void gt_rows(const float u[6], float w[3]) {
@@ -315,41 +346,51 @@ __device__ __forceinline__ void gt_rows(const float u[6], float w[3]) {
   w[2] = (s34 - s12) * (1.0f / 6.0f) + u[5];
 }
 
-// part[i] = sum over p of part[p * n + i], p ascending (in place: every thread owns its elements)
-__global__ __launch_bounds__(256) void wino_fold_kernel(float *__restrict__ part, int64_t n, int parts) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (i >= n) return;
-  float sum = part[i];
-  for (int p = 1; p < parts; ++p) sum += part[p * n + i];
-  part[i] = sum;
-}
-
-// dw[o][c][3][3] = G^T (sum of the partial dU, in ascending order) G; part[(p * 36 + xi) * O * C + o * C + c]
+// dw[o][c][3][3] = G^T (sum of the partial dU, in ascending order) G; part[(p * 36 + xi) * O * C + o * C + c].
+// A block takes 64 filter elements (o, c): its four waves each sum nine of the 36 points over the parts
+// (consecutive lanes read consecutive elements), the sums meet in LDS, and the first wave applies G^T . G and
+// stores the 64 x 9 results, which are contiguous in dw, as whole lines.
 __global__ __launch_bounds__(256) void wino_filter_grad_kernel(const float *__restrict__ part, float *__restrict__ dw,
                                                                int oc, int parts) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= oc) return;
-  float t[6][3];   // t[q][.] = G^T applied down column q
+  __shared__ float sums[kXi][64 + 1];
+  __shared__ float outs[64 * 9];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i0 = blockIdx.x * 64, i = i0 + lane;
+  if (i < oc) {
+    const int64_t step = static_cast<int64_t>(kXi) * oc;
+    float sum[9];
 #pragma unroll
-  for (int q = 0; q < 6; ++q) {
-    float col[6];
+    for (int j = 0; j < 9; ++j) sum[j] = part[static_cast<int64_t>(9 * wave + j) * oc + i];
+    for (int p = 1; p < parts; ++p) {
 #pragma unroll
-    for (int r = 0; r < 6; ++r) {
-      const float *src = part + static_cast<int64_t>(r * 6 + q) * oc + i;
-      float sum = src[0];
-      for (int p = 1; p < parts; ++p) sum += src[static_cast<int64_t>(p) * kXi * oc];
-      col[r] = sum;
+      for (int j = 0; j < 9; ++j) sum[j] += part[p * step + static_cast<int64_t>(9 * wave + j) * oc + i];
     }
-    gt_rows(col, t[q]);
-  }
 #pragma unroll
-  for (int r = 0; r < 3; ++r) {
-    const float row[6] = {t[0][r], t[1][r], t[2][r], t[3][r], t[4][r], t[5][r]};
-    float w[3];
-    gt_rows(row, w);
-#pragma unroll
-    for (int q = 0; q < 3; ++q) dw[static_cast<int64_t>(i) * 9 + r * 3 + q] = w[q];
+    for (int j = 0; j < 9; ++j) sums[9 * wave + j][lane] = sum[j];
   }
+  __syncthreads();
+  if (wave == 0 && i < oc) {
+    float t[6][3];   // t[q][.] = G^T applied down column q
+#pragma unroll
+    for (int q = 0; q < 6; ++q) {
+      float col[6];
+#pragma unroll
+      for (int r = 0; r < 6; ++r) col[r] = sums[r * 6 + q][lane];
+      gt_rows(col, t[q]);
+    }
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      const float row[6] = {t[0][r], t[1][r], t[2][r], t[3][r], t[4][r], t[5][r]};
+      float w[3];
+      gt_rows(row, w);
+#pragma unroll
+      for (int q = 0; q < 3; ++q) outs[lane * 9 + r * 3 + q] = w[q];
+    }
+  }
+  __syncthreads();
+  const int n = min(64, oc - i0) * 9;
+  float *dst = dw + static_cast<int64_t>(i0) * 9;
+  for (int k = threadIdx.x; k < n; k += 256) dst[k] = outs[k];
 }
 
 // ---------------------------------------------------------------- GEMM launch timing (opt-in)
@@ -532,8 +573,6 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
   float *VM = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(kXi) * (gathered + produced) * ld_max * 4));
   TS_REQUIRE(U && VM, "conv (Winograd): no scratch memory");
   float *V = VM, *M = VM + static_cast<int64_t>(kXi) * gathered * ld_max;
-  hipLaunchKernelGGL(wino_filter_kernel, dim3((produced * gathered + 255) / 256), dim3(256), 0, st, w, U, produced,
-                     gathered, rotated);
   for (int first = 0; first < imgs; first += run) {
     const int n = std::min(run, imgs - first);
     WinoGeo gi{gathered, H, W, th, tw, n * per_img, (n * per_img + 3) / 4 * 4,
@@ -541,10 +580,18 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
     WinoGeo go = gi;
     go.chans = produced;
     const float *xr = x + static_cast<int64_t>(first) * gathered * H * W;
+    // the filter transform rides in the first rows of the first run's input transform
+    const int nbx = (gi.ld + 255) / 256;
+    FilterJob job{w, U, produced, gathered, rotated, 0, 0};
+    if (first == 0) {
+      job.blocks = (produced * gathered + 255) / 256;
+      job.rows = (job.blocks + nbx - 1) / nbx;
+    }
+    const dim3 grid_in(nbx, job.rows + gathered);
     if ((W & 3) == 0 && (reinterpret_cast<uintptr_t>(xr) & 15) == 0)
-      hipLaunchKernelGGL(wino_input_kernel<true>, dim3((gi.ld + 255) / 256, gathered), dim3(256), 0, st, xr, V, gi);
+      hipLaunchKernelGGL(wino_input_kernel<true>, grid_in, dim3(256), 0, st, xr, V, gi, job);
     else
-      hipLaunchKernelGGL(wino_input_kernel<false>, dim3((gi.ld + 255) / 256, gathered), dim3(256), 0, st, xr, V, gi);
+      hipLaunchKernelGGL(wino_input_kernel<false>, grid_in, dim3(256), 0, st, xr, V, gi, job);
     {
       // every operand read once, the result written once
       const double flop = 2.0 * kXi * produced * static_cast<double>(gi.ld) * gathered;
@@ -596,15 +643,17 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
     WinoGeo gx{C, H, W, th, tw, n * per_img, (n * per_img + 3) / 4 * 4, false};
     WinoGeo gy = gx;
     gy.chans = O;
-    const dim3 grid_x((gx.ld + 255) / 256, C), grid_y((gx.ld + 255) / 256, O);
-    if ((W & 3) == 0 && (reinterpret_cast<uintptr_t>(xr) & 15) == 0)
-      hipLaunchKernelGGL(wino_input_kernel<true>, grid_x, dim3(256), 0, st, xr, V, gx);
+    const dim3 grid_xy((gx.ld + 255) / 256, C + O);
+    const bool qx = (W & 3) == 0 && (reinterpret_cast<uintptr_t>(xr) & 15) == 0;
+    const bool qy = (W & 3) == 0 && (reinterpret_cast<uintptr_t>(dyr) & 15) == 0;
+    if (qx && qy)
+      hipLaunchKernelGGL((wino_grad_pair_kernel<true, true>), grid_xy, dim3(256), 0, st, xr, V, gx, dyr, Y, gy);
+    else if (qx)
+      hipLaunchKernelGGL((wino_grad_pair_kernel<true, false>), grid_xy, dim3(256), 0, st, xr, V, gx, dyr, Y, gy);
+    else if (qy)
+      hipLaunchKernelGGL((wino_grad_pair_kernel<false, true>), grid_xy, dim3(256), 0, st, xr, V, gx, dyr, Y, gy);
     else
-      hipLaunchKernelGGL(wino_input_kernel<false>, grid_x, dim3(256), 0, st, xr, V, gx);
-    if ((W & 3) == 0 && (reinterpret_cast<uintptr_t>(dyr) & 15) == 0)
-      hipLaunchKernelGGL(wino_grad_kernel<true>, grid_y, dim3(256), 0, st, dyr, Y, gy);
-    else
-      hipLaunchKernelGGL(wino_grad_kernel<false>, grid_y, dim3(256), 0, st, dyr, Y, gy);
+      hipLaunchKernelGGL((wino_grad_pair_kernel<false, false>), grid_xy, dim3(256), 0, st, xr, V, gx, dyr, Y, gy);
     const int here = (gx.ld + kchunk - 1) / kchunk;
     {
       const bool split = plan.grid > 0 && split_bf16_enabled();
@@ -615,13 +664,8 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
     }
     parts += here;
   }
-  // many partial sums for few filter elements (narrow layers cut into many ranges): fold them with one
-  // thread per element first, so that the final transform's threads do not each walk all of them
-  if (parts > 1)
-    hipLaunchKernelGGL(wino_fold_kernel, dim3(static_cast<unsigned>((kXi * oc + 255) / 256)), dim3(256), 0, st, part,
-                       kXi * oc, parts);
-  hipLaunchKernelGGL(wino_filter_grad_kernel, dim3(static_cast<unsigned>((oc + 255) / 256)), dim3(256), 0, st, part, dw,
-                     static_cast<int>(oc), 1);
+  hipLaunchKernelGGL(wino_filter_grad_kernel, dim3(static_cast<unsigned>((oc + 63) / 64)), dim3(256), 0, st, part, dw,
+                     static_cast<int>(oc), parts);
   return 0;
 }
 
