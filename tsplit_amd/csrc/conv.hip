@@ -2262,8 +2262,9 @@ inline int winograd_forced() {
 }
 
 inline bool winograd_shape(const ConvGeo &g) {
+  // channels are a dimension of the transform kernels' grids (both tensors' together in the filter gradient)
   return g.kH == 3 && g.kW == 3 && g.s == 1 && g.ph == 1 && g.pw == 1 && g.oH == g.H && g.oW == g.W &&
-         static_cast<int64_t>(std::max(g.C, g.O)) * g.H * g.W < (1ll << 29);
+         static_cast<int64_t>(std::max(g.C, g.O)) * g.H * g.W < (1ll << 29) && g.C + g.O <= 32768;
 }
 
 // wide enough for the 36 GEMMs to outweigh the transforms (64 channels on both sides: with tiles as

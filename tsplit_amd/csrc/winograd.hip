@@ -69,6 +69,10 @@ __device__ __forceinline__ void wino_filter_block(const float *__restrict__ w, f
     for (int q = 0; q < 6; ++q) U[static_cast<int64_t>(r * 6 + q) * produced * gathered + i] = u[q];
   }
 }
+__global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restrict__ w, float *__restrict__ U, int produced,
+                                                          int gathered, bool rotated) {
+  wino_filter_block(w, U, produced, gathered, rotated, blockIdx.x);
+}
 // A filter transform that rides in the first rows of another kernel's grid (the input transform of a call's
 // first run: neither depends on the other, and a launch of its own would cost its ramp and tail).
 struct FilterJob {
@@ -586,6 +590,10 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
     if (first == 0) {
       job.blocks = (produced * gathered + 255) / 256;
       job.rows = (job.blocks + nbx - 1) / nbx;
+      if (job.rows + gathered > 65535) {   // a huge filter beside a narrow grid: a launch of its own
+        hipLaunchKernelGGL(wino_filter_kernel, dim3(job.blocks), dim3(256), 0, st, w, U, produced, gathered, rotated);
+        job.blocks = job.rows = 0;
+      }
     }
     const dim3 grid_in(nbx, job.rows + gathered);
     if ((W & 3) == 0 && (reinterpret_cast<uintptr_t>(xr) & 15) == 0)
