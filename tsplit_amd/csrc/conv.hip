@@ -2407,9 +2407,11 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
       double *tmp = reinterpret_cast<double *>(sink.part + static_cast<int64_t>(sink.capacity) * g.O * 2);
       const int slices = std::max(1, std::min(kStatsSlices, (sink.used + 63) / 64));
       const int chunk = (sink.used + slices - 1) / slices;
+      // one slice: its sums are the result (slice 0 of tmp has dst's layout), no second launch
       hipLaunchKernelGGL(conv_stats_fold_kernel, dim3((g.O + 31) / 32, slices), dim3(256), 0, st, sink.part, sink.used, g.O,
-                         tmp, chunk);
-      hipLaunchKernelGGL(conv_stats_final_kernel, dim3((g.O + 255) / 256), dim3(256), 0, st, tmp, slices, g.O, stats_dst);
+                         slices == 1 ? stats_dst : tmp, chunk);
+      if (slices > 1)
+        hipLaunchKernelGGL(conv_stats_final_kernel, dim3((g.O + 255) / 256), dim3(256), 0, st, tmp, slices, g.O, stats_dst);
     } else if (numel(y) > 0) {
       if (bn_channel_sums(y, stats_dst, st)) return -1;
     } else {
