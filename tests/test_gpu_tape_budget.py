@@ -105,6 +105,30 @@ def test_budgeted_graph_tracks_the_plain_tape_and_the_oracle(net, recompute, rng
     assert run.state.host_waits > 0 or not plan.away
 
 
+def test_schedules_change_between_steps_and_the_fastest_is_kept(rng):
+    """BudgetedRun.tune: every (lead, hold) schedule the budget admits trains real steps with the plain tape's
+    bits, a schedule that keeps everything on the device until the end is refused, and the run goes on
+    under the fastest."""
+    from tsplit_amd import graph, tape_budget as tb, workloads
+    build, inputs, lr = _cases(rng)["resnet"]
+    ops, leaves = tb.record(build, {k: v.shape for k, v in inputs.items()})
+    free_peak = tb.replay(ops, leaves)[0]
+    budget = leaves + int((free_peak - leaves) * 0.6)
+    # (values may only travel here: with recomputation allowed this budget is met without a copy, whatever the schedule)
+    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(5), budget, min_bytes=0, recompute=False)
+    best, timings, losses = run.tune(lr, candidates=((3, 1), (8, 4), (2, 6), (10000, 10000)), steps=2)
+    assert best in timings and (3, 1) in timings and (10000, 10000) not in timings and len(timings) >= 2
+    assert (run.plan.lead, run.plan.hold) == best
+    losses.append(run.step(lr))
+    got = [float(l.value.asnumpy()[0]) for l in losses]
+    assert len(got) == 2 * len(timings) + 1
+    plain_losses, plain_params = _plain(build, inputs, 5, len(got), lr, graph.GpuBackend())
+    assert got == plain_losses
+    run.binder.pull()
+    for k, v in plain_params.items():
+        np.testing.assert_array_equal(run.store.values[k], v)
+
+
 def test_pool_usage_stays_within_the_replayed_peak(rng):
     """A ResNet of two stages at 96x96, batch 16 (activations of tens of MB): the pool's `used` figure,
     read after every operator, against the planner's replay, unplanned and under half the budget."""

@@ -88,6 +88,28 @@ def test_sending_a_value_away_frees_it_between_its_uses():
     assert tb.replay(ops, leaves, (), 3, {j})[0] <= base
 
 
+def test_holding_and_fetching_ahead_cost_memory_that_the_plan_makes_room_for():
+    """A leaving value that keeps its memory for `hold` operators and a returning one that takes its memory
+    `lead` operators early raise the replayed peak of a given choice; the planner answers by sending more
+    away, still within the budget; a schedule that holds everything to the end of the sweep saves nothing."""
+    build, shapes = SHAPES["resnet"]
+    ops, leaves = tb.record(build, shapes)
+    free_peak = tb.replay(ops, leaves)[0]
+    budget = leaves + int((free_peak - leaves) * 0.6)
+    tight = tb.plan(ops, leaves, budget, lead=3, min_bytes=0, recompute=False, hold=1)
+    assert tight.away and tight.peak_bytes <= budget and (tight.lead, tight.hold) == (3, 1)
+    # the same choice replayed under lazier schedules: never a lower peak
+    peaks = [tb.replay(ops, leaves, tight.away, lead, (), hold)[0] for lead, hold in ((3, 1), (3, 4), (8, 4), (20, 12))]
+    assert peaks[0] == tight.peak_bytes and all(b >= a for a, b in zip(peaks, peaks[1:]))
+    lazy = tb.plan(ops, leaves, budget, lead=8, min_bytes=0, recompute=False, hold=4)
+    assert lazy.peak_bytes <= budget and len(lazy.away) >= len(tight.away) and (lazy.lead, lazy.hold) == (8, 4)
+    assert tb.replay(ops, leaves, lazy.away, 8, (), 4)[0] == lazy.peak_bytes
+    n = len(ops)
+    assert tb.replay(ops, leaves, tight.away, n, (), n)[0] == free_peak
+    with pytest.raises(ValueError):
+        tb.plan(ops, leaves, budget, lead=n, min_bytes=0, recompute=False, hold=n)
+
+
 def test_max_batch_grows_with_the_budget_and_with_planning():
     def build_for(batch):
         return _resnet

@@ -17,15 +17,19 @@ graphs of the reference's examples:
                       needs it, any other value is sent to pinned host memory;
   BudgetedTape        a Tape that follows the plan: values without a later reader are dropped as the
                       forward sweep passes their last use, values to be computed again likewise,
-                      values sent away go to pinned host memory behind the sweep and are fetched `lead`
-                      operators ahead of the backward sweep, and every value is dropped after the last
-                      backward operator (or recomputation) that reads it.
+                      values sent away go to pinned host memory behind the sweep (keeping their memory
+                      for `hold` more operators, while the copy runs) and are fetched `lead` operators
+                      ahead of the backward sweep, and every value is dropped after the last backward
+                      operator (or recomputation) that reads it;
+  BudgetedRun         trains step after step under a plan; BudgetedRun.tune runs a few steps under each
+                      of several (lead, hold) schedules and keeps the fastest.
 
 Schedule (replayed byte for byte by `replay`, measured against the pool by the tests):
   forward  of operator t : its output is allocated; then every value whose last reader in the forward
                            sweep was t and which no backward operator reads is released; a planned
                            value whose last forward reader was t starts leaving, and is released
-                           after operator t + 1 has been issued (the host waits for the copy then);
+                           after operator t + hold has been issued (the host waits for the copy then,
+                           if it is still on its way);
   backward of operator j : the values sent away that operators j - lead .. j need first (in the order
                            of the sweep) are allocated and start coming back; the host waits for
                            those operator j reads; dropped values operator j needs first are computed
@@ -33,10 +37,15 @@ Schedule (replayed byte for byte by `replay`, measured against the pool by the t
                            from the kept convolution output), which gives the same bits; j's backward
                            operators allocate the gradients of its inputs; then j's output gradient
                            and every value whose last reader was j are released.
-Ordering between the streams goes through the host (DLEventSync), as in the reference: before a
-value leaves, the host waits for the operator that last read it; before memory for a returning value
-is taken from the pool, the host waits for the compute stream, so that no kernel still in flight
-reads memory the pool hands out again.
+Ordering between the streams goes through the host (DLEventRecord / DLEventQuery / DLEventSync), as in
+the reference: a value's copy out is issued once the operator that last read it has run, a copy back
+once everything that was in flight when its memory was taken from the pool has run (so that no kernel
+reads memory the pool has handed out again).  The executor looks at those events as the sweeps pass
+and issues the copies that have become ready; the host waits only when a copy's time has come (a value
+due for release, or one its reader needs) and it has not been issued or has not finished.  With `hold`
+and `lead` of a few dozen operators the copies run beside the operators instead of between them; the
+memory that costs is part of the replay, so the planner makes room for it by sending more away.
+Which (lead, hold) is fastest depends on the graph and the budget: BudgetedRun.tune measures.
 
 The budget covers what the tape allocates: operator outputs, gradients, parameters and their
 gradients, inputs and constants.  The operator library's own scratch is outside it.
@@ -113,10 +122,11 @@ def record(build, inputs):
 
 
 class TapePlan(object):
-    def __init__(self, away, lead, peak_bytes, free_peak_bytes, budget_bytes, leaves_bytes, redo=()):
+    def __init__(self, away, lead, peak_bytes, free_peak_bytes, budget_bytes, leaves_bytes, redo=(), hold=1):
         self.away = frozenset(away)          # operator calls whose output leaves the device between the sweeps
         self.redo = frozenset(redo)          # operator calls whose output is dropped and computed again
-        self.lead = lead
+        self.lead = lead                     # operators ahead of its first reader at which a value starts coming back
+        self.hold = hold                     # operators behind its last reader after which a leaving value is released
         self.peak_bytes = peak_bytes
         self.free_peak_bytes = free_peak_bytes     # replayed peak with nothing sent away
         self.budget_bytes = budget_bytes
@@ -124,7 +134,8 @@ class TapePlan(object):
 
     def describe(self):
         gib = float(1 << 30)
-        return {"away": len(self.away), "recomputed": len(self.redo), "lead": self.lead, "peak_GiB": self.peak_bytes / gib,
+        return {"away": len(self.away), "recomputed": len(self.redo), "lead": self.lead, "hold": self.hold,
+                "peak_GiB": self.peak_bytes / gib,
                 "unplanned_peak_GiB": self.free_peak_bytes / gib,
                 "budget_GiB": None if self.budget_bytes is None else self.budget_bytes / gib}
 
@@ -162,7 +173,7 @@ def _needs(ops, redo):
     return last_fwd, need
 
 
-def replay(ops, leaves_bytes, away=(), lead=3, redo=()):
+def replay(ops, leaves_bytes, away=(), lead=3, redo=(), hold=1):
     """Peak of the executor's schedule with `away` sent to the host and `redo` dropped and computed
     again.  -> (peak bytes, moment of the peak, values resident and idle at that moment: list of
     (bytes, operator)).  A moment is an operator index for the forward sweep and 2n - 1 - j for the
@@ -186,23 +197,24 @@ def replay(ops, leaves_bytes, away=(), lead=3, redo=()):
     by_last_fwd = collections.defaultdict(list)
     for i in range(n):
         by_last_fwd[last_fwd[i]].append(i)
-    leaving = []                                        # values released after the next operator
+    leaving = []                                        # (operator after which it is released, value)
     # ---- forward
     for t, op in enumerate(ops):
         live += op.bytes
         resident[t] = op.bytes
         busy = set(i for i in op.inputs if i >= 0) | {t}
         note(t)
-        for i in leaving:
-            live -= resident.pop(i)
-        leaving = []
+        for due, i in leaving:
+            if due <= t:
+                live -= resident.pop(i)
+        leaving = [(due, i) for due, i in leaving if due > t]
         for i in by_last_fwd[t]:
             if not need[i] or i in redo:
                 if i != n - 1:                          # the loss stays for the caller
                     live -= resident.pop(i)
             elif i in away:
-                leaving.append(i)
-    for i in leaving:
+                leaving.append((t + hold, i))
+    for due, i in leaving:
         live -= resident.pop(i)
     # ---- backward
     grads = {}                                          # operator -> bytes of the gradient of its output
@@ -256,15 +268,15 @@ def replay(ops, leaves_bytes, away=(), lead=3, redo=()):
     return peak, peak_at, peak_set
 
 
-def plan(ops, leaves_bytes, budget_bytes, lead=3, min_bytes=1 << 20, recompute=True):
+def plan(ops, leaves_bytes, budget_bytes, lead=3, min_bytes=1 << 20, recompute=True, hold=1):
     """-> TapePlan.  Raises ValueError when the budget cannot be met (a single operator's operands,
     results and gradients do not fit with everything idle off the device)."""
-    free_peak, _, _ = replay(ops, leaves_bytes, (), lead)
+    free_peak, _, _ = replay(ops, leaves_bytes, (), lead, (), hold)
     away, redo, banned = set(), set(), set()
     n = len(ops)
     if budget_bytes is not None:
         while True:
-            peak, at, idle = replay(ops, leaves_bytes, away, lead, redo)
+            peak, at, idle = replay(ops, leaves_bytes, away, lead, redo, hold)
             if peak <= budget_bytes:
                 break
             last_fwd, need = _needs(ops, redo)
@@ -278,7 +290,7 @@ def plan(ops, leaves_bytes, budget_bytes, lead=3, min_bytes=1 << 20, recompute=T
                 cheap = recompute and ops[i].cheap and (i, "redo") not in banned
                 back_at = 2 * n - 1 - (max(need[i]) if cheap else min(n - 1, max(need[i]) + lead))
                 if not cheap:
-                    gone_from += 1                      # a copy takes one more operator to leave
+                    gone_from += hold                   # a copy takes that many more operators to leave
                     if (i, "away") in banned:
                         continue
                 if gone_from <= at < back_at:
@@ -289,15 +301,15 @@ def plan(ops, leaves_bytes, budget_bytes, lead=3, min_bytes=1 << 20, recompute=T
             # a value that can be computed again goes before one that has to travel, the larger first
             b, i, cheap = max(cands, key=lambda c: (c[2], c[0], c[1]))
             trial_away, trial_redo = (away, redo | {i}) if cheap else (away | {i}, redo)
-            new_peak, new_at, _ = replay(ops, leaves_bytes, trial_away, lead, trial_redo)
+            new_peak, new_at, _ = replay(ops, leaves_bytes, trial_away, lead, trial_redo, hold)
             if new_peak > peak or (new_peak == peak and new_at == at):
                 # keeping this value's inputs for the recomputation (or the move itself) does not help
                 # here: try the other way, then other values
                 banned.add((i, "redo" if cheap else "away"))
                 continue
             away, redo = set(trial_away), set(trial_redo)
-    peak, _, _ = replay(ops, leaves_bytes, away, lead, redo)
-    return TapePlan(away, lead, peak, free_peak, budget_bytes, leaves_bytes, redo)
+    peak, _, _ = replay(ops, leaves_bytes, away, lead, redo, hold)
+    return TapePlan(away, lead, peak, free_peak, budget_bytes, leaves_bytes, redo, hold)
 
 
 class BudgetedTape(graph.Tape):
@@ -341,7 +353,9 @@ class BudgetedTape(graph.Tape):
         for i in tape_plan.redo:
             if self.need[i]:
                 self.redo_at[self.first[i]].append(i)
-        self.leaving = []            # (operator, device array, copy-done event), released after the next operator
+        self.leaving = []            # (operator after which it is released, value, device array, event behind its
+                                     #  last reader, copy-done event or None while the copy has not been issued)
+        self.waiting_in = {}         # operator -> (event behind what was in flight when its memory was taken, array)
         self.arriving = {}           # operator -> copy-done event
         self.gone = set()            # values in host memory only
         self.recomputed = 0
@@ -350,11 +364,21 @@ class BudgetedTape(graph.Tape):
     def _compute_stream(self):
         return self.b.stream
 
-    def _host_wait_for_compute(self):
+    def _mark_compute(self):
+        """An event at the current end of the compute stream."""
         ev = create_event_handle(self.state.ctx)
         ev.record(self._compute_stream())
-        ev.sync()
-        self.state.host_waits += 1
+        return ev
+
+    def _reached(self, ev, wait):
+        """True once `ev` has been reached; with `wait` the host waits for it (and that is counted)."""
+        if ev.query():
+            return True
+        if wait:
+            ev.sync()
+            self.state.host_waits += 1
+            return True
+        return False
 
     def _note_pool(self):
         if self.track_pool:
@@ -364,19 +388,54 @@ class BudgetedTape(graph.Tape):
     def _var(self, i):
         return self._nodes[i].out
 
-    def _release_leaving(self):
-        for i, arr, ev in self.leaving:
-            ev.sync()                # the copy has left the device
-            self.state.host_waits += 1
-            del arr
-        self.leaving = []
+    # A copy is issued once the compute stream has passed the point recorded when the copy was decided: the
+    # last reader of a value that leaves, or everything that may still read the memory a returning value is
+    # given.  The hooks look at those points as they pass (_poll) and issue what has become ready, so the
+    # host waits only for a copy whose time has come: a value that is due for release, or one its reader needs.
+    def _issue_out(self, entry, wait):
+        due, i, arr, after, done = entry
+        if done is None and self._reached(after, wait):
+            host = self.state.host.get(i)
+            if host is None or host.shape != arr.shape:
+                host = self.state.host[i] = ndarray.empty(arr.shape, self.state.host_ctx)
+            arr.copyto(host, self.state.out_stream)
+            done = create_event_handle(self.state.ctx)
+            done.record(self.state.out_stream)
+        return (due, i, arr, after, done)
+
+    def _issue_in(self, i, wait):
+        pending = self.waiting_in.get(i)
+        if pending is not None and self._reached(pending[0], wait):
+            del self.waiting_in[i]
+            self.state.host[i].copyto(pending[1], self.state.in_stream)
+            ev = create_event_handle(self.state.ctx)
+            ev.record(self.state.in_stream)
+            self.arriving[i] = ev
+
+    def _poll(self):
+        self.leaving = [self._issue_out(e, False) for e in self.leaving]
+        for i in list(self.waiting_in):
+            self._issue_in(i, False)
+
+    def _release_leaving(self, t=None):
+        """Releases the values due after operator t (all of them without t) once their copies have left."""
+        keep = []
+        for entry in self.leaving:
+            if t is not None and entry[0] > t:
+                keep.append(entry)
+                continue
+            due, i, arr, after, done = self._issue_out(entry, True)
+            self._reached(done, True)            # the copy has left the device
+            del arr, entry
+        self.leaving = keep
 
     # ---- hooks
     def _after_forward(self, node):
         t = node.index
         assert t < len(self.ops) and _bytes(node.out.shape) == self.ops[t].bytes, "the graph differs from the recorded one"
         self._note_pool()
-        self._release_leaving()
+        self._poll()
+        self._release_leaving(t)
         n = len(self.ops)
         for i in self.by_last_fwd[t]:
             v = self._var(i)
@@ -384,37 +443,28 @@ class BudgetedTape(graph.Tape):
                 if i != n - 1:
                     v.value = None       # nobody reads it again, or it will be computed again
             elif i in self.plan.away:
-                # the operator that read it last has been issued: wait for it, then copy out
-                self._host_wait_for_compute()
-                host = self.state.host.get(i)
-                if host is None or host.shape != v.shape:
-                    host = self.state.host[i] = ndarray.empty(v.shape, self.state.host_ctx)
-                v.value.copyto(host, self.state.out_stream)
-                ev = create_event_handle(self.state.ctx)
-                ev.record(self.state.out_stream)
-                self.leaving.append((i, v.value, ev))
+                # the operator that read it last has been issued: the copy out starts once it has run
+                self.leaving.append((t + self.plan.hold, i, v.value, self._mark_compute(), None))
                 v.value = None
                 self.gone.add(i)
 
     def _fetch(self, i):
         v = self._var(i)
-        self._host_wait_for_compute()          # nothing in flight reads memory the pool may hand out now
+        # the memory is taken now (the plan counts it from here); the copy starts once nothing in flight can
+        # still read memory the pool may have handed out for it
         arr = ndarray.empty(v.shape, self.state.ctx)
-        self.state.host[i].copyto(arr, self.state.in_stream)
-        ev = create_event_handle(self.state.ctx)
-        ev.record(self.state.in_stream)
+        self.waiting_in[i] = (self._mark_compute(), arr)
         v.value = arr
-        self.arriving[i] = ev
         self.gone.discard(i)
 
     def _ensure(self, i):
         """Value i is on the device and complete when this returns."""
         if i in self.gone:                     # (a value the plan fetches later than this reader needs it)
             self._fetch(i)
+        self._issue_in(i, True)
         ev = self.arriving.pop(i, None)
         if ev is not None:
-            ev.sync()
-            self.state.host_waits += 1
+            self._reached(ev, True)
         if self._var(i).value is None and i in self.plan.redo:
             node = self._nodes[i]
             for u in node.inputs:
@@ -424,6 +474,7 @@ class BudgetedTape(graph.Tape):
             self.recomputed += 1
 
     def _before_backward(self, node):
+        self._poll()
         for i in sorted(self.redo_at[node.index]):      # producers before consumers
             self._ensure(i)
         for s in node.saved:
@@ -449,6 +500,7 @@ class BudgetedTape(graph.Tape):
             for i in sorted(self.fetch_at[j - 1], key=lambda i: -self.first[i]):
                 if i in self.gone:
                     self._fetch(i)
+        self._poll()
 
 
 class BudgetedRun(object):
@@ -456,12 +508,13 @@ class BudgetedRun(object):
     parameters come from `store` (workloads.ParamStore), inputs are numpy arrays uploaded once."""
 
     def __init__(self, build, inputs, store, budget_bytes, ctx=None, lead=3, track_pool=False, min_bytes=1 << 20,
-                 recompute=True):
+                 recompute=True, hold=1):
         from . import stream, workloads
         self.ctx = ctx or ndarray.gpu(0)
         self.build = build
         self.ops, self.leaves_bytes = record(build, {k: np.shape(v) for k, v in inputs.items()})
-        self.plan = plan(self.ops, self.leaves_bytes, budget_bytes, lead, min_bytes, recompute)
+        self.plan = plan(self.ops, self.leaves_bytes, budget_bytes, lead, min_bytes, recompute, hold)
+        self._plan_args = (budget_bytes, min_bytes, recompute)
         self.stream = stream.create_stream_handle(self.ctx)
         self.backend = graph.GpuBackend(self.ctx, self.stream)
         self.state = BudgetedTape.make_state(self.ctx)
@@ -486,6 +539,34 @@ class BudgetedRun(object):
         t.backward(loss)
         self.binder.sgd_step(lr)
         return loss
+
+    def tune(self, lr, candidates=((3, 1), (30, 30), (60, 30), (100, 30)), steps=2):
+        """Trains `steps` steps under each (lead, hold) schedule the budget admits and keeps the fastest.  Every
+        plan computes the same bits, so these are ordinary training steps: only their speed differs (how far
+        ahead of its reader a value starts coming back, how long a leaving value keeps its memory while its
+        copy runs, and what else has to leave to make room for that).  The first step of a schedule is not
+        timed (new pinned host buffers).  -> ((lead, hold), {(lead, hold): ms per step}), losses of the steps run."""
+        import time
+        budget_bytes, min_bytes, recompute = self._plan_args
+        timings, plans, losses = {}, {}, []
+        for lead, hold in candidates:
+            try:
+                plans[(lead, hold)] = plan(self.ops, self.leaves_bytes, budget_bytes, lead, min_bytes, recompute, hold)
+            except ValueError:
+                continue
+            self.plan = plans[(lead, hold)]
+            losses.append(self.step(lr))
+            self.sync()
+            t0 = time.perf_counter()
+            for _ in range(max(1, steps - 1)):
+                losses.append(self.step(lr))
+            self.sync()
+            timings[(lead, hold)] = (time.perf_counter() - t0) / max(1, steps - 1) * 1e3
+        if not timings:
+            raise ValueError("no schedule fits the budget")
+        best = min(timings, key=timings.get)
+        self.plan = plans[best]
+        return best, timings, losses
 
     def sync(self):
         self.backend.sync()

@@ -1,14 +1,16 @@
 """The branched example networks trained under device-memory budgets (one MI355X): the budgeted tape
 executor of tape_budget.py on ResNet-50 (batch 64), Inception-v4 (batch 32) and the Transformer (batch 32).
 
-    python -m tsplit_amd.tapebench --net resnet50|inception_v4|transformer [--fractions 0,0.75,0.5,0.35] [--steps 4] [--warmup 1] [--no-recompute]
-    python -m tsplit_amd.tapebench --net resnet50|inception_v4 --max-batch [--budgets 8,16] [--no-recompute]
+    python -m tsplit_amd.tapebench --net resnet50|inception_v4|transformer [--fractions 0,0.75,0.5,0.35] [--steps 4] [--warmup 1] [--no-recompute] [--tune | --lead L --hold H]
+    python -m tsplit_amd.tapebench --net resnet50|inception_v4 --max-batch [--budgets 8,16] [--no-recompute] [--tune]
 
 For every fraction f (0 = no limit) the budget is the leaves (parameters, their gradients' room is part
 of the replay, inputs, constants) plus f times what the operators' values and gradients take at the
 unplanned peak; the planner picks what is dropped and computed again and what leaves for pinned host memory
 (only the latter with --no-recompute), the executor trains on synthetic data.  One JSON object per budget: samples/s, the pool's measured peak over its level before the run,
-the replayed peak, values sent away, host waits per step.  With --max-batch the question is turned
+the replayed peak, values sent away, host waits per step.  --lead and --hold set the schedule (how many operators ahead of
+its reader a value starts coming back, for how many operators a leaving value keeps its memory while its copy runs);
+with --tune the run first trains two steps under each of a few schedules and keeps the fastest.  With --max-batch the question is turned
 around, as in the reference's batch-size sweeps per policy (examples/imagenet_resnet.py:139-154): for
 every budget in GiB, the largest batch that trains with everything resident and the largest one the
 planner fits, and the measured throughput at the latter.
@@ -58,11 +60,17 @@ def _net(name, batch=None):
     raise ValueError(name)
 
 
-def _measure(build, inputs, budget, steps, warmup, lr, recompute=True):
+def _measure(build, inputs, budget, steps, warmup, lr, recompute=True, lead=3, hold=1, tune=False):
     from . import tape_budget as tb, workloads
     from .gpu_memory_manager import pool_state
     base = pool_state().used
-    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(123), budget, track_pool=True, recompute=recompute)
+    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(123), budget, lead=lead, track_pool=True, recompute=recompute,
+                         hold=hold)
+    tuned = None
+    if tune and budget is not None:
+        best, timings, _ = run.tune(lr)
+        tuned = {"lead": best[0], "hold": best[1], "ms_per_schedule": {"%d,%d" % k: round(v, 2) for k, v in timings.items()}}
+        run.state.peak_used = 0          # the pool's peak below is that of the schedule kept
     for _ in range(warmup):
         run.step(lr)
     run.sync()
@@ -79,7 +87,8 @@ def _measure(build, inputs, budget, steps, warmup, lr, recompute=True):
             "planned_peak_GiB": d["peak_GiB"], "unplanned_peak_GiB": d["unplanned_peak_GiB"], "values_away": d["away"],
             "away_GiB": sum(run.ops[i].bytes for i in run.plan.away) / gib, "values_recomputed": len(run.plan.redo),
             "recomputed_GiB": sum(run.ops[i].bytes for i in run.plan.redo) / gib,
-            "host_waits_per_step": (run.state.host_waits - waits0) / steps, "loss": float(loss.value.asnumpy()[0])}
+            "host_waits_per_step": (run.state.host_waits - waits0) / steps, "loss": float(loss.value.asnumpy()[0]),
+            "lead": run.plan.lead, "hold": run.plan.hold, "tuned": tuned}
 
 
 def main():
@@ -93,6 +102,10 @@ def main():
     ap.add_argument("--lr", type=float, default=1e-4)
     ap.add_argument("--max-batch", action="store_true")
     ap.add_argument("--no-recompute", action="store_true", help="the plan may only send values to the host")
+    ap.add_argument("--lead", type=int, default=3, help="operators ahead of its first reader at which a value starts coming back")
+    ap.add_argument("--tune", action="store_true",
+                    help="train two steps under each of a few (lead, hold) schedules first and keep the fastest")
+    ap.add_argument("--hold", type=int, default=1, help="operators behind its last reader after which a leaving value is released")
     a = ap.parse_args()
     from . import tape_budget as tb
     build_for, inputs_for, default_batch, desc = _net(a.net)
@@ -111,7 +124,7 @@ def main():
                    "max_batch_resident": resident, "max_batch_planned": planned}
             if p is not None:
                 row.update(_measure(build_for(planned), inputs_for(planned, rng), budget, max(1, a.steps // 2), 1, a.lr,
-                                    not a.no_recompute))
+                                    not a.no_recompute, a.lead, a.hold, a.tune))
             print(json.dumps(row), flush=True)
         return
     n = a.batch or default_batch
@@ -124,7 +137,7 @@ def main():
         row = {"net": a.net, "workload": desc + ", batch %d" % n, "fraction": f,
                "budget_GiB": None if budget is None else budget / float(1 << 30), "recompute": not a.no_recompute}
         try:
-            row.update(_measure(build, inputs, budget, a.steps, a.warmup, a.lr, not a.no_recompute))
+            row.update(_measure(build, inputs, budget, a.steps, a.warmup, a.lr, not a.no_recompute, a.lead, a.hold, a.tune))
         except ValueError as e:
             row["error"] = str(e)
         print(json.dumps(row), flush=True)
