@@ -540,7 +540,7 @@ class BudgetedRun(object):
         self.binder.sgd_step(lr)
         return loss
 
-    def tune(self, lr, candidates=((3, 1), (30, 30), (60, 30), (100, 30)), steps=2):
+    def tune(self, lr, candidates=((3, 1), (30, 30), (60, 30), (100, 30), (200, 60), (400, 100)), steps=2):
         """Trains `steps` steps under each (lead, hold) schedule the budget admits and keeps the fastest.  Every
         plan computes the same bits, so these are ordinary training steps: only their speed differs (how far
         ahead of its reader a value starts coming back, how long a leaving value keeps its memory while its
