@@ -42,6 +42,14 @@ class OracleBackend(object):
         dx, dg, db = O.batchnorm_backward(dy, x, gamma, eps)
         return _s(dx), _s(dg).reshape(1, -1, 1, 1), _s(db).reshape(1, -1, 1, 1)
 
+    def bn_relu(self, x, gamma, beta, xs, eps):
+        y, mean, var = O.batchnorm_forward(x, gamma, beta, eps)
+        return _s(O.relu(y)), mean, var
+
+    def bn_relu_grad(self, dy, x, gamma, beta, mean, var, xs, eps):
+        y = O.batchnorm_forward(x, gamma, beta, eps)[0]
+        return self.bn_grad(O.relu_grad(y, dy), x, gamma, xs, eps)
+
     def relu(self, x, shape):
         return _s(O.relu(x))
 

@@ -20,12 +20,13 @@ def _onehot(rng, n, classes):
     return y
 
 
-def _plain(build, inputs, seed, steps, lr, backend):
+def _plain(build, inputs, seed, steps, lr, backend, fused=False):
     from tsplit_amd import graph, workloads
     store = workloads.ParamStore(seed)
     losses, binder, dev = [], None, None
     for _ in range(steps):
         t = graph.Tape(backend)
+        t.fuse_bn_relu = fused
         if binder is None:
             binder = workloads.Binder(t, store)
             dev = {k: binder.input(v) for k, v in inputs.items()}
@@ -127,6 +128,30 @@ def test_schedules_change_between_steps_and_the_fastest_is_kept(rng):
     run.binder.pull()
     for k, v in plain_params.items():
         np.testing.assert_array_equal(run.store.values[k], v)
+
+
+def test_budgeted_graph_with_fused_batchnorm_relu_nodes(rng):
+    """BatchNorm + Relu pairs as one node each: the recorded graph is shorter and its peak lower, and the run
+    under half of that gives the bits of the plain fused tape."""
+    from tsplit_amd import graph, tape_budget as tb, workloads
+    build, inputs, lr = _cases(rng)["resnet"]
+    shapes = {k: v.shape for k, v in inputs.items()}
+    ops2, leaves = tb.record(build, shapes)
+    ops1, _ = tb.record(build, shapes, fuse_bn_relu=True)
+    peak2, peak1 = tb.replay(ops2, leaves)[0], tb.replay(ops1, leaves)[0]
+    assert len(ops1) < len(ops2) and peak1 < 0.85 * peak2
+    budget = leaves + int((peak1 - leaves) * 0.5)
+    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(5), budget, min_bytes=0, fuse_bn_relu=True)
+    assert run.plan.away or run.plan.redo
+    got = [float(run.step(lr).value.asnumpy()[0]) for _ in range(3)]
+    run.binder.pull()
+    want, params = _plain(build, inputs, 5, 3, lr, graph.GpuBackend(), fused=True)
+    assert got == want
+    for k, v in params.items():
+        np.testing.assert_array_equal(run.store.values[k], v)
+    # and the fused tape tracks the oracle's two-node tape
+    ref, _ = _plain(build, inputs, 5, 3, lr, OracleBackend())
+    assert max(abs(a - b) / abs(b) for a, b in zip(got, ref)) <= 1e-3, (got, ref)
 
 
 def test_pool_usage_stays_within_the_replayed_peak(rng):

@@ -112,6 +112,17 @@ class GpuBackend(object):
         L.CuDNN_Batch_Normalization_gradient(dy, x, gamma, dx, dg, db, None, None, eps, self.stream)
         return dx, dg, db
 
+    def bn_relu(self, x, gamma, beta, xs, eps):
+        """-> (relu(bn(x)), saved mean, saved inverse deviation): one call, the BatchNorm output is never written."""
+        y, mean, istd = self.empty(xs), self.empty((1, xs[1], 1, 1)), self.empty((1, xs[1], 1, 1))
+        L.batch_norm_relu(x, gamma, beta, y, mean, istd, eps, stream=self.stream)
+        return y, mean, istd
+
+    def bn_relu_grad(self, dy, x, gamma, beta, mean, istd, xs, eps):
+        dx, dg, db = self.empty(xs), self.empty((1, xs[1], 1, 1)), self.empty((1, xs[1], 1, 1))
+        L.batch_norm_relu_gradient(dy, x, gamma, beta, dx, dg, db, mean, istd, eps, stream=self.stream)
+        return dx, dg, db
+
     def relu(self, x, shape):
         y = self.empty(shape)
         L.relu(x, y, self.stream)
@@ -267,6 +278,9 @@ class GpuBackend(object):
 
 
 class Tape(object):
+    # the builders' BatchNorm + Relu pairs as one node each (bn_then_relu); off: the reference's two nodes
+    fuse_bn_relu = False
+
     def __init__(self, backend):
         self.b = backend
         self._nodes = []     # every operator call, in order (Node)
@@ -330,6 +344,32 @@ class Tape(object):
             self._acc(gamma, dg)
             self._acc(beta, db)
         return self._out(fwd(), x.shape, [x, gamma, beta], back, saved=[x, gamma], redo=fwd)
+
+    def batch_norm_relu(self, x, gamma, beta, eps=0.01):
+        """BatchNorm and the Relu behind it as one node (TSplit_BatchNormRelu / _gradient; the reference's graph
+        has two nodes, gpu_ops/BatchNorm.py and gpu_ops/Relu.py): the BatchNorm output is never written, and
+        the gradient reads the BatchNorm's input, the parameters and the two saved statistics vectors."""
+        stats = [None, None]
+
+        def fwd():
+            r = self.b.bn_relu(x.value, gamma.value, beta.value, x.shape, eps)
+            if r is None:                      # a backend that only records shapes
+                return None
+            y, stats[0], stats[1] = r
+            return y
+
+        def back(g):
+            dx, dg, db = self.b.bn_relu_grad(g, x.value, gamma.value, beta.value, stats[0], stats[1], x.shape, eps)
+            self._acc(x, dx)
+            self._acc(gamma, dg)
+            self._acc(beta, db)
+        return self._out(fwd(), x.shape, [x, gamma, beta], back, saved=[x, gamma, beta], redo=fwd)
+
+    def bn_then_relu(self, x, gamma, beta, eps=0.01):
+        """The pair as the reference's graph has it (two nodes), or as one node when the tape was asked to fuse."""
+        if self.fuse_bn_relu:
+            return self.batch_norm_relu(x, gamma, beta, eps)
+        return self.relu(self.batch_norm(x, gamma, beta, eps))
 
     def relu(self, x):
         """gpu_ops/Relu.py:51,117."""

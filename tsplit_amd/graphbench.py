@@ -27,6 +27,8 @@ def main():
     ap.add_argument("--lr", type=float, default=1e-4)
     ap.add_argument("--record", action="store_true", help="record the step into a graph and time its replays")
     ap.add_argument("--split-bf16", action="store_true")
+    ap.add_argument("--fused", action="store_true",
+                    help="BatchNorm + Relu pairs of the conv nets as one node each (TSplit_BatchNormRelu / _gradient)")
     a = ap.parse_args()
     from . import gpu_links, graph, ndarray, stream, workloads
     ctx = ndarray.gpu(0)
@@ -90,6 +92,7 @@ def main():
     def one_step():
         nonlocal binder, dev_inputs
         t = graph.Tape(backend)
+        t.fuse_bn_relu = a.fused
         if binder is None:
             binder = workloads.Binder(t, store)
             dev_inputs = {k: binder.input(v) for k, v in inputs.items()}      # resident before timing
@@ -125,6 +128,7 @@ def main():
     loss_val = float(loss.value.asnumpy()[0])
     print(json.dumps({"net": a.net, "workload": desc, "samples_per_s": n * a.steps / dt, "ms_per_step": dt / a.steps * 1e3,
                       "steps": a.steps, "warmup": a.warmup, "final_loss": loss_val, "forward_ops_per_step": calls[0], "recorded": bool(a.record),
+                      "fused_bn_relu": bool(a.fused),
                       "dtype": "f32", "data": "synthetic"}))
 
 

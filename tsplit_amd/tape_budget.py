@@ -94,12 +94,13 @@ class _Zeros(object):
         return np.broadcast_to(np.float32(0), tuple(int(s) for s in shape))
 
 
-def record(build, inputs):
+def record(build, inputs, fuse_bn_relu=False):
     """Runs `build(tape, binder, cache)` (as graphbench.py's builders: cache maps input names to Vars)
     on shapes only.  inputs: name -> shape.  -> (list of OpRecord, bytes of the leaves: inputs,
-    parameters, constants)."""
+    parameters, constants).  fuse_bn_relu: the builders' BatchNorm + Relu pairs are one node each."""
     from .workloads import Binder
     t = graph.Tape(_ShapeOnly())
+    t.fuse_bn_relu = fuse_bn_relu
     b = Binder(t, _Zeros())
     cache = {k: t.const(None, shape) for k, shape in inputs.items()}
     loss, _ = build(t, b, cache)
@@ -508,11 +509,12 @@ class BudgetedRun(object):
     parameters come from `store` (workloads.ParamStore), inputs are numpy arrays uploaded once."""
 
     def __init__(self, build, inputs, store, budget_bytes, ctx=None, lead=3, track_pool=False, min_bytes=1 << 20,
-                 recompute=True, hold=1):
+                 recompute=True, hold=1, fuse_bn_relu=False):
         from . import stream, workloads
         self.ctx = ctx or ndarray.gpu(0)
         self.build = build
-        self.ops, self.leaves_bytes = record(build, {k: np.shape(v) for k, v in inputs.items()})
+        self.fuse_bn_relu = fuse_bn_relu
+        self.ops, self.leaves_bytes = record(build, {k: np.shape(v) for k, v in inputs.items()}, fuse_bn_relu)
         self.plan = plan(self.ops, self.leaves_bytes, budget_bytes, lead, min_bytes, recompute, hold)
         self._plan_args = (budget_bytes, min_bytes, recompute)
         self.stream = stream.create_stream_handle(self.ctx)
@@ -528,6 +530,7 @@ class BudgetedRun(object):
     def step(self, lr):
         """One forward + backward + SGD step; returns the loss Var (its value stays on the device)."""
         t = BudgetedTape(self.backend, self.plan, self.ops, self.state, self.track_pool)
+        t.fuse_bn_relu = self.fuse_bn_relu
         if self.binder is None:
             self.binder = self._workloads.Binder(t, self.store)
             self.dev_inputs = {k: self.binder.input(v) for k, v in self.inputs.items()}
@@ -573,13 +576,13 @@ class BudgetedRun(object):
 
 
 def max_batch(build_for, input_shapes_for, budget_bytes, planned=True, lead=3, limit=1 << 12, min_bytes=1 << 20,
-              recompute=True):
+              recompute=True, fuse_bn_relu=False):
     """Largest batch whose step fits `budget_bytes`: with `planned` the planner may send values to the
     host, without it the replayed peak of the plain schedule must fit.  build_for(batch) -> builder,
     input_shapes_for(batch) -> name -> shape.  The counterpart of the reference's batch-size sweeps per
     policy (examples/imagenet_resnet.py:139-154).  -> (batch, TapePlan) or (0, None)."""
     def fits(batch):
-        ops, leaves = record(build_for(batch), input_shapes_for(batch))
+        ops, leaves = record(build_for(batch), input_shapes_for(batch), fuse_bn_relu)
         if any(op.bytes >= (1 << 33) for op in ops):      # tensors are limited to 2^31 elements
             return None
         try:

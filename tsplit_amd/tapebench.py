@@ -60,12 +60,12 @@ def _net(name, batch=None):
     raise ValueError(name)
 
 
-def _measure(build, inputs, budget, steps, warmup, lr, recompute=True, lead=3, hold=1, tune=False):
+def _measure(build, inputs, budget, steps, warmup, lr, recompute=True, lead=3, hold=1, tune=False, fused=False):
     from . import tape_budget as tb, workloads
     from .gpu_memory_manager import pool_state
     base = pool_state().used
     run = tb.BudgetedRun(build, inputs, workloads.ParamStore(123), budget, lead=lead, track_pool=True, recompute=recompute,
-                         hold=hold)
+                         hold=hold, fuse_bn_relu=fused)
     tuned = None
     if tune and budget is not None:
         best, timings, _ = run.tune(lr)
@@ -103,6 +103,8 @@ def main():
     ap.add_argument("--max-batch", action="store_true")
     ap.add_argument("--no-recompute", action="store_true", help="the plan may only send values to the host")
     ap.add_argument("--lead", type=int, default=3, help="operators ahead of its first reader at which a value starts coming back")
+    ap.add_argument("--fused", action="store_true",
+                    help="BatchNorm + Relu pairs as one node each (TSplit_BatchNormRelu): the BatchNorm output is never written")
     ap.add_argument("--tune", action="store_true",
                     help="train two steps under each of a few (lead, hold) schedules first and keep the fastest")
     ap.add_argument("--hold", type=int, default=1, help="operators behind its last reader after which a leaving value is released")
@@ -118,26 +120,28 @@ def main():
 
             def shapes_for(n):
                 return {k: (n,) + tail for k, tail in one.items()}
-            resident, _ = tb.max_batch(build_for, shapes_for, budget, planned=False)
-            planned, p = tb.max_batch(build_for, shapes_for, budget, planned=True, recompute=not a.no_recompute)
+            resident, _ = tb.max_batch(build_for, shapes_for, budget, planned=False, fuse_bn_relu=a.fused)
+            planned, p = tb.max_batch(build_for, shapes_for, budget, planned=True, recompute=not a.no_recompute,
+                                      fuse_bn_relu=a.fused)
             row = {"net": a.net, "workload": desc, "budget_GiB": b, "recompute": not a.no_recompute,
                    "max_batch_resident": resident, "max_batch_planned": planned}
             if p is not None:
                 row.update(_measure(build_for(planned), inputs_for(planned, rng), budget, max(1, a.steps // 2), 1, a.lr,
-                                    not a.no_recompute, a.lead, a.hold, a.tune))
+                                    not a.no_recompute, a.lead, a.hold, a.tune, a.fused))
             print(json.dumps(row), flush=True)
         return
     n = a.batch or default_batch
     inputs = inputs_for(n, rng)
     build = build_for(n)
-    ops, leaves = tb.record(build, {k: v.shape for k, v in inputs.items()})
+    ops, leaves = tb.record(build, {k: v.shape for k, v in inputs.items()}, a.fused)
     free_peak = tb.replay(ops, leaves)[0]
     for f in [float(v) for v in a.fractions.split(",")]:
         budget = None if f == 0 else leaves + int((free_peak - leaves) * f)
         row = {"net": a.net, "workload": desc + ", batch %d" % n, "fraction": f,
-               "budget_GiB": None if budget is None else budget / float(1 << 30), "recompute": not a.no_recompute}
+               "budget_GiB": None if budget is None else budget / float(1 << 30), "recompute": not a.no_recompute,
+               "fused_bn_relu": a.fused}
         try:
-            row.update(_measure(build, inputs, budget, a.steps, a.warmup, a.lr, not a.no_recompute, a.lead, a.hold, a.tune))
+            row.update(_measure(build, inputs, budget, a.steps, a.warmup, a.lr, not a.no_recompute, a.lead, a.hold, a.tune, a.fused))
         except ValueError as e:
             row["error"] = str(e)
         print(json.dumps(row), flush=True)

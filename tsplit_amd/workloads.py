@@ -98,8 +98,7 @@ class Binder(object):
 # ------------------------------------------------------------------ ResNet (bottleneck)
 def _bn_relu(t, b, x, name, eps):
     c = x.shape[1]
-    x = t.batch_norm(x, b.get(name + "_scale", (1, c, 1, 1), "one"), b.get(name + "_bias", (1, c, 1, 1), "zero"), eps)
-    return t.relu(x)
+    return t.bn_then_relu(x, b.get(name + "_scale", (1, c, 1, 1), "one"), b.get(name + "_bias", (1, c, 1, 1), "zero"), eps)
 
 
 def _conv(t, b, x, cout, k, stride, pad, name):
@@ -149,8 +148,7 @@ def _conv_bn(t, b, x, cout, kh, kw, stride=1, same=True, eps=0.01):
     w = b.get(name + "_W", (cout, x.shape[1], kh, kw), "he")
     ph, pw = ((kh - stride) // 2, (kw - stride) // 2) if same else (0, 0)
     x = t.conv2d(x, w, ph, pw, stride)
-    x = t.batch_norm(x, b.get(name + "_scale", (1, cout, 1, 1), "one"), b.get(name + "_bias", (1, cout, 1, 1), "zero"), eps)
-    return t.relu(x)
+    return t.bn_then_relu(x, b.get(name + "_scale", (1, cout, 1, 1), "one"), b.get(name + "_bias", (1, cout, 1, 1), "zero"), eps)
 
 
 def _cat(t, parts):
