@@ -207,26 +207,33 @@ def main():
     for _ in range(a.warmup):
         t.step(gx, gy)
     t.sync()
-    # The timed region: K steps with event pairs only around the GEMM launches inside the Winograd routine (the
-    # step's largest kernel, recorded by the library on the compute stream).  The per-call events behind the
-    # kernels{} table cost about 3 us per launch (0.9 ms over the ~400 launches of a step), so they bracket a
-    # second pass of K steps after the timed region.
+    # The timed region: K steps with event pairs only around the launches of the step's largest kernel, the
+    # forward / data-gradient GEMM of the Winograd routine on 128 x 128 tiles (recorded by the library on the
+    # compute stream; 30 launches per step, about 5 us per pair).  The events of the routine's other GEMM kernels
+    # and the per-call events behind the kernels{} table (about 3 us per launch, 0.9 ms over the ~400 launches of
+    # a step) bracket a second pass of K steps after the timed region.
+    dominant_kind = 3 if a.split_bf16 else 0
     if timer:
-        L.winograd_gemm_timing(True)
+        L.winograd_gemm_timing(True, kind=dominant_kind)
     t0 = time.perf_counter()
     for _ in range(a.steps):
         t.step(gx, gy)
     t.sync()
     dt = time.perf_counter() - t0
-    gemm_times = {kind: L.winograd_gemm_times(kind=kind) for kind in range(5)} if timer else {}
+    gemm_times = {dominant_kind: L.winograd_gemm_times(kind=dominant_kind)} if timer else {}
     L.winograd_gemm_timing(False)
     if timer:
         timer.enabled = True
+        L.winograd_gemm_timing(True)
         t1 = time.perf_counter()
         for _ in range(a.steps):
             t.step(gx, gy)
         t.sync()
         dt_instrumented = time.perf_counter() - t1
+        for kind in range(5):
+            if kind != dominant_kind:
+                gemm_times[kind] = L.winograd_gemm_times(kind=kind)
+        L.winograd_gemm_timing(False)
     loss = float(t.loss.asnumpy()[0])
     ms_per_step = dt / a.steps * 1e3
 
@@ -336,9 +343,10 @@ def main():
             out["conv_mfma_util_direct_kernels_pct"] = pct(direct_flop, direct_ms)
         out["kernels"] = kernels
         out["instrumented_ms_per_step"] = dt_instrumented / a.steps * 1e3
-        out["timing_note"] = ("value and ms_per_step: K steps with event pairs around the Winograd GEMM launches only (the winograd_gemm* "
-                              "entries and roofline come from those); the other kernels{} entries: a second pass of K steps with "
-                              "one event per operator call, whose own cost shows in instrumented_ms_per_step")
+        out["timing_note"] = ("value and ms_per_step: K steps with event pairs around the launches of the roofline's kernel only (the "
+                              "Winograd routine's forward / data-gradient GEMM on 128 x 128 tiles: its kernels{} entry and roofline "
+                              "come from those); the other kernels{} entries, the routine's other GEMM kernels included: a second "
+                              "pass of K steps with one event per operator call, whose own cost shows in instrumented_ms_per_step")
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
         # the same 16-image sample, same seeded parameters, once through the GPU path (forward of the first

@@ -496,7 +496,8 @@ int TSplit_ConvTakesWinograd(int images, int in_channels, int out_channels, int 
 /* ---- Timing of the GEMM launches inside the Winograd routine.  NO counterpart in the reference;
  *      for benchmarks that report a kernel's duration measured inside their own timed region.
  *      TSplit_WinogradGemmTiming(1) makes every such launch record an event pair on its stream
- *      (not while the stream is being recorded into a graph); (0) stops and forgets them.
+ *      (not while the stream is being recorded into a graph), (2 + k) only the launches of kind k, so
+ *      that a timed region carries the events of the one kernel it reports; (0) stops and forgets them.
  *      TSplit_WinogradGemmTimes waits for the launches of kind `which` (0: forward and data
  *      gradient on 128 x 128 tiles, 1: filter gradient, 2: forward and data gradient of layers that
  *      produce at most 64 channels, which run on 64 x 256 tiles, 3 / 4: forward and data gradient /

@@ -408,14 +408,14 @@ struct TimedLaunch {
   double flop, bytes;
 };
 std::mutex g_timing_mu;
-bool g_timing_on = false;
+unsigned g_timing_kinds = 0;   // bit k: launches of kind k are timed
 std::vector<TimedLaunch> g_timed;
 
 class GemmTiming {
  public:
   GemmTiming(hipStream_t st, int which, double flop, double bytes) : st_(st) {
     std::lock_guard<std::mutex> lk(g_timing_mu);
-    if (!g_timing_on) return;
+    if (!((g_timing_kinds >> which) & 1u)) return;
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return;
     if (hipEventCreate(&t_.begin) != hipSuccess) return;
@@ -688,7 +688,8 @@ extern "C" int TSplit_SplitBf16(int on, int *was) {
   return 0;
 }
 
-// Switches the timing of the Winograd routine's GEMM launches on or off (and forgets what was recorded).
+// Switches the timing of the Winograd routine's GEMM launches on (1: every kind, 2 + k: kind k only) or off (0),
+// and forgets what was recorded.
 extern "C" int TSplit_WinogradGemmTiming(int on) {
   using namespace tsplit;
   std::lock_guard<std::mutex> lk(g_timing_mu);
@@ -697,7 +698,7 @@ extern "C" int TSplit_WinogradGemmTiming(int on) {
     (void)hipEventDestroy(t.end);
   }
   g_timed.clear();
-  g_timing_on = on != 0;
+  g_timing_kinds = on == 1 ? ~0u : (on >= 2 && on < 34) ? 1u << (on - 2) : 0u;
   return 0;
 }
 

@@ -425,9 +425,10 @@ def conv_takes_winograd(images, in_channels, out_channels, height, width, kernel
                                               int(kernel), int(kernel), int(pad), int(pad), int(stride), which))
 
 
-def winograd_gemm_timing(on):
-    """Switch the event timing of the GEMM launches inside the Winograd routine on or off."""
-    check_call(_LIB.TSplit_WinogradGemmTiming(int(bool(on))))
+def winograd_gemm_timing(on, kind=None):
+    """Switch the event timing of the GEMM launches inside the Winograd routine on or off; with `kind`
+    (see winograd_gemm_times) only the launches of that kind are timed."""
+    check_call(_LIB.TSplit_WinogradGemmTiming(0 if not on else 1 if kind is None else 2 + int(kind)))
 
 
 def split_bf16(on):
