@@ -41,3 +41,23 @@ def test_short_run_prints_the_contract_line():
     # the Winograd GEMM launches inside the timed steps add up to less than the steps themselves
     k = d["kernels"]["winograd_gemm"]
     assert 0 < k["ms_per_step"] < d["ms_per_step"]
+
+
+@pytest.mark.gpu
+def test_run_with_the_cpu_leg_reports_the_same_loss_on_the_same_sample():
+    """With the CPU leg, the line carries the CPU baseline (what was timed, on how many cores) and the first-step
+    loss of the GPU path on the very sample the CPU path ran (16 of the seeded images, 4 micro-tensors on the first
+    four convolutions): the two must agree within the 1e-3 relative bar of the end-to-end comparison."""
+    r = subprocess.run([sys.executable, BENCH, "--steps", "2", "--warmup", "1"], capture_output=True, text=True, cwd=ROOT,
+                       timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    d = json.loads([l for l in r.stdout.splitlines() if l.startswith("{")][-1])
+    base = d["cpu_baseline"]
+    for key in ("value", "unit", "cores", "kind", "sample"):
+        assert key in base, key
+    assert base["kind"] == "port" and base["unit"] == "samples/s" and base["cores"] >= 1 and base["value"] > 0
+    assert d["gpu_vs_cpu_loss_rel_diff"] <= 1e-3, (d["gpu_loss_on_cpu_sample"], base["loss"])
+    assert d["gpu_vs_cpu_loss_within_1e-3"] is True
+    assert d["roofline"]["measured_in"] == "timed region"
+    if "cpu_baseline_onednn" in d:          # the library path on the same sample: an independent third opinion
+        assert abs(d["cpu_baseline_onednn"]["loss"] - base["loss"]) <= 1e-3 * abs(base["loss"])

@@ -38,7 +38,19 @@ def test_mlp_20_steps_tracks_oracle():
 
 
 VGG_20_STEP_LR = 5e-7
-VGG_224_GRADIENT_L2_BAR = 0.25
+# Yardstick for quantities that are not stable functions of rounding (end-to-end gradients through
+# Relu / pooling decisions, the sum of 20 updates): the distance of the float32 run of the oracle from
+# its float64 run is what fp32 arithmetic by itself does to them; the GPU result may sit at most
+# YARDSTICK_FACTOR times as far from the float64 run (both measured norm-wise, relative to the float64
+# result), plus a floor of the operator tolerance for quantities fp32 arithmetic happens to hit.
+# Measured on VGG-16 at 224x224: the float32 oracle sits 0.37 - 0.49 % from the float64 gradients, the
+# device 1.0 - 1.24 % (2.3 - 3.1 times as far; the old fixed bar was 25 %).  The factor is above 2 for a
+# reason that can be named: the distance comes from Relu / pooling decisions that flip, their number
+# grows with the operators' own rounding error, and the Winograd routine's (about 1e-5 of the output,
+# inside the 2e-3 operator bar) is ten times a float32 direct sum's, so about sqrt(10) times the
+# distance is what the arithmetic predicts.
+YARDSTICK_FACTOR = 3.0
+YARDSTICK_FLOOR = 2e-3
 
 
 def _small_convnet():
@@ -96,7 +108,8 @@ def _vgg_20_step_oracle():
         Y = _onehot(rng.randint(0, 10, 8), 10)
         params = trainer.init_params(spec, seed=3)
         ref_losses, ref_params = nets.train(spec, params, X, Y, steps=20, lr=VGG_20_STEP_LR, momentum=0.9)
-        _VGG_20.update(spec=spec, X=X, Y=Y, params=params, ref_losses=ref_losses, ref_params=ref_params)
+        _, f32_params = nets.train(spec, params, X, Y, steps=20, lr=VGG_20_STEP_LR, momentum=0.9, dtype=np.float32)
+        _VGG_20.update(spec=spec, X=X, Y=Y, params=params, ref_losses=ref_losses, ref_params=ref_params, f32_params=f32_params)
     return _VGG_20
 
 
@@ -124,15 +137,17 @@ def test_vgg16_topology_20_steps_tracks_oracle(winograd, monkeypatch):
         got = t.params[k].asnumpy()
         if np.any(params[k] != 0):                 # BatchNorm biases start at zero: their value IS the change
             assert_close(got, ref_params[k], 2e-3, k)
-        # what the 20 updates changed: parameters are stored in fp32 on both sides, so a change is known
-        # to about 1e-3 of itself, and 20 steps of fp32 against float64 arithmetic add to that
-        # (norm-wise: with the Winograd routine forced onto 2x2 and 4x4 planes single entries move more);
-        # a parameter near 1 (the BatchNorm scales) is stored in steps of 2^-23, which each of the 20
-        # roundings may take differently on the two sides
-        d_got, d_ref = got.astype(np.float64) - params[k], ref_params[k].astype(np.float64) - params[k]
-        bound = 5e-2 * np.linalg.norm(d_ref) + np.sqrt(d_ref.size) * 20 * 2.0 ** -24 * np.max(np.abs(params[k]))
-        off = float(np.linalg.norm(d_got - d_ref))
-        assert off <= bound, "change of %s: off by %.3e in norm, bound %.3e" % (k, off, bound)
+        # what the 20 updates changed, against the yardstick: the same 20 steps of the oracle in float32
+        # arithmetic move away from its float64 run by `off_f32`; the device's fp32 run may be at most
+        # YARDSTICK_FACTOR times as far.  Parameters are stored in fp32 on all three sides; one near 1 (the
+        # BatchNorm scales) is stored in steps of 2^-23, which each of the 20 roundings may take differently,
+        # hence the second term
+        d_ref = ref_params[k].astype(np.float64) - params[k]
+        off = float(np.linalg.norm(got.astype(np.float64) - ref_params[k]))
+        off_f32 = float(np.linalg.norm(o["f32_params"][k].astype(np.float64) - ref_params[k]))
+        bound = YARDSTICK_FACTOR * off_f32 + YARDSTICK_FLOOR * np.linalg.norm(d_ref) + \
+            np.sqrt(d_ref.size) * 20 * 2.0 ** -24 * np.max(np.abs(params[k]))
+        assert off <= bound, "change of %s: off by %.3e in norm, the float32 oracle by %.3e, bound %.3e" % (k, off, off_f32, bound)
 
 
 def _rel_l2(got, ref):
@@ -156,10 +171,11 @@ def test_vgg16_224_natural_routing_every_operator_against_oracle():
 
     End to end, the loss is held to 1e-3 of the oracle's.  The end-to-end parameter gradients of this
     13-layer net at initialisation are not a stable function of rounding: which of two nearly equal
-    activations a pooling window or a Relu passes the gradient to flips with the last bit, and the
-    oracle itself, run in float32 instead of float64, moves some of them by several per cent of their
-    largest entry.  They are therefore held to a norm-wise bar, while the tight bars sit on the
-    operators above."""
+    activations a pooling window or a Relu passes the gradient to flips with the last bit.  How far
+    fp32 arithmetic by itself moves them is measured here, not assumed: the oracle runs a second time
+    in float32, and every parameter's gradient from the device must lie within YARDSTICK_FACTOR times
+    that run's distance from the float64 gradient (norm-wise, plus the operator tolerance as a floor).
+    The tight bars sit on the operators above."""
     from oracle import ops
     from tsplit_amd import gpu_links as L, ndarray, trainer
     from util import max_rel_err
@@ -243,7 +259,13 @@ def test_vgg16_224_natural_routing_every_operator_against_oracle():
     # end to end
     loss0, _, ref_grads = nets.forward_backward(spec, params, X, Y, eps)
     assert abs(gpu_loss - loss0) <= 1e-3 * abs(loss0), (gpu_loss, loss0)
+    _, _, f32_grads = nets.forward_backward(spec, params, X, Y, eps, dtype=np.float32)
     l2 = {k: _rel_l2(grads[k].reshape(g.shape), g) for k, g in ref_grads.items()}
-    assert max(l2.values()) <= VGG_224_GRADIENT_L2_BAR, sorted(l2.items(), key=lambda kv: -kv[1])[:5]
+    yard = {k: _rel_l2(f32_grads[k].reshape(g.shape), g) for k, g in ref_grads.items()}
+    over = {k: (l2[k], yard[k]) for k in l2 if l2[k] > YARDSTICK_FACTOR * yard[k] + YARDSTICK_FLOOR}
+    print("end-to-end gradients, relative L2 distance from the float64 oracle (device, float32 oracle):",
+          sorted(((k, round(l2[k], 6), round(yard[k], 6)) for k in l2), key=lambda r: -r[1])[:8])
+    print("largest ratio device / float32 oracle:", max(l2[k] / max(yard[k], 1e-300) for k in l2))
+    assert not over, sorted(over.items(), key=lambda kv: -kv[1][0])[:8]
     for k in ("vgg_fc3_weight", "vgg_fc2_weight", "vgg_fc1_weight"):      # nothing between them and the loss flips
         assert_close(grads[k], ref_grads[k], 2e-3, "gradient of " + k)

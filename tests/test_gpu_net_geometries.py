@@ -1,14 +1,19 @@
-"""Every distinct convolution of full-size ResNet-50 (batch 64, 224x224) and Inception-v4 (batch 32,
-299x299), as `tsplit_amd.workloads` builds them from the reference's examples
-(examples/imagenet_resnet.py:26-122, examples/imagenet_inceptionv4.py:84-234), through all three
-passes at the FULL batch, so that the kernels, tile shapes and cuts between blocks under test are the
-ones a training step of those nets launches:
+"""Every distinct convolution of full-size VGG-16 (batch 64, 224x224, the first four layers on the
+16-image micro-tensors the benchmark step gives them), ResNet-50 (batch 64, 224x224) and Inception-v4
+(batch 32, 299x299), as `tsplit_amd.workloads` builds them from the reference's examples
+(examples/imagenet_vgg.py:24-98, examples/imagenet_resnet.py:26-122,
+examples/imagenet_inceptionv4.py:84-234), through all three passes at the FULL batch, so that the
+kernels, tile shapes and cuts between blocks under test are the ones a training step of those nets
+launches:
 
-  * forward and data gradient of the first two images against the float64 oracle (images are
-    independent, so two images of the full-batch result pin the launch),
-  * the filter gradient, which sums over the batch, through the adjoint identity
-    <conv(x, w), dy> = <x, dx> = <w, dw> evaluated in float64 on the host, and against the oracle on a
-    two-image batch of the same geometry,
+  * forward and data gradient of the first two images and the last one against the float64 oracle
+    (images are independent, so a few images of the full-batch result pin the launch),
+  * the filter gradient, which sums over the batch: a block of 8 x 8 channel pairs of the full-batch
+    result against the oracle run on those channels of the whole batch, the adjoint identity
+    <conv(x, w), dy> = <x, dx> = <w, dw> evaluated in float64 on the host, and the whole gradient
+    against the oracle on a two-image batch of the same geometry,
+  * for VGG-16 every layer but the three-channel first one must take the Winograd routine in all
+    three passes (as in the benchmark step), so none of this can pass on another kernel,
 
 then one full-size training step of each branched example network (ResNet-50, Inception-v4, the
 Transformer): finite loss, a gradient for every parameter, and the same bits when the step is repeated.
@@ -25,7 +30,8 @@ from util import assert_close
 pytestmark = pytest.mark.gpu
 TOL = 2e-3
 
-GEOMETRIES = [("resnet50",) + g for g in workloads.conv_geometries("resnet50")] + \
+GEOMETRIES = [("vgg16",) + g for g in workloads.conv_geometries("vgg16")] + \
+             [("resnet50",) + g for g in workloads.conv_geometries("resnet50")] + \
              [("inception_v4",) + g for g in workloads.conv_geometries("inception_v4")]
 
 
@@ -56,10 +62,21 @@ def test_full_size_convolution(geo):
     x = rng.standard_normal((N, C, H, W), dtype=np.float32)
     w = (rng.standard_normal((Oc, C, kH, kW), dtype=np.float32) / np.float32(np.sqrt(C * kH * kW)))
     dy = rng.standard_normal((N, Oc, oH, oW), dtype=np.float32)
+    if net == "vgg16" and C >= 64:
+        from tsplit_amd import gpu_links as L
+        assert L.conv_takes_winograd(N, C, Oc, H, W), geo
+        assert L.conv_takes_winograd(N, C, Oc, H, W, data_gradient=True), geo
+        assert L.conv_takes_winograd(N, C, Oc, H, W, filter_gradient=True), geo
     y, dx, dw = _three_passes(x, w, dy, ph, pw, s)
-    # two images of the full-batch launches against the oracle
-    assert_close(y[:2], O.conv2d(x[:2], w, ph, pw, s), TOL, "forward %s" % (geo,))
-    assert_close(dx[:2], O.conv2d_grad_data(w, dy[:2], x[:2].shape, ph, pw, s), TOL, "data gradient %s" % (geo,))
+    # a few images of the full-batch launches against the oracle
+    pick = [0, 1, N - 1]
+    assert_close(y[pick], O.conv2d(x[pick], w, ph, pw, s), TOL, "forward %s" % (geo,))
+    assert_close(dx[pick], O.conv2d_grad_data(w, dy[pick], x[pick].shape, ph, pw, s), TOL, "data gradient %s" % (geo,))
+    # a block of the full-batch filter gradient: the sum over all images for 8 x 8 channel pairs
+    cs, os_ = np.sort(rng.choice(C, min(C, 8), replace=False)), np.sort(rng.choice(Oc, min(Oc, 8), replace=False))
+    block = O.conv2d_grad_filter(np.ascontiguousarray(x[:, cs]), np.ascontiguousarray(dy[:, os_]),
+                                 (len(os_), len(cs), kH, kW), ph, pw, s)
+    assert_close(dw[np.ix_(os_, cs)], block, TOL, "filter gradient over the whole batch, channel block %s" % (geo,))
     # the three passes are one bilinear form: <y, dy> = <x, dx> = <w, dw>
     form = _dot64(y, dy)
     scale = _norm64(y) * _norm64(dy)

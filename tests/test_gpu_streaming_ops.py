@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from oracle import ops as O
-from util import assert_close
+from util import assert_close, assert_close_entries
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4
@@ -38,10 +38,10 @@ def test_elementwise_family(ts, shape, rng):
     a.ravel()[::7] = 0.0                      # exercise relu'(0) = 0.5
     ga, gb, out = ts.arr(a), ts.arr(b), ts.empty(shape)
     L, s = ts.links, ts.stream
-    L.matrix_elementwise_add(ga, gb, out, s); assert_close(out.asnumpy(), O.add(a, b), TOL, "add")
-    L.matrix_elementwise_multiply(ga, gb, out, s); assert_close(out.asnumpy(), O.mul(a, b), TOL, "mul")
-    L.matrix_elementwise_add_by_const(ga, 1.5, out, s); assert_close(out.asnumpy(), O.add_const(a, 1.5), TOL, "addc")
-    L.matrix_elementwise_multiply_by_const(ga, -0.3, out, s); assert_close(out.asnumpy(), O.mul_const(a, -0.3), TOL, "mulc")
+    L.matrix_elementwise_add(ga, gb, out, s); assert_close_entries(out.asnumpy(), O.add(a, b), TOL, "add")
+    L.matrix_elementwise_multiply(ga, gb, out, s); assert_close_entries(out.asnumpy(), O.mul(a, b), TOL, "mul")
+    L.matrix_elementwise_add_by_const(ga, 1.5, out, s); assert_close_entries(out.asnumpy(), O.add_const(a, 1.5), TOL, "addc")
+    L.matrix_elementwise_multiply_by_const(ga, -0.3, out, s); assert_close_entries(out.asnumpy(), O.mul_const(a, -0.3), TOL, "mulc")
     L.array_set(out, 2.25, s); np.testing.assert_array_equal(out.asnumpy(), O.array_set(shape, 2.25))
     L.relu(ga, out, s); np.testing.assert_array_equal(out.asnumpy(), O.relu(a).astype(np.float32))
     L.relu_gradient(ga, gb, out, s); np.testing.assert_array_equal(out.asnumpy(), O.relu_grad(a, b).astype(np.float32))
@@ -76,20 +76,20 @@ def test_optimizers(ts, n, rng):
     for _ in range(3):
         L.sgd_update(p, gg, 0.1, s)
         ref = O.sgd_update(ref, g, 0.1).astype(np.float32)
-    assert_close(p.asnumpy(), ref, TOL, "sgd")
+    assert_close_entries(p.asnumpy(), ref, TOL, "sgd")
     for nesterov in (False, True):
         p, v = ts.arr(p0), ts.arr(np.zeros(n, np.float32))
         rp, rv = p0.copy(), np.zeros(n, np.float32)
         for _ in range(3):
             L.momentum_update(p, gg, v, 0.1, 0.9, nesterov, s)
             rp, rv = [t.astype(np.float32) for t in O.momentum_update(rp, g, rv, 0.1, 0.9, nesterov)]
-        assert_close(p.asnumpy(), rp, TOL, "momentum p"); assert_close(v.asnumpy(), rv, TOL, "momentum v")
+        assert_close_entries(p.asnumpy(), rp, TOL, "momentum p"); assert_close_entries(v.asnumpy(), rv, TOL, "momentum v")
     p, acc = ts.arr(p0), ts.arr(np.zeros(n, np.float32))
     rp, racc = p0.copy(), np.zeros(n, np.float32)
     for _ in range(3):
         L.adagrad_update(p, gg, acc, 0.1, 1e-7, s)
         rp, racc = [t.astype(np.float32) for t in O.adagrad_update(rp, g, racc, 0.1, 1e-7)]
-    assert_close(p.asnumpy(), rp, TOL, "adagrad p"); assert_close(acc.asnumpy(), racc, TOL, "adagrad acc")
+    assert_close_entries(p.asnumpy(), rp, TOL, "adagrad p"); assert_close_entries(acc.asnumpy(), racc, TOL, "adagrad acc")
     p, m, v = ts.arr(p0), ts.arr(np.zeros(n, np.float32)), ts.arr(np.zeros(n, np.float32))
     rp, rm, rv = p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
     b1t = b2t = 1.0
@@ -97,8 +97,8 @@ def test_optimizers(ts, n, rng):
         b1t *= 0.9; b2t *= 0.999
         L.adam_update(p, gg, m, v, 0.01, 0.9, 0.999, b1t, b2t, 1e-7, s)
         rp, rm, rv = [t.astype(np.float32) for t in O.adam_update(rp, g, rm, rv, 0.01, 0.9, 0.999, b1t, b2t, 1e-7)]
-    assert_close(p.asnumpy(), rp, TOL, "adam p"); assert_close(m.asnumpy(), rm, TOL, "adam m")
-    assert_close(v.asnumpy(), rv, TOL, "adam v")
+    assert_close_entries(p.asnumpy(), rp, TOL, "adam p"); assert_close_entries(m.asnumpy(), rm, TOL, "adam m")
+    assert_close_entries(v.asnumpy(), rv, TOL, "adam v")
 
 
 # rows of at least 2048 columns in multiples of 4 take the block-per-row cross-entropy kernels
@@ -110,17 +110,17 @@ def test_softmax_and_cross_entropy(ts, rows, cols, rng):
     gy, gl = ts.arr(y), ts.arr(lab)
     out = ts.empty((rows, cols))
     ts.links.softmax(gy, out, ts.stream)
-    assert_close(out.asnumpy(), O.softmax(y), TOL, "softmax")
+    assert_close_entries(out.asnumpy(), O.softmax(y), TOL, "softmax")
     loss = ts.empty((1,))
     ts.links.softmax_cross_entropy(gy, gl, loss, ts.stream)
-    assert_close(loss.asnumpy(), O.softmax_ce(y, lab), TOL, "ce")
+    assert_close_entries(loss.asnumpy(), O.softmax_ce(y, lab), TOL, "ce")
     g = ts.arr(np.array([1.7], np.float32))
     ts.links.softmax_cross_entropy_gradient(gy, gl, g, out, ts.stream)
-    assert_close(out.asnumpy(), O.softmax_ce_grad(y, lab, np.array([1.7], np.float32)), TOL, "ce grad")
+    assert_close_entries(out.asnumpy(), O.softmax_ce_grad(y, lab, np.array([1.7], np.float32)), TOL, "ce grad")
     # smoothed (non one-hot) labels
     sm = (lab * 0.9 + 0.1 / cols).astype(np.float32)
     ts.links.softmax_cross_entropy(gy, ts.arr(sm), loss, ts.stream)
-    assert_close(loss.asnumpy(), O.softmax_ce(y, sm), TOL, "ce smoothed")
+    assert_close_entries(loss.asnumpy(), O.softmax_ce(y, sm), TOL, "ce smoothed")
 
 
 @pytest.mark.parametrize("cols", [1000, 4096])
@@ -174,15 +174,15 @@ def test_batchnorm_forward_backward(ts, shape, saved, rng):
     sv = ts.empty((1, C, 1, 1)) if saved else None
     ts.links.CuDNN_Batch_Normalization(gx, gg, gb, y, sm, sv, 0.99, eps, ts.stream)
     ry, mean, var = O.batchnorm_forward(x, gamma, beta, eps)
-    assert_close(y.asnumpy(), ry, TOL, "bn fwd")
+    assert_close_entries(y.asnumpy(), ry, TOL, "bn fwd")
     if saved:
-        assert_close(sm.asnumpy().ravel(), mean, TOL, "saved mean")
-        assert_close(sv.asnumpy().ravel(), 1 / np.sqrt(var + eps), TOL, "saved inv-std")
+        assert_close_entries(sm.asnumpy().ravel(), mean, TOL, "saved mean")
+        assert_close_entries(sv.asnumpy().ravel(), 1 / np.sqrt(var + eps), TOL, "saved inv-std")
     ts.links.CuDNN_Batch_Normalization_gradient(gdy, gx, gg, dx, dg, db, sm, sv, eps, ts.stream)
     rdx, rdg, rdb = O.batchnorm_backward(dy, x, gamma, eps)
-    assert_close(dx.asnumpy(), rdx, TOL, "bn dx")
-    assert_close(dg.asnumpy().ravel(), rdg, TOL, "bn dgamma")
-    assert_close(db.asnumpy().ravel(), rdb, TOL, "bn dbeta")
+    assert_close_entries(dx.asnumpy(), rdx, TOL, "bn dx")
+    assert_close_entries(dg.asnumpy().ravel(), rdg, TOL, "bn dgamma")
+    assert_close_entries(db.asnumpy().ravel(), rdb, TOL, "bn dbeta")
 
 
 def test_batchnorm_on_micro_tensor_views_differs_from_full_batch(ts, rng):
@@ -408,3 +408,33 @@ def test_optimizer_update_of_many_parameters_in_one_launch(ts, kind, rng):
     # the rows of the 5 x 3 arrays that were not listed are untouched
     np.testing.assert_array_equal(base_many.asnumpy()[[0, 2, 4]], base_one.asnumpy()[[0, 2, 4]])
     L.optimizer_update_multi([], [], None, lr, stream=s)         # nothing to do
+
+
+def test_optimizer_update_of_many_parameters_survives_stream_destruction(ts, rng):
+    """The list of arrays a stream last updated is remembered so that it is uploaded once.  A stream
+    that is destroyed takes its device copy with it: a new stream updating the very same arrays
+    uploads the list again (streams are created and destroyed several times so that a handle value
+    is likely to come back), and a changed list on a live stream is uploaded too."""
+    from tsplit_amd import stream as S
+    L = ts.links
+    shapes = [(7,), (4096,), (64, 3, 3, 3), (100003,)]
+    ps = [rng.normal(size=sh).astype(np.float32) for sh in shapes]
+    one, many = [ts.arr(p) for p in ps], [ts.arr(p) for p in ps]
+    v_one, v_many = [ts.arr(np.zeros_like(p)) for p in ps], [ts.arr(np.zeros_like(p)) for p in ps]
+    lr, mom = 0.05, 0.9
+    for round_ in range(4):
+        s = S.create_stream_handle(ts.ctx)
+        gs = [ts.arr(rng.normal(size=sh)) for sh in shapes]
+        for p, g, v in zip(one, gs, v_one):
+            L.momentum_update(p, g, v, lr, mom, False, s)
+        L.optimizer_update_multi(many, gs, v_many, lr, mom, False, s)
+        # a shorter list on the same stream, then the full one again
+        L.momentum_update(one[1], gs[1], v_one[1], lr, mom, False, s)
+        L.optimizer_update_multi(many[1:2], gs[1:2], v_many[1:2], lr, mom, False, s)
+        for p, g, v in zip(one, gs, v_one):
+            L.momentum_update(p, g, v, lr, mom, False, s)
+        L.optimizer_update_multi(many, gs, v_many, lr, mom, False, s)
+        s.sync()
+        for a, b in zip(one + v_one, many + v_many):
+            np.testing.assert_array_equal(b.asnumpy(), a.asnumpy())
+        del s       # DLStreamDestroy

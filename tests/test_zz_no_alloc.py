@@ -57,3 +57,35 @@ def test_no_alloc_refuses_more_rows_than_its_array_holds(capfd):
     out = ndarray.empty((1,), ctx)
     assert _no_alloc(gz, glab, out) == -1
     assert "fixed scratch array" in capfd.readouterr().err
+
+
+def test_no_alloc_call_allocates_no_device_memory():
+    """What the entry point is for: after the library's init call and one warm-up call, a call changes
+    neither the device pool's accounting nor the device's free memory (hipMemGetInfo, asked through the
+    HIP runtime the library itself is linked against)."""
+    from tsplit_amd import gpu_links as L, gpu_memory_manager as M, ndarray, stream
+    from tsplit_amd._base import _LIB
+    hip = ctypes.CDLL("libamdhip64.so")
+    ctx = ndarray.gpu(0)
+    st = stream.create_stream_handle(ctx)
+    _LIB.cudnn_init(0, None)                      # void in the reference ABI; looks the array up on device 0
+
+    def device_free():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    rng = np.random.RandomState(5)
+    cases = [_case(rng, 2048, 1000, ctx), _case(rng, 64, 4096, ctx)]
+    out = ndarray.empty((1,), ctx)
+    for _, _, gz, glab in cases:                       # warm-up: code objects loaded, kernels resolved
+        assert _no_alloc(gz, glab, out, st) == 0
+    st.sync()
+    pool_before, free_before = M.pool_state(), device_free()
+    for _ in range(3):
+        for _, _, gz, glab in cases:
+            assert _no_alloc(gz, glab, out, st) == 0
+            assert _no_alloc(gz, glab, out, None) == 0
+    st.sync()
+    assert M.pool_state() == pool_before
+    assert device_free() == free_before

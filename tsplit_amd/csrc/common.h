@@ -27,6 +27,10 @@ inline float mib(int64_t elems) { return static_cast<float>(elems) * 4.0f / (102
 // that stream without waiting; ops on different streams never share one.
 void *scratch_get(hipStream_t stream, int slot, size_t bytes);
 
+// Forgets the table of arrays TSplit_OptimizerUpdateMulti keeps for a stream (elementwise.hip);
+// called by DLStreamDestroy once the stream has drained, before its scratch is dropped.
+void multi_update_drop_stream(hipStream_t stream);
+
 // whether contractions take their products in split bf16 (TSplit_SplitBf16; winograd.hip)
 bool split_bf16_enabled();
 

@@ -311,13 +311,44 @@ __global__ __launch_bounds__(kThreads) void ew_multi_kernel(Op op, const MultiTe
   }
 }
 
-// The table of one stream's last multi-array call: uploaded again only when the arrays changed (a
-// trainer passes the same parameters every step, and a recorded step must not copy from the host).
+// The table of one stream's last multi-array call: uploaded again only when the arrays or the device
+// buffer under it changed (a trainer passes the same parameters every step, and a recorded step must
+// not copy from the host).  The copy reads a pinned staging buffer of its own, rewritten only after
+// the previous upload has finished.
 struct MultiTable {
-  std::vector<char> host;
+  std::vector<char> host;          // the table as last uploaded
+  char *dev = nullptr;             // the device buffer it was uploaded into
+  char *pinned = nullptr;          // staging buffer the asynchronous copy reads
+  size_t pinned_bytes = 0;
+  hipEvent_t uploaded = nullptr;   // recorded behind the last upload
+  bool in_graph = false;           // a recorded step launches with this table at `dev`
 };
 std::mutex g_multi_mu;
 std::map<hipStream_t, MultiTable> g_multi;
+
+void multi_table_release(MultiTable &mt) {
+  if (mt.uploaded) {
+    (void)hipEventSynchronize(mt.uploaded);
+    (void)hipEventDestroy(mt.uploaded);
+  }
+  if (mt.pinned) (void)hipHostFree(mt.pinned);
+  mt = MultiTable{};
+}
+
+bool stream_is_recording(hipStream_t s) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  return s && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+}
+
+// The stream is about to be destroyed (it has drained): its table's device buffer goes with the
+// stream's scratch, and a later stream may get the same handle value.
+void tsplit::multi_update_drop_stream(hipStream_t stream) {
+  std::lock_guard<std::mutex> lk(g_multi_mu);
+  auto it = g_multi.find(stream);
+  if (it == g_multi.end()) return;
+  multi_table_release(it->second);
+  g_multi.erase(it);
+}
 
 // arrays[k][i]: array k of tensor i.  Tensors whose arrays are not all 16-byte aligned go through the
 // single-array launch.
@@ -353,15 +384,47 @@ int launch_multi(Op op, const std::vector<std::array<float *, Op::N>> &arrays, c
   std::vector<char> table(tbytes + bbytes);
   std::memcpy(table.data(), tensors.data(), tensors.size() * sizeof(MultiTensor<N>));
   std::memcpy(table.data() + tbytes, blocks.data(), bbytes);
+  const bool recording = stream_is_recording(s);
+  {
+    std::lock_guard<std::mutex> lk(g_multi_mu);
+    MultiTable &mt = g_multi[s];
+    if (mt.in_graph && mt.host != table && !recording) {
+      // a recorded step replays with the table that lies in the device buffer: other arrays on this
+      // stream go through one launch each and leave that table alone
+      for (const MultiTensor<N> &t : tensors) {
+        Ptrs<N> a;
+        for (int k = 0; k < N; ++k) a.p[k] = t.p[k];
+        launch(op, a, t.n, s);
+      }
+      return 0;
+    }
+  }
   char *dev = static_cast<char *>(scratch_get(s, 8, table.size()));
   TS_REQUIRE(dev, "%s: no scratch memory", who);
   {
     std::lock_guard<std::mutex> lk(g_multi_mu);
     MultiTable &mt = g_multi[s];
-    if (mt.host != table) {
-      mt.host = table;      // kept: the copy below reads it
-      TS_HIP(hipMemcpyAsync(dev, mt.host.data(), mt.host.size(), hipMemcpyHostToDevice, s));
+    if (mt.dev != dev || mt.host != table) {
+      TS_REQUIRE(!recording, "%s: the list of arrays changed while a step is being recorded; run the step once before recording it", who);
+      if (mt.uploaded) TS_HIP(hipEventSynchronize(mt.uploaded));   // the staging buffer is free again
+      if (mt.pinned_bytes < table.size()) {
+        if (mt.pinned) (void)hipHostFree(mt.pinned);
+        mt.pinned = nullptr;
+        mt.pinned_bytes = 0;
+        const size_t want = (table.size() + 4095) / 4096 * 4096;
+        TS_HIP(hipHostMalloc(reinterpret_cast<void **>(&mt.pinned), want, hipHostMallocDefault));
+        mt.pinned_bytes = want;
+      }
+      if (!mt.uploaded) TS_HIP(hipEventCreateWithFlags(&mt.uploaded, hipEventDisableTiming));
+      std::memcpy(mt.pinned, table.data(), table.size());
+      mt.dev = nullptr;   // until the copy below is queued nothing valid lies there
+      TS_HIP(hipMemcpyAsync(dev, mt.pinned, table.size(), hipMemcpyHostToDevice, s));
+      TS_HIP(hipEventRecord(mt.uploaded, s));
+      mt.host = table;
+      mt.dev = dev;
+      mt.in_graph = false;
     }
+    mt.in_graph |= recording;
   }
   hipLaunchKernelGGL(ew_multi_kernel<Op>, dim3(static_cast<unsigned>(blocks.size())), dim3(kThreads), 0, s, op,
                      reinterpret_cast<const MultiTensor<N> *>(dev), reinterpret_cast<const MultiBlock *>(dev + tbytes));

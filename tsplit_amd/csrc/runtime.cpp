@@ -326,6 +326,7 @@ int DLStreamDestroy(DLStreamHandle handle) {
   hipStream_t *s = static_cast<hipStream_t *>(handle->handle);
   if (s) {
     (void)hipStreamSynchronize(*s);
+    multi_update_drop_stream(*s);
     scratch_drop_stream(*s);
     TS_HIP(hipStreamDestroy(*s));
     delete s;

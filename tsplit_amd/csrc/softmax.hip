@@ -212,12 +212,18 @@ float *softmax_noalloc_scratch(int dev) {
   if (dev < 0 || dev >= kNoAllocMaxDevices) return nullptr;
   std::lock_guard<std::mutex> lk(g_noalloc_mu);
   if (g_noalloc_ptr[dev]) return g_noalloc_ptr[dev];
+  int caller_dev = -1;
+  if (hipGetDevice(&caller_dev) != hipSuccess) {
+    (void)hipGetLastError();
+    caller_dev = -1;
+  }
   if (hipSetDevice(dev) != hipSuccess) {
     (void)hipGetLastError();
     return nullptr;
   }
   void *ptr = nullptr;
   const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (caller_dev >= 0 && caller_dev != dev) (void)hipSetDevice(caller_dev);   // the caller's device stays current
   if (e != hipSuccess || ptr == nullptr) {
     (void)hipGetLastError();
     std::fprintf(stderr, "[libc_runtime_api] hipGetSymbolAddress(scratch) failed on device %d: %s\n", dev,

@@ -378,8 +378,24 @@ class _ShapeStore(object):
 def conv_geometries(net, batch=None):
     """The distinct convolution geometries of a full-size example network, in order of first use:
     tuples (images, Cin, H, W, Cout, kH, kW, pad_h, pad_w, stride).  net: "resnet50" (batch 64,
-    224x224) or "inception_v4" (batch 32, 299x299), the sizes of the benchmark configurations."""
+    224x224), "inception_v4" (batch 32, 299x299) or "vgg16" (batch 64, 224x224, the first four
+    layers on a quarter of the batch each: the micro-tensors of the benchmark configuration,
+    examples/imagenet_vgg.py:24-98), the sizes of the benchmark configurations."""
     from . import graph
+    if net == "vgg16":
+        from . import trainer
+        n, hw, seen, out, ci = batch or 64, 224, set(), [], 0
+        for layer in trainer.vgg16_spec():
+            if layer[0] == "conv":
+                _, _, cin, cout, k, pad, stride = layer
+                g = ((n + 3) // 4 if ci < 4 else n, cin, hw, hw, cout, k, k, pad, pad, stride)
+                ci += 1
+                if g not in seen:
+                    seen.add(g)
+                    out.append(g)
+            elif layer[0] == "maxpool":
+                hw //= 2
+        return out
     backend = _ShapeBackend()
     t = graph.Tape(backend)
     b = Binder(t, _ShapeStore())
