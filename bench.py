@@ -76,6 +76,33 @@ def traffic_bytes_per_launch(tag):
     return total / launches if launches else None
 
 
+MFMA_PROFILE = os.path.join(ROOT, "profiles", "vgg16_b64_train_step_mfma_counters.txt")
+
+
+def mfma_counters_per_launch(tag, profile=MFMA_PROFILE):
+    """(FLOP the matrix pipes executed per launch, MFMA-busy %) of the class's kernel, from the rocprofv3 counter
+    summary committed under profiles/ (SQ_INSTS_VALU_MFMA_MOPS_F32 x 512 and the MfmaUtil expression; columns:
+    kernel, launches, avg us, MFMA GFLOP, TFLOP/s, of 157.3, MFMA busy %), averaged by launch count over the
+    kernel's variants.  (None, None) when the summary does not list the kernel."""
+    names = TRAFFIC_KERNELS.get(tag)
+    if not names or not os.path.exists(profile):
+        return None, None
+    launches = flop = busy = 0.0
+    with open(profile) as f:
+        for line in f:
+            if not any(line.startswith(n) for n in names):
+                continue
+            cols = line.split()
+            try:
+                n, g, b = float(cols[-6]), float(cols[-4]), float(cols[-1])
+            except (ValueError, IndexError):
+                continue
+            launches += n
+            flop += n * g * 1e9
+            busy += n * b
+    return (flop / launches, busy / launches) if launches else (None, None)
+
+
 def vgg_workload(batch, seed=123):
     from tsplit_amd import trainer
     rng = np.random.RandomState(seed)
@@ -316,6 +343,12 @@ def main():
                            # batch sizes, --fused, --no-split) its figures are those of the second, instrumented pass
                            "measured_in": "timed region" if dom == {0: "winograd_gemm", 3: "winograd_gemm_split_bf16"}[dominant_kind]
                            else "second pass (one event per operator call)"}
+        if split and a.batch == 64 and not a.fused and not a.split_bf16 and dd["unit"] == "flop":
+            # what the matrix pipes executed per launch and the share of cycles they were busy, by counter
+            # (committed summary of a rocprofv3 --pmc run of this command); per_launch above is arithmetic
+            counted, busy = mfma_counters_per_launch(dom)
+            out["roofline"]["per_launch_by_mfma_counter"] = counted
+            out["roofline"]["mfma_busy_pct"] = busy
         # Conv utilisation, two ways.  The thin first layer (Cin*kH*kW = 27) is timed in bytes because
         # HBM bounds it, so its FLOP (forward and filter gradient) are added to both counts.
         conv = {tag: d for tag, d in k.items() if tag.startswith("conv_")}      # the Winograd GEMMs' time is inside these

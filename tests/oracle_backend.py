@@ -131,8 +131,20 @@ class OracleBackend(object):
     def softmax_ce(self, logits, labels):
         return _s(O.softmax_ce(logits, labels)).reshape(1)
 
-    def softmax_ce_grad(self, logits, labels, shape):
-        return _s(O.softmax_ce_grad(logits, labels, np.ones(1, np.float32)))
+    def softmax_ce_grad(self, logits, labels, shape, seed=1.0):
+        return _s(O.softmax_ce_grad(logits, labels, np.full(1, seed, np.float32)))
+
+    # ---- batch micro-tensors: rows [i * n / pieces, (i + 1) * n / pieces) as a view, and a copy into one
+    def piece(self, x, pieces, index):
+        rows = x.shape[0] // pieces
+        assert rows * pieces == x.shape[0]
+        return x[index * rows:(index + 1) * rows]
+
+    def assign(self, dst, src):
+        dst[...] = src
+
+    def empty(self, shape):
+        return np.empty(tuple(int(v) for v in shape), np.float32)
 
     def sgd(self, p, g, lr):
         p[...] = _s(O.sgd_update(p, g, lr))

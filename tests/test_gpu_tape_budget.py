@@ -181,3 +181,100 @@ def test_pool_usage_stays_within_the_replayed_peak(rng):
         assert peaks[tag] >= run.plan.peak_bytes * 0.8, (tag, peaks[tag], run.plan.peak_bytes)
         del run
     assert peaks["half"] < 0.65 * peaks["free"] and peaks["half recomputing"] < 0.65 * peaks["free"]
+
+
+def _transformer_case(rng, batch, **over):
+    from tsplit_amd import workloads
+    kw = dict(len1=12, len2=10, d_model=32, heads=4, d_ff=64, blocks=1, vocab=600, mask_value=-1.0, embed_std=0.05,
+              pos_amplitude=0.2)
+    kw.update(over)
+
+    def build_for(n):
+        cfg = workloads.TransformerConfig(batch=n, **kw)
+        return lambda t, b, c: workloads.transformer(t, b, cfg, c["xs"], c["yi"], c["yo"])
+    ids = lambda length: rng.randint(0, kw["vocab"], size=(batch, length)).astype(np.float32)
+    xs, yi, yo = ids(kw["len1"]), ids(kw["len2"]), ids(kw["len2"])
+    xs[:, -2:] = 0
+    return build_for, {"xs": xs, "yi": yi, "yo": yo}
+
+
+@pytest.mark.parametrize("where", ["tail", "whole graph"])
+def test_transformer_in_micro_tensors_tracks_the_whole_batch_and_the_oracle(where, rng):
+    """The end of the Transformer graph (from the logits on, with the operators in front of it planned under a
+    budget; or as much of the graph as the planner likes: all of it) run on 4 batch micro-tensors of 8 samples: three training steps
+    against the plain tape on the library at the whole batch (same operators on row ranges of the same values:
+    losses and parameters agree to rounding, 1e-5) and against the oracle tape (loss 1e-3, parameters 2e-3)."""
+    from tsplit_amd import graph, tape_budget as tb, workloads
+    batch, pieces, lr, steps = 32, 4, 0.01, 3
+    build_for, inputs = _transformer_case(rng, batch)
+    build = build_for(batch)
+    ops, leaves = tb.record(build, {k: v.shape for k, v in inputs.items()})
+    if where == "tail":
+        # the stretch from the logits' product on, under the tightest budget the rest can then be planned in
+        names = [op.name for op in ops]
+        start = max(i for i, nm in enumerate(names) if nm == "matmul") - 1
+        run = None
+        for frac in (0.2, 0.3, 0.4, 0.5, 0.6, 0.8):
+            budget = leaves + int((tb.replay(ops, leaves)[0] - leaves) * frac)
+            try:
+                run = tb.BudgetedRun(build, inputs, workloads.ParamStore(5), budget, min_bytes=0, piece_build=build_for(batch // pieces),
+                                     pieces=pieces, track_pool=True, split_from=start)
+                break
+            except ValueError:
+                continue
+        assert run is not None and run.plan.split_from == start and run.plan.peak_bytes <= budget
+        assert run.plan.away or run.plan.redo          # the operators in front of the stretch are planned as before
+    else:
+        run = tb.BudgetedRun(build, inputs, workloads.ParamStore(5), None, piece_build=build_for(batch // pieces), pieces=pieces,
+                             split_always=True, track_pool=True)
+        assert run.plan.split_from is not None
+    assert run.plan.pieces == pieces and len(run.ops) == run.plan.split_from + 1
+    from tsplit_amd.gpu_memory_manager import pool_state
+    base = pool_state().used
+    got = []
+    for _ in range(steps):
+        loss = run.step(lr)
+        got.append(float(loss.value.asnumpy()[0]))
+    run.binder.pull()
+    plain_losses, plain_params = _plain(build, inputs, 5, steps, lr, graph.GpuBackend())
+    np.testing.assert_allclose(got, plain_losses, rtol=1e-5)
+    for k, v in plain_params.items():
+        assert_close(run.store.values[k].reshape(v.shape), v, 1e-5, k)
+    ref_losses, ref_params = _plain(build, inputs, 5, steps, lr, OracleBackend())
+    assert max(abs(a - b) / abs(b) for a, b in zip(got, ref_losses)) <= 1e-3, (got, ref_losses)
+    for k, v in ref_params.items():
+        assert_close(run.store.values[k].reshape(v.shape), v, 2e-3, k)
+    # the pool stayed within what the planner replayed (its rounding and the library's own scratch aside)
+    assert run.state.peak_used - base <= run.plan.peak_bytes * 1.05 + (4 << 20), (run.state.peak_used - base, run.plan.peak_bytes)
+
+
+def test_full_size_transformer_in_micro_tensors_of_8(rng):
+    """The benchmark configuration's own clause: the Transformer at batch 32 (6+6 blocks, d_model 512, vocabulary
+    32 000, length 256) with the end of the graph on micro-tensors of 8 samples, under a budget below what any plan
+    over whole values needs (the three 1 GB arrays around the loss at once).  The step must fit that budget in
+    the pool, and its loss must equal the whole batch's on the plain tape to rounding."""
+    from tsplit_amd import graph, tape_budget as tb, workloads
+    from tsplit_amd.gpu_memory_manager import pool_state
+    batch, pieces = 32, 4
+
+    def build_for(n):
+        cfg = workloads.TransformerConfig(batch=n, mask_value=0.0, embed_std=0.0002, pos_amplitude=0.003)
+        return lambda t, b, c: workloads.transformer(t, b, cfg, c["xs"], c["yi"], c["yo"])
+    ids = lambda: rng.randint(1, 32000, size=(batch, 256)).astype(np.float32)
+    inputs = {"xs": ids(), "yi": ids(), "yo": ids()}
+    build = build_for(batch)
+    ops, leaves = tb.record(build, {k: v.shape for k, v in inputs.items()})
+    budget = leaves + int(2.0 * (1 << 30))                       # whole values need 3.17 GiB
+    with pytest.raises(ValueError):
+        tb.plan(ops, leaves, budget)
+    base = pool_state().used
+    run = tb.BudgetedRun(build, inputs, workloads.ParamStore(123), budget, piece_build=build_for(batch // pieces), pieces=pieces,
+                         track_pool=True)
+    assert run.plan.split_from is not None and run.plan.pieces == pieces and run.plan.peak_bytes <= budget
+    loss = float(run.step(1e-4).value.asnumpy()[0])
+    run.sync()
+    assert run.state.peak_used - base <= budget * 1.03 + (8 << 20), ((run.state.peak_used - base) / 2.0 ** 30, budget / 2.0 ** 30)
+    del run
+    plain_losses, _ = _plain(build, inputs, 123, 1, 1e-4, graph.GpuBackend())
+    assert abs(loss - plain_losses[0]) <= 1e-5 * abs(plain_losses[0]), (loss, plain_losses)
+    assert abs(loss - np.log(32000.0)) < 1.0

@@ -22,7 +22,14 @@ graphs of the reference's examples:
                       ahead of the backward sweep, and every value is dropped after the last backward
                       operator (or recomputation) that reads it;
   BudgetedRun         trains step after step under a plan; BudgetedRun.tune runs a few steps under each
-                      of several (lead, hold) schedules and keeps the fastest.
+                      of several (lead, hold) schedules and keeps the fastest;
+  plan_split          when moving and recomputing whole values cannot meet the budget (one operator's
+                      operands, results and gradients do not fit), the END of the graph - from some
+                      operator on, up to the loss - runs per batch micro-tensor (graph.MicroTape: forward
+                      and backward of one micro-tensor back to back, so that stretch's values and
+                      gradients exist for one micro-tensor at a time); the planner takes the shortest
+                      such stretch under which the rest can be planned, measuring what a stretch holds by
+                      running it on a backend that only counts bytes (measure_tail).
 
 Schedule (replayed byte for byte by `replay`, measured against the pool by the tests):
   forward  of operator t : its output is allocated; then every value whose last reader in the forward
@@ -68,9 +75,14 @@ def _bytes(shape):
 
 class OpRecord(object):
     """One operator call of a recorded graph.  Indices refer to operator calls (-1: a leaf)."""
-    __slots__ = ["bytes", "inputs", "saved", "has_backward", "grad_inputs", "leaf_grad_bytes", "cheap"]
+    __slots__ = ["bytes", "inputs", "saved", "has_backward", "grad_inputs", "leaf_grad_bytes", "cheap", "name",
+                 "transient", "early_grads", "early_leaf_grad_bytes"]
 
-    def __init__(self, nbytes, inputs, saved, has_backward, grad_inputs, leaf_grad_bytes, cheap=False):
+    def __init__(self, nbytes, inputs, saved, has_backward, grad_inputs, leaf_grad_bytes, cheap=False, name=None):
+        self.name = name                   # the Tape method of the call
+        # a stretch of operators run per micro-tensor (split_tail): bytes it holds on top of its inputs while it
+        # runs, the outside values whose gradients it leaves behind, and the parameter gradients it creates
+        self.transient, self.early_grads, self.early_leaf_grad_bytes = 0, (), 0
         self.cheap = cheap                 # the operator can compute its output again from its inputs
         self.bytes = nbytes                # of the output
         self.inputs = inputs               # producers of the values the forward operator reads
@@ -80,11 +92,7 @@ class OpRecord(object):
         self.leaf_grad_bytes = leaf_grad_bytes   # bytes of parameter gradients this operator's backward creates
 
 
-class _ShapeOnly(object):
-    """Backend that computes nothing: every primitive returns None."""
-
-    def __getattr__(self, name):
-        return lambda *a, **k: None
+_ShapeOnly = graph._ShapeOnly
 
 
 class _Zeros(object):
@@ -98,15 +106,17 @@ def record(build, inputs, fuse_bn_relu=False):
     """Runs `build(tape, binder, cache)` (as graphbench.py's builders: cache maps input names to Vars)
     on shapes only.  inputs: name -> shape.  -> (list of OpRecord, bytes of the leaves: inputs,
     parameters, constants).  fuse_bn_relu: the builders' BatchNorm + Relu pairs are one node each."""
-    from .workloads import Binder
+    from .workloads import ShapeBinder
     t = graph.Tape(_ShapeOnly())
     t.fuse_bn_relu = fuse_bn_relu
-    b = Binder(t, _Zeros())
+    t._log = []
+    b = ShapeBinder(t, _Zeros())
     cache = {k: t.const(None, shape) for k, shape in inputs.items()}
     loss, _ = build(t, b, cache)
+    assert len(t._log) == len(t._nodes)          # every operator call is one node
     ops = []
     seen_param_grads = set()
-    for node in t._nodes:
+    for node, call in zip(t._nodes, t._log):
         leaf_grad = 0
         for v in node.inputs:
             if v.node < 0 and v.needs_grad and node.back is not None and id(v) not in seen_param_grads:
@@ -115,7 +125,7 @@ def record(build, inputs, fuse_bn_relu=False):
         ops.append(OpRecord(_bytes(node.out.shape), [v.node for v in node.inputs], [v.node for v in node.saved],
                             node.back is not None,
                             [v.node for v in node.inputs if v.node >= 0 and v.needs_grad] if node.back is not None else [],
-                            leaf_grad, node.redo is not None))
+                            leaf_grad, node.redo is not None, call[0]))
     leaves = sum(_bytes(s) for s in inputs.values()) + sum(_bytes(v.shape) for v in b.vars.values())
     leaves += sum(_bytes(shape) for _, shape in b._consts.values())
     assert loss.node == len(ops) - 1
@@ -132,13 +142,15 @@ class TapePlan(object):
         self.free_peak_bytes = free_peak_bytes     # replayed peak with nothing sent away
         self.budget_bytes = budget_bytes
         self.leaves_bytes = leaves_bytes
+        self.split_from, self.pieces = None, 1   # plan_split: operators from split_from on run per micro-tensor
 
     def describe(self):
         gib = float(1 << 30)
         return {"away": len(self.away), "recomputed": len(self.redo), "lead": self.lead, "hold": self.hold,
                 "peak_GiB": self.peak_bytes / gib,
                 "unplanned_peak_GiB": self.free_peak_bytes / gib,
-                "budget_GiB": None if self.budget_bytes is None else self.budget_bytes / gib}
+                "budget_GiB": None if self.budget_bytes is None else self.budget_bytes / gib,
+                "split_from": self.split_from, "pieces": self.pieces}
 
 
 def _uses(ops):
@@ -200,11 +212,24 @@ def replay(ops, leaves_bytes, away=(), lead=3, redo=(), hold=1):
         by_last_fwd[last_fwd[i]].append(i)
     leaving = []                                        # (operator after which it is released, value)
     # ---- forward
+    grads = {}                                          # operator -> bytes of the gradient of its output
     for t, op in enumerate(ops):
         live += op.bytes
         resident[t] = op.bytes
         busy = set(i for i in op.inputs if i >= 0) | {t}
         note(t)
+        if op.transient:
+            # a stretch run per micro-tensor: what one piece holds at its worst moment, then the
+            # gradients it leaves behind (of outside values, released as the backward sweep passes their
+            # producers, and of parameters)
+            live += op.transient
+            note(t)
+            live -= op.transient
+            for i in op.early_grads:
+                grads[i] = ops[i].bytes
+                live += ops[i].bytes
+            live += op.early_leaf_grad_bytes
+            note(t)
         for due, i in leaving:
             if due <= t:
                 live -= resident.pop(i)
@@ -218,7 +243,6 @@ def replay(ops, leaves_bytes, away=(), lead=3, redo=(), hold=1):
     for due, i in leaving:
         live -= resident.pop(i)
     # ---- backward
-    grads = {}                                          # operator -> bytes of the gradient of its output
     fetch_at = collections.defaultdict(list)
     for i in away:
         if need[i]:
@@ -313,7 +337,171 @@ def plan(ops, leaves_bytes, budget_bytes, lead=3, min_bytes=1 << 20, recompute=T
     return TapePlan(away, lead, peak, free_peak, budget_bytes, leaves_bytes, redo, hold)
 
 
-class BudgetedTape(graph.Tape):
+def first_splittable(ops):
+    """Smallest operator index from which on no operator couples the samples of a batch: a stretch
+    run per micro-tensor may start there or later."""
+    s = len(ops) - 1
+    while s > 0 and ops[s - 1].name not in graph.COUPLES_SAMPLES:
+        s -= 1
+    return s
+
+
+def split_tail(ops, split_from, transient_bytes):
+    """The recorded graph with the operators from `split_from` on as ONE operator, run per micro-tensor
+    with forward and backward back to back (graph.MicroTape): it reads the outside values the stretch
+    reads, its output is the loss, nothing is kept for the backward sweep, and while it runs it holds
+    `transient_bytes` (measure_tail) on top of them; the gradients of the outside values and of the
+    stretch's parameters exist from then on."""
+    tail = ops[split_from:]
+    assert tail and ops[-1].name == "softmax_ce" and not any(op.name in graph.COUPLES_SAMPLES for op in tail)
+    outside = sorted({i for op in tail for i in op.inputs if 0 <= i < split_from})
+    sup = OpRecord(ops[-1].bytes, outside, [], False, [], 0, False, "micro_tensor_tail")
+    sup.transient = int(transient_bytes)
+    sup.early_grads = tuple(sorted({i for op in tail for i in op.grad_inputs if 0 <= i < split_from}))
+    sup.early_leaf_grad_bytes = sum(op.leaf_grad_bytes for op in tail)
+    return list(ops[:split_from]) + [sup]
+
+
+class _Counter(object):
+    def __init__(self):
+        self.live = self.peak = 0
+
+
+class _FakeArray(object):
+    """Stands for a device array of `nbytes`: counted while it is referenced, as the pool counts the real one."""
+    __slots__ = ["nbytes", "counter", "owner"]
+
+    def __init__(self, nbytes, counter, owner=None):
+        self.nbytes, self.counter, self.owner = nbytes, counter, owner
+        counter.live += nbytes
+        counter.peak = max(counter.peak, counter.live)
+
+    def __del__(self):
+        self.counter.live -= self.nbytes
+
+
+class _NoLinks(object):
+    def __getattr__(self, name):
+        return lambda *a, **k: None
+
+
+class CountingBackend(graph.GpuBackend):
+    """graph.GpuBackend with every library call taken out: the same Python runs, allocating and dropping
+    stand-in arrays at the same points, so the bytes a tape holds can be read off without a device."""
+    L = _NoLinks()
+
+    def __init__(self):
+        self.ctx, self.stream, self.counter = None, None, _Counter()
+
+    def empty(self, shape):
+        return _FakeArray((_bytes(shape) + 255) // 256 * 256, self.counter)
+
+    def from_numpy(self, a):
+        return self.empty(np.shape(a))
+
+    def piece(self, x, pieces, index):
+        return _FakeArray(0, self.counter, x)            # a view: no memory of its own, keeps its parent
+
+    def assign(self, dst, src):
+        pass
+
+    def sync(self):
+        pass
+
+
+def measure_tail(build, inputs, piece_calls, split_from, pieces, fuse_bn_relu=False):
+    """Bytes the stretch of operators from `split_from` on holds at its worst moment, beyond what is
+    resident when it starts, when run per micro-tensor: found by running the builder on a MicroTape over
+    a backend that only counts (the executor's own Python, stand-in arrays)."""
+    from .workloads import ShapeBinder
+    backend = CountingBackend()
+    level = {}
+
+    class Probe(graph.MicroTape):
+        def _run_pieces(self, loss_var):
+            level["start"] = backend.counter.live
+            backend.counter.peak = backend.counter.live
+            out = graph.MicroTape._run_pieces(self, loss_var)
+            level["peak"] = backend.counter.peak
+            return out
+
+    t = Probe(backend, split_from, pieces, piece_calls, len(piece_calls))
+    t.fuse_bn_relu = fuse_bn_relu
+    b = ShapeBinder(t, _Zeros())
+    cache = {k: t.const(backend.empty(shape), shape) for k, shape in inputs.items()}
+    build(t, b, cache)
+    return level["peak"] - level["start"]
+
+
+def trace_pieces(piece_build, piece_inputs, fuse_bn_relu=False):
+    """The operator calls of the builder at the micro-tensors' batch size (graph.trace)."""
+    from .workloads import ShapeBinder
+    return graph.trace(piece_build, piece_inputs, lambda t: ShapeBinder(t, _Zeros()), fuse_bn_relu)
+
+
+LINK_BYTES_PER_S = 57e9             # pinned host memory <-> HBM through DLArrayCopyFromTo, each way
+HBM_BYTES_PER_S = 5e12              # what the streaming kernels that recompute a value sustain
+SPLIT_ISSUE_MS_PER_OPERATOR = 0.04  # host time to issue one operator's forward and backward once more
+
+
+def plan_split(ops, leaves_bytes, budget_bytes, build, inputs, piece_calls, pieces, lead=3, min_bytes=1 << 20,
+               recompute=True, hold=1, fuse_bn_relu=False, always=False, split_from=None):
+    """-> (TapePlan, the operators the plan refers to).  The plan over whole values is kept when it moves and
+    recomputes nothing.  Otherwise (or with `always`) the end of the graph may run per micro-tensor: stretches
+    that start 1, 2, 4, 8 ... operators before the loss, and at the first operator from which on nothing
+    couples the samples of a batch, are planned as well, and the plan with the smallest estimated cost per step
+    wins: bytes sent to the host and back at the link's rate, bytes recomputed at three passes over HBM, and, for
+    a stretch, the host's time to issue its operators once more per extra micro-tensor (the kernels themselves do
+    the same work on row ranges; SPLIT_ISSUE_MS_PER_OPERATOR was measured on the Transformer at batch 32, where a
+    stretch over the whole graph in 4 pieces adds 73 ms to a 42 ms step).  plan.split_from / plan.pieces say what
+    was chosen.  With `split_from` the stretch starts at that operator and nothing else is tried."""
+    always = always or split_from is not None
+
+    def cost(p, cut):
+        ms = 2e3 * sum(cut[i].bytes for i in p.away) / LINK_BYTES_PER_S + 3e3 * sum(cut[i].bytes for i in p.redo) / HBM_BYTES_PER_S
+        if p.split_from is not None:
+            ms += (len(ops) - p.split_from) * (p.pieces - 1) * SPLIT_ISSUE_MS_PER_OPERATOR
+        return ms
+
+    best = None
+    if not always:
+        try:
+            p = plan(ops, leaves_bytes, budget_bytes, lead, min_bytes, recompute, hold)
+            if not p.away and not p.redo:
+                return p, ops
+            best = (cost(p, ops), p, ops)
+        except ValueError:
+            pass
+    n = len(ops)
+    assert len(piece_calls) == n, "the builder makes other calls at the micro-tensors' batch size"
+    lowest = first_splittable(ops)
+    starts, step = [], 1
+    while n - 1 - step > lowest:
+        starts.append(n - 1 - step)
+        step *= 2
+    starts.append(lowest)
+    if split_from is not None:
+        assert lowest <= split_from < n - 1, "a stretch run per micro-tensor starts at operator %d or later" % lowest
+        starts = [split_from]
+    last_error = None
+    for s in starts:
+        if s >= n - 1:
+            continue
+        cut = split_tail(ops, s, measure_tail(build, inputs, piece_calls, s, pieces, fuse_bn_relu))
+        try:
+            p = plan(cut, leaves_bytes, budget_bytes, lead, min_bytes, recompute, hold)
+        except ValueError as e:
+            last_error = e
+            continue
+        p.split_from, p.pieces = s, pieces
+        if best is None or cost(p, cut) < best[0]:
+            best = (cost(p, cut), p, cut)
+    if best is None:
+        raise last_error or ValueError("no operator of this graph can run per micro-tensor")
+    return best[1], best[2]
+
+
+class BudgetedTape(graph.MicroTape):
     """A Tape that executes `plan` (see the module description).  One instance per step; the streams
     and the pinned host buffers live in `state`, shared by the steps (BudgetedTape.make_state)."""
 
@@ -331,8 +519,11 @@ class BudgetedTape(graph.Tape):
     def make_state(ctx):
         return BudgetedTape.State(ctx)
 
-    def __init__(self, backend, tape_plan, ops, state, track_pool=False):
-        graph.Tape.__init__(self, backend)
+    def __init__(self, backend, tape_plan, ops, state, track_pool=False, piece_calls=None):
+        if tape_plan.split_from is None:
+            graph.MicroTape.__init__(self, backend)
+        else:
+            graph.MicroTape.__init__(self, backend, tape_plan.split_from, tape_plan.pieces, piece_calls, len(piece_calls))
         self.plan, self.ops, self.state = tape_plan, ops, state
         self.track_pool = track_pool
         n = len(ops)
@@ -380,6 +571,9 @@ class BudgetedTape(graph.Tape):
             self.state.host_waits += 1
             return True
         return False
+
+    def _inside_piece(self):
+        self._note_pool()
 
     def _note_pool(self):
         if self.track_pool:
@@ -489,7 +683,7 @@ class BudgetedTape(graph.Tape):
         for i in sorted(self.fetch_at[n - 1], key=lambda i: -self.first[i]):     # planned for the first operator
             if i in self.gone:
                 self._fetch(i)
-        graph.Tape.backward(self, loss)
+        graph.MicroTape.backward(self, loss)
 
     def _after_backward(self, node):
         # the sweep reaches operator j - 1 next: issue what the plan fetches there before its operators
@@ -509,13 +703,24 @@ class BudgetedRun(object):
     parameters come from `store` (workloads.ParamStore), inputs are numpy arrays uploaded once."""
 
     def __init__(self, build, inputs, store, budget_bytes, ctx=None, lead=3, track_pool=False, min_bytes=1 << 20,
-                 recompute=True, hold=1, fuse_bn_relu=False):
+                 recompute=True, hold=1, fuse_bn_relu=False, piece_build=None, pieces=1, split_always=False, split_from=None):
+        """piece_build, pieces: the same builder for batch / pieces samples.  With them the planner may run the end
+        of the graph per batch micro-tensor when whole values cannot meet the budget (plan_split), or does so
+        in any case with `split_always`."""
         from . import stream, workloads
         self.ctx = ctx or ndarray.gpu(0)
         self.build = build
         self.fuse_bn_relu = fuse_bn_relu
-        self.ops, self.leaves_bytes = record(build, {k: np.shape(v) for k, v in inputs.items()}, fuse_bn_relu)
-        self.plan = plan(self.ops, self.leaves_bytes, budget_bytes, lead, min_bytes, recompute, hold)
+        shapes = {k: tuple(np.shape(v)) for k, v in inputs.items()}
+        self.ops, self.leaves_bytes = record(build, shapes, fuse_bn_relu)
+        self.piece_calls = None
+        if piece_build is not None and pieces > 1:
+            assert all(sh[0] % pieces == 0 for sh in shapes.values()), "the batch must divide by the number of micro-tensors"
+            self.piece_calls = trace_pieces(piece_build, {k: (sh[0] // pieces,) + sh[1:] for k, sh in shapes.items()}, fuse_bn_relu)
+            self.plan, self.ops = plan_split(self.ops, self.leaves_bytes, budget_bytes, build, shapes, self.piece_calls, pieces,
+                                             lead, min_bytes, recompute, hold, fuse_bn_relu, split_always, split_from)
+        else:
+            self.plan = plan(self.ops, self.leaves_bytes, budget_bytes, lead, min_bytes, recompute, hold)
         self._plan_args = (budget_bytes, min_bytes, recompute)
         self.stream = stream.create_stream_handle(self.ctx)
         self.backend = graph.GpuBackend(self.ctx, self.stream)
@@ -529,7 +734,7 @@ class BudgetedRun(object):
 
     def step(self, lr):
         """One forward + backward + SGD step; returns the loss Var (its value stays on the device)."""
-        t = BudgetedTape(self.backend, self.plan, self.ops, self.state, self.track_pool)
+        t = BudgetedTape(self.backend, self.plan, self.ops, self.state, self.track_pool, self.piece_calls)
         t.fuse_bn_relu = self.fuse_bn_relu
         if self.binder is None:
             self.binder = self._workloads.Binder(t, self.store)
@@ -557,6 +762,7 @@ class BudgetedRun(object):
                 plans[(lead, hold)] = plan(self.ops, self.leaves_bytes, budget_bytes, lead, min_bytes, recompute, hold)
             except ValueError:
                 continue
+            plans[(lead, hold)].split_from, plans[(lead, hold)].pieces = self.plan.split_from, self.plan.pieces
             self.plan = plans[(lead, hold)]
             losses.append(self.step(lr))
             self.sync()

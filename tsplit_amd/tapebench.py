@@ -3,6 +3,7 @@ executor of tape_budget.py on ResNet-50 (batch 64), Inception-v4 (batch 32) and 
 
     python -m tsplit_amd.tapebench --net resnet50|inception_v4|transformer [--fractions 0,0.75,0.5,0.35] [--steps 4] [--warmup 1] [--no-recompute] [--tune | --lead L --hold H]
     python -m tsplit_amd.tapebench --net resnet50|inception_v4 --max-batch [--budgets 8,16] [--no-recompute] [--tune]
+    python -m tsplit_amd.tapebench --net transformer --fractions 0.5,0.35,0.25,0.15 --split 4 [--split-always]
 
 For every fraction f (0 = no limit) the budget is the leaves (parameters, their gradients' room is part
 of the replay, inputs, constants) plus f times what the operators' values and gradients take at the
@@ -60,12 +61,13 @@ def _net(name, batch=None):
     raise ValueError(name)
 
 
-def _measure(build, inputs, budget, steps, warmup, lr, recompute=True, lead=3, hold=1, tune=False, fused=False):
+def _measure(build, inputs, budget, steps, warmup, lr, recompute=True, lead=3, hold=1, tune=False, fused=False,
+             piece_build=None, pieces=1, split_always=False):
     from . import tape_budget as tb, workloads
     from .gpu_memory_manager import pool_state
     base = pool_state().used
     run = tb.BudgetedRun(build, inputs, workloads.ParamStore(123), budget, lead=lead, track_pool=True, recompute=recompute,
-                         hold=hold, fuse_bn_relu=fused)
+                         hold=hold, fuse_bn_relu=fused, piece_build=piece_build, pieces=pieces, split_always=split_always)
     tuned = None
     if tune and budget is not None:
         best, timings, _ = run.tune(lr)
@@ -88,7 +90,10 @@ def _measure(build, inputs, budget, steps, warmup, lr, recompute=True, lead=3, h
             "away_GiB": sum(run.ops[i].bytes for i in run.plan.away) / gib, "values_recomputed": len(run.plan.redo),
             "recomputed_GiB": sum(run.ops[i].bytes for i in run.plan.redo) / gib,
             "host_waits_per_step": (run.state.host_waits - waits0) / steps, "loss": float(loss.value.asnumpy()[0]),
-            "lead": run.plan.lead, "hold": run.plan.hold, "tuned": tuned}
+            "lead": run.plan.lead, "hold": run.plan.hold, "tuned": tuned,
+            # operators from split_from on (of operators_whole in the graph) run per batch micro-tensor, `pieces` of them
+            "split_from": run.plan.split_from, "pieces": run.plan.pieces,
+            "operators_whole": len(run.piece_calls) if run.piece_calls else len(run.ops)}
 
 
 def main():
@@ -108,6 +113,9 @@ def main():
     ap.add_argument("--tune", action="store_true",
                     help="train two steps under each of a few (lead, hold) schedules first and keep the fastest")
     ap.add_argument("--hold", type=int, default=1, help="operators behind its last reader after which a leaving value is released")
+    ap.add_argument("--split", type=int, default=0,
+                    help="the planner may run the end of the graph on this many batch micro-tensors when whole values cannot meet the budget")
+    ap.add_argument("--split-always", action="store_true", help="with --split: run a stretch per micro-tensor under every budget")
     a = ap.parse_args()
     from . import tape_budget as tb
     build_for, inputs_for, default_batch, desc = _net(a.net)
@@ -141,7 +149,8 @@ def main():
                "budget_GiB": None if budget is None else budget / float(1 << 30), "recompute": not a.no_recompute,
                "fused_bn_relu": a.fused}
         try:
-            row.update(_measure(build, inputs, budget, a.steps, a.warmup, a.lr, not a.no_recompute, a.lead, a.hold, a.tune, a.fused))
+            row.update(_measure(build, inputs, budget, a.steps, a.warmup, a.lr, not a.no_recompute, a.lead, a.hold, a.tune, a.fused,
+                                build_for(n // a.split) if a.split > 1 else None, max(1, a.split), a.split_always))
         except ValueError as e:
             row["error"] = str(e)
         print(json.dumps(row), flush=True)

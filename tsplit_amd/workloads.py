@@ -95,6 +95,21 @@ class Binder(object):
                 self.store.values[k] = np.ascontiguousarray(self.t.b.to_numpy(v.value), dtype=np.float32).reshape(v.shape)
 
 
+class ShapeBinder(Binder):
+    """A Binder for runs that only need shapes (recording a graph, counting bytes): a constant's array is
+    built once per process to learn its shape and never again."""
+    _shapes = {}
+
+    def constant(self, key, make):
+        if key not in ShapeBinder._shapes:
+            ShapeBinder._shapes[key] = tuple(np.shape(make()))
+        shape = ShapeBinder._shapes[key]
+        if key not in self._consts:
+            self._consts[key] = (self.t.b.from_numpy(np.broadcast_to(np.float32(0), shape)), shape)
+        value, shape = self._consts[key]
+        return self.t.const(value, shape)
+
+
 # ------------------------------------------------------------------ ResNet (bottleneck)
 def _bn_relu(t, b, x, name, eps):
     c = x.shape[1]
