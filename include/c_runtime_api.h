@@ -482,6 +482,16 @@ int TSplit_OptimizerUpdateMulti(DLArrayHandle *params, const DLArrayHandle *grad
                                 DLArrayHandle *velocities, int count, float lr, float momentum,
                                 int nesterov, DLStreamHandle stream_handle);
 
+/* ---- No counterpart in the reference: reports how CuDNN_DLGpuBatch_Normalization obtained its batch
+ *      statistics.  A forward convolution whose epilogue sums its output per channel leaves those sums
+ *      noted for the memory it wrote; a BatchNorm called next on exactly that tensor (the outputs of
+ *      consecutive batch micro-tensors count as one tensor), on the same stream and with no other
+ *      library call in between that could have written it, takes mean and variance from them and reads
+ *      the tensor once instead of twice.  *calls_served: BatchNorm calls served that way since the
+ *      library was loaded; *notes_live: non-zero while such a note is pending.  Either pointer may be
+ *      NULL.  TSPLIT_BN_LOOKBEHIND=0 in the environment switches the mechanism off. ---- */
+int TSplit_BatchNormLookBehind(long long *calls_served, int *notes_live);
+
 /* ---- Which routine a convolution takes.  NO counterpart in the reference (cuDNN's choice is
  *      internal there, src/ops/CudnnConv2d.cu:66).  Returns 1 when CuDNN_DLGpuConv2d (pass 0),
  *      CuDNN_DLGpuConv2d_Gradient_of_Data (pass 1) or CuDNN_DLGpuConv2d_Gradient_of_Filter (pass 2)

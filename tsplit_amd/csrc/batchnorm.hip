@@ -833,7 +833,16 @@ int bn_channel_sums(const DLArray *y, double *dst, hipStream_t st) {
 
 using namespace tsplit;
 
+// BatchNorm calls served from a convolution's note (TSplit_BatchNormLookBehind reports it)
+static std::atomic<long long> g_bn_from_notes{0};
+
 extern "C" {
+
+int TSplit_BatchNormLookBehind(long long *calls_served, int *notes_live) {
+  if (calls_served) *calls_served = g_bn_from_notes.load(std::memory_order_relaxed);
+  if (notes_live) *notes_live = tsplit::g_conv_notes_live.load(std::memory_order_relaxed);
+  return 0;
+}
 
 // coefficients from the partial sums (pair k of channel c at part[(c * part_c + k * part_k) * 2]), then
 // the streaming pass y = a*x + b (+ Relu)
@@ -889,7 +898,27 @@ static int bn_forward(const char *who, bool relu, const DLArrayHandle input_X, c
   TS_REQUIRE(!save_mean_arr || numel(save_mean_arr) == C, "%s: save_mean must hold C elements", who);
   TS_REQUIRE(!save_var_arr || numel(save_var_arr) == C, "%s: save_var must hold C elements", who);
   TS_REQUIRE(!relu || (save_mean_arr && save_var_arr), "%s: the fused form needs both save arrays", who);
+  // sums a convolution left for exactly this tensor on this stream (common.h): looked up before
+  // stream_of() ends all notes, since this call writes too
+  const double *note_sums = nullptr;
+  int note_slots = 0;
+  if (numel(input_X) > 0 && !one_pass_ok(input_X) && C <= INT32_MAX && input_X->shape[2] * input_X->shape[3] <= INT32_MAX)
+    note_slots = conv_notes_take(stream_keep_notes(stream_handle), input_X->data, static_cast<size_t>(numel(input_X)) * sizeof(float),
+                                 static_cast<int>(C), static_cast<int>(input_X->shape[2] * input_X->shape[3]), &note_sums);
   hipStream_t s = stream_of(stream_handle);
+  if (note_slots > 0) {
+    // the later convolutions that reuse the sums' memory are ordered behind this call on its stream
+    g_bn_from_notes.fetch_add(1, std::memory_order_relaxed);
+    ProfileScope psn(p, s, numel(input_X) + 2 * C, numel(output_Y), 0);
+    const bool aln = aligned16(input_X->data) && aligned16(output_Y->data);
+    Plan apn;
+    TS_REQUIRE(make_plan(input_X, aln, 4 * kThreads, 1 << 22, apn), "%s: unsupported shape", who);
+    float *coefn = static_cast<float *>(scratch_get(s, 1, static_cast<size_t>(C) * 2 * sizeof(float)));
+    TS_REQUIRE(coefn, "%s: no scratch memory", who);
+    bn_apply_from(note_sums, note_slots, 1, C, coefn, apn, relu, input_X, bn_scale, bn_bias, output_Y, eps, save_mean_arr,
+                  save_var_arr, s);
+    return psn.finish();
+  }
   if (one_pass_ok(input_X)) {
     const uint32_t hw = static_cast<uint32_t>(input_X->shape[2] * input_X->shape[3]);
     const uint32_t m = static_cast<uint32_t>(input_X->shape[0]) * hw;

@@ -3,6 +3,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 
@@ -16,8 +17,44 @@ inline int64_t numel(const DLArray *a) {
   return n;
 }
 
-inline hipStream_t stream_of(DLStreamHandle h) {
+// ---- what a convolution leaves behind for the BatchNorm that follows it (runtime.cpp) ----
+// A forward convolution whose epilogue can sum its output per channel at no extra pass notes, for the
+// range of memory it wrote, where those sums lie.  CuDNN_DLGpuBatch_Normalization on exactly that range
+// (one note, or the notes of consecutive batch micro-tensors that tile it in ascending order), on the same
+// stream, takes its batch statistics from them instead of reading the tensor twice.  A note may only be
+// used while nothing has written the range since: EVERY operator of the library obtains its stream through
+// stream_of(), which drops all notes (a convolution drops the notes its own output overlaps and keeps the
+// others, so that micro-tensors accumulate); so do copies without a stream, graph launches and stream
+// destruction.  Only calls made through this library are seen: memory written behind its back (another
+// library in the process) is not, as with any of its scratch buffers.  TSPLIT_BN_LOOKBEHIND=0 switches
+// the notes off.
+struct ConvNote {
+  hipStream_t stream;
+  const char *begin;     // the convolution's output
+  size_t bytes;
+  int images, channels, plane;
+  const double *sums;    // [channels][2]: sum and sum of squares over this output
+};
+extern std::atomic<int> g_conv_notes_live;
+void conv_notes_drop_all();
+// drops the notes that overlap [begin, begin + bytes)
+void conv_notes_drop_overlapping(const void *begin, size_t bytes);
+// room for one more note's sums on `stream` (nullptr: none; the caller then makes no note)
+double *conv_note_sums(hipStream_t stream, int channels);
+void conv_note_add(const ConvNote &note);
+// the notes that tile [begin, begin + bytes) of a [*, channels, plane] tensor on `stream`: returns their
+// number (0: none) and the first one's sums, behind which the others' lie at channels * 2 doubles each
+int conv_notes_take(hipStream_t stream, const void *begin, size_t bytes, int channels, int plane, const double **sums);
+bool conv_notes_enabled();
+
+inline hipStream_t stream_keep_notes(DLStreamHandle h) {
   return h ? *static_cast<hipStream_t *>(h->handle) : static_cast<hipStream_t>(nullptr);
+}
+
+// The stream an operator runs on.  Every operator writes somewhere: the notes above end here.
+inline hipStream_t stream_of(DLStreamHandle h) {
+  if (g_conv_notes_live.load(std::memory_order_relaxed)) conv_notes_drop_all();
+  return stream_keep_notes(h);
 }
 
 inline float mib(int64_t elems) { return static_cast<float>(elems) * 4.0f / (1024.0f * 1024.0f); }

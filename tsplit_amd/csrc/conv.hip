@@ -2343,13 +2343,28 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
                  DLStreamHandle sh, ProfilerHandle p, double *stats_dst = nullptr) {
   ConvGeo g;
   if (geo_from(who, x, w, y, ph, pw, s, g)) return -1;
-  hipStream_t st = stream_of(sh);
+  // Without a caller's array for the sums this call may leave a note for the BatchNorm that follows (see
+  // common.h): it then keeps the notes of other ranges (earlier micro-tensors of the same tensor) and
+  // drops those of the range it writes.
+  const bool may_note = !stats_dst && conv_notes_enabled() && numel(y) > 0;
+  hipStream_t st = may_note ? stream_keep_notes(sh) : stream_of(sh);
+  if (may_note) conv_notes_drop_overlapping(y->data, static_cast<size_t>(numel(y)) * sizeof(float));
   ProfileScope ps(p, st, numel(x) + numel(w), numel(y), 0);
   StatsSink sink{nullptr, g.O, 0, 0};
   StatsSink *sk = nullptr;
-  if (stats_dst && numel(y) > 0 && !thin_fwd_ok(g) &&
+  // routes whose epilogue sums the output per channel at (almost) no cost
+  const bool sums_in_epilogue = numel(y) > 0 && !thin_fwd_ok(g) &&
       (winograd_pays(g, g.C) ||
-       (g.C % BK == 0 && tap_kernel_images(g, static_cast<int64_t>(g.C) * g.H * g.W, numel(w)) > 0))) {
+       (g.C % BK == 0 && tap_kernel_images(g, static_cast<int64_t>(g.C) * g.H * g.W, numel(w)) > 0));
+  double *note_dst = nullptr;
+  // (a BatchNorm over at most 16384 values per channel holds them in registers and reads its input once
+  // anyway; this output may be one of a few batch micro-tensors of the BatchNorm's input, hence a quarter)
+  if (may_note && sums_in_epilogue && static_cast<int64_t>(g.imgs) * g.oH * g.oW > 4096 && g.O <= 4096 &&
+      numel(y) < (1ll << 31)) {
+    note_dst = conv_note_sums(st, g.O);
+    stats_dst = note_dst;
+  }
+  if (stats_dst && sums_in_epilogue) {
     // one partial per 32 output positions at most, and a ragged group per run of images
     sink.capacity = static_cast<int>((static_cast<int64_t>(g.imgs) * g.oH * g.oW + 31) / 32) + g.imgs;
     const size_t bytes = static_cast<size_t>(sink.capacity) * g.O * 2 * sizeof(float) +
@@ -2419,6 +2434,9 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
                          static_cast<const double *>(nullptr), 0, g.O, stats_dst);
     }
   }
+  if (note_dst)
+    conv_note_add(ConvNote{st, static_cast<const char *>(y->data), static_cast<size_t>(numel(y)) * sizeof(float), g.imgs, g.O,
+                           g.oH * g.oW, note_dst});
   return ps.finish();
 }
 

@@ -1,5 +1,6 @@
 // Runtime half of the C ABI: array lifecycle, copies, streams, events, the pooled
 // allocator's public face, micro-tensor views.  No kernels here.
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -267,6 +268,99 @@ void scratch_drop_stream(hipStream_t stream) {
   }
 }
 
+// ---------------------------------------------------------------- notes of convolutions for BatchNorm
+namespace {
+std::mutex g_notes_mu;
+std::vector<ConvNote> g_notes;
+// the sums of the notes of a stream lie one behind the other in that stream's scratch slot 9
+constexpr size_t kNoteBytes = 1 << 20;
+std::map<hipStream_t, size_t> g_note_used;
+}  // namespace
+std::atomic<int> g_conv_notes_live{0};
+
+bool conv_notes_enabled() {
+  static const bool on = [] {
+    const char *e = std::getenv("TSPLIT_BN_LOOKBEHIND");
+    return !(e && e[0] == '0');
+  }();
+  return on;
+}
+
+void conv_notes_drop_all() {
+  std::lock_guard<std::mutex> lk(g_notes_mu);
+  g_notes.clear();
+  g_note_used.clear();
+  g_conv_notes_live.store(0, std::memory_order_relaxed);
+}
+
+void conv_notes_drop_overlapping(const void *begin, size_t bytes) {
+  if (!g_conv_notes_live.load(std::memory_order_relaxed)) return;
+  std::lock_guard<std::mutex> lk(g_notes_mu);
+  const char *b = static_cast<const char *>(begin), *e = b + bytes;
+  bool dropped = false;
+  for (auto it = g_notes.begin(); it != g_notes.end();) {
+    if (it->begin < e && b < it->begin + it->bytes) {
+      it = g_notes.erase(it);
+      dropped = true;
+    } else {
+      ++it;
+    }
+  }
+  if (g_notes.empty()) {
+    g_note_used.clear();
+    g_conv_notes_live.store(0, std::memory_order_relaxed);
+  } else if (dropped) {
+    // the remaining notes keep their sums; nothing is handed out twice because offsets only grow until
+    // the list is empty
+  }
+}
+
+double *conv_note_sums(hipStream_t stream, int channels) {
+  const size_t want = static_cast<size_t>(channels) * 2 * sizeof(double);
+  size_t used;
+  {
+    std::lock_guard<std::mutex> lk(g_notes_mu);
+    used = g_note_used[stream];
+    if (used + want > kNoteBytes) return nullptr;
+    g_note_used[stream] = used + want;
+  }
+  char *base = static_cast<char *>(scratch_get(stream, 9, kNoteBytes));
+  return base ? reinterpret_cast<double *>(base + used) : nullptr;
+}
+
+void conv_note_add(const ConvNote &note) {
+  std::lock_guard<std::mutex> lk(g_notes_mu);
+  g_notes.push_back(note);
+  g_conv_notes_live.store(1, std::memory_order_relaxed);
+}
+
+int conv_notes_take(hipStream_t stream, const void *begin, size_t bytes, int channels, int plane, const double **sums) {
+  if (!g_conv_notes_live.load(std::memory_order_relaxed)) return 0;
+  std::lock_guard<std::mutex> lk(g_notes_mu);
+  const char *at = static_cast<const char *>(begin), *end = at + bytes;
+  const double *first = nullptr, *expect = nullptr;
+  int n = 0;
+  // the notes are in the order their convolutions were issued: the pieces must come in ascending order,
+  // one behind the other in memory and in the sums' buffer
+  for (const ConvNote &c : g_notes) {
+    if (c.begin != at) continue;
+    if (c.stream != stream || c.channels != channels || c.plane != plane || at + c.bytes > end) return 0;
+    if (c.bytes != static_cast<size_t>(c.images) * channels * plane * sizeof(float)) return 0;
+    if (n == 0) {
+      first = c.sums;
+    } else if (c.sums != expect) {
+      return 0;
+    }
+    expect = c.sums + static_cast<size_t>(channels) * 2;
+    at += c.bytes;
+    ++n;
+    if (at == end) break;
+  }
+  if (n == 0 || at != end) return 0;
+  *sums = first;
+  return n;
+}
+
 void scratch_recording_opened() {
   std::lock_guard<std::mutex> lk(g_mu);
   ++g_open_recordings;
@@ -326,6 +420,7 @@ int DLStreamDestroy(DLStreamHandle handle) {
   hipStream_t *s = static_cast<hipStream_t *>(handle->handle);
   if (s) {
     (void)hipStreamSynchronize(*s);
+    conv_notes_drop_all();            // their sums lie in this stream's scratch
     multi_update_drop_stream(*s);
     scratch_drop_stream(*s);
     TS_HIP(hipStreamDestroy(*s));
@@ -336,7 +431,7 @@ int DLStreamDestroy(DLStreamHandle handle) {
 }
 
 int DLStreamSync(DLStreamHandle handle) {
-  TS_HIP(hipStreamSynchronize(stream_of(handle)));
+  TS_HIP(hipStreamSynchronize(stream_keep_notes(handle)));   // waiting writes nothing
   return 0;
 }
 
@@ -368,7 +463,8 @@ int DLEventDestroy(DLEventHandle handle) {
 
 int DLEventRecord(DLStreamHandle stream_handle, DLEventHandle event_handle) {
   TS_REQUIRE(event_handle != nullptr, "DLEventRecord: NULL event");
-  TS_HIP(hipEventRecord(*static_cast<hipEvent_t *>(event_handle->handle), stream_of(stream_handle)));
+  // (marking a point on a stream writes nothing: the convolutions' notes stay)
+  TS_HIP(hipEventRecord(*static_cast<hipEvent_t *>(event_handle->handle), stream_keep_notes(stream_handle)));
   return 0;
 }
 
@@ -535,6 +631,7 @@ int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle strea
   if (stream) {
     TS_HIP(hipMemcpyAsync(to->data, from->data, bytes, kind, stream_of(stream)));
   } else {
+    conv_notes_drop_all();            // (the branch above went through stream_of)
     TS_HIP(hipMemcpy(to->data, from->data, bytes, kind));
   }
   return 0;

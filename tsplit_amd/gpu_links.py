@@ -425,6 +425,14 @@ def conv_takes_winograd(images, in_channels, out_channels, height, width, kernel
                                               int(kernel), int(kernel), int(pad), int(pad), int(stride), which))
 
 
+def batch_norm_look_behind():
+    """(BatchNorm calls that took their statistics from the sums the convolution in front of them left,
+    whether such sums are pending right now)."""
+    served, live = ctypes.c_longlong(0), ctypes.c_int(0)
+    check_call(_LIB.TSplit_BatchNormLookBehind(ctypes.byref(served), ctypes.byref(live)))
+    return int(served.value), bool(live.value)
+
+
 def winograd_gemm_timing(on, kind=None):
     """Switch the event timing of the GEMM launches inside the Winograd routine on or off; with `kind`
     (see winograd_gemm_times) only the launches of that kind are timed."""
