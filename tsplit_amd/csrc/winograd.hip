@@ -264,6 +264,12 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const float *__restric
   }
 }
 
+}  // namespace
+}  // namespace tsplit
+namespace tsplit {
+namespace {
+#include "wino_fused.h"
+
 // ---------------------------------------------------------------- filter gradient
 // The forward map is linear in the filter, y = A^T [(G g G^T) . (B^T d B)] A per tile, so the filter
 // gradient is its adjoint: dg = G^T [ sum over tiles (A dy A^T) . (B^T d B) ] G.
@@ -563,6 +569,21 @@ bool split_bf16_enabled() {
   return v != 0;
 }
 
+// Which layers take the one-kernel form: bands of 64 produced channels from 64 or 128 gathered ones, where the
+// three-kernel routine is bound by the traffic of its transformed tensors.  TSPLIT_WINOGRAD_FUSED=0 switches it
+// off, =2 also sends wider layers (any multiple of 64 / 16 channels) through it.
+namespace {
+inline bool fused_wanted(int gathered, int produced) {
+  static const int mode = [] {
+    const char *e = std::getenv("TSPLIT_WINOGRAD_FUSED");
+    return e ? std::atoi(e) : 1;
+  }();
+  if (mode == 0 || produced % fused::kBand || gathered % fused::kChunk) return false;
+  if (mode >= 2) return true;
+  return std::min(gathered, produced) == 64 && std::max(gathered, produced) <= 128;
+}
+}  // namespace
+
 // y[n][produced][H][W] = conv3x3(x[n][gathered][H][W], filter), stride 1, pad 1.  `rotated` selects
 // the data-gradient reading of the filter (stored [gathered][produced][3][3], rotated 180 degrees).
 // With a sink, every block of the output transform adds one partial (sum, sum of squares) per channel.
@@ -570,6 +591,33 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
                       bool rotated, hipStream_t st, StatsSink *sink) {
   const int th = (H + 3) / 4, tw = (W + 3) / 4;
   const int per_img = th * tw;
+  {
+    // few channels: the one-kernel form, whose transformed tensors never leave the chip (wino_fused.h)
+    int gw = 0, gh = 0;
+    if (fused_wanted(gathered, produced) && (H & 3) == 0 && (W & 3) == 0 && aligned16(x) && aligned16(y) &&
+        fused::fused_group(tw, th, gw, gh) && static_cast<int64_t>(imgs) * std::max(gathered, produced) * H * W < (1ll << 31)) {
+      const fused::FusedGeo fg{gathered, produced, H, W, tw, th, gw, gh, tw / gw, (tw / gw) * (th / gh)};
+      float *Uf = static_cast<float *>(scratch_get(st, 3, fused::fused_filter_floats(produced, gathered) * 4));
+      TS_REQUIRE(Uf, "conv (Winograd): no scratch memory");
+      hipLaunchKernelGGL(fused::wino_filter_fused_kernel, dim3((produced * gathered + 255) / 256), dim3(256), 0, st, w, Uf, produced,
+                         gathered, rotated);
+      const unsigned blocks = static_cast<unsigned>(imgs) * fg.groups * (produced / fused::kBand);
+      const double flop = 2.0 * kXi * produced * static_cast<double>(imgs) * per_img * gathered;
+      const double bytes = 4.0 * (static_cast<double>(gathered + produced) * imgs * H * W + static_cast<double>(kXi) * produced * gathered);
+      GemmTiming timed(st, 5, flop, bytes);
+      if (sink) {
+        const int parts = imgs * fg.groups;
+        TS_REQUIRE(sink->used + parts <= sink->capacity, "conv (Winograd): statistics buffer too small");
+        hipLaunchKernelGGL(fused::wino_fused_kernel<true>, dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg,
+                           sink->part + static_cast<int64_t>(sink->used) * produced * 2);
+        sink->used += parts;
+      } else {
+        hipLaunchKernelGGL(fused::wino_fused_kernel<false>, dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg,
+                           static_cast<float *>(nullptr));
+      }
+      return 0;
+    }
+  }
   const int run = run_images(imgs, per_img, gathered, produced);
   TS_REQUIRE(run > 0, "conv (Winograd): one image's tiles do not fit 32-bit offsets");
   const int ld_max = (run * per_img + 3) / 4 * 4;

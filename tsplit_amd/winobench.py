@@ -10,6 +10,8 @@ ones; the GEMM inside a Winograd call by the library's own event pairs (TSplit_W
 GEMM rates count executed FLOP (2 * 36 * rows * tiles * depth) against the 157.3 TFLOP/s fp32 matrix peak.
 With --split-bf16 the GEMMs of layers with more than 64 channels on both sides take their products as six
 bf16 x bf16 terms (TSplit_SplitBf16); their rate is then the fp32-equivalent one (the same FLOP count).
+Layers with 64 channels on one side run forward and data gradient as one kernel (transforms inside): its "GEMM" time
+is the whole call's.
 Prints one JSON object per layer and pass and a final table.
 """
 import argparse
@@ -26,6 +28,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--iters", type=int, default=10)
     ap.add_argument("--split-bf16", action="store_true")
+    ap.add_argument("--layers", type=int, default=len(LAYERS), help="only the first so many layers")
     a = ap.parse_args()
     from . import gpu_links as L, ndarray, stream
     from .timing import EventTimer
@@ -35,7 +38,7 @@ def main():
     timer = EventTimer(ctx)
     rng = np.random.RandomState(0)
     rows = []
-    for n, c, o, hw in LAYERS:
+    for n, c, o, hw in LAYERS[:a.layers]:
         x = ndarray.array(rng.standard_normal((n, c, hw, hw)).astype(np.float32), ctx)
         w = ndarray.array((rng.standard_normal((o, c, 3, 3)) / np.sqrt(9.0 * c)).astype(np.float32), ctx)
         dy = ndarray.array(rng.standard_normal((n, o, hw, hw)).astype(np.float32), ctx)
@@ -66,7 +69,7 @@ def main():
                 fn()
             st.sync()
             launches = ms = gf = 0
-            for k in ((1, 4) if kind == 1 else (0, 2, 3)):
+            for k in ((1, 4) if kind == 1 else (0, 2, 3, 5)):
                 ln, m, f, _ = L.winograd_gemm_times(kind=k)
                 launches, ms, gf = launches + ln, ms + m, gf + f
             L.winograd_gemm_timing(False)
