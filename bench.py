@@ -50,6 +50,7 @@ TRAFFIC_KERNELS = {
     "winograd_gemm": ("wino_gemm_kernel<128, 128>",),
     "winograd_filter_grad_gemm": ("wino_grad_gemm_kernel<3>",),
     "winograd_gemm_64_rows": ("wino_gemm_kernel<64, 256>",),
+    "winograd_fused": ("wino_fused_kernel<",),
 }
 
 
@@ -235,11 +236,11 @@ def main():
         t.step(gx, gy)
     t.sync()
     # The timed region: K steps with event pairs only around the launches of the step's largest kernel, the
-    # forward / data-gradient GEMM of the Winograd routine on 128 x 128 tiles (recorded by the library on the
-    # compute stream; 30 launches per step, about 5 us per pair).  The events of the routine's other GEMM kernels
+    # one-kernel Winograd convolution of the layers with up to 256 channels (forward and data gradient; recorded
+    # by the library on the compute stream; 30 launches per step, about 5 us per pair).  The events of the routine's other GEMM kernels
     # and the per-call events behind the kernels{} table (about 3 us per launch, 0.9 ms over the ~400 launches of
     # a step) bracket a second pass of K steps after the timed region.
-    dominant_kind = 3 if a.split_bf16 else 0
+    dominant_kind = 3 if a.split_bf16 else 5
     if timer:
         L.winograd_gemm_timing(True, kind=dominant_kind)
     t0 = time.perf_counter()
@@ -257,7 +258,7 @@ def main():
             t.step(gx, gy)
         t.sync()
         dt_instrumented = time.perf_counter() - t1
-        for kind in range(5):
+        for kind in range(6):
             if kind != dominant_kind:
                 gemm_times[kind] = L.winograd_gemm_times(kind=kind)
         L.winograd_gemm_timing(False)
@@ -297,7 +298,7 @@ def main():
         # the GEMM kernels inside the Winograd calls, timed by the library with event pairs on the
         # compute stream around each launch; their work is the FLOP they execute
         wino_exec_flop = 0.0
-        for tag, kind in (("winograd_gemm", 0), ("winograd_filter_grad_gemm", 1), ("winograd_gemm_64_rows", 2)):
+        for tag, kind in (("winograd_gemm", 0), ("winograd_filter_grad_gemm", 1), ("winograd_gemm_64_rows", 2), ("winograd_fused", 5)):
             launches, ms, flop, nbytes = gemm_times[kind]
             if launches:
                 wino_exec_flop += flop
@@ -307,6 +308,14 @@ def main():
                                 "achieved": k[tag]["rate"], "unit": "TFLOP/s", "frac": k[tag]["rate"] / PEAK_TFLOPS_FP32_MFMA,
                                 "note": "one kernel inside the *_winograd calls above (its time is part of theirs); "
                                         "executed FLOP"}
+                if kind == 5:
+                    # forward / data gradient of the layers with 64 channels on one side as ONE kernel (transforms inside,
+                    # the transformed tensors never leave the chip): its time is the whole call's, its bytes the activations'
+                    kernels[tag]["hbm_achieved_gbs"] = nbytes / (ms * 1e-3) / 1e9
+                    kernels[tag]["hbm_frac"] = kernels[tag]["hbm_achieved_gbs"] / PEAK_HBM_GBS
+                    kernels[tag]["note"] = ("the whole forward / data-gradient call of the layers with 64 channels on one side: one kernel "
+                                            "with the Winograd transforms inside; executed FLOP (2 * 36 * O * C * tiles), and the "
+                                            "activations' and filter's bytes for hbm_*")
                 if kind == 2:
                     # 64 or 128 channels summed over on 64-row tiles: 16 - 21 executed FLOP per algorithmic byte, at
                     # the ratio of the two peaks (19.7), so both fractions are given
@@ -341,7 +350,7 @@ def main():
                            # which pass the launch durations behind `achieved` come from: the timed region carries event
                            # pairs only for the kernel expected to be the largest; if another one turns out larger (other
                            # batch sizes, --fused, --no-split) its figures are those of the second, instrumented pass
-                           "measured_in": "timed region" if dom == {0: "winograd_gemm", 3: "winograd_gemm_split_bf16"}[dominant_kind]
+                           "measured_in": "timed region" if dom == {5: "winograd_fused", 3: "winograd_gemm_split_bf16"}[dominant_kind]
                            else "second pass (one event per operator call)"}
         if split and a.batch == 64 and not a.fused and not a.split_bf16 and dd["unit"] == "flop":
             # what the matrix pipes executed per launch and the share of cycles they were busy, by counter
@@ -382,8 +391,8 @@ def main():
         out["kernels"] = kernels
         out["instrumented_ms_per_step"] = dt_instrumented / a.steps * 1e3
         out["timing_note"] = ("value and ms_per_step: K steps with event pairs around the launches of the roofline's kernel only (the "
-                              "Winograd routine's forward / data-gradient GEMM on 128 x 128 tiles: its kernels{} entry and roofline "
-                              "come from those); the other kernels{} entries, the routine's other GEMM kernels included: a second "
+                              "one-kernel Winograd convolution, wino_fused_kernel: its kernels{} entry and roofline come from "
+                              "those); the other kernels{} entries, the routine's GEMM kernels included: a second "
                               "pass of K steps with one event per operator call, whose own cost shows in instrumented_ms_per_step")
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()

@@ -2420,7 +2420,8 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
       // the slices' sums live behind the partials in the same scratch buffer (8-byte aligned: the
       // partials are pairs of floats)
       double *tmp = reinterpret_cast<double *>(sink.part + static_cast<int64_t>(sink.capacity) * g.O * 2);
-      const int slices = std::max(1, std::min(kStatsSlices, (sink.used + 63) / 64));
+      // (one slice per 512 partials: the second kernel walks the slices one after the other)
+      const int slices = std::max(1, std::min(kStatsSlices, (sink.used + 511) / 512));
       const int chunk = (sink.used + slices - 1) / slices;
       // one slice: its sums are the result (slice 0 of tmp has dst's layout), no second launch
       hipLaunchKernelGGL(conv_stats_fold_kernel, dim3((g.O + 31) / 32, slices), dim3(256), 0, st, sink.part, sink.used, g.O,

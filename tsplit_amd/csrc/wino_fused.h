@@ -35,7 +35,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kThreadsF = 256;
 constexpr int kSlots = 16;      // tile slots per block
 constexpr int kChunk = 16;      // gathered channels per step
-constexpr int kAhead = 6;       // filter words a wave keeps in flight
+#ifndef FUSED_AHEAD
+#define FUSED_AHEAD 6
+#endif
+constexpr int kAhead = FUSED_AHEAD;       // filter words a wave keeps in flight (must divide 36)
 constexpr int kBand = 64;       // produced channels per block
 
 // Filter transform into the layout the kernel reads: word (chunk, xi, ob, lane) holds, for produced channel
@@ -111,7 +114,9 @@ __device__ __forceinline__ void load_patch(__amdgpu_buffer_rsrc_t rx, const Patc
 // (c % 4) * 16 + slot of every wave reads it as element c / 4 of its 16-byte word.
 // The columns beside the quads come from the neighbouring lanes, which hold the neighbouring tiles of the
 // same row of the group; at the group's edges they are fetched here (lines the neighbouring block's quads
-// brought into the cache; zero beyond the plane) rather than held in registers through the products.
+// brought into the cache; zero beyond the plane) rather than held in registers through the products
+// (fetching them with the quads, a step ahead, measured 8 % slower: six more loads in front of the
+// filter words, which return in order).
 __device__ __forceinline__ void transform_patch(const Patch &p, __amdgpu_buffer_rsrc_t rx, const PatchAddr &pa, unsigned chunk_off,
                                                 bool at_left, bool at_right, int c, int slot, float *__restrict__ Vl) {
   float edge[6];
@@ -199,14 +204,15 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
   for (int j = 0; j < kAhead; ++j) ua[j] = buf_load4(ru, uoff, static_cast<unsigned>(j) * 4096u);
 
   for (int ch = 0; ch < chunks; ++ch) {
+#if !defined(FUSED_VARIANT) || FUSED_VARIANT != 3
     transform_patch(patch, rx, pa, static_cast<unsigned>(ch) * chunk_bytes, at_left, at_right, cl, slot, Vl);
+#endif
     __syncthreads();
     if (ch + 1 < chunks) load_patch(rx, pa, static_cast<unsigned>(ch + 1) * chunk_bytes, patch);
     const unsigned ubase = static_cast<unsigned>(ch * kXi + kAhead) * 4096u;     // the word kAhead points on
     // (the scheduling barriers keep every filter word's load kAhead points ahead of its use and the LDS
     // reads a pair of points ahead: left alone the compiler sinks them next to their uses to save
-    // registers and every point then waits out the cache's latency.  Two points go through the matrix
-    // pipe interleaved, so that no instruction waits for the one before it.)
+    // registers and every point then waits out the cache's latency; a single point ahead was slower)
     f32x4 vb0 = vw[0], vb1 = vw[64];
 #pragma unroll
     for (int xi = 0; xi < kXi; xi += 2) {
@@ -219,6 +225,10 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
       ua[xi % kAhead] = buf_load4(ru, uoff, ubase + static_cast<unsigned>(xi) * 4096u);       // (behind the last chunk: the slack words)
       ua[(xi + 1) % kAhead] = buf_load4(ru, uoff, ubase + static_cast<unsigned>(xi + 1) * 4096u);
       __builtin_amdgcn_sched_barrier(0);
+#if defined(FUSED_VARIANT) && FUSED_VARIANT == 4
+      acc[xi] += a0 * b0;
+      acc[xi + 1] += a1 * b1;
+#else
       acc[xi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.x, b0.x, acc[xi], 0, 0, 0);
       acc[xi + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.x, b1.x, acc[xi + 1], 0, 0, 0);
       acc[xi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.y, b0.y, acc[xi], 0, 0, 0);
@@ -227,6 +237,7 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
       acc[xi + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.z, b1.z, acc[xi + 1], 0, 0, 0);
       acc[xi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.w, b0.w, acc[xi], 0, 0, 0);
       acc[xi + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.w, b1.w, acc[xi + 1], 0, 0, 0);
+#endif
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();

@@ -569,9 +569,11 @@ bool split_bf16_enabled() {
   return v != 0;
 }
 
-// Which layers take the one-kernel form: bands of 64 produced channels from 64 or 128 gathered ones, where the
-// three-kernel routine is bound by the traffic of its transformed tensors.  TSPLIT_WINOGRAD_FUSED=0 switches it
-// off, =2 also sends wider layers (any multiple of 64 / 16 channels) through it.
+// Which layers take the one-kernel form: up to 256 channels on either side (in bands of 64 produced channels and
+// chunks of 16 gathered ones).  Measured per 16- or 64-image call against the three-kernel routine: 64 -> 64 at
+// 224 x 224 forward 467 -> 251 us, 128 -> 128 at 112 x 112 284 -> 232, 128 -> 256 at 56 x 56 486 -> 382, 256 -> 256
+// at 56 x 56 778 -> 708; beyond that the three-kernel routine's GEMM, which runs at 120 TFLOP/s against 90 here,
+// outweighs the transforms it pays for.  TSPLIT_WINOGRAD_FUSED=0 switches the form off, =2 lifts the limit.
 namespace {
 inline bool fused_wanted(int gathered, int produced) {
   static const int mode = [] {
@@ -579,8 +581,7 @@ inline bool fused_wanted(int gathered, int produced) {
     return e ? std::atoi(e) : 1;
   }();
   if (mode == 0 || produced % fused::kBand || gathered % fused::kChunk) return false;
-  if (mode >= 2) return true;
-  return std::min(gathered, produced) == 64 && std::max(gathered, produced) <= 128;
+  return mode >= 2 || std::max(gathered, produced) <= 256;
 }
 }  // namespace
 
@@ -594,7 +595,9 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
   {
     // few channels: the one-kernel form, whose transformed tensors never leave the chip (wino_fused.h)
     int gw = 0, gh = 0;
-    if (fused_wanted(gathered, produced) && (H & 3) == 0 && (W & 3) == 0 && aligned16(x) && aligned16(y) &&
+    // (with the opt-in split-bf16 products the layers they cover keep the three-kernel routine, whose GEMM takes them)
+    const bool split_products = produced > 64 && (gathered & 7) == 0 && split_bf16_enabled();
+    if (!split_products && fused_wanted(gathered, produced) && (H & 3) == 0 && (W & 3) == 0 && aligned16(x) && aligned16(y) &&
         fused::fused_group(tw, th, gw, gh) && static_cast<int64_t>(imgs) * std::max(gathered, produced) * H * W < (1ll << 31)) {
       const fused::FusedGeo fg{gathered, produced, H, W, tw, th, gw, gh, tw / gw, (tw / gw) * (th / gh)};
       float *Uf = static_cast<float *>(scratch_get(st, 3, fused::fused_filter_floats(produced, gathered) * 4));
