@@ -32,18 +32,24 @@ namespace fused {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// the value of the lane below / above within a row of 16 lanes (a data-parallel move, no trip through LDS);
+// the row's first / last lane gets its own value back and does not use it
+__device__ __forceinline__ float from_lane_below(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float from_lane_above(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x101, 0xf, 0xf, false));
+}
+
 constexpr int kThreadsF = 256;
 constexpr int kSlots = 16;      // tile slots per block
 constexpr int kChunk = 16;      // gathered channels per step
-#ifndef FUSED_AHEAD
-#define FUSED_AHEAD 6
-#endif
-constexpr int kAhead = FUSED_AHEAD;       // filter words a wave keeps in flight (must divide 36)
+constexpr int kAhead = 6;       // filter words a wave keeps in flight (divides 36; 4 ran the same, 9 and 12 spill and ran 25 - 40 % slower)
 constexpr int kBand = 64;       // produced channels per block
 
 // Filter transform into the layout the kernel reads: word (chunk, xi, ob, lane) holds, for produced channel
 // o = 16 * ob + lane % 16 and gathered channels c = 16 * chunk + 4 * kk + lane / 16 (kk = 0 .. 3), the four
-// U[xi][o][c].  `bands` bands of 64 produced channels lie one behind the other; kAhead words of slack behind
+// U[xi][o][c].  `bands` bands of 64 produced channels lie one behind the other; `slack_words` words behind
 // each band's last word are read ahead by the kernel and never used.
 inline size_t fused_filter_floats(int produced, int gathered) {
   const size_t band = static_cast<size_t>(gathered / kChunk) * kXi * 4 * 64 * 4;
@@ -51,7 +57,7 @@ inline size_t fused_filter_floats(int produced, int gathered) {
 }
 
 __global__ __launch_bounds__(256) void wino_filter_fused_kernel(const float *__restrict__ w, float *__restrict__ Uf, int produced,
-                                                                int gathered, bool rotated) {
+                                                                int gathered, bool rotated, int slack_words) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= produced * gathered) return;
   const int o = i / gathered, c = i - o * gathered;
@@ -64,7 +70,7 @@ __global__ __launch_bounds__(256) void wino_filter_fused_kernel(const float *__r
   for (int col = 0; col < 3; ++col) g_rows(k[col], k[3 + col], k[6 + col], t[col]);
   const int band = o / kBand, ob = (o % kBand) / 16, chunk = c / kChunk, kk = (c % kChunk) / 4;
   const int lane = (c % 4) * 16 + o % 16;
-  const size_t band_floats = static_cast<size_t>(gathered / kChunk) * kXi * 4 * 64 * 4 + static_cast<size_t>(kAhead) * 4 * 64 * 4;
+  const size_t band_floats = static_cast<size_t>(gathered / kChunk) * kXi * 4 * 64 * 4 + static_cast<size_t>(slack_words) * 4 * 64 * 4;
   float *dst = Uf + band * band_floats + ((static_cast<size_t>(chunk) * kXi * 4 + ob) * 64 + lane) * 4 + kk;
 #pragma unroll
   for (int r = 0; r < 6; ++r) {
@@ -81,6 +87,7 @@ struct FusedGeo {
   int tw, th;               // tiles per plane
   int gw, gh;               // tiles per group, gw * gh <= 16; tw % gw == 0, th % gh == 0
   int groups_w, groups;     // groups per row of groups, per image
+  int items;                // images * groups * bands: one per block
 };
 
 // the six quads of one thread's patch: the middle four columns of its six rows
@@ -128,7 +135,7 @@ __device__ __forceinline__ void transform_patch(const Patch &p, __amdgpu_buffer_
   float d[6][6];
 #pragma unroll
   for (int r = 0; r < 6; ++r) {
-    const float from_left = __shfl_up(p.mid[r].w, 1), from_right = __shfl_down(p.mid[r].x, 1);
+    const float from_left = from_lane_below(p.mid[r].w), from_right = from_lane_above(p.mid[r].x);
     d[r][0] = at_left ? edge[r] : from_left;        // (zero beyond the plane: no edge value is fetched there)
     d[r][1] = p.mid[r].x;
     d[r][2] = p.mid[r].y;
@@ -153,15 +160,21 @@ __device__ __forceinline__ void transform_patch(const Patch &p, __amdgpu_buffer_
   }
 }
 
-// grid: images * groups * bands blocks; block b: band = b % bands (the blocks of one group of tiles, which
-// read the same activations, follow each other), then the group, then the image.
+// grid: images * groups * bands work items rounded up to a multiple of 8 blocks; item i: band = i % bands (the
+// items of one group of tiles, which read the same activations, follow each other), then the group, then the image.
 template <bool STATS>
 __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *__restrict__ x, const float *__restrict__ Uf,
                                                                float *__restrict__ y, FusedGeo g, float *__restrict__ stats) {
   __shared__ __attribute__((aligned(16))) float Vl[kXi * 64 * 4];      // 36 864 bytes
   const int bands = g.produced / kBand;
-  const int band = blockIdx.x % bands;
-  const int grp = (blockIdx.x / bands) % g.groups, n = blockIdx.x / bands / g.groups;
+  // Workgroup ids go round the 8 XCDs, each with its own L2: block b takes work item (b % 8) * per_xcd + b / 8,
+  // so that an XCD owns a contiguous stretch of groups and the rows and columns neighbouring groups share
+  // (a patch overlaps its neighbours by two rows and two columns) come from that L2 and not from memory again.
+  const int per_xcd = gridDim.x >> 3;
+  const int item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (item >= g.items) return;
+  const int band = item % bands;
+  const int grp = (item / bands) % g.groups, n = item / bands / g.groups;
   const int GY = grp / g.groups_w, GX = grp - GY * g.groups_w;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   // ---- the loader's tile and channel: lanes 16 apart hold the channels that share c % 4
@@ -204,9 +217,7 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
   for (int j = 0; j < kAhead; ++j) ua[j] = buf_load4(ru, uoff, static_cast<unsigned>(j) * 4096u);
 
   for (int ch = 0; ch < chunks; ++ch) {
-#if !defined(FUSED_VARIANT) || FUSED_VARIANT != 3
     transform_patch(patch, rx, pa, static_cast<unsigned>(ch) * chunk_bytes, at_left, at_right, cl, slot, Vl);
-#endif
     __syncthreads();
     if (ch + 1 < chunks) load_patch(rx, pa, static_cast<unsigned>(ch + 1) * chunk_bytes, patch);
     const unsigned ubase = static_cast<unsigned>(ch * kXi + kAhead) * 4096u;     // the word kAhead points on
@@ -225,10 +236,6 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
       ua[xi % kAhead] = buf_load4(ru, uoff, ubase + static_cast<unsigned>(xi) * 4096u);       // (behind the last chunk: the slack words)
       ua[(xi + 1) % kAhead] = buf_load4(ru, uoff, ubase + static_cast<unsigned>(xi + 1) * 4096u);
       __builtin_amdgcn_sched_barrier(0);
-#if defined(FUSED_VARIANT) && FUSED_VARIANT == 4
-      acc[xi] += a0 * b0;
-      acc[xi + 1] += a1 * b1;
-#else
       acc[xi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.x, b0.x, acc[xi], 0, 0, 0);
       acc[xi + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.x, b1.x, acc[xi + 1], 0, 0, 0);
       acc[xi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.y, b0.y, acc[xi], 0, 0, 0);
@@ -237,7 +244,6 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
       acc[xi + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.z, b1.z, acc[xi + 1], 0, 0, 0);
       acc[xi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.w, b0.w, acc[xi], 0, 0, 0);
       acc[xi + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.w, b1.w, acc[xi + 1], 0, 0, 0);
-#endif
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
@@ -284,7 +290,7 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
       }
     }
     if ((lane & 15) == 0) {
-      const int64_t k = blockIdx.x / bands;     // partial index: (image, group)
+      const int64_t k = item / bands;     // partial index: (image, group)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         float *dst = stats + (k * g.produced + o0 + r4) * 2;

@@ -575,13 +575,14 @@ bool split_bf16_enabled() {
 // at 56 x 56 778 -> 708; beyond that the three-kernel routine's GEMM, which runs at 120 TFLOP/s against 90 here,
 // outweighs the transforms it pays for.  TSPLIT_WINOGRAD_FUSED=0 switches the form off, =2 lifts the limit.
 namespace {
-inline bool fused_wanted(int gathered, int produced) {
+// 0: not this layer; otherwise the value of TSPLIT_WINOGRAD_FUSED (1 unless set)
+inline int fused_form(int gathered, int produced) {
   static const int mode = [] {
     const char *e = std::getenv("TSPLIT_WINOGRAD_FUSED");
     return e ? std::atoi(e) : 1;
   }();
-  if (mode == 0 || produced % fused::kBand || gathered % fused::kChunk) return false;
-  return mode >= 2 || std::max(gathered, produced) <= 256;
+  if (mode == 0 || produced % fused::kBand || gathered % fused::kChunk) return 0;
+  return (mode == 2 || std::max(gathered, produced) <= 256) ? mode : 0;
 }
 }  // namespace
 
@@ -597,28 +598,32 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
     int gw = 0, gh = 0;
     // (with the opt-in split-bf16 products the layers they cover keep the three-kernel routine, whose GEMM takes them)
     const bool split_products = produced > 64 && (gathered & 7) == 0 && split_bf16_enabled();
-    if (!split_products && fused_wanted(gathered, produced) && (H & 3) == 0 && (W & 3) == 0 && aligned16(x) && aligned16(y) &&
-        fused::fused_group(tw, th, gw, gh) && static_cast<int64_t>(imgs) * std::max(gathered, produced) * H * W < (1ll << 31)) {
-      const fused::FusedGeo fg{gathered, produced, H, W, tw, th, gw, gh, tw / gw, (tw / gw) * (th / gh)};
-      float *Uf = static_cast<float *>(scratch_get(st, 3, fused::fused_filter_floats(produced, gathered) * 4));
-      TS_REQUIRE(Uf, "conv (Winograd): no scratch memory");
-      hipLaunchKernelGGL(fused::wino_filter_fused_kernel, dim3((produced * gathered + 255) / 256), dim3(256), 0, st, w, Uf, produced,
-                         gathered, rotated);
-      const unsigned blocks = static_cast<unsigned>(imgs) * fg.groups * (produced / fused::kBand);
-      const double flop = 2.0 * kXi * produced * static_cast<double>(imgs) * per_img * gathered;
-      const double bytes = 4.0 * (static_cast<double>(gathered + produced) * imgs * H * W + static_cast<double>(kXi) * produced * gathered);
-      GemmTiming timed(st, 5, flop, bytes);
-      if (sink) {
-        const int parts = imgs * fg.groups;
-        TS_REQUIRE(sink->used + parts <= sink->capacity, "conv (Winograd): statistics buffer too small");
-        hipLaunchKernelGGL(fused::wino_fused_kernel<true>, dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg,
-                           sink->part + static_cast<int64_t>(sink->used) * produced * 2);
-        sink->used += parts;
-      } else {
-        hipLaunchKernelGGL(fused::wino_fused_kernel<false>, dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg,
-                           static_cast<float *>(nullptr));
+    const int form = fused_form(gathered, produced);
+    if (!split_products && form && (H & 3) == 0 && (W & 3) == 0 && aligned16(x) && aligned16(y) &&
+        static_cast<int64_t>(imgs) * std::max(gathered, produced) * H * W < (1ll << 31)) {
+      if (fused::fused_group(tw, th, gw, gh)) {
+        const int items = imgs * (tw / gw) * (th / gh) * (produced / fused::kBand);
+        const fused::FusedGeo fg{gathered, produced, H, W, tw, th, gw, gh, tw / gw, (tw / gw) * (th / gh), items};
+        float *Uf = static_cast<float *>(scratch_get(st, 3, fused::fused_filter_floats(produced, gathered) * 4));
+        TS_REQUIRE(Uf, "conv (Winograd): no scratch memory");
+        hipLaunchKernelGGL(fused::wino_filter_fused_kernel, dim3((produced * gathered + 255) / 256), dim3(256), 0, st, w, Uf, produced,
+                           gathered, rotated, fused::kAhead);
+        const unsigned blocks = static_cast<unsigned>((items + 7) / 8 * 8);
+        const double flop = 2.0 * kXi * produced * static_cast<double>(imgs) * per_img * gathered;
+        const double bytes = 4.0 * (static_cast<double>(gathered + produced) * imgs * H * W + static_cast<double>(kXi) * produced * gathered);
+        GemmTiming timed(st, 5, flop, bytes);
+        if (sink) {
+          const int parts = imgs * fg.groups;
+          TS_REQUIRE(sink->used + parts <= sink->capacity, "conv (Winograd): statistics buffer too small");
+          hipLaunchKernelGGL(fused::wino_fused_kernel<true>, dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg,
+                             sink->part + static_cast<int64_t>(sink->used) * produced * 2);
+          sink->used += parts;
+        } else {
+          hipLaunchKernelGGL(fused::wino_fused_kernel<false>, dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg,
+                             static_cast<float *>(nullptr));
+        }
+        return 0;
       }
-      return 0;
     }
   }
   const int run = run_images(imgs, per_img, gathered, produced);
