@@ -41,6 +41,7 @@ PEAK_HBM_GBS = 8000.0
 # Kernel names (as rocprofv3 prints them) behind the operator classes that can be the step's largest
 # single kernel; their HBM bytes per launch are read from the counter summary under profiles/.
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "vgg16_b64_train_step_hbm_traffic.txt")
+TRAFFIC_PROFILE_FUSED = os.path.join(ROOT, "profiles", "vgg16_b64_fused_bn_relu_train_step_hbm_traffic.txt")      # bench.py --fused
 TRAFFIC_KERNELS = {
     "conv_fwd_128x128": ("conv_tap_kernel<128, 128, 2, 2, false",),
     "conv_bwd_data_128x128": ("conv_tap_kernel<128, 128, 2, 2, true",),
@@ -54,16 +55,16 @@ TRAFFIC_KERNELS = {
 }
 
 
-def traffic_bytes_per_launch(tag):
+def traffic_bytes_per_launch(tag, profile=TRAFFIC_PROFILE):
     """HBM bytes one launch of the class's kernel moves (read + write, mean over the launches of a step),
     from the FETCH_SIZE / WRITE_SIZE summary committed under profiles/ (columns: kernel, launches, read MB,
     write MB; several variants of one kernel are averaged by launch count).  None when the summary does
     not list the kernel: the figure is never a constant typed in here."""
     names = TRAFFIC_KERNELS.get(tag)
-    if not names or not os.path.exists(TRAFFIC_PROFILE):
+    if not names or not os.path.exists(profile):
         return None
     launches = total = 0.0
-    with open(TRAFFIC_PROFILE) as f:
+    with open(profile) as f:
         for line in f:
             if not any(line.startswith(n) for n in names):
                 continue
@@ -78,6 +79,7 @@ def traffic_bytes_per_launch(tag):
 
 
 MFMA_PROFILE = os.path.join(ROOT, "profiles", "vgg16_b64_train_step_mfma_counters.txt")
+MFMA_PROFILE_FUSED = os.path.join(ROOT, "profiles", "vgg16_b64_fused_bn_relu_train_step_mfma_counters.txt")       # bench.py --fused
 
 
 def mfma_counters_per_launch(tag, profile=MFMA_PROFILE):
@@ -345,17 +347,18 @@ def main():
                            "achieved": dd["rate"], "peak": dom_peak,
                            "unit": "TFLOP/s" if dd["unit"] == "flop" else "GB/s",
                            "frac": dd["rate"] / dom_peak,
-                           "traffic": traffic_bytes_per_launch(dom) if split and a.batch == 64 and not a.fused and not a.split_bf16 else None,
+                           "traffic": traffic_bytes_per_launch(dom, TRAFFIC_PROFILE_FUSED if a.fused else TRAFFIC_PROFILE)
+                           if split and a.batch == 64 and not a.split_bf16 else None,
                            "per_launch": dd["work_per_call"], "ms_avg": dd["ms_avg"],
                            # which pass the launch durations behind `achieved` come from: the timed region carries event
                            # pairs only for the kernel expected to be the largest; if another one turns out larger (other
                            # batch sizes, --fused, --no-split) its figures are those of the second, instrumented pass
                            "measured_in": "timed region" if dom == {5: "winograd_fused", 3: "winograd_gemm_split_bf16"}[dominant_kind]
                            else "second pass (one event per operator call)"}
-        if split and a.batch == 64 and not a.fused and not a.split_bf16 and dd["unit"] == "flop":
+        if split and a.batch == 64 and not a.split_bf16 and dd["unit"] == "flop":
             # what the matrix pipes executed per launch and the share of cycles they were busy, by counter
             # (committed summary of a rocprofv3 --pmc run of this command); per_launch above is arithmetic
-            counted, busy = mfma_counters_per_launch(dom)
+            counted, busy = mfma_counters_per_launch(dom, MFMA_PROFILE_FUSED if a.fused else MFMA_PROFILE)
             out["roofline"]["per_launch_by_mfma_counter"] = counted
             out["roofline"]["mfma_busy_pct"] = busy
         # Conv utilisation, two ways.  The thin first layer (Cin*kH*kW = 27) is timed in bytes because

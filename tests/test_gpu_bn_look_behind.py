@@ -36,8 +36,9 @@ def _served(ts):
     return ts.L.batch_norm_look_behind()[0]
 
 
-def _layer(rng, n=8, c=64, o=64, hw=56):
-    """A layer the Winograd routine takes (its output transform sums per channel): 8 x 64 x 56 x 56."""
+def _layer(rng, n=8, c=64, o=64, hw=128):
+    """A layer the Winograd routine takes (its epilogue sums per channel) and whose output, 8 x 64 x 128 x 128 = 32 MiB,
+    is large enough for a note (smaller outputs leave none: the pass a note saves costs no more than the fold launch)."""
     x = rng.normal(size=(n, c, hw, hw)).astype(np.float32)
     w = (rng.normal(size=(o, c, 3, 3)) / np.sqrt(9 * c)).astype(np.float32)
     g = rng.normal(size=(1, o, 1, 1)).astype(np.float32)
@@ -54,8 +55,8 @@ def _bn(ts, y, g, b, stream=None):
 def test_batchnorm_behind_a_convolution_uses_its_sums_and_matches_the_oracle(ts, rng):
     x, w, g, b = _layer(rng)
     gx, gw, gg, gb = ts.arr(x), ts.arr(w), ts.arr(g), ts.arr(b)
-    y = ts.empty((8, 64, 56, 56))
-    assert ts.L.conv_takes_winograd(8, 64, 64, 56, 56)
+    y = ts.empty((8, 64, 128, 128))
+    assert ts.L.conv_takes_winograd(8, 64, 64, 128, 128)
     before = _served(ts)
     ts.L.CuDNN_conv2d(gx, gw, y, 1, 1, 1, ts.stream)
     assert ts.L.batch_norm_look_behind()[1]                 # a note is pending
@@ -67,10 +68,10 @@ def test_batchnorm_behind_a_convolution_uses_its_sums_and_matches_the_oracle(ts,
     assert _served(ts) == before + 1
     assert_close(got, again, 1e-6, "with and without the shortcut")
     # the direct (tap-major) kernels leave sums too: 1x1 filter, 128 -> 128
-    x1 = rng.normal(size=(8, 128, 56, 56)).astype(np.float32)
+    x1 = rng.normal(size=(8, 128, 96, 96)).astype(np.float32)
     w1 = (rng.normal(size=(128, 128, 1, 1)) / np.sqrt(128)).astype(np.float32)
     g1, b1 = rng.normal(size=(1, 128, 1, 1)).astype(np.float32), rng.normal(size=(1, 128, 1, 1)).astype(np.float32)
-    y1, gx1, gw1, gg1, gb1 = ts.empty((8, 128, 56, 56)), ts.arr(x1), ts.arr(w1), ts.arr(g1), ts.arr(b1)
+    y1, gx1, gw1, gg1, gb1 = ts.empty((8, 128, 96, 96)), ts.arr(x1), ts.arr(w1), ts.arr(g1), ts.arr(b1)
     ts.L.CuDNN_conv2d(gx1, gw1, y1, 0, 0, 1, ts.stream)       # (an upload between the two calls would end the note)
     got1 = _bn(ts, y1, gg1, gb1)
     assert _served(ts) == before + 2
@@ -78,9 +79,10 @@ def test_batchnorm_behind_a_convolution_uses_its_sums_and_matches_the_oracle(ts,
 
 
 def test_micro_tensor_convolutions_add_up_and_the_fused_call_takes_them_too(ts, rng):
-    x, w, g, b = _layer(rng)
+    # 32 images in four micro-tensors of 8: every piece is large enough for a note
+    x, w, g, b = _layer(rng, n=32)
     gx, gw, gg, gb = ts.arr(x), ts.arr(w), ts.arr(g), ts.arr(b)
-    y = ts.empty((8, 64, 56, 56))
+    y = ts.empty((32, 64, 128, 128))
     gx.split_tensor(4)
     y.split_tensor(4)
     before = _served(ts)
@@ -96,22 +98,40 @@ def test_micro_tensor_convolutions_add_up_and_the_fused_call_takes_them_too(ts, 
         ts.L.CuDNN_conv2d(gx.sTensor[i], gw, y.sTensor[i], 1, 1, 1, ts.stream)
     assert_close(_bn(ts, y, gg, gb), got, 1e-6, "pieces out of order")
     assert _served(ts) == before + 1
-    # a BatchNorm over ONE micro-tensor (small enough here for the kernel that holds a channel in registers and
-    # reads its input once anyway: no shortcut) sees that micro-tensor only, and all notes end with it
+    # a BatchNorm over ONE micro-tensor sees that micro-tensor's sums only, and all notes end with it
     for i in range(4):
         ts.L.CuDNN_conv2d(gx.sTensor[i], gw, y.sTensor[i], 1, 1, 1, ts.stream)
     one = _bn(ts, y.sTensor[2], gg, gb)
-    assert _served(ts) == before + 1 and not ts.L.batch_norm_look_behind()[1]
-    assert_close_entries(one, O.batchnorm_forward(conv[4:6], g, b, EPS)[0], 1e-4, "one micro-tensor")
+    assert _served(ts) == before + 2 and not ts.L.batch_norm_look_behind()[1]
+    assert_close_entries(one, O.batchnorm_forward(conv[16:24], g, b, EPS)[0], 1e-4, "one micro-tensor")
     # the fused BatchNorm + Relu symbol
     for i in range(4):
         ts.L.CuDNN_conv2d(gx.sTensor[i], gw, y.sTensor[i], 1, 1, 1, ts.stream)
     out, sm, sv = ts.empty(y.shape), ts.empty((1, 64, 1, 1)), ts.empty((1, 64, 1, 1))
     ts.L.batch_norm_relu(y, gg, gb, out, sm, sv, EPS, stream=ts.stream)
-    assert _served(ts) == before + 2
+    assert _served(ts) == before + 3
     assert_close(out.asnumpy(), np.maximum(ref, 0), 1e-4, "fused BatchNorm + Relu from the sums")
     assert_close(sm.asnumpy().ravel(), mean, 1e-4, "saved mean")
     assert_close(sv.asnumpy().ravel(), 1 / np.sqrt(var + EPS), 1e-4, "saved inverse deviation")
+
+
+def test_small_outputs_leave_no_note(ts, rng):
+    """At most 16 384 values per channel (the BatchNorm reads such a tensor once anyway) or less than 32 MiB in all (the
+    saved pass is no longer than the extra launch): the convolution neither sums nor notes."""
+    for n, hw in ((4, 56), (8, 56), (4, 128)):
+        _no_note(ts, rng, n, hw)
+
+
+def _no_note(ts, rng, n, hw):
+    x, w, g, b = _layer(rng, n=n, hw=hw)
+    gx, gw, gg, gb = ts.arr(x), ts.arr(w), ts.arr(g), ts.arr(b)
+    y = ts.empty((n, 64, hw, hw))
+    before = _served(ts)
+    ts.L.CuDNN_conv2d(gx, gw, y, 1, 1, 1, ts.stream)
+    assert not ts.L.batch_norm_look_behind()[1]
+    got = _bn(ts, y, gg, gb)
+    assert _served(ts) == before
+    assert_close_entries(got, O.batchnorm_forward(y.asnumpy(), g, b, EPS)[0], 1e-4, "small tensor, no note")
 
 
 @pytest.mark.parametrize("how", ["device copy on the stream", "device copy without a stream", "host upload", "operator in place",
@@ -119,8 +139,8 @@ def test_micro_tensor_convolutions_add_up_and_the_fused_call_takes_them_too(ts, 
 def test_sums_are_never_used_once_the_tensor_may_have_changed(ts, how, rng):
     x, w, g, b = _layer(rng)
     gx, gw, gg, gb = ts.arr(x), ts.arr(w), ts.arr(g), ts.arr(b)
-    y = ts.empty((8, 64, 56, 56))
-    other = rng.normal(size=(8, 64, 56, 56)).astype(np.float32) * 3 + 1
+    y = ts.empty((8, 64, 128, 128))
+    other = rng.normal(size=(8, 64, 128, 128)).astype(np.float32) * 3 + 1
     g_other = ts.arr(other)
     before = _served(ts)
     ts.L.CuDNN_conv2d(gx, gw, y, 1, 1, 1, ts.stream)

@@ -2295,15 +2295,16 @@ inline bool winograd_filter_grad_pays(const ConvGeo &g) {
 // in two steps with a fixed order: `slices` blocks per group of 32 channels each sum a contiguous range
 // of k in double (lanes of a wave read neighbouring channels), then one thread per channel adds the
 // slices in ascending order and writes dst[c * 2], dst[c * 2 + 1] as doubles.
-__global__ __launch_bounds__(256) void conv_stats_fold_kernel(const float *__restrict__ part, int used, int C,
-                                                              double *__restrict__ tmp, int chunk) {
-  __shared__ double sm[8][32][2];
+constexpr int kFoldRows = 32;      // partials a block of 32 x kFoldRows threads reads at a time
+__global__ __launch_bounds__(32 * kFoldRows) void conv_stats_fold_kernel(const float *__restrict__ part, int used, int C,
+                                                                         double *__restrict__ tmp, int chunk) {
+  __shared__ double sm[kFoldRows][32][2];
   const int cc = threadIdx.x & 31, kk = threadIdx.x >> 5;
   const int c = blockIdx.x * 32 + cc, slice = blockIdx.y;
   const int kend = min(used, (slice + 1) * chunk);
   double s = 0.0, q = 0.0;
   if (c < C)
-    for (int k = slice * chunk + kk; k < kend; k += 8) {
+    for (int k = slice * chunk + kk; k < kend; k += kFoldRows) {
       const float2 v = *reinterpret_cast<const float2 *>(part + (static_cast<int64_t>(k) * C + c) * 2);
       s += static_cast<double>(v.x);
       q += static_cast<double>(v.y);
@@ -2313,7 +2314,7 @@ __global__ __launch_bounds__(256) void conv_stats_fold_kernel(const float *__res
   __syncthreads();
   if (kk == 0 && c < C) {
 #pragma unroll
-    for (int j = 1; j < 8; ++j) {
+    for (int j = 1; j < kFoldRows; ++j) {
       s += sm[j][cc][0];
       q += sm[j][cc][1];
     }
@@ -2358,9 +2359,11 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
        (g.C % BK == 0 && tap_kernel_images(g, static_cast<int64_t>(g.C) * g.H * g.W, numel(w)) > 0));
   double *note_dst = nullptr;
   // (a BatchNorm over at most 16384 values per channel holds them in registers and reads its input once
-  // anyway; this output may be one of a few batch micro-tensors of the BatchNorm's input, hence a quarter)
-  if (may_note && sums_in_epilogue && static_cast<int64_t>(g.imgs) * g.oH * g.oW > 4096 && g.O <= 4096 &&
-      numel(y) < (1ll << 31)) {
+  // anyway, so an output that small gets no note: the fold launch behind the epilogue would be paid for
+  // nothing, and networks of many small layers have hundreds of such calls a step.  For the same reason an
+  // output below 32 MiB gets none: the pass over it that the note saves takes about as long as that launch)
+  if (may_note && sums_in_epilogue && static_cast<int64_t>(g.imgs) * g.oH * g.oW > 16384 && g.O <= 4096 &&
+      numel(y) >= (8ll << 20) && numel(y) < (1ll << 31)) {
     note_dst = conv_note_sums(st, g.O);
     stats_dst = note_dst;
   }
@@ -2424,7 +2427,7 @@ int conv_forward(const char *who, const DLArray *x, const DLArray *w, DLArray *y
       const int slices = std::max(1, std::min(kStatsSlices, (sink.used + 511) / 512));
       const int chunk = (sink.used + slices - 1) / slices;
       // one slice: its sums are the result (slice 0 of tmp has dst's layout), no second launch
-      hipLaunchKernelGGL(conv_stats_fold_kernel, dim3((g.O + 31) / 32, slices), dim3(256), 0, st, sink.part, sink.used, g.O,
+      hipLaunchKernelGGL(conv_stats_fold_kernel, dim3((g.O + 31) / 32, slices), dim3(32 * kFoldRows), 0, st, sink.part, sink.used, g.O,
                          slices == 1 ? stats_dst : tmp, chunk);
       if (slices > 1)
         hipLaunchKernelGGL(conv_stats_final_kernel, dim3((g.O + 255) / 256), dim3(256), 0, st, tmp, slices, g.O, stats_dst);

@@ -1,5 +1,5 @@
 // Winograd F(4x4, 3x3) in ONE kernel for layers that produce their output in bands of 64 channels from
-// 64 or 128 gathered channels: the input transform happens on the way into LDS and the output transform
+// a multiple of 16 gathered channels (the caller takes it up to 256 on either side): the input transform happens on the way into LDS and the output transform
 // comes straight from the accumulators, so neither V nor M (2.25 times the activations each) touches
 // memory.  With so few channels the three-kernel routine is bound by exactly that traffic (a 64 -> 64
 // layer at 224 x 224 moves 2.3 GB for 0.4 GB of activations); here the activations are read once per

@@ -100,24 +100,39 @@ def main():
         g = rng.normal(scale=0.1, size=(1, 64, 1, 1)).astype(np.float32)
         b = rng.normal(scale=0.1, size=(1, 64, 1, 1)).astype(np.float32)
         gx, gg, gb, out = dev(x), dev(g), dev(b), ndarray.empty(x.shape, ctx)
+        up = rng.normal(scale=0.1, size=x.shape).astype(np.float32)            # the gradient arriving from above
+        gup = dev(up)
+        tup = torch.from_numpy(up) if torch is not None else None
         dg, db = ndarray.empty(g.shape, ctx), ndarray.empty(g.shape, ctx)
         n = float(x.size)
         tx = torch.from_numpy(x) if torch is not None else None
         tg, tb = (torch.from_numpy(g.reshape(-1)), torch.from_numpy(b.reshape(-1))) if torch is not None else (None, None)
+        if torch is not None:
+            _, tmean, tistd = torch.ops.aten.native_batch_norm(tx, tg, tb, None, None, True, 0.1, 0.01)
         case("batchnorm 224x224x64 forward", B, 8 * n, "byte",
              lambda: L.CuDNN_Batch_Normalization(gx, gg, gb, out, None, None, 0.99, 0.01, st, prof),
              (lambda: F.batch_norm(tx, None, None, tg, tb, training=True, eps=0.01)) if torch is not None else None)
         case("batchnorm 224x224x64 gradient", B, 12 * n, "byte",
-             lambda: L.CuDNN_Batch_Normalization_gradient(gx, gx, gg, out, dg, db, None, None, 0.01, st, prof), None)
+             lambda: L.CuDNN_Batch_Normalization_gradient(gup, gx, gg, out, dg, db, None, None, 0.01, st, prof),
+             (lambda: torch.ops.aten.native_batch_norm_backward(tup, tx, tg, None, None, tmean, tistd, True, 0.01, [True, True, True]))
+             if torch is not None else None)
         case("relu 224x224x64 forward", B, 8 * n, "byte", lambda: L.relu(gx, out, st, prof),
              (lambda: F.relu(tx)) if torch is not None else None)
-        case("relu 224x224x64 gradient", B, 12 * n, "byte", lambda: L.relu_gradient(gx, gx, out, st, prof), None)
+        case("relu 224x224x64 gradient", B, 12 * n, "byte", lambda: L.relu_gradient(gx, gup, out, st, prof),
+             (lambda: torch.ops.aten.threshold_backward(tup, tx, 0.0)) if torch is not None else None)
         pooled = ndarray.empty((B, 64, 112, 112), ctx)
+        pup = rng.normal(scale=0.1, size=(B, 64, 112, 112)).astype(np.float32)
+        gpup = dev(pup)
+        if torch is not None:
+            tpup = torch.from_numpy(pup)
+            _, tidx = F.max_pool2d(tx, 2, 2, return_indices=True)
         case("maxpool 2x2/2 224x224x64 forward", B, 4 * (n + n / 4), "byte", lambda: L.CuDNN_max_pooling2d(gx, 2, 2, pooled, 0, 2, st, prof),
              (lambda: F.max_pool2d(tx, 2, 2)) if torch is not None else None)
         case("maxpool 2x2/2 224x224x64 gradient", B, 4 * (2 * n + n / 4), "byte",
-             lambda: L.CuDNN_max_pooling2d_gradient(pooled, pooled, gx, 2, 2, out, 0, 2, st, prof), None)
-        del gx, out, pooled
+             lambda: L.CuDNN_max_pooling2d_gradient(pooled, gpup, gx, 2, 2, out, 0, 2, st, prof),
+             (lambda: torch.ops.aten.max_pool2d_with_indices_backward(tpup, tx, [2, 2], [2, 2], [0, 0], [1, 1], False, tidx))
+             if torch is not None else None)
+        del gx, out, pooled, gup, gpup
         for rows_, k, cols in ((B, 1024, 1024), (100, 4096, 4096)):
             if rows_ == 100 and B != int(a.batches.split(",")[0]):
                 continue
@@ -133,6 +148,9 @@ def main():
         print("%-40s %6d %10.3f %9.1f %-7s %7.1f%% %10s %9s" % (r["op"], r["batch"], r["gpu_ms"], r["achieved"], r["unit"], 100 * r["frac"],
                                                                "%.1f" % r["cpu_ms"] if "cpu_ms" in r else "-",
                                                                "%.0fx" % r["speedup"] if "speedup" in r else "-"))
+    print("conv rates count the direct algorithm's FLOP (2 * B * O * H * W * C * 9); layers the Winograd routine takes execute a quarter of "
+          "them, so such a call can read above 100 % of the matrix peak.  BatchNorm forward on a tensor no convolution of this library has "
+          "just written reads it twice (statistics, then apply): 12 B per element moved for the 8 counted.")
     if rows and "cpu_cores" in rows[0]:
         print("CPU: PyTorch %s (bundled oneDNN), %d threads" % (torch.__version__, rows[0]["cpu_cores"]))
 
