@@ -52,6 +52,7 @@ TRAFFIC_KERNELS = {
     "winograd_filter_grad_gemm": ("wino_grad_gemm_kernel<3>",),
     "winograd_gemm_64_rows": ("wino_gemm_kernel<64, 256>",),
     "winograd_fused": ("wino_fused_kernel<",),
+    "winograd_filter_grad_fused": ("wino_fgrad_fused_kernel",),
 }
 
 
@@ -260,7 +261,7 @@ def main():
             t.step(gx, gy)
         t.sync()
         dt_instrumented = time.perf_counter() - t1
-        for kind in range(6):
+        for kind in range(7):
             if kind != dominant_kind:
                 gemm_times[kind] = L.winograd_gemm_times(kind=kind)
         L.winograd_gemm_timing(False)
@@ -300,7 +301,8 @@ def main():
         # the GEMM kernels inside the Winograd calls, timed by the library with event pairs on the
         # compute stream around each launch; their work is the FLOP they execute
         wino_exec_flop = 0.0
-        for tag, kind in (("winograd_gemm", 0), ("winograd_filter_grad_gemm", 1), ("winograd_gemm_64_rows", 2), ("winograd_fused", 5)):
+        for tag, kind in (("winograd_gemm", 0), ("winograd_filter_grad_gemm", 1), ("winograd_gemm_64_rows", 2), ("winograd_fused", 5),
+                          ("winograd_filter_grad_fused", 6)):
             launches, ms, flop, nbytes = gemm_times[kind]
             if launches:
                 wino_exec_flop += flop
@@ -318,6 +320,14 @@ def main():
                     kernels[tag]["note"] = ("the whole forward / data-gradient call of the layers with 64 channels on one side: one kernel "
                                             "with the Winograd transforms inside; executed FLOP (2 * 36 * O * C * tiles), and the "
                                             "activations' and filter's bytes for hbm_*")
+                if kind == 6:
+                    # filter gradient of the layers with at most 128 channels as ONE kernel plus the final transform of
+                    # the filter: both transforms on the way into LDS, products there
+                    kernels[tag]["hbm_achieved_gbs"] = nbytes / (ms * 1e-3) / 1e9
+                    kernels[tag]["hbm_frac"] = kernels[tag]["hbm_achieved_gbs"] / PEAK_HBM_GBS
+                    kernels[tag]["note"] = ("the filter-gradient call of the layers with at most 128 channels but for its final 3x3 transform: "
+                                            "one kernel with both Winograd transforms inside; executed FLOP (2 * 36 * O * C * tiles), and "
+                                            "the activations', gradients' and partial sums' bytes for hbm_*")
                 if kind == 2:
                     # 64 or 128 channels summed over on 64-row tiles: 16 - 21 executed FLOP per algorithmic byte, at
                     # the ratio of the two peaks (19.7), so both fractions are given

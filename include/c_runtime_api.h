@@ -512,8 +512,10 @@ int TSplit_ConvTakesWinograd(int images, int in_channels, int out_channels, int 
  *      gradient on 128 x 128 tiles, 1: filter gradient, 2: forward and data gradient of layers that
  *      produce at most 64 channels, which run on 64 x 256 tiles, 3 / 4: forward and data gradient /
  *      filter gradient with split-bf16 products, see TSplit_SplitBf16; 5: forward and data gradient of
- *      layers with 64 channels on one side and at most 128 on the other, which run as ONE kernel with the
- *      transforms inside, so that its milliseconds cover the whole call: one kernel per kind) and returns
+ *      layers with at most 256 channels, which run as ONE kernel with the transforms inside, so that its
+ *      milliseconds cover the whole call; 6: filter gradient of layers with at most 128 channels, one
+ *      kernel with both transforms inside, followed by the filter's final 3x3 transform: one kernel per
+ *      kind) and returns
  *      their count, summed milliseconds and summed executed FLOP (2 * 36 * rows * columns * depth
  *      per launch);
  *      TSplit_WinogradGemmBytes returns their summed algorithmic bytes (both operands read once,

@@ -223,6 +223,46 @@ def test_conv_winograd_is_per_image_and_repeatable(rng, monkeypatch):
         np.testing.assert_array_equal(whole[1], other[1])
 
 
+@pytest.mark.parametrize("shape", [(4, 64, 128, 128, 128),      # 4096 tiles, rows of 32 tiles: whole steps of 8
+                                   (6, 128, 64, 120, 92),       # 4140 tiles, rows of 23: steps wrap rows and images, ragged end
+                                   (5, 128, 128, 116, 116)])    # 4205 tiles, four band pairs
+def test_conv_winograd_filter_gradient_in_one_kernel(shape, rng):
+    """Layers with at most 128 channels and at least 4096 tiles take the filter gradient that transforms both
+    tensors on the way into LDS (wino_fgrad_fused.h).  Channel blocks of 8 x 8 filters (a filter's gradient depends
+    on its two channels only), chosen inside bands, across the band boundary and at the end, against the oracle;
+    the whole result against the direct kernels; twice for the same bits."""
+    from tsplit_amd import gpu_links as L, ndarray
+    import os
+    N, C, Oc, H, W = shape
+    ctx = ndarray.gpu(0)
+    x = rng.normal(size=(N, C, H, W)).astype(np.float32)
+    dy = rng.normal(size=(N, Oc, H, W)).astype(np.float32)
+    gx, gdy = ndarray.array(x, ctx), ndarray.array(dy, ctx)
+    assert L.conv_takes_winograd(N, C, Oc, H, W, filter_gradient=True)
+    L.winograd_gemm_timing(True, kind=6)
+    got = []
+    for _ in range(2):
+        dw = ndarray.empty((Oc, C, 3, 3), ctx)
+        L.CuDNN_conv2d_gradient_of_filter(gx, gdy, dw, 1, 1, 1)
+        got.append(dw.asnumpy())
+    launches = L.winograd_gemm_times(kind=6)[0]
+    L.winograd_gemm_timing(False)
+    assert launches == 2, "the one-kernel filter gradient did not run"
+    np.testing.assert_array_equal(got[0], got[1])
+    scale = np.max(np.abs(got[0]))
+    for o0, c0 in ((0, 0), (Oc - 8, C - 8), (min(60, Oc - 8), min(60, C - 8)), (17, C - 8)):
+        ref = O.conv2d_grad_filter(x[:, c0:c0 + 8], dy[:, o0:o0 + 8], (8, 8, 3, 3), 1, 1, 1)
+        err = np.max(np.abs(got[0][o0:o0 + 8, c0:c0 + 8] - ref)) / scale
+        assert err <= 1e-4, (o0, c0, err)
+    os.environ["TSPLIT_CONV_WINOGRAD"] = "0"
+    try:
+        direct = ndarray.empty((Oc, C, 3, 3), ctx)
+        L.CuDNN_conv2d_gradient_of_filter(gx, gdy, direct, 1, 1, 1)
+        assert_close(got[0], direct.asnumpy(), 1e-4, f"one-kernel Winograd filter gradient vs direct {shape}")
+    finally:
+        del os.environ["TSPLIT_CONV_WINOGRAD"]
+
+
 @pytest.mark.parametrize("case", [c for c in CASES if c[7] == c[8]][:8])
 def test_conv_plain_family(case, rng):
     _run(case, "plain", rng)

@@ -336,6 +336,8 @@ __device__ __forceinline__ void wino_grad_block(const float *__restrict__ dy, fl
     for (int q = 0; q < 6; ++q) out[(r * 6 + q) * plane_stride] = v[q];
   }
 }
+#include "wino_fgrad_fused.h"
+
 // Both transforms of a filter-gradient run in one launch, grid (ceil(ld / 256), gx.chans + gy.chans): rows
 // below gx.chans transform a channel of x, the others a channel of dy (the two share nothing but the tiling)
 template <bool QUADS_X, bool QUADS_Y>
@@ -410,7 +412,8 @@ struct TimedLaunch {
   hipEvent_t begin, end;
   int which;       // 0: forward / data-gradient GEMMs on 128 x 128 tiles, 1: filter-gradient GEMMs,
                    // 2: forward / data-gradient GEMMs on 64 x 256 tiles (at most 64 channels produced),
-                   // 3 / 4: forward / data-gradient and filter-gradient GEMMs in split bf16
+                   // 3 / 4: forward / data-gradient and filter-gradient GEMMs in split bf16,
+                   // 5 / 6: forward / data gradient and filter gradient as one kernel each (wino_fused.h, wino_fgrad_fused.h)
   double flop, bytes;
 };
 std::mutex g_timing_mu;
@@ -688,6 +691,38 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
                                   hipStream_t st) {
   const int th = (H + 3) / 4, tw = (W + 3) / 4;
   const int per_img = th * tw;
+  const int64_t oc = static_cast<int64_t>(O) * C;
+  {
+    // few channels: the one-kernel form, whose transformed tensors never leave the chip (wino_fgrad_fused.h)
+    const bool split_products = O > 64 && C > 64 && split_bf16_enabled();
+    // Taken where it was measured faster than the three-kernel routine: at most 128 channels on both sides (with more
+    // bands every band pair reads the activations again, and the routine's deep GEMMs run at three quarters of the
+    // matrix peak) and at least 4096 tiles (below, its launch of ranges and their partial sums weigh more than the
+    // transformed tensors' way through memory).  TSPLIT_WINOGRAD_FGRAD_FUSED: 0 never, 2 wherever the kernel can run.
+    static const int fgrad_mode = [] {
+      const char *e = std::getenv("TSPLIT_WINOGRAD_FGRAD_FUSED");
+      return e ? std::atoi(e) : 1;
+    }();
+    const int64_t tiles = static_cast<int64_t>(imgs) * per_img;
+    const bool pays = fgrad_mode == 2 ? tiles >= 16 * fgrad::kStep : (std::max(C, O) <= 128 && tiles >= 4096);
+    if (fgrad_mode != 0 && pays && !split_products && fused_form(C, O) && (C % fgrad::kBandF) == 0 && (H & 3) == 0 && (W & 3) == 0 &&
+        aligned16(x) && aligned16(dy) && static_cast<int64_t>(imgs) * std::max(C, O) * H * W < (1ll << 29)) {
+      fgrad::FGradGeo fg{C, O, H, W, tw, th, imgs * per_img, 0, 0, C / fgrad::kBandF, O / fgrad::kBandF, 0};
+      fgrad::fgrad_plan(fg, compute_units());
+      float *part = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(fg.ranges) * kXi * oc * 4));
+      TS_REQUIRE(part, "conv (Winograd): no scratch memory");
+      {
+        const double flop = 2.0 * kXi * O * static_cast<double>(fg.tiles) * C;
+        const double bytes = 4.0 * (static_cast<double>(C + O) * imgs * H * W + static_cast<double>(kXi) * oc * fg.ranges);
+        GemmTiming timed(st, 6, flop, bytes);
+        hipLaunchKernelGGL(fgrad::wino_fgrad_fused_kernel, dim3(static_cast<unsigned>((fg.items + 7) / 8 * 8)), dim3(256), 0, st, x, dy, part,
+                           fg);
+      }
+      hipLaunchKernelGGL(wino_filter_grad_kernel, dim3(static_cast<unsigned>((oc + 63) / 64)), dim3(256), 0, st, part, dw,
+                         static_cast<int>(oc), fg.ranges);
+      return 0;
+    }
+  }
   const int run = run_images(imgs, per_img, C, O);
   TS_REQUIRE(run > 0, "conv (Winograd): one image's tiles do not fit 32-bit offsets");
   const int runs = (imgs + run - 1) / run;
@@ -695,7 +730,6 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
   const GradPlan plan = plan_grad_gemm(O, C, ld_max, compute_units());
   const int kchunk = plan.kchunk;
   const int parts_max = runs * ((ld_max + kchunk - 1) / kchunk);
-  const int64_t oc = static_cast<int64_t>(O) * C;
   float *VY = static_cast<float *>(scratch_get(st, 2, static_cast<size_t>(kXi) * (C + O) * ld_max * 4));
   float *part = static_cast<float *>(scratch_get(st, 3, static_cast<size_t>(parts_max) * kXi * oc * 4));
   TS_REQUIRE(VY && part, "conv (Winograd): no scratch memory");

@@ -451,7 +451,8 @@ def winograd_gemm_times(filter_gradient=False, kind=None):
     """-> (launches, total ms, total executed FLOP, total algorithmic bytes) of the timed GEMM launches of
     kind 0 (forward / data gradient on 128 x 128 tiles), 1 (filter gradient), 2 (forward / data gradient
     of layers that produce at most 64 channels, on 64 x 256 tiles), 3 / 4 (forward and data gradient /
-    filter gradient with split-bf16 products)."""
+    filter gradient with split-bf16 products), 5 (forward / data gradient as one kernel), 6 (filter gradient as
+    one kernel)."""
     which = int(bool(filter_gradient)) if kind is None else int(kind)
     n, ms, flop, nbytes = ctypes.c_double(), ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
     check_call(_LIB.TSplit_WinogradGemmTimes(which, ctypes.byref(n), ctypes.byref(ms), ctypes.byref(flop)))

@@ -69,7 +69,7 @@ def main():
                 fn()
             st.sync()
             launches = ms = gf = 0
-            for k in ((1, 4) if kind == 1 else (0, 2, 3, 5)):
+            for k in ((1, 4, 6) if kind == 1 else (0, 2, 3, 5)):
                 ln, m, f, _ = L.winograd_gemm_times(kind=k)
                 launches, ms, gf = launches + ln, ms + m, gf + f
             L.winograd_gemm_timing(False)
