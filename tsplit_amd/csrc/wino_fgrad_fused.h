@@ -26,7 +26,7 @@
 //     two values are tiles 2 j, 2 j + 1, j = lane / 16: the depth index of two successive matrix instructions)
 //     and four of X (the four blocks of 16 gathered channels), then 8 v_mfma_f32_16x16x4_f32.
 // At the end the block stores its 6 x 64 x 64 partial sums; wino_filter_grad_kernel adds the ranges' partial
-// sums in ascending order and applies G^T . G, as for the three-kernel routine.
+// sums in a fixed order and applies G^T . G, as for the three-kernel routine.
 //
 // Included by winograd.hip behind wino_fused.h (buffer loads, lane shifts) and the filter gradient's
 // transforms (a_rows).

@@ -358,30 +358,46 @@ __device__ __forceinline__ void gt_rows(const float u[6], float w[3]) {
   w[2] = (s34 - s12) * (1.0f / 6.0f) + u[5];
 }
 
-// dw[o][c][3][3] = G^T (sum of the partial dU, in ascending order) G; part[(p * 36 + xi) * O * C + o * C + c].
-// A block takes 64 filter elements (o, c): its four waves each sum nine of the 36 points over the parts
-// (consecutive lanes read consecutive elements), the sums meet in LDS, and the first wave applies G^T . G and
-// stores the 64 x 9 results, which are contiguous in dw, as whole lines.
-__global__ __launch_bounds__(256) void wino_filter_grad_kernel(const float *__restrict__ part, float *__restrict__ dw,
-                                                               int oc, int parts) {
+// dw[o][c][3][3] = G^T (sum of the partial dU) G; part[(p * 36 + xi) * O * C + o * C + c].
+// A block of 1024 threads takes 64 filter elements (o, c): wave w sums nine of the 36 points (w % 4) over a
+// quarter of the parts (w / 4: contiguous stretches, each in ascending order; consecutive lanes read consecutive
+// elements), the quarters are added in ascending order in LDS, and the first wave applies G^T . G and stores the
+// 64 x 9 results, which are contiguous in dw, as whole lines.  (One wave per nine points over all parts took
+// 19 us with the 85 parts of a one-kernel filter gradient.)
+constexpr int kPartSlices = 4;
+__global__ __launch_bounds__(256 * kPartSlices) void wino_filter_grad_kernel(const float *__restrict__ part, float *__restrict__ dw,
+                                                                             int oc, int parts) {
+  __shared__ float slices[kPartSlices][kXi][64 + 1];
   __shared__ float sums[kXi][64 + 1];
   __shared__ float outs[64 * 9];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3, slice = threadIdx.x >> 8;
   const int i0 = blockIdx.x * 64, i = i0 + lane;
   if (i < oc) {
     const int64_t step = static_cast<int64_t>(kXi) * oc;
+    const int per = (parts + kPartSlices - 1) / kPartSlices;
+    const int p0 = slice * per, p1 = min(parts, p0 + per);
     float sum[9];
 #pragma unroll
-    for (int j = 0; j < 9; ++j) sum[j] = part[static_cast<int64_t>(9 * wave + j) * oc + i];
-    for (int p = 1; p < parts; ++p) {
+    for (int j = 0; j < 9; ++j) sum[j] = 0.0f;
+    for (int p = p0; p < p1; ++p) {
 #pragma unroll
       for (int j = 0; j < 9; ++j) sum[j] += part[p * step + static_cast<int64_t>(9 * wave + j) * oc + i];
     }
 #pragma unroll
-    for (int j = 0; j < 9; ++j) sums[9 * wave + j][lane] = sum[j];
+    for (int j = 0; j < 9; ++j) slices[slice][9 * wave + j][lane] = sum[j];
   }
   __syncthreads();
-  if (wave == 0 && i < oc) {
+  if (slice == 0 && i < oc) {
+#pragma unroll
+    for (int j = 0; j < 9; ++j) {
+      float total = slices[0][9 * wave + j][lane];
+#pragma unroll
+      for (int q = 1; q < kPartSlices; ++q) total += slices[q][9 * wave + j][lane];
+      sums[9 * wave + j][lane] = total;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 64 && i < oc) {
     float t[6][3];   // t[q][.] = G^T applied down column q
 #pragma unroll
     for (int q = 0; q < 6; ++q) {
@@ -402,7 +418,7 @@ __global__ __launch_bounds__(256) void wino_filter_grad_kernel(const float *__re
   __syncthreads();
   const int n = min(64, oc - i0) * 9;
   float *dst = dw + static_cast<int64_t>(i0) * 9;
-  for (int k = threadIdx.x; k < n; k += 256) dst[k] = outs[k];
+  for (int k = threadIdx.x; k < n; k += 256 * kPartSlices) dst[k] = outs[k];
 }
 
 // ---------------------------------------------------------------- GEMM launch timing (opt-in)
@@ -718,7 +734,7 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
         hipLaunchKernelGGL(fgrad::wino_fgrad_fused_kernel, dim3(static_cast<unsigned>((fg.items + 7) / 8 * 8)), dim3(256), 0, st, x, dy, part,
                            fg);
       }
-      hipLaunchKernelGGL(wino_filter_grad_kernel, dim3(static_cast<unsigned>((oc + 63) / 64)), dim3(256), 0, st, part, dw,
+      hipLaunchKernelGGL(wino_filter_grad_kernel, dim3(static_cast<unsigned>((oc + 63) / 64)), dim3(256 * kPartSlices), 0, st, part, dw,
                          static_cast<int>(oc), fg.ranges);
       return 0;
     }
@@ -762,7 +778,7 @@ int conv_winograd_3x3_filter_grad(const float *x, const float *dy, float *dw, in
     }
     parts += here;
   }
-  hipLaunchKernelGGL(wino_filter_grad_kernel, dim3(static_cast<unsigned>((oc + 63) / 64)), dim3(256), 0, st, part, dw,
+  hipLaunchKernelGGL(wino_filter_grad_kernel, dim3(static_cast<unsigned>((oc + 63) / 64)), dim3(256 * kPartSlices), 0, st, part, dw,
                      static_cast<int>(oc), parts);
   return 0;
 }
