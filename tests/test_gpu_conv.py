@@ -225,7 +225,8 @@ def test_conv_winograd_is_per_image_and_repeatable(rng, monkeypatch):
 
 @pytest.mark.parametrize("shape", [(4, 64, 128, 128, 128),      # 4096 tiles, rows of 32 tiles: whole steps of 8
                                    (6, 128, 64, 120, 92),       # 4140 tiles, rows of 23: steps wrap rows and images, ragged end
-                                   (5, 128, 128, 116, 116)])    # 4205 tiles, four band pairs
+                                   (5, 128, 128, 116, 116),     # 4205 tiles, four band pairs
+                                   (300, 64, 64, 16, 16)])      # 4800 tiles, rows of 4: a step of 8 covers two rows of tiles
 def test_conv_winograd_filter_gradient_in_one_kernel(shape, rng):
     """Layers with at most 128 channels and at least 4096 tiles take the filter gradient that transforms both
     tensors on the way into LDS (wino_fgrad_fused.h).  Channel blocks of 8 x 8 filters (a filter's gradient depends
