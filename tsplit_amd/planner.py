@@ -54,7 +54,7 @@ class CostModel(object):
     event wait costs the compute stream (the host has to catch up with its launches afterwards;
     a swapped tensor brings one such wait on the way out and one on the way in)."""
 
-    def __init__(self, conv_tflops=110.0, conv_tflops_narrow=90.0, matmul_tflops=45.0, stream_gbs=5900.0,
+    def __init__(self, conv_tflops=110.0, conv_tflops_narrow=90.0, matmul_tflops=45.0, stream_gbs=6000.0,
                  link_gbs=55.0, host_wait_ms=0.2, thin_gbs=2900.0):
         self.host_wait_ms = host_wait_ms
         self.conv_tflops = conv_tflops
@@ -71,12 +71,12 @@ class CostModel(object):
         falls and the GEMMs' depth grows with the channel count; the 14 x 14 planes leave a sparse last round."""
         lo, hi = min(cin, cout), max(cin, cout)
         if lo < 128:
-            return 125.0 if hi < 128 else 157.0
+            return 262.0 if hi < 128 else 237.0      # one kernel per pass
         if lo < 256:
-            return 207.0 if hi < 256 else 255.0
+            return 291.0 if hi < 256 else 302.0      # forward / data gradient one kernel; filter gradient too up to 128
         if lo < 512:
-            return 311.0
-        return 368.0 if plane >= 28 else 231.0
+            return 332.0 if hi < 512 else 313.0
+        return 368.0 if plane >= 28 else 235.0
 
     def copy_ms(self, nbytes):
         return nbytes / (self.link_gbs * 1e9) * 1e3
