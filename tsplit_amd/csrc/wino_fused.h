@@ -7,9 +7,10 @@
 //
 // Included by winograd.hip behind its transforms (g_rows, bt_rows, at_rows).
 //
-// One block of 256 threads (4 waves) owns a group of gw x gh tiles of one image (at most 16: 8 x 2 at
-// 224 x 224, 4 x 4 at 112 x 112; a group is a rectangle of tiles so that neighbouring lanes hold neighbouring
-// tiles) and one band of 64 produced channels, for all 36 points xi.  Two blocks share a compute unit (a wave
+// One block of 256 threads (4 waves) owns a group of at most 16 tiles of one image (a rectangle of gw x gh tiles:
+// 8 x 2 at 224 x 224, 4 x 4 at 112 x 112; or, where no rectangle fills the 16 slots as well, 16 consecutive tiles
+// row after row: 56 x 56; either way neighbouring lanes hold neighbouring tiles) and one band of 64 produced
+// channels, for all 36 points xi.  Two blocks share a compute unit (a wave
 // needs 256 registers: 144 of them accumulators) and run out of step, so that one multiplies while the other
 // transforms or waits for its activations:
 //   * the gathered channels go by in chunks of 16.  A thread loads the 6 x 6 patch of one tile slot in one
@@ -85,8 +86,8 @@ struct FusedGeo {
   int gathered, produced;   // channels
   int H, W;                 // plane (multiples of 4)
   int tw, th;               // tiles per plane
-  int gw, gh;               // tiles per group, gw * gh <= 16; tw % gw == 0, th % gh == 0
-  int groups_w, groups;     // groups per row of groups, per image
+  int gw, gh;               // tiles per group, gw * gh <= 16; tw % gw == 0, th % gh == 0; gw = 0: runs of 16 tiles
+  int groups_w, groups;     // groups per row of groups (rectangles only), per image
   int items;                // images * groups * bands: one per block
 };
 
@@ -124,6 +125,7 @@ __device__ __forceinline__ void load_patch(__amdgpu_buffer_rsrc_t rx, const Patc
 // brought into the cache; zero beyond the plane) rather than held in registers through the products
 // (fetching them with the quads, a step ahead, measured 8 % slower: six more loads in front of the
 // filter words, which return in order).
+template <bool RUNS>
 __device__ __forceinline__ void transform_patch(const Patch &p, __amdgpu_buffer_rsrc_t rx, const PatchAddr &pa, unsigned chunk_off,
                                                 bool at_left, bool at_right, int c, int slot, float *__restrict__ Vl) {
   float edge[6];
@@ -136,12 +138,14 @@ __device__ __forceinline__ void transform_patch(const Patch &p, __amdgpu_buffer_
 #pragma unroll
   for (int r = 0; r < 6; ++r) {
     const float from_left = from_lane_below(p.mid[r].w), from_right = from_lane_above(p.mid[r].x);
-    d[r][0] = at_left ? edge[r] : from_left;        // (zero beyond the plane: no edge value is fetched there)
+    // (zero beyond the plane: no edge value is fetched there.  In a run of consecutive tiles a thread can be at the
+    // run's end on one side and at the plane's edge on the other: the one value it fetched belongs to one side only)
+    d[r][0] = !at_left ? from_left : (!RUNS || pa.edge < 0) ? edge[r] : 0.0f;
     d[r][1] = p.mid[r].x;
     d[r][2] = p.mid[r].y;
     d[r][3] = p.mid[r].z;
     d[r][4] = p.mid[r].w;
-    d[r][5] = at_right ? edge[r] : from_right;
+    d[r][5] = !at_right ? from_right : (!RUNS || pa.edge > 0) ? edge[r] : 0.0f;
   }
   float tmp[6][6];
 #pragma unroll
@@ -162,7 +166,7 @@ __device__ __forceinline__ void transform_patch(const Patch &p, __amdgpu_buffer_
 
 // grid: images * groups * bands work items rounded up to a multiple of 8 blocks; item i: band = i % bands (the
 // items of one group of tiles, which read the same activations, follow each other), then the group, then the image.
-template <bool STATS>
+template <bool STATS, bool RUNS>
 __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *__restrict__ x, const float *__restrict__ Uf,
                                                                float *__restrict__ y, FusedGeo g, float *__restrict__ stats) {
   __shared__ __attribute__((aligned(16))) float Vl[kXi * 64 * 4];      // 36 864 bytes
@@ -175,20 +179,36 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
   if (item >= g.items) return;
   const int band = item % bands;
   const int grp = (item / bands) % g.groups, n = item / bands / g.groups;
-  const int GY = grp / g.groups_w, GX = grp - GY * g.groups_w;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   // ---- the loader's tile and channel: lanes 16 apart hold the channels that share c % 4
   const int slot = t & 15, cl = (((t >> 4) & 3) << 2) | wave;
-  const int gy = slot / g.gw, gx = slot - gy * g.gw;
-  const bool live = slot < g.gw * g.gh;
-  const int ty = GY * g.gh + gy, tx = GX * g.gw + gx;
+  // a slot's tile, whether it exists, and whether the tile to its left / right sits in the neighbouring lane
+  const auto tile_of = [&](int s, int &ty_, int &tx_, bool &left_, bool &right_) {
+    if (RUNS) {      // a run of 16 consecutive tiles of the image, row after row
+      const int idx = grp * kSlots + s;
+      ty_ = idx / g.tw;
+      tx_ = idx - ty_ * g.tw;
+      left_ = s == 0 || tx_ == 0;
+      right_ = s == kSlots - 1 || tx_ == g.tw - 1;
+      return idx < g.tw * g.th;
+    }
+    const int GY = grp / g.groups_w, GX = grp - GY * g.groups_w;
+    const int gy = s / g.gw, gx = s - gy * g.gw;
+    ty_ = GY * g.gh + gy;
+    tx_ = GX * g.gw + gx;
+    left_ = gx == 0;
+    right_ = gx == g.gw - 1;
+    return s < g.gw * g.gh;
+  };
+  int ty, tx;
+  bool at_left, at_right;      // the column beside the quad does not come from the neighbouring lane
+  const bool live = tile_of(slot, ty, tx, at_left, at_right);
   const int64_t plane_elems = static_cast<int64_t>(g.H) * g.W;
   const unsigned plane_bytes = static_cast<unsigned>(plane_elems) * 4u;
   // the image's gathered planes as one buffer: rows outside the plane get an offset beyond it and read as zeros
   const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<float *>(x) + static_cast<int64_t>(n) * g.gathered * plane_elems, 0, static_cast<int>(g.gathered * plane_bytes), kBufFlagsF);
   PatchAddr pa;
-  const bool at_left = gx == 0, at_right = gx == g.gw - 1;
   pa.edge = !live ? 0 : (at_left && tx > 0) ? -4 : (at_right && tx < g.tw - 1) ? 16 : 0;
 #pragma unroll
   for (int r = 0; r < 6; ++r) {
@@ -217,7 +237,7 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
   for (int j = 0; j < kAhead; ++j) ua[j] = buf_load4(ru, uoff, static_cast<unsigned>(j) * 4096u);
 
   for (int ch = 0; ch < chunks; ++ch) {
-    transform_patch(patch, rx, pa, static_cast<unsigned>(ch) * chunk_bytes, at_left, at_right, cl, slot, Vl);
+    transform_patch<RUNS>(patch, rx, pa, static_cast<unsigned>(ch) * chunk_bytes, at_left, at_right, cl, slot, Vl);
     __syncthreads();
     if (ch + 1 < chunks) load_patch(rx, pa, static_cast<unsigned>(ch + 1) * chunk_bytes, patch);
     const unsigned ubase = static_cast<unsigned>(ch * kXi + kAhead) * 4096u;     // the word kAhead points on
@@ -251,10 +271,10 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
 
   // ---- output transform from the accumulators: lane holds channels o0 .. o0 + 3 of tile slot `os`
   const int os = lane & 15;
-  const int oy = os / g.gw, ox = os - oy * g.gw;
-  const bool olive = os < g.gw * g.gh;
+  int oty, otx;
+  bool unused_left, unused_right;
+  const bool olive = tile_of(os, oty, otx, unused_left, unused_right);
   const int o0 = band * kBand + ob * 16 + (lane >> 4) * 4;
-  const int oty = GY * g.gh + oy, otx = GX * g.gw + ox;
   float s[4] = {0.0f, 0.0f, 0.0f, 0.0f}, sq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
   for (int r4 = 0; r4 < 4; ++r4) {
@@ -301,8 +321,11 @@ __global__ __launch_bounds__(kThreadsF, 2) void wino_fused_kernel(const float *_
   }
 }
 
-// the largest group of at most 16 tiles (wider first, at least two wide) that tiles the plane's tw x th tiles exactly
-inline bool fused_group(int tw, int th, int &gw, int &gh) {
+// How a plane's tw x th tiles are dealt to groups of at most 16: the largest rectangle (wider first, at least two wide)
+// that tiles the plane exactly, or - where that leaves more slots empty - runs of 16 consecutive tiles, row after
+// row (gw = 0; 14 x 14 tiles: 13 runs with 196 of 208 slots filled, where rows of 14 fill 14 of 16).  False if
+// less than three quarters of the slots would carry a tile.
+inline bool fused_group(int tw, int th, int &gw, int &gh, int &groups) {
   int best = 0;
   for (int w = 2; w <= tw && w <= kSlots; ++w) {
     if (tw % w) continue;
@@ -315,7 +338,14 @@ inline bool fused_group(int tw, int th, int &gw, int &gh) {
       }
     }
   }
-  return best >= 12;    // at least three quarters of the slots carry a tile
+  const int tiles = tw * th, runs = (tiles + kSlots - 1) / kSlots;
+  if (best > 0 && best * runs >= tiles) {        // the rectangles fill their slots at least as well
+    groups = (tw / gw) * (th / gh);
+    return best >= 12;
+  }
+  gw = gh = 0;
+  groups = runs;
+  return 4 * tiles >= 3 * runs * kSlots;
 }
 
 }  // namespace fused

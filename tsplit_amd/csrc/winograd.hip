@@ -620,9 +620,10 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
     const int form = fused_form(gathered, produced);
     if (!split_products && form && (H & 3) == 0 && (W & 3) == 0 && aligned16(x) && aligned16(y) &&
         static_cast<int64_t>(imgs) * std::max(gathered, produced) * H * W < (1ll << 31)) {
-      if (fused::fused_group(tw, th, gw, gh)) {
-        const int items = imgs * (tw / gw) * (th / gh) * (produced / fused::kBand);
-        const fused::FusedGeo fg{gathered, produced, H, W, tw, th, gw, gh, tw / gw, (tw / gw) * (th / gh), items};
+      int groups = 0;
+      if (fused::fused_group(tw, th, gw, gh, groups)) {
+        const int items = imgs * groups * (produced / fused::kBand);
+        const fused::FusedGeo fg{gathered, produced, H, W, tw, th, gw, gh, gw ? tw / gw : 0, groups, items};
         float *Uf = static_cast<float *>(scratch_get(st, 3, fused::fused_filter_floats(produced, gathered) * 4));
         TS_REQUIRE(Uf, "conv (Winograd): no scratch memory");
         hipLaunchKernelGGL(fused::wino_filter_fused_kernel, dim3((produced * gathered + 255) / 256), dim3(256), 0, st, w, Uf, produced,
@@ -631,14 +632,21 @@ int conv_winograd_3x3(const float *x, const float *w, float *y, int imgs, int ga
         const double flop = 2.0 * kXi * produced * static_cast<double>(imgs) * per_img * gathered;
         const double bytes = 4.0 * (static_cast<double>(gathered + produced) * imgs * H * W + static_cast<double>(kXi) * produced * gathered);
         GemmTiming timed(st, 5, flop, bytes);
+        const bool runs = gw == 0;
         if (sink) {
           const int parts = imgs * fg.groups;
           TS_REQUIRE(sink->used + parts <= sink->capacity, "conv (Winograd): statistics buffer too small");
-          hipLaunchKernelGGL(fused::wino_fused_kernel<true>, dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg,
-                             sink->part + static_cast<int64_t>(sink->used) * produced * 2);
+          float *stats = sink->part + static_cast<int64_t>(sink->used) * produced * 2;
+          if (runs)
+            hipLaunchKernelGGL((fused::wino_fused_kernel<true, true>), dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg, stats);
+          else
+            hipLaunchKernelGGL((fused::wino_fused_kernel<true, false>), dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg, stats);
           sink->used += parts;
+        } else if (runs) {
+          hipLaunchKernelGGL((fused::wino_fused_kernel<false, true>), dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg,
+                             static_cast<float *>(nullptr));
         } else {
-          hipLaunchKernelGGL(fused::wino_fused_kernel<false>, dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg,
+          hipLaunchKernelGGL((fused::wino_fused_kernel<false, false>), dim3(blocks), dim3(fused::kThreadsF), 0, st, x, Uf, y, fg,
                              static_cast<float *>(nullptr));
         }
         return 0;
