@@ -278,12 +278,16 @@ __device__ __forceinline__ void fgrad_block(const float *__restrict__ x, const f
   const f32x2 *Yv = reinterpret_cast<const f32x2 *>(Yl) + wave * kBlockVecs + lane_vec;
 
   for (int step = step0 + 1; step <= step1; ++step) {
+    // two LDS buffers take turns, so that one barrier a step is enough: a wave writes the points of the next step
+    // while slower waves still read the other buffer, and by the time it writes this buffer again every wave
+    // has passed the barrier behind the step in between, that is, has finished reading it
+    const int buf = (step & 1) * (2 * kOperandWords);
     {
       Half after;
       first_pass<R>(raw, after);
       after.has_left = at.tx > 0;
       after.has_right = at.tx < g.tw - 1;
-      second_pass(cur, before_x3, after, slot, cg, Xl, Yl);
+      second_pass(cur, before_x3, after, slot, cg, Xl + buf, Yl + buf);
 #pragma unroll
       for (int k = 0; k < 2; ++k) before_x3[k] = cur.x[k][3];
       cur = after;
@@ -295,16 +299,17 @@ __device__ __forceinline__ void fgrad_block(const float *__restrict__ x, const f
     // every point's LDS reads one point ahead of its products: left alone the compiler sinks the loads behind
     // the products and the reads next to their uses)
     __builtin_amdgcn_sched_barrier(0);
-    f32x2 a = Yv[0], b[4];
+    const f32x2 *Xb = Xv + buf / 2, *Yb = Yv + buf / 2;
+    f32x2 a = Yb[0], b[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b[j] = Xv[j * kBlockVecs];
+    for (int j = 0; j < 4; ++j) b[j] = Xb[j * kBlockVecs];
 #pragma unroll
     for (int e = 0; e < kPts; ++e) {
       f32x2 an = a, bn[4] = {b[0], b[1], b[2], b[3]};
       if (e + 1 < kPts) {
-        an = Yv[(e + 1) * kPointVecs];
+        an = Yb[(e + 1) * kPointVecs];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) bn[j] = Xv[(e + 1) * kPointVecs + j * kBlockVecs];
+        for (int j = 0; j < 4; ++j) bn[j] = Xb[(e + 1) * kPointVecs + j * kBlockVecs];
       }
       __builtin_amdgcn_sched_barrier(0);
       // (a matrix instruction that accumulates into the result of the one before it waits for it: the four
@@ -318,7 +323,6 @@ __device__ __forceinline__ void fgrad_block(const float *__restrict__ x, const f
 #pragma unroll
       for (int j = 0; j < 4; ++j) b[j] = bn[j];
     }
-    __syncthreads();
   }
 
   // partial sums of this range: part[((range * 36) + point) * O * C + o * C + c]
@@ -337,7 +341,7 @@ __device__ __forceinline__ void fgrad_block(const float *__restrict__ x, const f
 // the 8 XCDs in contiguous stretches so that the blocks of one range (which read the same activations) share an L2
 __global__ __launch_bounds__(256, 2) void wino_fgrad_fused_kernel(const float *__restrict__ x, const float *__restrict__ dy,
                                                                   float *__restrict__ part, FGradGeo g) {
-  __shared__ __attribute__((aligned(16))) float lds[2 * kOperandWords];      // 36 864 bytes
+  __shared__ __attribute__((aligned(16))) float lds[2 * 2 * kOperandWords];      // two buffers of 36 864 bytes
   const int per_xcd = gridDim.x >> 3;
   const int item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (item >= g.items) return;
