@@ -253,7 +253,11 @@ int DLGpuSliceGradient(const DLArrayHandle in_arr, DLArrayHandle out_arr, int64_
                        DLStreamHandle stream_handle, ProfilerHandle p);
 
 /* ---- Optimizer updates, in place, no ProfilerHandle (ref: c_runtime_api.h:371-380; impl
- *      src/ops/Optimizers.cu:9,48,87,122).  beta1t/beta2t are the host-accumulated powers. ---- */
+ *      src/ops/Optimizers.cu:9,48,87,122).  beta1t/beta2t are the host-accumulated powers.
+ *      SGD and Momentum calls issued back to back are queued on their stream as ONE launch when the
+ *      next call of any other kind reaches the library (DLStreamSync, DLEventRecord and copies
+ *      included), so every effect visible through this interface keeps its order; environment
+ *      TSPLIT_LAZY_UPDATES=0 issues each call at once. ---- */
 int SGDOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, float lr,
                        DLStreamHandle stream_handle);
 int MomentumOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, DLArrayHandle velocity,

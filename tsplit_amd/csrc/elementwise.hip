@@ -340,6 +340,14 @@ bool stream_is_recording(hipStream_t s) {
   return s && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
 }
 
+std::atomic<int> tsplit::g_updates_pending{0};
+int pending_run_locked();
+extern std::mutex g_pending_mu;
+void tsplit::updates_flush_all() {
+  std::lock_guard<std::mutex> lk(g_pending_mu);
+  if (pending_run_locked()) std::fprintf(stderr, "tsplit: a deferred optimizer update could not be launched\n");
+}
+
 // The stream is about to be destroyed (it has drained): its table's device buffer goes with the
 // stream's scratch, and a later stream may get the same handle value.
 void tsplit::multi_update_drop_stream(hipStream_t stream) {
@@ -429,6 +437,121 @@ int launch_multi(Op op, const std::vector<std::array<float *, Op::N>> &arrays, c
   hipLaunchKernelGGL(ew_multi_kernel<Op>, dim3(static_cast<unsigned>(blocks.size())), dim3(kThreads), 0, s, op,
                      reinterpret_cast<const MultiTensor<N> *>(dev), reinterpret_cast<const MultiBlock *>(dev + tbytes));
   return 0;
+}
+
+// ---- the list of optimizer updates that wait for their neighbours (common.h)
+struct PendingUpdates {
+  hipStream_t stream = nullptr;
+  int device = 0;
+  int rule = 0;                     // 0: SGD, 1: momentum, 2: Nesterov momentum
+  float lr = 0.0f, momentum = 0.0f;
+  std::vector<std::array<float *, 3>> arrays;      // param, grad, velocity (SGD: velocity unused)
+  std::vector<int64_t> sizes;
+};
+std::mutex g_pending_mu;
+PendingUpdates g_pending;
+
+bool lazy_updates_enabled() {
+  static const bool on = [] {
+    const char *e = std::getenv("TSPLIT_LAZY_UPDATES");
+    return !e || std::atoi(e) != 0;
+  }();
+  return on;
+}
+
+// one array of the list as a launch of its own
+void pending_run_one(const PendingUpdates &job, size_t i) {
+  Ptrs<3> a{{job.arrays[i][0], job.arrays[i][1], job.arrays[i][2]}};
+  if (job.rule == 0)
+    launch(SgdOp{job.lr}, Ptrs<2>{{a.p[0], a.p[1]}}, job.sizes[i], job.stream);
+  else if (job.rule == 1)
+    launch(MomentumOp{job.lr, job.momentum}, a, job.sizes[i], job.stream);
+  else
+    launch(NesterovOp{job.lr, job.momentum}, a, job.sizes[i], job.stream);
+}
+
+// runs the list (the caller holds g_pending_mu)
+int pending_run_locked() {
+  if (g_pending.arrays.empty()) return 0;
+  PendingUpdates job;
+  std::swap(job, g_pending);
+  tsplit::g_updates_pending.store(0, std::memory_order_relaxed);
+  int now = job.device;
+  (void)hipGetDevice(&now);
+  if (now != job.device) (void)hipSetDevice(job.device);      // the list runs on the device its stream lives on
+  // Arrays the one launch can take (16-byte aligned, below its size limit) go into it; the others, and all of
+  // them if the launch cannot be set up, run one by one: no update is ever dropped or done twice.
+  PendingUpdates many;
+  many.stream = job.stream, many.rule = job.rule, many.lr = job.lr, many.momentum = job.momentum;
+  std::vector<size_t> listed;
+  for (size_t i = 0; i < job.arrays.size(); ++i) {
+    const bool takes = job.arrays.size() > 1 && job.sizes[i] < (1ll << 33) && aligned16(job.arrays[i][0]) &&
+                       aligned16(job.arrays[i][1]) && (job.rule == 0 || aligned16(job.arrays[i][2]));
+    if (!takes) {
+      pending_run_one(job, i);
+      continue;
+    }
+    many.arrays.push_back(job.arrays[i]);
+    many.sizes.push_back(job.sizes[i]);
+    listed.push_back(i);
+  }
+  int rc = 0;
+  if (listed.size() == 1) {
+    pending_run_one(job, listed[0]);
+  } else if (!listed.empty()) {
+    const char *who = "optimizer update";
+    if (job.rule == 0) {
+      std::vector<std::array<float *, 2>> two(many.arrays.size());
+      for (size_t i = 0; i < two.size(); ++i) two[i] = {many.arrays[i][0], many.arrays[i][1]};
+      rc = launch_multi(SgdOp{job.lr}, two, many.sizes, job.stream, who);
+    } else {
+      rc = job.rule == 1 ? launch_multi(MomentumOp{job.lr, job.momentum}, many.arrays, many.sizes, job.stream, who)
+                         : launch_multi(NesterovOp{job.lr, job.momentum}, many.arrays, many.sizes, job.stream, who);
+    }
+    if (rc)       // set-up failed before the launch: nothing of the list has run
+      for (size_t i : listed) pending_run_one(job, i);
+  }
+  if (now != job.device) (void)hipSetDevice(now);
+  return 0;
+}
+
+// Puts one update on the list (running the list first if this one does not fit it).  False: the caller runs
+// the update itself, now (recording streams, or the list switched off).
+bool pending_add(hipStream_t s, int rule, float lr, float momentum, float *param, float *grad, float *velocity, int64_t n) {
+  if (!lazy_updates_enabled() || stream_is_recording(s)) {
+    tsplit::updates_flush_if_any();
+    return false;
+  }
+  int device = 0;
+  (void)hipGetDevice(&device);
+  std::lock_guard<std::mutex> lk(g_pending_mu);
+  bool fits = g_pending.arrays.empty() || (g_pending.stream == s && g_pending.device == device && g_pending.rule == rule &&
+                                           g_pending.lr == lr && g_pending.momentum == momentum);
+  if (fits) {
+    // one launch updates all listed arrays at once: an array this update writes must not be read or written by a
+    // listed one, nor may it read what a listed one writes (the same parameter updated twice in a row)
+    const auto overlap = [](const float *a, int64_t na, const float *b, int64_t nb) {
+      return a && b && a < b + nb && b < a + na;
+    };
+    for (size_t i = 0; fits && i < g_pending.arrays.size(); ++i) {
+      const std::array<float *, 3> &o = g_pending.arrays[i];
+      const int64_t m = g_pending.sizes[i];
+      for (int k = 0; k < 3 && fits; ++k) {
+        if (overlap(param, n, o[k], m) || overlap(velocity, n, o[k], m)) fits = false;      // writes against anything listed
+        if (k != 1 && overlap(grad, n, o[k], m)) fits = false;                              // reads against listed writes
+      }
+    }
+  }
+  if (!fits) (void)pending_run_locked();
+  g_pending.stream = s;
+  g_pending.device = device;
+  g_pending.rule = rule;
+  g_pending.lr = lr;
+  g_pending.momentum = momentum;
+  g_pending.arrays.push_back({param, grad, velocity});
+  g_pending.sizes.push_back(n);
+  tsplit::g_updates_pending.store(1, std::memory_order_relaxed);
+  return true;
 }
 
 #define SAME_SIZE(a, b, name) \
@@ -580,7 +703,8 @@ int DLGpuWhere(const DLArrayHandle cond, const DLArrayHandle arr1, const DLArray
 int SGDOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, float lr, DLStreamHandle stream_handle) {
   TS_REQUIRE(param && grad, "SGDOptimizerUpdate: NULL array");
   SAME_SIZE(param, grad, "SGDOptimizerUpdate");
-  hipStream_t s = stream_of(stream_handle);
+  hipStream_t s = stream_of_update(stream_handle);
+  if (numel(param) > 0 && pending_add(s, 0, lr, 0.0f, fp(param), fp(grad), nullptr, numel(param))) return 0;
   ProfileScope ps(nullptr, s, 0, 0, 0);
   launch(SgdOp{lr}, Ptrs<2>{{fp(param), fp(grad)}}, numel(param), s);
   return ps.finish();
@@ -591,7 +715,8 @@ int MomentumOptimizerUpdate(DLArrayHandle param, const DLArrayHandle grad, DLArr
   TS_REQUIRE(param && grad && velocity, "MomentumOptimizerUpdate: NULL array");
   SAME_SIZE(param, grad, "MomentumOptimizerUpdate");
   SAME_SIZE(param, velocity, "MomentumOptimizerUpdate");
-  hipStream_t s = stream_of(stream_handle);
+  hipStream_t s = stream_of_update(stream_handle);
+  if (numel(param) > 0 && pending_add(s, nesterov ? 2 : 1, lr, momentum, fp(param), fp(grad), fp(velocity), numel(param))) return 0;
   ProfileScope ps(nullptr, s, 0, 0, 0);
   Ptrs<3> a{{fp(param), fp(grad), fp(velocity)}};
   if (nesterov)

@@ -419,6 +419,7 @@ int DLStreamDestroy(DLStreamHandle handle) {
   if (!handle) return 0;
   hipStream_t *s = static_cast<hipStream_t *>(handle->handle);
   if (s) {
+    updates_flush_if_any();           // optimizer updates that waited on this stream run before it drains
     (void)hipStreamSynchronize(*s);
     conv_notes_drop_all();            // their sums lie in this stream's scratch
     multi_update_drop_stream(*s);
@@ -597,6 +598,9 @@ int DLArrayAllocSelf(DLArrayHandle handle, int MEMORY_MANAGE_RULE) {
 
 int DLArrayFree(DLArrayHandle handle, int MEMORY_MANAGE_RULE) {
   API_BEGIN();
+  // An optimizer update that waits may name this array.  Memory of the pool stays mapped and is next written by a
+  // call that runs the waiting updates first; memory that goes back to the driver must be done with now.
+  if (MEMORY_MANAGE_RULE == 0) updates_flush_if_any();
   if (handle) {
     void *d = handle->data;
     DLContext ctx = handle->ctx;
@@ -609,6 +613,7 @@ int DLArrayFree(DLArrayHandle handle, int MEMORY_MANAGE_RULE) {
 
 int DLArrayFreeSelf(DLArrayHandle handle, int MEMORY_MANAGE_RULE) {
   API_BEGIN();
+  if (MEMORY_MANAGE_RULE == 0) updates_flush_if_any();
   void *d = handle->data;
   handle->data = nullptr;
   data_free(handle->ctx, d, MEMORY_MANAGE_RULE);
@@ -632,6 +637,7 @@ int DLArrayCopyFromTo(DLArrayHandle from, DLArrayHandle to, DLStreamHandle strea
     TS_HIP(hipMemcpyAsync(to->data, from->data, bytes, kind, stream_of(stream)));
   } else {
     conv_notes_drop_all();            // (the branch above went through stream_of)
+    updates_flush_if_any();
     TS_HIP(hipMemcpy(to->data, from->data, bytes, kind));
   }
   return 0;
