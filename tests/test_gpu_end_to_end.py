@@ -3,7 +3,7 @@ Tolerance from the task statement: loss within 1e-3 relative over 20 steps."""
 import numpy as np
 import pytest
 
-from oracle import nets
+from oracle import nets, ops as O
 from util import assert_close
 
 pytestmark = pytest.mark.gpu
@@ -51,6 +51,7 @@ VGG_20_STEP_LR = 5e-7
 # distance is what the arithmetic predicts.
 YARDSTICK_FACTOR = 3.0
 YARDSTICK_FLOOR = 2e-3
+LAST_STEP_LOSS_BAR = 1e-4     # measured: 2e-6 on the direct kernels, 2e-5 through the Winograd routine
 
 
 def _small_convnet():
@@ -83,13 +84,17 @@ def test_convnet_momentum_tracks_oracle_with_and_without_split(split, fuse):
         assert_close(t.params[k].asnumpy(), ref_params[k], 2e-3, k)
 
 
-def _train_gpu(spec, params, X, Y, steps, opt, split=None, fuse=False):
+def _train_gpu(spec, params, X, Y, steps, opt, split=None, fuse=False, before_last=None):
+    """`before_last`: a dict that receives the parameters and velocities as they are before the last step."""
     from tsplit_amd import ndarray, trainer
     ctx = ndarray.gpu(0)
     t = trainer.Trainer(spec, params, X.shape, Y.shape[1], ctx, optimizer=opt, split=split, fuse_bn_relu=fuse)
     gx, gy = ndarray.array(X, ctx), ndarray.array(Y, ctx)
     losses = []
-    for _ in range(steps):
+    for i in range(steps):
+        if before_last is not None and i == steps - 1:
+            before_last["params"] = {k: v.asnumpy() for k, v in t.params.items()}
+            before_last["velocity"] = {k: v.asnumpy() for k, v in t.state.items()}
         t.step(gx, gy)
         losses.append(t.loss_value())
     return t, losses
@@ -129,10 +134,17 @@ def test_vgg16_topology_20_steps_tracks_oracle(winograd, monkeypatch):
     spec, params, ref_losses, ref_params = o["spec"], o["params"], o["ref_losses"], o["ref_params"]
     assert ref_losses[-1] < 0.5 * ref_losses[0], ref_losses       # the run does train
     conv_idx = [i for i, l in enumerate(spec) if l[0] == "conv"]
+    before = {}
     t, losses = _train_gpu(spec, params, o["X"], o["Y"], 20, ("momentum", VGG_20_STEP_LR, 0.9),
-                           split={i: 2 for i in conv_idx[:4]})
-    rel = np.max(np.abs(np.array(losses) - np.array(ref_losses)) / np.abs(ref_losses))
-    assert rel <= 1e-3, (rel, losses, ref_losses)
+                           split={i: 2 for i in conv_idx[:4]}, before_last=before)
+    rel = np.abs(np.array(losses) - np.array(ref_losses)) / np.abs(ref_losses)
+    assert np.max(rel) <= 1e-3, (rel, losses, ref_losses)
+    # This run amplifies whatever differs (the oracle's own float32 run leaves its float64 run by 2e-7 of the loss at
+    # the first step and by 2e-4 to 4e-4 at the last ones), so the last step is also held to the oracle without any
+    # history: its loss from the parameters the device itself had before it.
+    l_ref, _, _ = nets.forward_backward(spec, before["params"], o["X"], o["Y"], want_grads=False)
+    assert abs(losses[-1] - l_ref) <= LAST_STEP_LOSS_BAR * abs(l_ref), (losses[-1], l_ref)
+    assert losses[-1] < 0.5 * losses[0]
     for k in params:
         got = t.params[k].asnumpy()
         if np.any(params[k] != 0):                 # BatchNorm biases start at zero: their value IS the change

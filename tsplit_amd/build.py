@@ -75,6 +75,16 @@ def build(force=False, jobs=8, verbose=True):
                                capture_output=True, text=True)
             if r.returncode != 0:
                 raise RuntimeError(f"g++ failed on pool_capi.cpp:\n{r.stderr}")
+    # stand-alone measurement programs (csrc/probes/*.hip -> lib/<name>)
+    probes = os.path.join(CSRC, "probes")
+    for f in sorted(os.listdir(probes)) if os.path.isdir(probes) else []:
+        if not f.endswith(".hip"):
+            continue
+        exe, src = os.path.join(LIBDIR, f[:-4]), os.path.join(probes, f)
+        if force or not os.path.exists(exe) or os.path.getmtime(exe) < os.path.getmtime(src):
+            r = subprocess.run([HIPCC, *[x for x in FLAGS if x != "-fPIC"], "-Wno-unused-value", src, "-o", exe], capture_output=True, text=True)
+            if r.returncode != 0:
+                raise RuntimeError(f"hipcc failed on probes/{f}:\n{r.stdout}\n{r.stderr}")
     if verbose:
         print(f"built {LIB} ({sum(c for _, c in results)}/{len(srcs)} objects recompiled)")
     return LIB
