@@ -42,6 +42,8 @@ PEAK_HBM_GBS = 8000.0
 # single kernel; their HBM bytes per launch are read from the counter summary under profiles/.
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "vgg16_b64_train_step_hbm_traffic.txt")
 TRAFFIC_PROFILE_FUSED = os.path.join(ROOT, "profiles", "vgg16_b64_fused_bn_relu_train_step_hbm_traffic.txt")      # bench.py --fused
+TRAFFIC_PROFILE_SPLIT = os.path.join(ROOT, "profiles", "vgg16_b64_split_bf16_train_step_hbm_traffic.txt")          # --split-bf16
+TRAFFIC_PROFILE_FUSED_SPLIT = os.path.join(ROOT, "profiles", "vgg16_b64_fused_split_bf16_train_step_hbm_traffic.txt")
 TRAFFIC_KERNELS = {
     "conv_fwd_128x128": ("conv_tap_kernel<128, 128, 2, 2, false",),
     "conv_bwd_data_128x128": ("conv_tap_kernel<128, 128, 2, 2, true",),
@@ -53,6 +55,8 @@ TRAFFIC_KERNELS = {
     "winograd_gemm_64_rows": ("wino_gemm_kernel<64, 256>",),
     "winograd_fused": ("wino_fused_kernel<",),
     "winograd_filter_grad_fused": ("wino_fgrad_fused_kernel",),
+    "winograd_gemm_split_bf16": ("wino_gemm_split_kernel",),
+    "winograd_filter_grad_gemm_split_bf16": ("wino_grad_gemm_split_kernel<3>",),
 }
 
 
@@ -357,8 +361,10 @@ def main():
                            "achieved": dd["rate"], "peak": dom_peak,
                            "unit": "TFLOP/s" if dd["unit"] == "flop" else "GB/s",
                            "frac": dd["rate"] / dom_peak,
-                           "traffic": traffic_bytes_per_launch(dom, TRAFFIC_PROFILE_FUSED if a.fused else TRAFFIC_PROFILE)
-                           if split and a.batch == 64 and not a.split_bf16 else None,
+                           "traffic": traffic_bytes_per_launch(dom, {(False, False): TRAFFIC_PROFILE, (True, False): TRAFFIC_PROFILE_FUSED,
+                                                                     (False, True): TRAFFIC_PROFILE_SPLIT,
+                                                                     (True, True): TRAFFIC_PROFILE_FUSED_SPLIT}[(a.fused, a.split_bf16)])
+                           if split and a.batch == 64 else None,
                            "per_launch": dd["work_per_call"], "ms_avg": dd["ms_avg"],
                            # which pass the launch durations behind `achieved` come from: the timed region carries event
                            # pairs only for the kernel expected to be the largest; if another one turns out larger (other
