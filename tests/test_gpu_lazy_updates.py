@@ -130,3 +130,22 @@ def test_another_stream_sees_the_update_behind_an_event(ts):
     # the default stream (no handle)
     ts.L.sgd_update(p, g, 0.5, None)
     np.testing.assert_array_equal(p.asnumpy(), (p0 - np.float32(0.5) * g0) - np.float32(0.5) * g0)
+
+
+def test_lists_that_change_from_call_to_call(ts):
+    """Two sets of parameters updated in turn, and lists of a different length every time: the table of arrays the
+    one launch reads is uploaded again each time, through staging buffers that take turns."""
+    rng = np.random.RandomState(7)
+    sizes = [4, 1000, 4096, 33000, 64, 12, 70000, 256]
+    host = [(rng.normal(size=n).astype(np.float32), rng.normal(size=n).astype(np.float32)) for n in sizes]
+    dev = [(ts.arr(p), ts.arr(g)) for p, g in host]
+    want = [p.copy() for p, _ in host]
+    lr = np.float32(0.125)
+    for round_ in range(12):
+        chosen = [i for i in range(len(sizes)) if (i + round_) % 2 == 0][:2 + round_ % 3]
+        for i in chosen:
+            ts.L.sgd_update(dev[i][0], dev[i][1], float(lr), ts.stream)
+            want[i] = want[i] - lr * host[i][1]
+        ts.L.array_set(ts.arr(np.zeros(4, np.float32)), 1.0, ts.stream)      # any other call: the list runs
+    for (p, _), w in zip(dev, want):
+        np.testing.assert_array_equal(p.asnumpy(), w)

@@ -318,20 +318,26 @@ __global__ __launch_bounds__(kThreads) void ew_multi_kernel(Op op, const MultiTe
 struct MultiTable {
   std::vector<char> host;          // the table as last uploaded
   char *dev = nullptr;             // the device buffer it was uploaded into
-  char *pinned = nullptr;          // staging buffer the asynchronous copy reads
-  size_t pinned_bytes = 0;
-  hipEvent_t uploaded = nullptr;   // recorded behind the last upload
+  // two staging buffers the asynchronous copies read in turn, each with an event recorded behind its last upload:
+  // the host waits only for the upload before the last one (lists that change from call to call would
+  // otherwise tie the host to the stream)
+  char *pinned[2] = {nullptr, nullptr};
+  size_t pinned_bytes[2] = {0, 0};
+  hipEvent_t uploaded[2] = {nullptr, nullptr};
+  int turn = 0;
   bool in_graph = false;           // a recorded step launches with this table at `dev`
 };
 std::mutex g_multi_mu;
 std::map<hipStream_t, MultiTable> g_multi;
 
 void multi_table_release(MultiTable &mt) {
-  if (mt.uploaded) {
-    (void)hipEventSynchronize(mt.uploaded);
-    (void)hipEventDestroy(mt.uploaded);
+  for (int i = 0; i < 2; ++i) {
+    if (mt.uploaded[i]) {
+      (void)hipEventSynchronize(mt.uploaded[i]);
+      (void)hipEventDestroy(mt.uploaded[i]);
+    }
+    if (mt.pinned[i]) (void)hipHostFree(mt.pinned[i]);
   }
-  if (mt.pinned) (void)hipHostFree(mt.pinned);
   mt = MultiTable{};
 }
 
@@ -414,20 +420,22 @@ int launch_multi(Op op, const std::vector<std::array<float *, Op::N>> &arrays, c
     MultiTable &mt = g_multi[s];
     if (mt.dev != dev || mt.host != table) {
       TS_REQUIRE(!recording, "%s: the list of arrays changed while a step is being recorded; run the step once before recording it", who);
-      if (mt.uploaded) TS_HIP(hipEventSynchronize(mt.uploaded));   // the staging buffer is free again
-      if (mt.pinned_bytes < table.size()) {
-        if (mt.pinned) (void)hipHostFree(mt.pinned);
-        mt.pinned = nullptr;
-        mt.pinned_bytes = 0;
+      const int b = mt.turn;
+      mt.turn ^= 1;
+      if (mt.uploaded[b]) TS_HIP(hipEventSynchronize(mt.uploaded[b]));   // this staging buffer is free again
+      if (mt.pinned_bytes[b] < table.size()) {
+        if (mt.pinned[b]) (void)hipHostFree(mt.pinned[b]);
+        mt.pinned[b] = nullptr;
+        mt.pinned_bytes[b] = 0;
         const size_t want = (table.size() + 4095) / 4096 * 4096;
-        TS_HIP(hipHostMalloc(reinterpret_cast<void **>(&mt.pinned), want, hipHostMallocDefault));
-        mt.pinned_bytes = want;
+        TS_HIP(hipHostMalloc(reinterpret_cast<void **>(&mt.pinned[b]), want, hipHostMallocDefault));
+        mt.pinned_bytes[b] = want;
       }
-      if (!mt.uploaded) TS_HIP(hipEventCreateWithFlags(&mt.uploaded, hipEventDisableTiming));
-      std::memcpy(mt.pinned, table.data(), table.size());
+      if (!mt.uploaded[b]) TS_HIP(hipEventCreateWithFlags(&mt.uploaded[b], hipEventDisableTiming));
+      std::memcpy(mt.pinned[b], table.data(), table.size());
       mt.dev = nullptr;   // until the copy below is queued nothing valid lies there
-      TS_HIP(hipMemcpyAsync(dev, mt.pinned, table.size(), hipMemcpyHostToDevice, s));
-      TS_HIP(hipEventRecord(mt.uploaded, s));
+      TS_HIP(hipMemcpyAsync(dev, mt.pinned[b], table.size(), hipMemcpyHostToDevice, s));
+      TS_HIP(hipEventRecord(mt.uploaded[b], s));
       mt.host = table;
       mt.dev = dev;
       mt.in_graph = false;
