@@ -55,6 +55,18 @@ def test_pooling_and_convolution_on_an_empty_batch():
     dw = nd.array(np.full((32, 16, 3, 3), 7.0, np.float32), ctx)
     L.CuDNN_conv2d_gradient_of_filter(x, out, dw, 1, 1, 1)
     assert not dw.asnumpy().any()
+    # every route of the dispatcher: a first layer on 3 channels (1x1 stride 2 and 3x3), a 1x1 and a strided layer on
+    # many channels, a channel count that is no multiple of 16, a layer the Winograd routine would take
+    for (C, O, k, pad, s, H) in [(3, 24, 1, 0, 2, 12), (3, 64, 3, 1, 1, 16), (64, 256, 1, 0, 1, 8), (32, 48, 3, 1, 2, 9),
+                                 (20, 10, 5, 2, 1, 7), (64, 64, 3, 1, 1, 64)]:
+        oH = (H + 2 * pad - k) // s + 1
+        x, y, dx = e(0, C, H, H), e(0, O, oH, oH), e(0, C, H, H)
+        w = nd.array(np.ones((O, C, k, k), np.float32), ctx)
+        dw = nd.array(np.full((O, C, k, k), 7.0, np.float32), ctx)
+        L.CuDNN_conv2d(x, w, y, pad, pad, s)
+        L.CuDNN_conv2d_gradient_of_data(w, y, dx, pad, pad, s)
+        L.CuDNN_conv2d_gradient_of_filter(x, y, dw, pad, pad, s)
+        assert not dw.asnumpy().any(), (C, O, k, pad, s, H)
 
 
 def test_matrix_products_with_an_empty_dimension():

@@ -2519,7 +2519,11 @@ int conv_bwd_filter(const char *who, const DLArray *x, const DLArray *dy, DLArra
   int64_t ws = 0;
   ProfileScope ps(p, st, numel(x) + numel(dy), numel(dw), 0);
   int rc = 0;
-  if (numel(dw) > 0) {
+  if (numel(dw) > 0 && (numel(x) == 0 || numel(dy) == 0)) {
+    // a sum over no positions (an empty batch: the last of more micro-tensors than there are images)
+    const int64_t n = numel(dw);
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, mf(dw), n);
+  } else if (numel(dw) > 0) {
     if (wgrad_narrow_ok(g)) {
       rc = launch_wgrad_narrow(g, cf(x), cf(dy), mf(dw), st, &ws);
     } else if (winograd_filter_grad_pays(g)) {
